@@ -1,0 +1,188 @@
+/* C ABI of libviola_hip.so: hand-written HIP kernels for gfx950 (MI355X) behind the
+ * Python operator seam of chinoll/viola's low-precision hot path.
+ *
+ * The reference has no FFI layer; its seam is a set of Python wrapper functions that
+ * take torch tensors and launch one TileLang kernel each. Every entry point below
+ * replaces one of those wrappers (cited as path:line under the reference tree).
+ *
+ * Conventions
+ *   - plain pointers and sizes only; all pointers are device pointers unless noted;
+ *   - the library never allocates or frees device memory and never synchronises:
+ *     each call enqueues kernels on `stream` (a hipStream_t) and returns;
+ *   - a null pointer means "absent" (no bias, no aux, no source scale ...);
+ *   - return 0 on success, VIOLA_EINVAL / VIOLA_EUNSUPPORTED for rejected arguments
+ *     (nothing was launched), or a positive hipError_t from the launch;
+ *   - matrices are row-major and contiguous unless a stride is passed.
+ */
+#ifndef VIOLA_HIP_H
+#define VIOLA_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* viola_stream_t; /* hipStream_t */
+
+enum { VIOLA_F32 = 0, VIOLA_BF16 = 1, VIOLA_F16 = 2, VIOLA_E4M3 = 3, VIOLA_E5M2 = 4 };
+enum { VIOLA_SILU = 0, VIOLA_GELU = 1, VIOLA_RELU = 2 };
+enum { VIOLA_NEAREST = 0, VIOLA_STOCHASTIC = 1 };
+enum { VIOLA_EINVAL = -1, VIOLA_EUNSUPPORTED = -2 };
+
+int viola_abi_version(void);
+const char* viola_error_string(int code);
+
+/* ---------------------------------------------------------------- group quantization
+ * viola/nn/_grouped_kernels.py:127-158 `quantize` (encode_kernel :53-92,
+ * transpose_encode_kernel :95-124).
+ * x is [rows, cols] of x_dtype (f32/bf16/f16, or fp8 codes when source_scale is given:
+ * then value = code * source_scale[r / source_gr, c / source_gc]). With transposed = 0
+ * the output q is [rows, cols] and scale is [ceil(rows/gr), ceil(cols/gc)]; with
+ * transposed = 1 the output is the quantized transpose, q [cols, rows] and scale
+ * [ceil(cols/gr), ceil(rows/gc)], groups laid along the new last dimension.
+ * Per group: s = max(amax, 1e-30) / limit; q = fp8(isnan(v/s) ? NaN : clamp(v/s, +-limit)). */
+int viola_group_quantize(const void* x, int x_dtype, int64_t rows, int64_t cols,
+                         void* q, int q_dtype, float* scale, int gr, int gc, float limit, int transposed,
+                         const float* source_scale, int source_gr, int source_gc, viola_stream_t stream);
+
+/* One read pass that emits both layouts of a row-major matrix with 1-D groups: the row-wise
+ * codes/scales (q [rows, cols], scale [rows, ceil(cols/gc)]) and the quantized transpose
+ * (qt [cols, rows], scale_t [cols, ceil(rows/gc)]). Same arithmetic per group as two calls of
+ * viola_group_quantize (viola/nn/_grouped_linear.py:21,46-47 and :73,92 make those two calls). */
+int viola_group_quantize_dual(const void* x, int x_dtype, int64_t rows, int64_t cols,
+                              void* q, float* scale, void* qt, float* scale_t, int q_dtype, int gc,
+                              float limit, viola_stream_t stream);
+
+/* viola/nn/_grouped_kernels.py:44-50 `dequantize` (decode_kernel :24-41): out = f32(q) * scale[r/gr, c/gc]. */
+int viola_group_dequantize(const void* q, int q_dtype, const float* scale, int64_t rows, int64_t cols,
+                           int gr, int gc, float* out, viola_stream_t stream);
+
+/* viola/nn/_linear_kernels.py:107-121,253-257 `transpose`: byte-matrix transpose, out [cols, rows]. */
+int viola_fp8_transpose(const void* x, void* out, int64_t rows, int64_t cols, viola_stream_t stream);
+
+/* ---------------------------------------------------------------- grouped-scale FP8 GEMM
+ * viola/nn/_grouped_kernels.py:310-328 `gemm` (gemm_kernel :195-293).
+ * out[m, n] = sum over 32-wide K groups kg of (sum_{k in kg} a[m,k]*b[n,k]) * sa[m/ar, k/ak] * sb[n/br, k/bk]
+ *             (+ bias[n]);  a is [m, k], b is [n, k] ("NT"), both FP8 codes; ak and bk are multiples of 32. */
+int viola_group_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,
+                     int64_t m, int64_t n, int64_t k, int ar, int ak, int br, int bk,
+                     const void* bias, int bias_dtype, void* out, int out_dtype, viola_stream_t stream);
+
+/* viola/nn/_mlp_kernels.py:243-277 `gemm` (kernel :16-231), grouped FP32-scale path.
+ * forward (backward = 0): b is [2h, k]; g = a.b[0:h]^T, u = a.b[h:2h]^T (+bias), each rounded to
+ *   out_dtype; aux[m, 0:h] = g, aux[m, h:2h] = u when aux != NULL; out[m, h] = act(g) * u.
+ * backward (backward = 1): b is [h, k]; d = round(a.b^T); g, u read from aux [m, 2h];
+ *   out[m, 0:h] = d*u*act'(g), out[m, h:2h] = d*act(g). aux and out share out_dtype. */
+int viola_gated_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,
+                     int64_t m, int64_t h, int64_t k, int ar, int ak, int br, int bk,
+                     const void* bias, int bias_dtype, void* aux, void* out, int out_dtype,
+                     int activation, int backward, viola_stream_t stream);
+
+/* Variable-group (MoE-expert style) GEMM: `groups` independent problems that share n and k and
+ * differ in their row range. Group g owns rows [offsets[g], offsets[g+1]) of a and out
+ * (offsets: groups+1 int64 on the device, ascending) and operand b + g*b_group_stride (elements),
+ * sb + g*sb_group_stride (floats). Same arithmetic per group as viola_group_gemm. The reference
+ * has no such kernel (its "grouped" is group-scaled quantization); this serves the
+ * variable-group linear named by the build's target workload. m_total bounds the grid. */
+int viola_varlen_group_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,
+                            const int64_t* offsets, int groups, int64_t m_total, int64_t n, int64_t k,
+                            int ar, int ak, int br, int bk, int64_t b_group_stride, int64_t sb_group_stride,
+                            void* out, int out_dtype, viola_stream_t stream);
+
+/* Variable-group weight gradient: for each group g, out[g] ([n, kout]) = sum over the group's
+ * tokens of at[:, t] * bt[:, t], with at [n, t_total] and bt [kout, t_total] the quantized
+ * transposes whose 32-token scale groups start at each group's own padded offset:
+ * group g owns token columns [poffsets[g], poffsets[g+1]) (multiples of 32, zero codes in the
+ * padding); sat [n, t_total/32], sbt [kout, t_total/32]. */
+int viola_varlen_wgrad_gemm(const void* at, int a_dtype, const void* bt, int b_dtype, const float* sat, const float* sbt,
+                            const int64_t* poffsets, int groups, int64_t t_total, int64_t n, int64_t kout,
+                            void* out, int out_dtype, viola_stream_t stream);
+
+/* Segmented transposed quantize for the variable-group path: x [rows, cols] row-major; group g owns
+ * rows [offsets[g], offsets[g+1]) and writes its quantized transpose into token columns
+ * [poffsets[g], poffsets[g+1]) of qt [cols, t_total] (scale_t [cols, t_total/32]), 32-token groups
+ * counted from the group's own first row; padding columns get zero codes and scale 1e-30/limit. */
+int viola_varlen_quantize_transposed(const void* x, int x_dtype, int64_t rows, int64_t cols,
+                                     const int64_t* offsets, const int64_t* poffsets, int groups, int64_t t_total,
+                                     void* qt, float* scale_t, int q_dtype, float limit, viola_stream_t stream);
+
+/* ---------------------------------------------------------------- gated activations (elementwise)
+ * viola/nn/_gated_kernels.py:16-36 forward_kernel: out[r, c] = act(z[r, c]) * z[r, c + h].
+ * viola/nn/_gated_kernels.py:39-67 backward_kernel: dz = [dy*u*act'(g), dy*act(g)]. */
+int viola_gated_forward(const void* z, void* out, int64_t rows, int64_t h, int dtype, int activation, viola_stream_t stream);
+int viola_gated_backward(const void* z, const void* dy, void* dz, int64_t rows, int64_t h, int dtype, int activation,
+                         viola_stream_t stream);
+
+/* ---------------------------------------------------------------- FP8Muon kernels
+ * viola/optim/_kernels.py:300-315 `momentum_update` (_momentum_1d_kernel :88-144,
+ * _momentum_2d_kernel :147-200). granularity 0: 1-D tiles of tile_size over the flat tensor
+ * (q padded to whole tiles); granularity 1: tr x tc blocks over [planes, rows, cols] (unpadded).
+ * old_q/new_q and old_scale/new_scale may alias. Pointers need only element alignment. */
+int viola_momentum_update(const void* grad, int grad_dtype, const void* old_q, const float* old_scale,
+                          void* new_q, float* new_scale, void* update /* bf16 */,
+                          int64_t n, float beta, float inv_loss_scale, int nesterov,
+                          int granularity, int tile_size, int64_t planes, int64_t rows, int64_t cols, int tr, int tc,
+                          int rounding, int64_t rounding_step, int64_t rounding_key, viola_stream_t stream);
+
+/* viola/optim/_kernels.py:325-328 `weight_update` (_weight_kernel :227-255). */
+int viola_weight_update(void* weight, int weight_dtype, const void* grad, int grad_dtype, int64_t n,
+                        float lr, float decay, float update_scale, int rounding, int64_t rounding_step,
+                        int64_t rounding_key, int64_t offset, viola_stream_t stream);
+
+/* viola/optim/_kernels.py:331-337 `adam_update` (_adam_kernel :258-293); inv_c1/inv_c2 are the
+ * host-computed bias corrections; rounding_step is step - 1. */
+int viola_adam_update(void* weight, int weight_dtype, const void* grad, int grad_dtype,
+                      void* first, void* second, int state_dtype, int64_t n,
+                      float lr, float decay, float b1, float b2, float inv_c1, float inv_c2, float eps,
+                      int rounding, int64_t rounding_step, int64_t rounding_key, int64_t offset,
+                      int adamw, int maximize, viola_stream_t stream);
+
+/* viola/optim/_kernels.py:318-322 `copy_scaled` (_copy_scaled_kernel :203-222). */
+int viola_copy_scaled(const void* update, int update_dtype, void* out, int out_dtype,
+                      int64_t src, int64_t dst, int64_t count, float scale, viola_stream_t stream);
+
+/* viola/optim/_kernels.py:73-83 `dequantize` (diagnostic): e4m3 payload * per-tile scale -> fp32 [n]. */
+int viola_momentum_dequantize(const void* q, const float* scale, float* out, int64_t n,
+                              int granularity, int tile_size, int64_t planes, int64_t rows, int64_t cols, int tr, int tc,
+                              viola_stream_t stream);
+
+/* ---------------------------------------------------------------- Newton-Schulz GEMM chain
+ * viola/optim/_orthogonalize_kernels.py:53-66 `_matmul` (matmul_kernel :16-50): batched
+ * out[b] = a[b] . (transpose_b ? bmat[b]^T : bmat[b]) with fp32 accumulation, rounded to dtype,
+ * then epilogue 0: nothing; 1: -4.7750*residual + 2.0315*value; 2: value + 3.4445*residual; rounded
+ * to dtype. a [batch, m, k]; bmat [batch, n, k] if transpose_b else [batch, k, n]; dtype bf16 or f16.
+ * out_diag (nullable) receives a second copy of the result with add_diag added to its diagonal after
+ * rounding (Q = Z + 3.4445 I, viola/optim/_orthogonalize.py:45-47). */
+int viola_ns_gemm(const void* a, const void* bmat, const void* residual, void* out, int dtype,
+                  int transpose_b, int epilogue, int64_t batch, int64_t m, int64_t n, int64_t k,
+                  float add_diag, void* out_diag, viola_stream_t stream);
+
+/* viola/optim/_orthogonalize.py:12-16 / _orthogonalize_kernels.py:80-84: x = dtype(matrix), optionally
+ * transposed so rows <= cols, divided by (Frobenius norm + 1e-7), all in the working dtype.
+ * in [batch, rows, cols] of in_dtype; out [batch, min, max] of dtype; workspace: batch floats. */
+int viola_ns_prepare(const void* in, int in_dtype, void* out, int dtype, int64_t batch, int64_t rows, int64_t cols,
+                     float* workspace, viola_stream_t stream);
+
+/* ---------------------------------------------------------------- FP8 gradient wire codec
+ * viola/distributed/_fp8_kernels.py:84-87 `pack` (_pack :18-43) and :90-93 `unpack` (_unpack :46-69).
+ * packet: rows x stride bytes, stride = ceil16(groups*(tile+4)): per row groups*tile codes, then
+ * groups fp32 scales. pack reads x[n] fp32 at index row*groups*tile + group*tile + i (0 past n).
+ * unpack writes out[n]; with reduce != 0 it sums the rows into out[0 : groups*tile]. */
+int viola_comm_pack(const float* x, int64_t n, void* packet, int64_t rows, int64_t groups, int tile, int fp8_dtype,
+                    viola_stream_t stream);
+int viola_comm_unpack(const void* packet, float* out, int64_t n, int64_t rows, int64_t groups, int tile, int fp8_dtype,
+                      int reduce, viola_stream_t stream);
+
+/* ---------------------------------------------------------------- self checks (test support)
+ * Compare the hardware FP8 conversion instructions with the software codecs over every fp32 bit
+ * pattern of magnitude <= the format's clamp range (encode) and all 256 codes (decode); writes
+ * mismatch counts to counts[4] (device): {e4m3 encode, e5m2 encode, e4m3 decode, e5m2 decode}. */
+int viola_selftest_fp8(uint64_t* counts, viola_stream_t stream);
+/* philox(element, step, key) word 0 for `count` triples (device arrays) -> out. */
+int viola_selftest_philox(const uint64_t* triples, uint32_t* out, int64_t count, viola_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VIOLA_HIP_H */

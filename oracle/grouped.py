@@ -1,0 +1,90 @@
+"""Group-scaled FP8 quantization and GEMM on CPU tensors. TEST INFRASTRUCTURE ONLY.
+
+Restates the reference's group quantizer and the "dequantize then FP32 matmul"
+recipe its checks use as the expected value.
+"""
+
+import torch
+import torch.nn.functional as F
+
+FP8 = {"e4m3": torch.float8_e4m3fn, "e5m2": torch.float8_e5m2}
+
+
+def scale_shape(shape, group):
+    """ceil(n / g) per dimension (viola/nn/_grouped_kernels.py:16-17)."""
+    return tuple((n + g - 1) // g for n, g in zip(shape, group))
+
+
+def dequantize(q, scale, group):
+    """float(q) * scale[r // gr, c // gc]  (viola/nn/_grouped_kernels.py:37-40,49-50)."""
+    expanded = scale.float().repeat_interleave(group[0], 0).repeat_interleave(group[1], 1)
+    return q.float() * expanded[:q.shape[0], :q.shape[1]]
+
+
+def quantize(x, dtype, group, *, limit=None, transposed=False, source_scale=None, source_group=(1, 32)):
+    """Group amax quantization (viola/nn/_grouped_kernels.py:127-158).
+
+    Follows the CPU branch at :135-151 (pad -> reshape (nr, gr, nc, gc) -> amax ->
+    clamp_min(1e-30) / limit -> divide -> clamp -> cast), except for NaN inside a
+    group, where the device kernel's behaviour is restated instead
+    (encode_kernel :69-91): the abs-max reduction ignores NaN, so only the NaN
+    element itself becomes a NaN code. Every step is an IEEE fp32 operation.
+    """
+    limit = torch.finfo(dtype).max if limit is None else limit
+    value = dequantize(x, source_scale, source_group) if source_scale is not None else x.float()
+    value = value.T if transposed else value
+    shape = tuple(value.shape)
+    gr, gc = group
+    nr, nc = scale_shape(shape, group)
+    blocks = F.pad(value, (0, nc * gc - shape[1], 0, nr * gr - shape[0])).reshape(nr, gr, nc, gc)
+    magnitude = torch.where(blocks.isnan(), torch.zeros_like(blocks), blocks.abs())
+    scales = magnitude.amax((1, 3)).clamp_min(1e-30) / limit
+    codes = (blocks / scales[:, None, :, None]).clamp(-limit, limit)      # clamp keeps NaN
+    q = codes.reshape(nr * gr, nc * gc)[:shape[0], :shape[1]].to(dtype)
+    return q.contiguous(), scales.contiguous()
+
+
+def transpose_group(group):
+    """2-D blocks transpose exactly; 1-D row groups keep their shape (:161-163)."""
+    return group[::-1] if group[0] >= 32 else group
+
+
+def transpose(q, scale, group, *, limit=None):
+    """Byte transpose + scale.T for 2-D blocks, otherwise re-encode (:166-171)."""
+    if group[0] >= 32:
+        return q.T.contiguous(), scale.T.contiguous()
+    return quantize(q, q.dtype, group, limit=limit, transposed=True, source_scale=scale, source_group=group)
+
+
+def gemm(a, b, sa, sb, group_a, group_b, *, out_dtype=torch.float32, bias=None, witness=False):
+    """(deq(a) @ deq(b).T + bias) -> out dtype (checks/check_grouped_linear.py:32,39).
+
+    witness=True evaluates the same sum in fp64 (the reference's FP64 witness,
+    viola/nn/_grouped_tuning.py:40-46).
+    """
+    da, db = dequantize(a, sa, group_a), dequantize(b, sb, group_b)
+    if witness:
+        da, db = da.double(), db.double()
+    out = da @ db.T
+    if bias is not None:
+        out = out + bias.to(out.dtype)
+    return out.to(out_dtype)
+
+
+def gemm_kgroup_order(a, b, sa, sb, group_a, group_b, *, bias=None):
+    """The device kernel's own summation order: per 32-wide K group, the raw code
+    product is formed first and then scaled, total += (acc*sa)*sb, K groups in
+    ascending order (viola/nn/_grouped_kernels.py:268-292). Used to show that the
+    order does not matter beyond fp32 rounding."""
+    m, k = a.shape
+    n = b.shape[0]
+    total = torch.zeros(m, n)
+    af, bf = a.float(), b.float()
+    rows = torch.arange(m) // group_a[0]
+    cols = torch.arange(n) // group_b[0]
+    for k0 in range(0, k, 32):
+        acc = af[:, k0:k0 + 32] @ bf[:, k0:k0 + 32].T
+        total = total + (acc * sa[rows, k0 // group_a[1]][:, None]) * sb[cols, k0 // group_b[1]][None, :]
+    if bias is not None:
+        total = total + bias.float()
+    return total

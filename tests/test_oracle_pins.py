@@ -1,0 +1,340 @@
+"""Pins for the CPU oracle itself: every check here is something the oracle's own formula does not
+decide (golden vectors held by the reference, an independent implementation, a closed form, an
+invariant), so that a dropped term / wrong index / wrong sign in the oracle fails. No GPU."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import comm, fp8, grouped, linear, ns, optim
+from conftest import rel_l2
+
+E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
+
+
+# ----------------------------------------------------------------------------- FP8 casts
+@pytest.mark.parametrize("name,dtype", [("e4m3", E4), ("e5m2", E5)])
+def test_decode_table_matches_torch(name, dtype):
+    table = fp8.decode_table(name)
+    ours = torch.from_numpy(table)
+    theirs = torch.arange(256, dtype=torch.uint8).view(dtype).float()
+    assert torch.equal(ours.isnan(), theirs.isnan())
+    assert torch.equal(ours.nan_to_num(7.0), theirs.nan_to_num(7.0))
+
+
+@pytest.mark.parametrize("name,dtype", [("e4m3", E4), ("e5m2", E5)])
+def test_torch_cast_is_rne_on_the_grid(name, dtype):
+    """torch's CPU cast (what the reference's CPU oracles call) == exact nearest-even search."""
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(200000, generator=g) * torch.exp2(torch.randint(-20, 18, (200000,), generator=g).float())
+    table = torch.from_numpy(fp8.decode_table(name))
+    finite = table[table.isfinite()]
+    mids = (finite.sort().values[:-1] + finite.sort().values[1:]) / 2             # every tie point
+    special = torch.tensor([0.0, -0.0, 447.9, 448.0, 463.9, 464.0, 464.1, 479.9, 480.0, 500.0, 57344.0, 61439.0,
+                            61440.0, 65536.0, 1e30, -1e30, float("inf"), -float("inf"), float("nan"), 2.0 ** -10,
+                            2.0 ** -9, 1.5 * 2.0 ** -10, 2.0 ** -17, 2.0 ** -16, 3 * 2.0 ** -17])
+    x = torch.cat([x, finite, mids, torch.nextafter(mids, mids + 1), torch.nextafter(mids, mids - 1), special])
+    ours = torch.from_numpy(fp8.encode(x.numpy(), name))
+    theirs = x.to(dtype).view(torch.uint8)
+    nan_ours = torch.from_numpy(np.isnan(fp8.decode_table(name)))[ours.long()]
+    nan_theirs = torch.from_numpy(np.isnan(fp8.decode_table(name)))[theirs.long()]
+    assert torch.equal(nan_ours, nan_theirs)
+    keep = ~nan_ours
+    assert torch.equal(ours[keep], theirs[keep])
+
+
+def test_cast_cases_the_quantizers_rely_on():
+    x = torch.tensor([447.9, 448.0, 464.0, float("nan"), -float("nan")])
+    codes = x.to(E4).view(torch.uint8)
+    assert codes[:3].tolist() == [0x7E, 0x7E, 0x7E] and (codes[3] & 0x7F) == 0x7F
+    assert torch.tensor([500.0]).clamp(-448, 448).to(E4).view(torch.uint8).item() == 0x7E
+    assert torch.tensor([float("nan")]).clamp(-448, 448).isnan().item()          # clamp keeps NaN
+
+
+# ----------------------------------------------------------------------------- group quantize
+@pytest.mark.parametrize("dtype", [E4, E5])
+@pytest.mark.parametrize("group,shape", [((1, 32), (65, 96)), ((32, 32), (96, 70)), ((1, 64), (33, 130)), ((32, 64), (64, 160))])
+def test_quantize_invariants(dtype, group, shape):
+    torch.manual_seed(1)
+    x = (torch.randn(*shape) * torch.exp2(torch.randint(-5, 6, (shape[0], 1)).float())).bfloat16()
+    q, s = grouped.quantize(x, dtype, group)
+    assert q.shape == x.shape and tuple(s.shape) == grouped.scale_shape(shape, group)
+    limit = torch.finfo(dtype).max
+    # the largest element of each group maps to +-limit and the scale is amax/limit exactly
+    gr, gc = group
+    pad = F.pad(x.float(), (0, s.shape[1] * gc - shape[1], 0, s.shape[0] * gr - shape[0]))
+    amax = pad.reshape(s.shape[0], gr, s.shape[1], gc).abs().amax((1, 3))
+    assert torch.equal(s, amax.clamp_min(1e-30) / limit)
+    qpad = F.pad(q.float(), (0, s.shape[1] * gc - shape[1], 0, s.shape[0] * gr - shape[0]))
+    assert torch.equal(qpad.reshape(s.shape[0], gr, s.shape[1], gc).abs().amax((1, 3))[amax > 0],
+                       torch.full_like(amax, limit)[amax > 0])
+    # element-wise against a scalar loop on a sample of positions (independent indexing)
+    table = fp8.decode_table("e4m3" if dtype == E4 else "e5m2")
+    for r, c in [(0, 0), (shape[0] - 1, shape[1] - 1), (shape[0] // 2, shape[1] // 3), (1, shape[1] - 1)]:
+        sc = s[r // gr, c // gc].item()
+        v = np.float32(x[r, c].float().item()) / np.float32(sc)
+        expect = fp8.encode(np.clip(np.array([v], dtype=np.float32), -limit, limit), "e4m3" if dtype == E4 else "e5m2")[0]
+        assert q.view(torch.uint8)[r, c].item() == expect
+    # quantization error bound: half a grid step at the element's magnitude
+    deq = grouped.dequantize(q, s, group)
+    mant = 3 if dtype == E4 else 2
+    assert rel_l2(deq, x.float()) < 2.0 ** -(mant + 1)
+
+
+def test_quantize_exact_roundtrip_and_transpose():
+    """Representable values times a power-of-two scale come back exactly; transposed == quantize(x.T)."""
+    torch.manual_seed(2)
+    codes = torch.randint(0, 0x7F, (64, 64), dtype=torch.uint8)
+    codes[::32, ::32] = 0x7E                                   # every (32,32) block and (1,32) row tile holds 448
+    codes[:, ::32] = 0x7E
+    value = codes.view(E4).float() * 0.25
+    for group in ((1, 32), (32, 32)):
+        q, s = grouped.quantize(value, E4, group)
+        assert torch.equal(grouped.dequantize(q, s, group), value)
+    x = torch.randn(70, 45).bfloat16()
+    qt, st = grouped.quantize(x, E4, (1, 32), transposed=True)
+    q2, s2 = grouped.quantize(x.T.contiguous(), E4, (1, 32))
+    assert torch.equal(qt.view(torch.uint8), q2.view(torch.uint8)) and torch.equal(st, s2)
+    assert qt.shape == (45, 70) and st.shape == (45, 3)
+
+
+def test_quantize_nan_inf_follow_the_device_kernel():
+    x = torch.ones(2, 64)
+    x[0, 3], x[1, 40] = float("nan"), float("inf")
+    q, s = grouped.quantize(x, E4, (1, 32))
+    d = q.float()
+    assert d[0, 3].isnan() and d[0, :3].eq(448).all() and s[0, 0] == 1 / 448     # NaN stays local
+    assert s[1, 1].isinf() and d[1, 40].isnan() and d[1, 33] == 0                  # inf/inf = NaN, finite/inf = 0
+
+
+def test_reencode_and_transpose_rules():
+    torch.manual_seed(3)
+    w = torch.randn(64, 96)
+    q, s = grouped.quantize(w, E4, (32, 32))
+    qt, st = grouped.transpose(q, s, (32, 32))
+    assert torch.equal(grouped.dequantize(qt, st, (32, 32)), grouped.dequantize(q, s, (32, 32)).T)
+    q1, s1 = grouped.quantize(w, E4, (1, 32))
+    qt1, st1 = grouped.transpose(q1, s1, (1, 32))               # 1-D groups must be re-encoded
+    again, sa = grouped.quantize(grouped.dequantize(q1, s1, (1, 32)), E4, (1, 32), transposed=True)
+    assert torch.equal(qt1.view(torch.uint8), again.view(torch.uint8)) and torch.equal(st1, sa)
+
+
+# ----------------------------------------------------------------------------- grouped GEMM
+@pytest.mark.parametrize("ga,gb,fa,fb,shape", [((1, 32), (32, 32), E4, E4, (65, 96, 128)), ((1, 64), (32, 64), E5, E4, (96, 65, 64)),
+                                                ((32, 64), (64, 32), E4, E5, (64, 160, 96))])
+def test_gemm_oracle_vs_fp64_and_kernel_order(ga, gb, fa, fb, shape):
+    """fp32 dequantize-matmul == fp64 witness == the device kernel's per-K-group order, to fp32 rounding."""
+    m, k, n = shape
+    torch.manual_seed(2041)
+    a = (torch.randn(m, k) * torch.exp2(torch.randint(-5, 6, (m, 1)).float())).bfloat16()
+    b = (torch.randn(n, k) * torch.exp2(torch.randint(-5, 6, (n, 1)).float())).bfloat16()
+    qa, sa = grouped.quantize(a, fa, ga)
+    qb, sb = grouped.quantize(b, fb, gb)
+    bias = torch.randn(n)
+    plain = grouped.gemm(qa, qb, sa, sb, ga, gb, bias=bias)
+    witness = grouped.gemm(qa, qb, sa, sb, ga, gb, bias=bias, witness=True, out_dtype=torch.float64)
+    ordered = grouped.gemm_kgroup_order(qa, qb, sa, sb, ga, gb, bias=bias) if ga[1] % 32 == 0 and k % 32 == 0 else plain
+    assert rel_l2(plain, witness) < 2e-6 and rel_l2(ordered, witness) < 2e-6
+    # brute force on a few entries, written with scalar indexing
+    da, db = qa.float().double(), qb.float().double()
+    for i, j in [(0, 0), (m - 1, n - 1), (m // 2, n // 3)]:
+        total = sum(da[i, kk] * sa[i // ga[0], kk // ga[1]].double() * db[j, kk] * sb[j // gb[0], kk // gb[1]].double()
+                    for kk in range(k)) + bias[j].double()
+        assert abs(witness[i, j] - total) <= 1e-6 * max(1.0, abs(total))   # dequantize rounds code*scale to fp32
+
+
+# ----------------------------------------------------------------------------- Philox / stochastic rounding
+def test_philox_known_answers():
+    """Random123 kat_vectors for philox4x32-10, word 0 (held by the reference, checks/quantization.py:77-81)."""
+    triples = [(0, 0, 0), (0xffffffffffffffff,) * 3, (0x85a308d3243f6a88, 0x0370734413198a2e, 0x299f31d0a4093822)]
+    answers = [int(optim.philox(np.array([e], dtype=np.uint64), s, k)[0]) for e, s, k in triples]
+    assert answers == [0x6627e8d5, 0x408f276d, 0xd16cfe09]
+
+
+def test_stochastic_round_probability_and_adjacency():
+    n = 256 * 1024
+    x = np.full(n, 1 + .27 * .125, dtype=np.float32)
+    out = optim.stochastic_round_e4m3(x, np.arange(n, dtype=np.uint64), 7, 42)
+    assert set(np.unique(out)) == {np.float32(1.0), np.float32(1.125)}
+    assert abs((out == 1.125).mean() - .27) < .005                                # checks/quantization.py:114-136
+    assert not np.array_equal(out, optim.stochastic_round_e4m3(x, np.arange(n, dtype=np.uint64), 8, 42))
+    table = fp8.decode_table("e4m3")[:127]
+    values = np.tile(table[:-1] * .7 + table[1:] * .3, 64).astype(np.float32)
+    both = np.concatenate([values, -values, np.tile(table, 64)])
+    out = optim.stochastic_round_e4m3(both, np.arange(both.size, dtype=np.uint64), 0, 0)
+    idx = np.searchsorted(table, np.abs(both)).clip(max=126)
+    lower, upper = table[np.maximum(idx - 1, 0)], table[idx]
+    assert (((np.abs(out) == lower) | (np.abs(out) == upper))).all()              # checks/quantization.py:138-153
+    assert ((np.sign(out) == np.sign(both)) | (out == 0)).all()
+
+
+@pytest.mark.parametrize("fn,spacing", [(optim.stochastic_bf16, 2.0 ** -8), (optim.stochastic_fp16, 2.0 ** -11)])
+def test_stochastic_storage_rounding_fraction(fn, spacing):
+    """One quarter of a grid step below 1: kept about 25 % of the time (checks/precision_kernels.py:48-58)."""
+    n = 131072
+    x = np.full(n, 1.0 - spacing / 4, dtype=np.float32)
+    out = fn(x, np.arange(n, dtype=np.uint64), 17, 29)
+    assert set(np.unique(out)) <= {np.float32(1.0), np.float32(1.0 - spacing)}
+    assert abs((out != 1.0).mean() - .25) < .005
+    cut = 13001
+    replay = np.concatenate([fn(x[:cut], np.arange(cut, dtype=np.uint64), 17, 29),
+                             fn(x[cut:], np.arange(n - cut, dtype=np.uint64) + np.uint64(cut), 17, 29)])
+    assert np.array_equal(out, replay)
+
+
+# ----------------------------------------------------------------------------- momentum / weight / adam
+@pytest.mark.parametrize("granularity,size", [("tile", 64), ("tile", 256), ("tile", 1024), ("block", (8, 8)), ("block", (16, 32)), ("block", (64, 64))])
+@pytest.mark.parametrize("shape", [(17, 31), (2, 33, 67)])
+def test_momentum_against_the_reference_checks(granularity, size, shape):
+    """The closed forms of checks/quantization.py:27-53,83-112 written independently of oracle.optim's body."""
+    torch.manual_seed(79)
+    quant = dict(granularity=granularity, tile_size=size if granularity == "tile" else 256,
+                 block_shape=size if granularity == "block" else (16, 16))
+    qn, sn = optim.state_sizes(shape, **quant)
+    n = math.prod(shape)
+    q, scale = torch.zeros(qn, dtype=torch.uint8), torch.ones(sn)
+    for step in range(4):
+        g = torch.randn(n) * (1e-8 if step < 1 else 1.)
+        old = optim.dequantize(q, scale, shape, **quant)
+        fresh = .95 * old.double() + .05 * g.double()
+        q, scale, u = optim.momentum_update(g, q, scale, beta=.95, shape=shape, **quant)
+        if granularity == "tile":
+            tiles = F.pad(fresh, (0, qn - n)).view(-1, size)
+        else:
+            rows, cols = shape[-2:]
+            tr, tc = size
+            p = F.pad(fresh.view(-1, rows, cols), (0, (-cols) % tc, 0, (-rows) % tr))
+            tiles = p.view(-1, p.shape[1] // tr, tr, p.shape[2] // tc, tc).permute(0, 1, 3, 2, 4).reshape(-1, tr * tc)
+        expected_scale = (tiles.abs().amax(1).clamp_min(1e-30) / 448).float()
+        torch.testing.assert_close(scale, expected_scale, rtol=2e-6, atol=1e-30)
+        torch.testing.assert_close(u.float(), (.05 * g.double() + .95 * fresh).float().bfloat16().float(), rtol=.01, atol=2e-7)
+        current = optim.dequantize(q, scale, shape, **quant)
+        assert ((current - fresh).norm() / fresh.norm()).item() < .06
+        assert q.numel() == qn and scale.numel() == sn
+
+
+def test_momentum_zero_stays_zero_and_loss_scale():
+    q, scale, u = optim.momentum_update(torch.zeros(300), torch.zeros(512, dtype=torch.uint8), torch.ones(2), beta=.95,
+                                        shape=(300,), tile_size=256)
+    assert q.count_nonzero() == 0 and u.count_nonzero() == 0 and torch.equal(scale, torch.full((2,), 1e-30) / 448)
+    g = torch.randn(257).half()
+    _, _, u = optim.momentum_update(g, torch.zeros(512, dtype=torch.uint8), torch.ones(2), beta=.95, shape=(257,),
+                                    tile_size=256, loss_scale=32.0, nesterov=False)
+    torch.testing.assert_close(u.float(), (.05 * g.float() / 32).bfloat16().float(), rtol=.01, atol=2e-7)
+
+
+def test_weight_and_adam_closed_forms():
+    torch.manual_seed(107)
+    for wdtype in (torch.float32, torch.bfloat16, torch.float16):
+        w = (torch.randn(1025) * .1).to(wdtype)
+        g = (torch.randn(1025) * .01)
+        new = optim.weight_update(w, g, .001, .01, update_scale=3.0)
+        target = w.double() * (1 - .001 * .01) - .001 * 3.0 * g.double()
+        assert (new.double() - target).abs().max() <= 1.01 * (torch.finfo(wdtype).eps * target.abs().max())
+        m, v = torch.zeros(1025), torch.zeros(1025)
+        cur = w
+        for step in range(1, 4):
+            rm = .9 * m.double() + .1 * g.double()
+            rv = .95 * v.double() + .05 * g.double().square()
+            value = cur.double() * (1 - .001 * .01) - .001 * (rm / (1 - .9 ** step)) / ((rv / (1 - .95 ** step)).sqrt() + 1e-8)
+            cur, m, v = optim.adam_update(cur, g, m, v, lr=.001, weight_decay=.01, betas=(.9, .95), eps=1e-8, step=step)
+            torch.testing.assert_close(m.double(), rm, rtol=2e-6, atol=1e-12)
+            torch.testing.assert_close(v.double(), rv, rtol=2e-6, atol=1e-12)
+            assert (cur.double() - value).abs().max() <= 1.01 * torch.finfo(wdtype).eps * value.abs().max()
+    out = optim.copy_scaled(torch.arange(20.).bfloat16(), torch.zeros(30), 11, 3, 5, 3.2)
+    assert torch.equal(out[3:8], torch.arange(11., 16.) * torch.tensor(3.2)) and out[:3].eq(0).all() and out[8:].eq(0).all()
+
+
+# ----------------------------------------------------------------------------- wire codec
+@pytest.mark.parametrize("tile,n", [(64, 1), (64, 31), (256, 513), (1024, 8193), (256, 65539)])
+@pytest.mark.parametrize("dtype", [E4, E5])
+def test_comm_roundtrip_matches_reference_formula(tile, n, dtype):
+    """pack -> unpack == pad / amax / cast / multiply back (checks/fp8_communication.py:32-38)."""
+    torch.manual_seed(300)
+    x = torch.randn(n) * torch.logspace(-5, 5, n)
+    x[::31] *= 64
+    groups = math.ceil(n / tile)
+    packet = comm.pack(x, 1, groups, tile, dtype)
+    assert packet.shape == (1, comm.packet_bytes(groups, tile)) and packet.shape[1] % 16 == 0
+    out = comm.unpack(packet, n, tile, dtype)
+    assert torch.equal(out, comm.roundtrip(x, tile, dtype))
+    # rows = R with reduce: the sum of the R single-row decodes, rank order
+    rows = 3
+    g3 = math.ceil(n / (rows * tile))
+    packet3 = comm.pack(x, rows, g3, tile, dtype)
+    parts = F.pad(x, (0, rows * g3 * tile - n)).view(rows, -1)
+    expect = sum(comm.roundtrip(parts[r], tile, dtype) for r in range(rows))
+    assert torch.allclose(comm.unpack(packet3, g3 * tile, tile, dtype, reduce=True), expect, rtol=1e-6, atol=0)
+
+
+def test_comm_nonfinite_survive():
+    x = torch.ones(1025)
+    x[3], x[600] = float("nan"), float("inf")
+    for dtype in (E4, E5):
+        out = comm.unpack(comm.pack(x, 1, 5, 256, dtype), 1025, 256, dtype)
+        assert not out[3].isfinite() and not out[600].isfinite() and out[900].isfinite()     # fp8_communication.py:80-92
+
+
+def test_packet_layout_constants():
+    assert comm.packet_bytes(25600, 256) == 6656000 and comm.packet_bytes(1, 64) == 80
+
+
+# ----------------------------------------------------------------------------- Newton-Schulz
+def test_ns_matches_reference_golden(golden_dir):
+    """Vectors written by tests/golden/make_ns_golden.py from the reference's own eager recipe."""
+    rows = torch.load(golden_dir / "ns_golden.pt", weights_only=True)
+    assert len(rows) >= 8
+    for row in rows:
+        out = ns.METHODS[row["method"]](row["input"], steps=row["steps"])
+        assert out.dtype == row["output"].dtype and torch.equal(out, row["output"]), (row["method"], row["input"].shape)
+
+
+@pytest.mark.parametrize("method", ["standard", "gram"])
+@pytest.mark.parametrize("shape", [(64, 256), (192, 64), (96, 96)])
+def test_ns_invariants_and_chain(method, shape):
+    torch.manual_seed(1)
+    g = torch.randn(*shape)
+    out = ns.METHODS[method](g, steps=5).float()
+    sv = torch.linalg.svdvals(out)
+    assert sv.max() < 1.3 and .6 < sv.median() < 1.25                             # singular values pushed towards 1
+    if shape[0] != shape[1]:
+        assert sv.min() > .45                                                     # (a square Gaussian matrix is nearly singular)
+    u, _, vh = torch.linalg.svd(g, full_matrices=False)
+    assert F.cosine_similarity(out.flatten(), (u @ vh).flatten(), dim=0) > .97      # same singular vectors as G
+    transposed = ns.METHODS[method](g.T.contiguous(), steps=5).float()
+    # ns(A^T) = ns(A)^T: exact when the recipe transposes the tall case itself, approximate for a square input
+    assert rel_l2(transposed.T, out) < (1e-6 if shape[0] != shape[1] else .08)
+    # fp64 evaluation of the same polynomial (loose: half-precision trajectory)
+    x = g.double() if shape[0] <= shape[1] else g.double().T
+    x = x / (x.norm() + 1e-7)
+    for _ in range(5):
+        a = x @ x.T
+        x = 3.4445 * x + (-4.7750 * a + 2.0315 * a @ a) @ x
+    x = x if shape[0] <= shape[1] else x.T
+    assert rel_l2(out, x) < (.05 if method == "standard" else .01)
+    chain = ns.chain(g, 5, method).float()
+    assert rel_l2(chain, out) < (.06 if method == "standard" else .01)       # eager vs fused-epilogue rounding points
+
+
+# ----------------------------------------------------------------------------- composition
+def test_linear_oracle_against_float_math():
+    torch.manual_seed(4)
+    x = torch.randn(65, 128).bfloat16()
+    w = torch.randn(96, 128) / 11
+    dy = torch.randn(65, 96).bfloat16()
+    qw, sw = grouped.quantize(w, E4, (32, 32))
+    r = linear.linear(x, grouped.dequantize(qw, sw, (32, 32)), torch.zeros(96), dy)
+    assert rel_l2(r["y"], x.float() @ w.T) < .06 and rel_l2(r["dx"], dy.float() @ w) < .06
+    assert rel_l2(r["dw"], dy.float().T @ x.float()) < .06 and torch.equal(r["db"], dy.sum(0, dtype=torch.bfloat16))
+    g, u = torch.randn(33, 40), torch.randn(33, 40)
+    for name in ("silu", "gelu", "relu"):
+        gg = g.clone().requires_grad_(); uu = u.clone().requires_grad_()
+        out = linear.activation(name)(gg) * uu
+        d = torch.randn(33, 40)
+        out.backward(d)
+        assert rel_l2(linear.gated_forward(g, u, name), out.detach()) < 1e-6
+        dg, du = linear.gated_backward(d, g, u, name)
+        assert rel_l2(dg, gg.grad) < 1e-5 and rel_l2(du, uu.grad) < 1e-6

@@ -1,0 +1,195 @@
+// Device helpers shared by every kernel file: storage-type loads/stores, OCP FP8
+// codecs, Philox4x32-10, wavefront reductions. gfx950 only (64-wide wavefronts).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/viola_hip.h"
+
+#define VIOLA_CHECK_ARG(cond) \
+    do {                      \
+        if (!(cond)) return VIOLA_EINVAL; \
+    } while (0)
+
+static inline int viola_launch_status() {
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : (int)e;
+}
+
+static inline bool viola_is_fp8(int dtype) { return dtype == VIOLA_E4M3 || dtype == VIOLA_E5M2; }
+static inline bool viola_is_float(int dtype) { return dtype == VIOLA_F32 || dtype == VIOLA_BF16 || dtype == VIOLA_F16; }
+static inline int viola_dtype_size(int dtype) { return dtype == VIOLA_F32 ? 4 : (dtype == VIOLA_BF16 || dtype == VIOLA_F16) ? 2 : 1; }
+
+namespace viola {
+
+constexpr int WAVE = 64;
+
+// ------------------------------------------------------------------ storage types
+struct bf16_t { uint16_t bits; };
+struct f16_t { _Float16 value; };
+struct e4m3_t { uint8_t bits; };
+struct e5m2_t { uint8_t bits; };
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits) { return __uint_as_float(bits << 16); }
+
+// Round-to-nearest-even, NaN -> quiet NaN with the sign dropped (the rule of PyTorch's cast).
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float x) {
+    uint32_t u = __float_as_uint(x);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;
+    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
+// ------------------------------------------------------------------ FP8 (OCP) codecs
+// Software encoders: exact RNE onto the grid. e4m3fn has no Inf: anything that
+// rounds above 448 becomes NaN (0x7f), as in PyTorch's cast; callers clamp first
+// where the reference clamps.
+__device__ __forceinline__ uint8_t f32_to_e4m3(float x) {
+    uint32_t u = __float_as_uint(x);
+    const uint32_t sign = (u >> 24) & 0x80u;
+    u &= 0x7fffffffu;
+    uint32_t r;
+    if (u >= 0x43f00000u) {                       // >= 480, Inf, NaN
+        r = 0x7f;
+    } else if (u < 0x3c800000u) {                 // < 2^-6: subnormal target, spacing 2^-9
+        const float magic = __uint_as_float(141u << 23);
+        r = __float_as_uint(__uint_as_float(u) + magic) - (141u << 23);
+    } else {
+        const uint32_t odd = (u >> 20) & 1u;
+        u += ((uint32_t)(7 - 127) << 23) + 0x7ffffu + odd;
+        r = u >> 20;
+    }
+    return (uint8_t)(r | sign);
+}
+
+__device__ __forceinline__ uint8_t f32_to_e5m2(float x) {
+    uint32_t u = __float_as_uint(x);
+    const uint32_t sign = (u >> 24) & 0x80u;
+    u &= 0x7fffffffu;
+    uint32_t r;
+    if (u >= (143u << 23)) {                      // >= 65536, Inf, NaN
+        r = u > 0x7f800000u ? 0x7f : 0x7c;
+    } else if (u < (113u << 23)) {                // < 2^-14: subnormal target, spacing 2^-16
+        const float magic = __uint_as_float(134u << 23);
+        r = __float_as_uint(__uint_as_float(u) + magic) - (134u << 23);
+    } else {
+        const uint32_t odd = (u >> 21) & 1u;
+        u += ((uint32_t)(15 - 127) << 23) + 0xfffffu + odd;
+        r = u >> 21;
+    }
+    return (uint8_t)(r | sign);
+}
+
+__device__ __forceinline__ float e4m3_to_f32(uint32_t c) {
+    const uint32_t sign = (c & 0x80u) << 24;
+    const uint32_t mag = c & 0x7fu;
+    float v;
+    if (mag == 0x7f) v = __uint_as_float(0x7fc00000u);
+    else if (mag < 8) v = (float)mag * 0x1p-9f;
+    else v = __uint_as_float((mag << 20) + (120u << 23));
+    return __uint_as_float(__float_as_uint(v) | sign);
+}
+
+__device__ __forceinline__ float e5m2_to_f32(uint32_t c) {
+    const uint32_t sign = (c & 0x80u) << 24;
+    const uint32_t mag = c & 0x7fu;
+    float v;
+    if (mag >= 0x7c) v = __uint_as_float(mag == 0x7c ? 0x7f800000u : 0x7fc00000u);
+    else if (mag < 4) v = (float)mag * 0x1p-16f;
+    else v = __uint_as_float((mag << 21) + (112u << 23));
+    return __uint_as_float(__float_as_uint(v) | sign);
+}
+
+template <typename T> __device__ __forceinline__ float to_f32(T v);
+template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ float to_f32<bf16_t>(bf16_t v) { return bf16_bits_to_f32(v.bits); }
+template <> __device__ __forceinline__ float to_f32<f16_t>(f16_t v) { return (float)v.value; }
+template <> __device__ __forceinline__ float to_f32<e4m3_t>(e4m3_t v) { return e4m3_to_f32(v.bits); }
+template <> __device__ __forceinline__ float to_f32<e5m2_t>(e5m2_t v) { return e5m2_to_f32(v.bits); }
+
+template <typename T> __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return bf16_t{f32_to_bf16_bits(v)}; }
+template <> __device__ __forceinline__ f16_t from_f32<f16_t>(float v) { return f16_t{(_Float16)v}; }
+template <> __device__ __forceinline__ e4m3_t from_f32<e4m3_t>(float v) { return e4m3_t{f32_to_e4m3(v)}; }
+template <> __device__ __forceinline__ e5m2_t from_f32<e5m2_t>(float v) { return e5m2_t{f32_to_e5m2(v)}; }
+
+template <typename T> struct fp8_traits;
+template <> struct fp8_traits<e4m3_t> { static constexpr float max = 448.0f; };
+template <> struct fp8_traits<e5m2_t> { static constexpr float max = 57344.0f; };
+
+// ------------------------------------------------------------------ wavefront reductions
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int offset = WAVE / 2; offset > 0; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, WAVE));
+    return v;
+}
+
+// max over aligned sub-groups of WIDTH lanes (WIDTH a power of two <= 64)
+template <int WIDTH> __device__ __forceinline__ float group_max(float v) {
+#pragma unroll
+    for (int offset = WIDTH / 2; offset > 0; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, WAVE));
+    return v;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int offset = WAVE / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, WAVE);
+    return v;
+}
+
+// ------------------------------------------------------------------ Philox4x32-10 + stochastic rounding
+// counter = (element_lo, element_hi, step_lo, step_hi), key = (key_lo, key_hi); word 0.
+__device__ __forceinline__ uint32_t philox(uint64_t element, uint64_t step, uint64_t key) {
+    uint32_t a = (uint32_t)element, b = (uint32_t)(element >> 32), c = (uint32_t)step, d = (uint32_t)(step >> 32);
+    uint32_t k0 = (uint32_t)key, k1 = (uint32_t)(key >> 32);
+#pragma unroll
+    for (int round = 0; round < 10; ++round) {
+        const uint32_t lo0 = 0xD2511F53u * a, hi0 = __umulhi(0xD2511F53u, a);
+        const uint32_t lo1 = 0xCD9E8D57u * c, hi1 = __umulhi(0xCD9E8D57u, c);
+        a = hi1 ^ b ^ k0; b = lo1; c = hi0 ^ d ^ k1; d = lo0;
+        k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+    }
+    return a;
+}
+
+__device__ __forceinline__ bool finite_f32(float x) { return (__float_as_uint(x) & 0x7f800000u) != 0x7f800000u; }
+
+// Stochastic rounding onto a grid with MANT explicit mantissa bits and minimum spacing 2^MIN_EXP.
+template <int MANT, int MIN_EXP>
+__device__ __forceinline__ float stochastic_grid(float x, uint64_t element, uint64_t step, uint64_t key) {
+    const float a = fabsf(x);
+    const int exponent = (int)((__float_as_uint(a) >> 23) & 255u) - 127;
+    const int e = exponent - MANT > MIN_EXP ? exponent - MANT : MIN_EXP;
+    const float spacing = __uint_as_float((uint32_t)(e + 127) << 23);
+    const float lower = floorf(a / spacing) * spacing;
+    const float probability = (a - lower) / spacing;
+    const float uniform = (float)(philox(element, step, key) >> 8) * 0x1p-24f;
+    return copysignf(lower + (uniform < probability ? spacing : 0.0f), x);
+}
+
+__device__ __forceinline__ float stochastic_e4m3(float x, uint64_t element, uint64_t step, uint64_t key) {
+    return finite_f32(x) ? stochastic_grid<3, -9>(x, element, step, key) : x;
+}
+
+__device__ __forceinline__ float stochastic_bf16(float x, uint64_t element, uint64_t step, uint64_t key) {
+    if (!finite_f32(x)) return x;
+    return __uint_as_float((__float_as_uint(x) + (philox(element, step, key) >> 16)) & 0xffff0000u);
+}
+
+__device__ __forceinline__ float stochastic_fp16(float x, uint64_t element, uint64_t step, uint64_t key) {
+    if (!finite_f32(x) || fabsf(x) > 65504.0f) return x;
+    return stochastic_grid<10, -24>(x, element, step, key);
+}
+
+// Store a fp32 result in storage type T, optionally with stochastic rounding (bf16 / fp16 only).
+template <typename T, bool STOCHASTIC>
+__device__ __forceinline__ T round_store(float v, uint64_t element, uint64_t step, uint64_t key) {
+    if constexpr (STOCHASTIC && sizeof(T) == 2) {
+        if constexpr (__is_same(T, bf16_t)) v = stochastic_bf16(v, element, step, key);
+        else v = stochastic_fp16(v, element, step, key);
+    }
+    return from_f32<T>(v);
+}
+
+}  // namespace viola

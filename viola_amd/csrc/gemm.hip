@@ -1,0 +1,447 @@
+// Grouped-scale FP8 GEMM for gfx950 ("NT": out[m, n] = sum_k a[m, k] * b[n, k]) with FP32 scales
+// per (row group, 32-wide K group) on both operands.
+//
+// Per 32-wide K group the raw code product is formed on the matrix cores
+// (v_mfma_f32_32x32x16_fp8_fp8 twice) and folded into an FP32 total with one VALU FMA per output
+// element: total += acc * (sa * sb). The FP32 scales cannot be applied inside a wider MFMA, so the
+// K = 32 instructions are the ones that fit this contract.
+//
+// Orientation: the B matrix (rows n) is fed as the MFMA "A" operand and the A matrix (rows m) as
+// the MFMA "B" operand, so a lane's 16 accumulators of a 32 x 32 tile share one m and cover 16
+// values of n inside one 32-row block of b. With 2-D weight blocks (br a multiple of 32) the scale
+// product sa[m] * sb[block] is then a single per-lane scalar per K group.
+//
+// Block: 256 threads = 2 x 2 wavefronts, tile 128 (m) x 128 (b rows) x 64 (k), two LDS stages,
+// global loads for chunk i+1 issued before the math of chunk i.
+//
+// One kernel template serves: the plain GEMM, the gated-MLP forward (two 64-row panels of b, gate
+// and up, sharing a; epilogue act(g)*u), the gated-MLP backward (epilogue reads g,u and writes
+// [d*u*act'(g), d*act(g)]), the variable-group row-range GEMM and the variable-group wgrad.
+#include "common.hpp"
+
+namespace viola {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 128, BN = 128, BK = 64, LDK = BK + 8, KG = BK / 32;
+enum { MODE_PLAIN = 0, MODE_GATED_FWD = 1, MODE_GATED_BWD = 2 };
+
+struct GemmArgs {
+    const uint8_t* a; const uint8_t* b; const float* sa; const float* sb;
+    const void* bias; void* out; void* aux;
+    int64_t m, n, k;              // n: rows of one b panel (h for the gated modes)
+    int64_t lda, ldb;             // bytes between rows of a / b
+    int64_t ldsa, ldsb;           // floats between rows of sa / sb
+    int64_t ldo;                  // elements between rows of out
+    int ar, br, ak_shift, bk_shift;
+    int activation;
+    // variable-group row ranges (grid.y walks the tiles of all groups)
+    const int64_t* offsets; int groups; int64_t b_group_stride, sb_group_stride;
+    // variable-group K ranges (grid.z = group): k range [koffsets[g], koffsets[g+1])
+    const int64_t* koffsets; int64_t out_group_stride;
+};
+
+template <bool A_BF8, bool B_BF8>
+__device__ __forceinline__ f32x16 mfma32(long x, long y, f32x16 c) {
+    // x: 8 codes of the b matrix (MFMA srcA), y: 8 codes of the a matrix (MFMA srcB)
+    if constexpr (!B_BF8 && !A_BF8) return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(x, y, c, 0, 0, 0);
+    else if constexpr (!B_BF8 && A_BF8) return __builtin_amdgcn_mfma_f32_32x32x16_fp8_bf8(x, y, c, 0, 0, 0);
+    else if constexpr (B_BF8 && !A_BF8) return __builtin_amdgcn_mfma_f32_32x32x16_bf8_fp8(x, y, c, 0, 0, 0);
+    else return __builtin_amdgcn_mfma_f32_32x32x16_bf8_bf8(x, y, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ float load_dtype(const void* p, int64_t i, int dtype) {
+    if (dtype == VIOLA_F32) return static_cast<const float*>(p)[i];
+    if (dtype == VIOLA_BF16) return bf16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
+    return (float)static_cast<const _Float16*>(p)[i];
+}
+
+__device__ __forceinline__ void activation_pair(int activation, float g, float& act, float& derivative) {
+    if (activation == VIOLA_SILU) {
+        const float s = 1.0f / (1.0f + expf(-g));
+        act = g * s;
+        derivative = s * (1.0f + g * (1.0f - s));
+    } else if (activation == VIOLA_GELU) {
+        const float t = tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g));
+        act = 0.5f * g * (1.0f + t);
+        derivative = 0.5f * (1.0f + t) + 0.5f * g * (1.0f - t * t) * 0.7978845608028654f * (1.0f + 0.134145f * g * g);
+    } else {
+        act = fmaxf(g, 0.0f);
+        derivative = g > 0.0f ? 1.0f : 0.0f;
+    }
+}
+
+template <typename TO> __device__ __forceinline__ float round_through(float v) { return to_f32(from_f32<TO>(v)); }
+
+// A_BF8/B_BF8: operand formats (false = e4m3, true = e5m2). B_ROWSCALE: b scales vary inside a 32-row block.
+// VEC: 16-byte global loads are legal (k ranges and row strides multiples of 16, aligned bases).
+template <int MODE, bool A_BF8, bool B_BF8, bool B_ROWSCALE, bool VEC, typename TO>
+__global__ __launch_bounds__(256, 2) void group_gemm_kernel(GemmArgs p, int bias_dtype) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds_a[2][BM * LDK];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_b[2][BN * LDK];
+    __shared__ __attribute__((aligned(16))) float lds_sa[2][KG][BM];
+    __shared__ __attribute__((aligned(16))) float lds_sb[2][KG][BN];
+
+    constexpr int PANEL = MODE == MODE_GATED_FWD ? BN / 2 : BN;       // b rows per panel in the tile
+    const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+    const int wm = wave / 2, wn = wave % 2;
+    const int l32 = lane % 32, lhi = lane / 32;
+
+    // ---- which problem / tile
+    int64_t m_begin = (int64_t)blockIdx.y * BM, m_end = p.m;
+    int64_t k_begin = 0, k_end = p.k;
+    const uint8_t* bptr = p.b;
+    const float* sbptr = p.sb;
+    uint8_t* outptr = static_cast<uint8_t*>(p.out);
+    if (p.offsets) {
+        int64_t tile = blockIdx.y;
+        int g = 0;
+        bool found = false;
+        for (; g < p.groups; ++g) {
+            const int64_t lo = p.offsets[g], hi = p.offsets[g + 1];
+            const int64_t tiles = (hi - lo + BM - 1) / BM;
+            if (tile < tiles) { m_begin = lo + tile * BM; m_end = hi; found = true; break; }
+            tile -= tiles;
+        }
+        if (!found) return;
+        bptr += (int64_t)g * p.b_group_stride;
+        sbptr += (int64_t)g * p.sb_group_stride;
+    }
+    if (p.koffsets) {
+        const int g = blockIdx.z;
+        k_begin = p.koffsets[g];
+        k_end = p.koffsets[g + 1];
+        outptr += (int64_t)g * p.out_group_stride * (int64_t)sizeof(TO);
+    }
+    if (m_begin >= m_end) return;
+    const int64_t n_begin = (int64_t)blockIdx.x * PANEL;
+
+    // global row of tile-local b row `lr`
+    auto b_row = [&](int lr) -> int64_t {
+        if constexpr (MODE == MODE_GATED_FWD) return (int64_t)(lr / PANEL) * p.n + n_begin + lr % PANEL;
+        else return n_begin + lr;
+    };
+    const int64_t b_rows_total = MODE == MODE_GATED_FWD ? 2 * p.n : p.n;
+    auto b_row_valid = [&](int lr) -> bool {
+        if constexpr (MODE == MODE_GATED_FWD) return n_begin + lr % PANEL < p.n;
+        else return n_begin + lr < p.n;
+    };
+
+    // ---- staging registers for the next chunk
+    uint4 ra[2], rb[2];
+    float rsa, rsb;
+    auto fetch = [&](int64_t k0) {
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int id = it * 256 + tid;
+            const int lr = id / 4, c = id % 4;
+            const int64_t kk = k0 + c * 16;
+            int64_t am = m_begin + lr;
+            am = am < m_end ? am : m_end - 1;
+            int64_t bn = b_row(lr);
+            bn = bn < b_rows_total ? bn : b_rows_total - 1;
+            if constexpr (VEC) {
+                ra[it] = kk < k_end ? *reinterpret_cast<const uint4*>(p.a + am * p.lda + kk) : make_uint4(0, 0, 0, 0);
+                rb[it] = kk < k_end ? *reinterpret_cast<const uint4*>(bptr + bn * p.ldb + kk) : make_uint4(0, 0, 0, 0);
+            } else {
+                uint32_t wa[4] = {0, 0, 0, 0}, wb[4] = {0, 0, 0, 0};
+                for (int i = 0; i < 16; ++i) {
+                    if (kk + i < k_end) {
+                        wa[i / 4] |= (uint32_t)p.a[am * p.lda + kk + i] << (8 * (i % 4));
+                        wb[i / 4] |= (uint32_t)bptr[bn * p.ldb + kk + i] << (8 * (i % 4));
+                    }
+                }
+                ra[it] = make_uint4(wa[0], wa[1], wa[2], wa[3]);
+                rb[it] = make_uint4(wb[0], wb[1], wb[2], wb[3]);
+            }
+        }
+        {
+            const int kg = tid / BM, lr = tid % BM;                    // KG * 128 == 256 entries each
+            const int64_t kk = k0 + kg * 32;
+            int64_t am = m_begin + lr;
+            am = am < m_end ? am : m_end - 1;
+            int64_t bn = b_row(lr);
+            bn = bn < b_rows_total ? bn : b_rows_total - 1;
+            rsa = kk < k_end ? p.sa[am / p.ar * p.ldsa + (kk >> p.ak_shift)] : 0.0f;
+            rsb = kk < k_end ? sbptr[bn / p.br * p.ldsb + (kk >> p.bk_shift)] : 0.0f;
+        }
+    };
+    auto stash = [&](int s) {
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int id = it * 256 + tid;
+            const int lr = id / 4, c = id % 4;
+            uint2* da = reinterpret_cast<uint2*>(&lds_a[s][lr * LDK + c * 16]);
+            da[0] = make_uint2(ra[it].x, ra[it].y);
+            da[1] = make_uint2(ra[it].z, ra[it].w);
+            uint2* db = reinterpret_cast<uint2*>(&lds_b[s][lr * LDK + c * 16]);
+            db[0] = make_uint2(rb[it].x, rb[it].y);
+            db[1] = make_uint2(rb[it].z, rb[it].w);
+        }
+        lds_sa[s][tid / BM][tid % BM] = rsa;
+        lds_sb[s][tid / BM][tid % BM] = rsb;
+    };
+
+    // tile-local b row of this wavefront's sub-tile i (32 rows each)
+    auto b_sub = [&](int i) -> int {
+        if constexpr (MODE == MODE_GATED_FWD) return i * PANEL + wn * 32;   // i = 0 gate, 1 up
+        else return wn * 64 + i * 32;
+    };
+
+    f32x16 total[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) total[i][j][r] = 0.0f;
+
+    const int64_t chunks = (k_end - k_begin + BK - 1) / BK;
+    if (chunks > 0) {
+        fetch(k_begin);
+        stash(0);
+    }
+    __syncthreads();
+    for (int64_t chunk = 0; chunk < chunks; ++chunk) {
+        const int s = (int)(chunk & 1);
+        if (chunk + 1 < chunks) fetch(k_begin + (chunk + 1) * BK);
+#pragma unroll
+        for (int kg = 0; kg < KG; ++kg) {
+            f32x16 acc[2][2];
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                const int koff = kg * 32 + ks * 16 + lhi * 8;
+                long opb[2], opa[2];
+#pragma unroll
+                for (int i = 0; i < 2; ++i) opb[i] = *reinterpret_cast<const long*>(&lds_b[s][(b_sub(i) + l32) * LDK + koff]);
+#pragma unroll
+                for (int j = 0; j < 2; ++j) opa[j] = *reinterpret_cast<const long*>(&lds_a[s][(wm * 64 + j * 32 + l32) * LDK + koff]);
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        if (ks == 0) {
+                            f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                            acc[i][j] = mfma32<A_BF8, B_BF8>(opb[i], opa[j], zero);
+                        } else {
+                            acc[i][j] = mfma32<A_BF8, B_BF8>(opb[i], opa[j], acc[i][j]);
+                        }
+                    }
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const float sa_l = lds_sa[s][kg][wm * 64 + j * 32 + l32];
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    if constexpr (!B_ROWSCALE) {
+                        const float sc = sa_l * lds_sb[s][kg][b_sub(i)];
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) total[i][j][r] = fmaf(acc[i][j][r], sc, total[i][j][r]);
+                    } else {
+#pragma unroll
+                        for (int r4 = 0; r4 < 4; ++r4) {
+                            const float4 sb4 = *reinterpret_cast<const float4*>(&lds_sb[s][kg][b_sub(i) + r4 * 8 + lhi * 4]);
+                            total[i][j][r4 * 4 + 0] = fmaf(acc[i][j][r4 * 4 + 0], sa_l * sb4.x, total[i][j][r4 * 4 + 0]);
+                            total[i][j][r4 * 4 + 1] = fmaf(acc[i][j][r4 * 4 + 1], sa_l * sb4.y, total[i][j][r4 * 4 + 1]);
+                            total[i][j][r4 * 4 + 2] = fmaf(acc[i][j][r4 * 4 + 2], sa_l * sb4.z, total[i][j][r4 * 4 + 2]);
+                            total[i][j][r4 * 4 + 3] = fmaf(acc[i][j][r4 * 4 + 3], sa_l * sb4.w, total[i][j][r4 * 4 + 3]);
+                        }
+                    }
+                }
+            }
+        }
+        if (chunk + 1 < chunks) stash(s ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: lane holds m = l32 of sub-tile j, n = (r/4)*8 + lhi*4 + r%4 of sub-tile i
+    TO* out = reinterpret_cast<TO*>(outptr);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int64_t mrow = m_begin + wm * 64 + j * 32 + l32;
+        if (mrow >= m_end) continue;
+        if constexpr (MODE == MODE_GATED_FWD) {
+            TO* aux = static_cast<TO*>(p.aux);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int64_t ncol = n_begin + wn * 32 + (r / 4) * 8 + lhi * 4 + r % 4;
+                if (ncol >= p.n) continue;
+                float gv = total[0][j][r], uv = total[1][j][r];
+                if (p.bias) {
+                    gv += load_dtype(p.bias, ncol, bias_dtype);
+                    uv += load_dtype(p.bias, p.n + ncol, bias_dtype);
+                }
+                const TO gq = from_f32<TO>(gv), uq = from_f32<TO>(uv);
+                if (aux) {
+                    aux[mrow * 2 * p.n + ncol] = gq;
+                    aux[mrow * 2 * p.n + p.n + ncol] = uq;
+                }
+                float act, derivative;
+                activation_pair(p.activation, to_f32(gq), act, derivative);
+                out[mrow * p.ldo + ncol] = from_f32<TO>(act * to_f32(uq));
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int64_t ncol = n_begin + wn * 64 + i * 32 + (r / 4) * 8 + lhi * 4 + r % 4;
+                    if (ncol >= p.n) continue;
+                    float v = total[i][j][r];
+                    if constexpr (MODE == MODE_PLAIN) {
+                        if (p.bias) v += load_dtype(p.bias, ncol, bias_dtype);
+                        out[mrow * p.ldo + ncol] = from_f32<TO>(v);
+                    } else {
+                        const TO* aux = static_cast<const TO*>(p.aux);
+                        const float d = round_through<TO>(v);
+                        const float g = to_f32(aux[mrow * 2 * p.n + ncol]);
+                        const float u = to_f32(aux[mrow * 2 * p.n + p.n + ncol]);
+                        float act, derivative;
+                        activation_pair(p.activation, g, act, derivative);
+                        out[mrow * p.ldo + ncol] = from_f32<TO>(d * u * derivative);
+                        out[mrow * p.ldo + p.n + ncol] = from_f32<TO>(d * act);
+                    }
+                }
+            }
+        }
+    }
+}
+
+static int shift_of(int v) {
+    int s = 0;
+    while ((1 << s) < v) ++s;
+    return s;
+}
+
+template <int MODE, bool B_ROWSCALE, bool VEC, typename TO>
+static void launch_formats(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, dim3 grid, hipStream_t stream) {
+    const bool a5 = a_dtype == VIOLA_E5M2, b5 = b_dtype == VIOLA_E5M2;
+    if (!a5 && !b5) hipLaunchKernelGGL((group_gemm_kernel<MODE, false, false, B_ROWSCALE, VEC, TO>), grid, dim3(256), 0, stream, p, bias_dtype);
+    else if (a5 && !b5) hipLaunchKernelGGL((group_gemm_kernel<MODE, true, false, B_ROWSCALE, VEC, TO>), grid, dim3(256), 0, stream, p, bias_dtype);
+    else if (!a5 && b5) hipLaunchKernelGGL((group_gemm_kernel<MODE, false, true, B_ROWSCALE, VEC, TO>), grid, dim3(256), 0, stream, p, bias_dtype);
+    else hipLaunchKernelGGL((group_gemm_kernel<MODE, true, true, B_ROWSCALE, VEC, TO>), grid, dim3(256), 0, stream, p, bias_dtype);
+}
+
+template <int MODE, typename TO>
+static void launch_paths(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, bool rowscale, bool vec, dim3 grid,
+                         hipStream_t stream) {
+    if (rowscale) {
+        if (vec) launch_formats<MODE, true, true, TO>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
+        else launch_formats<MODE, true, false, TO>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
+    } else {
+        if (vec) launch_formats<MODE, false, true, TO>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
+        else launch_formats<MODE, false, false, TO>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
+    }
+}
+
+template <int MODE>
+static int launch_out(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, bool rowscale, bool vec,
+                      dim3 grid, hipStream_t stream) {
+    switch (out_dtype) {
+        case VIOLA_F32: launch_paths<MODE, float>(p, a_dtype, b_dtype, bias_dtype, rowscale, vec, grid, stream); break;
+        case VIOLA_BF16: launch_paths<MODE, bf16_t>(p, a_dtype, b_dtype, bias_dtype, rowscale, vec, grid, stream); break;
+        case VIOLA_F16: launch_paths<MODE, f16_t>(p, a_dtype, b_dtype, bias_dtype, rowscale, vec, grid, stream); break;
+        default: return VIOLA_EINVAL;
+    }
+    return viola_launch_status();
+}
+
+static bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+static bool pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
+
+}  // namespace viola
+
+using namespace viola;
+
+extern "C" int viola_group_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,
+                                int64_t m, int64_t n, int64_t k, int ar, int ak, int br, int bk, const void* bias,
+                                int bias_dtype, void* out, int out_dtype, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_fp8(a_dtype) && viola_is_fp8(b_dtype) && viola_is_float(out_dtype));
+    VIOLA_CHECK_ARG(m >= 0 && n >= 0 && k >= 0 && ar > 0 && br > 0 && pow2(ak) && pow2(bk) && ak >= 32 && bk >= 32);
+    VIOLA_CHECK_ARG(!bias || viola_is_float(bias_dtype));
+    if (m == 0 || n == 0) return 0;
+    VIOLA_CHECK_ARG(out && (k == 0 || (a && b && sa && sb)));
+    const int64_t gy = (m + BM - 1) / BM, gx = (n + BN - 1) / BN;
+    VIOLA_CHECK_ARG(gy <= 65535);
+    GemmArgs p = {};
+    p.a = static_cast<const uint8_t*>(a); p.b = static_cast<const uint8_t*>(b); p.sa = sa; p.sb = sb;
+    p.bias = bias; p.out = out; p.m = m; p.n = n; p.k = k; p.lda = k; p.ldb = k;
+    p.ldsa = (k + ak - 1) / ak; p.ldsb = (k + bk - 1) / bk; p.ldo = n;
+    p.ar = ar; p.br = br; p.ak_shift = shift_of(ak); p.bk_shift = shift_of(bk);
+    const bool vec = k % 16 == 0 && aligned16(a) && aligned16(b);
+    const bool rowscale = br % 32 != 0;
+    return launch_out<MODE_PLAIN>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, vec, dim3((unsigned)gx, (unsigned)gy), stream);
+}
+
+extern "C" int viola_gated_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,
+                                int64_t m, int64_t h, int64_t k, int ar, int ak, int br, int bk, const void* bias,
+                                int bias_dtype, void* aux, void* out, int out_dtype, int activation, int backward,
+                                viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_fp8(a_dtype) && viola_is_fp8(b_dtype) && viola_is_float(out_dtype));
+    VIOLA_CHECK_ARG(m >= 0 && h >= 0 && k >= 0 && ar > 0 && br > 0 && pow2(ak) && pow2(bk) && ak >= 32 && bk >= 32);
+    VIOLA_CHECK_ARG(activation >= VIOLA_SILU && activation <= VIOLA_RELU && (!bias || viola_is_float(bias_dtype)));
+    if (m == 0 || h == 0) return 0;
+    VIOLA_CHECK_ARG(out && (k == 0 || (a && b && sa && sb)) && (!backward || aux));
+    GemmArgs p = {};
+    p.a = static_cast<const uint8_t*>(a); p.b = static_cast<const uint8_t*>(b); p.sa = sa; p.sb = sb;
+    p.bias = backward ? nullptr : bias; p.out = out; p.aux = aux; p.m = m; p.n = h; p.k = k; p.lda = k; p.ldb = k;
+    p.ldsa = (k + ak - 1) / ak; p.ldsb = (k + bk - 1) / bk; p.ldo = backward ? 2 * h : h;
+    p.ar = ar; p.br = br; p.ak_shift = shift_of(ak); p.bk_shift = shift_of(bk); p.activation = activation;
+    const bool vec = k % 16 == 0 && aligned16(a) && aligned16(b);
+    const int64_t gy = (m + BM - 1) / BM;
+    VIOLA_CHECK_ARG(gy <= 65535);
+    if (backward) {
+        const bool rowscale = br % 32 != 0;
+        return launch_out<MODE_GATED_BWD>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, vec,
+                                          dim3((unsigned)((h + BN - 1) / BN), (unsigned)gy), stream);
+    }
+    const bool rowscale = br % 32 != 0 || h % 32 != 0;
+    return launch_out<MODE_GATED_FWD>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, vec,
+                                      dim3((unsigned)((h + BN / 2 - 1) / (BN / 2)), (unsigned)gy), stream);
+}
+
+extern "C" int viola_varlen_group_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa,
+                                       const float* sb, const int64_t* offsets, int groups, int64_t m_total, int64_t n,
+                                       int64_t k, int ar, int ak, int br, int bk, int64_t b_group_stride,
+                                       int64_t sb_group_stride, void* out, int out_dtype, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_fp8(a_dtype) && viola_is_fp8(b_dtype) && viola_is_float(out_dtype));
+    VIOLA_CHECK_ARG(m_total >= 0 && n >= 0 && k >= 0 && groups > 0 && ar == 1 && br > 0 && pow2(ak) && pow2(bk) && ak >= 32 && bk >= 32);
+    if (m_total == 0 || n == 0) return 0;
+    VIOLA_CHECK_ARG(out && offsets && (k == 0 || (a && b && sa && sb)));
+    const int64_t gy = (m_total + BM - 1) / BM + groups;
+    VIOLA_CHECK_ARG(gy <= 65535);
+    GemmArgs p = {};
+    p.a = static_cast<const uint8_t*>(a); p.b = static_cast<const uint8_t*>(b); p.sa = sa; p.sb = sb;
+    p.out = out; p.m = m_total; p.n = n; p.k = k; p.lda = k; p.ldb = k;
+    p.ldsa = (k + ak - 1) / ak; p.ldsb = (k + bk - 1) / bk; p.ldo = n;
+    p.ar = ar; p.br = br; p.ak_shift = shift_of(ak); p.bk_shift = shift_of(bk);
+    p.offsets = offsets; p.groups = groups; p.b_group_stride = b_group_stride; p.sb_group_stride = sb_group_stride;
+    const bool vec = k % 16 == 0 && aligned16(a) && aligned16(b) && b_group_stride % 16 == 0;
+    const bool rowscale = br % 32 != 0;
+    return launch_out<MODE_PLAIN>(p, a_dtype, b_dtype, VIOLA_F32, out_dtype, rowscale, vec,
+                                  dim3((unsigned)((n + BN - 1) / BN), (unsigned)gy), stream);
+}
+
+extern "C" int viola_varlen_wgrad_gemm(const void* at, int a_dtype, const void* bt, int b_dtype, const float* sat,
+                                       const float* sbt, const int64_t* poffsets, int groups, int64_t t_total, int64_t n,
+                                       int64_t kout, void* out, int out_dtype, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_fp8(a_dtype) && viola_is_fp8(b_dtype) && viola_is_float(out_dtype));
+    VIOLA_CHECK_ARG(t_total >= 0 && t_total % 32 == 0 && n >= 0 && kout >= 0 && groups > 0 && groups <= 65535);
+    if (n == 0 || kout == 0) return 0;
+    VIOLA_CHECK_ARG(out && poffsets && (t_total == 0 || (at && bt && sat && sbt)));
+    const int64_t gy = (n + BM - 1) / BM;
+    VIOLA_CHECK_ARG(gy <= 65535);
+    GemmArgs p = {};
+    p.a = static_cast<const uint8_t*>(at); p.b = static_cast<const uint8_t*>(bt); p.sa = sat; p.sb = sbt;
+    p.out = out; p.m = n; p.n = kout; p.k = t_total; p.lda = t_total; p.ldb = t_total;
+    p.ldsa = t_total / 32; p.ldsb = t_total / 32; p.ldo = kout;
+    p.ar = 1; p.br = 1; p.ak_shift = 5; p.bk_shift = 5;
+    p.koffsets = poffsets; p.out_group_stride = n * kout;
+    const bool vec = t_total % 16 == 0 && aligned16(at) && aligned16(bt);
+    return launch_out<MODE_PLAIN>(p, a_dtype, b_dtype, VIOLA_F32, out_dtype, true, vec,
+                                  dim3((unsigned)((kout + BN - 1) / BN), (unsigned)gy, (unsigned)groups), stream);
+}

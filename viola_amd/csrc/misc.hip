@@ -1,0 +1,263 @@
+// FP8 gradient wire codec, elementwise gated activations, and device self checks for gfx950.
+// Built with -ffp-contract=off.
+#include "common.hpp"
+
+namespace viola {
+
+// ------------------------------------------------------------------ wire codec
+// LANES lanes share one tile of `tile` fp32 values; each lane walks it with stride LANES.
+template <typename TQ, int LANES>
+__global__ __launch_bounds__(256) void comm_pack_kernel(const float* __restrict__ x, int64_t n, uint8_t* __restrict__ packet,
+                                                         int64_t rows, int64_t groups, int tile, int64_t stride) {
+    const int64_t unit = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / LANES;     // (row, group) pair
+    if (unit >= rows * groups) return;                                                   // LANES-aligned sets leave together
+    const int sub = threadIdx.x % LANES;
+    const int64_t row = unit / groups, group = unit % groups;
+    const int64_t base = row * groups * tile + group * tile;
+    float amax = 0.0f;
+    for (int i = sub; i < tile; i += LANES) {
+        const float v = base + i < n ? x[base + i] : 0.0f;
+        amax = fmaxf(amax, v != v ? __uint_as_float(0x7f800000u) : fabsf(v));
+    }
+    amax = group_max<LANES>(amax);
+    const float s = fmaxf(amax, 1e-30f) / fp8_traits<TQ>::max;
+    uint8_t* codes = packet + row * stride + group * tile;
+    for (int i = sub; i < tile; i += LANES) {
+        const float v = base + i < n ? x[base + i] : 0.0f;
+        codes[i] = from_f32<TQ>(v / s).bits;
+    }
+    if (sub == 0) reinterpret_cast<float*>(packet + row * stride + groups * tile)[group] = s;
+}
+
+// tile == 256, x 16-byte aligned: one wavefront per tile, one float4 per lane.
+template <typename TQ>
+__global__ __launch_bounds__(256) void comm_pack256_kernel(const float* __restrict__ x, int64_t n, uint8_t* __restrict__ packet,
+                                                            int64_t rows, int64_t groups, int64_t stride) {
+    const int64_t unit = (int64_t)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (unit >= rows * groups) return;
+    const int lane = threadIdx.x % WAVE;
+    const int64_t row = unit / groups, group = unit % groups;
+    const int64_t base = (row * groups + group) * 256 + lane * 4;
+    float v[4] = {0, 0, 0, 0};
+    if (base + 3 < n) {
+        const float4 raw = *reinterpret_cast<const float4*>(x + base);
+        v[0] = raw.x; v[1] = raw.y; v[2] = raw.z; v[3] = raw.w;
+    } else {
+        for (int i = 0; i < 4; ++i)
+            if (base + i < n) v[i] = x[base + i];
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) amax = fmaxf(amax, v[i] != v[i] ? __uint_as_float(0x7f800000u) : fabsf(v[i]));
+    amax = wave_max(amax);
+    const float s = fmaxf(amax, 1e-30f) / fp8_traits<TQ>::max;
+    uint32_t w = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w |= (uint32_t)from_f32<TQ>(v[i] / s).bits << (8 * i);
+    *reinterpret_cast<uint32_t*>(packet + row * stride + group * 256 + lane * 4) = w;
+    if (lane == 0) reinterpret_cast<float*>(packet + row * stride + groups * 256)[group] = s;
+}
+
+template <typename TQ>
+__global__ __launch_bounds__(256) void comm_unpack_kernel(const uint8_t* __restrict__ packet, float* __restrict__ out, int64_t n,
+                                                           int64_t rows, int64_t groups, int tile, int64_t stride, int reduce) {
+    const int64_t width = groups * tile;
+    const int64_t total = reduce ? width : rows * width;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t row = idx / width, col = idx % width;
+        if (reduce) {
+            if (col >= n) continue;
+            float result = 0.0f;
+            for (int64_t rank = 0; rank < rows; ++rank) {
+                const float s = reinterpret_cast<const float*>(packet + rank * stride + width)[col / tile];
+                result += to_f32(TQ{packet[rank * stride + col]}) * s;
+            }
+            out[col] = result;
+        } else {
+            if (idx >= n) continue;
+            const float s = reinterpret_cast<const float*>(packet + row * stride + width)[col / tile];
+            out[idx] = to_f32(TQ{packet[row * stride + col]}) * s;
+        }
+    }
+}
+
+// ------------------------------------------------------------------ gated activations
+__device__ __forceinline__ float load_half(const void* p, int64_t i, int dtype) {
+    if (dtype == VIOLA_F32) return static_cast<const float*>(p)[i];
+    if (dtype == VIOLA_BF16) return bf16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
+    return (float)static_cast<const _Float16*>(p)[i];
+}
+__device__ __forceinline__ void store_half(void* p, int64_t i, int dtype, float v) {
+    if (dtype == VIOLA_F32) static_cast<float*>(p)[i] = v;
+    else if (dtype == VIOLA_BF16) static_cast<uint16_t*>(p)[i] = f32_to_bf16_bits(v);
+    else static_cast<_Float16*>(p)[i] = (_Float16)v;
+}
+
+__global__ __launch_bounds__(256) void gated_forward_kernel(const void* __restrict__ z, void* __restrict__ out, int64_t rows,
+                                                             int64_t h, int dtype, int activation) {
+    const int64_t total = rows * h;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t r = idx / h, c = idx % h;
+        const float g = load_half(z, r * 2 * h + c, dtype), u = load_half(z, r * 2 * h + h + c, dtype);
+        float a;
+        if (activation == VIOLA_SILU) a = g / (1.0f + expf(-g));
+        else if (activation == VIOLA_GELU) a = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+        else a = fmaxf(g, 0.0f);
+        store_half(out, idx, dtype, a * u);
+    }
+}
+
+__global__ __launch_bounds__(256) void gated_backward_kernel(const void* __restrict__ z, const void* __restrict__ dy,
+                                                              void* __restrict__ dz, int64_t rows, int64_t h, int dtype,
+                                                              int activation) {
+    const int64_t total = rows * h;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t r = idx / h, c = idx % h;
+        const float g = load_half(z, r * 2 * h + c, dtype), u = load_half(z, r * 2 * h + h + c, dtype);
+        const float d = load_half(dy, idx, dtype);
+        float a, derivative;
+        if (activation == VIOLA_SILU) {
+            const float s = 1.0f / (1.0f + expf(-g));
+            a = g * s;
+            derivative = s * (1.0f + g * (1.0f - s));
+        } else if (activation == VIOLA_GELU) {
+            const float t = tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g));
+            a = 0.5f * g * (1.0f + t);
+            derivative = 0.5f * (1.0f + t) + 0.5f * g * (1.0f - t * t) * 0.7978845608028654f * (1.0f + 0.134145f * g * g);
+        } else {
+            a = fmaxf(g, 0.0f);
+            derivative = g > 0.0f ? 1.0f : 0.0f;
+        }
+        store_half(dz, r * 2 * h + c, dtype, d * u * derivative);
+        store_half(dz, r * 2 * h + h + c, dtype, d * a);
+    }
+}
+
+// ------------------------------------------------------------------ self checks
+// Hardware v_cvt_pk_{fp8,bf8}_f32 / v_cvt_f32_{fp8,bf8} against the software codecs.
+__global__ __launch_bounds__(256) void selftest_fp8_kernel(unsigned long long* counts) {
+    unsigned long long bad[4] = {0, 0, 0, 0};
+    const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t bits = gid; bits < (1ull << 32); bits += stride) {
+        const float x = __uint_as_float((uint32_t)bits);
+        const float a = fabsf(x);
+        if (a <= 448.0f) {
+            const uint32_t hw = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(x, x, 0, false) & 0xffu;
+            if (hw != f32_to_e4m3(x)) ++bad[0];
+        }
+        if (a <= 57344.0f) {
+            const uint32_t hw = (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(x, x, 0, false) & 0xffu;
+            if (hw != f32_to_e5m2(x)) ++bad[1];
+        }
+    }
+    if (gid < 256) {
+        const uint32_t c = (uint32_t)gid;
+        const float hw4 = __builtin_amdgcn_cvt_f32_fp8((int)c, 0), sw4 = e4m3_to_f32(c);
+        const float hw5 = __builtin_amdgcn_cvt_f32_bf8((int)c, 0), sw5 = e5m2_to_f32(c);
+        const bool nan4 = sw4 != sw4, nan5 = sw5 != sw5;
+        if (nan4 ? hw4 == hw4 : __float_as_uint(hw4) != __float_as_uint(sw4)) ++bad[2];
+        if (nan5 ? hw5 == hw5 : __float_as_uint(hw5) != __float_as_uint(sw5)) ++bad[3];
+    }
+    for (int i = 0; i < 4; ++i)
+        if (bad[i]) atomicAdd(&counts[i], bad[i]);
+}
+
+__global__ void selftest_philox_kernel(const uint64_t* __restrict__ triples, uint32_t* __restrict__ out, int64_t count) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) out[i] = philox(triples[3 * i], triples[3 * i + 1], triples[3 * i + 2]);
+}
+
+static unsigned grid_for(int64_t n) {
+    const int64_t blocks = (n + 255) / 256;
+    return (unsigned)(blocks < 1 ? 1 : blocks > 65536 * 8 ? 65536 * 8 : blocks);
+}
+
+template <typename TQ>
+static int launch_pack(const float* x, int64_t n, uint8_t* packet, int64_t rows, int64_t groups, int tile, int64_t stride,
+                       hipStream_t stream) {
+    const int64_t units = rows * groups;
+    if (tile == 256 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(packet) % 4 == 0) {
+        hipLaunchKernelGGL(comm_pack256_kernel<TQ>, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x, n, packet, rows, groups, stride);
+    } else if (tile >= 64) {
+        hipLaunchKernelGGL((comm_pack_kernel<TQ, 64>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x, n, packet, rows, groups, tile, stride);
+    } else {
+        hipLaunchKernelGGL((comm_pack_kernel<TQ, 32>), dim3((unsigned)((units + 7) / 8)), dim3(256), 0, stream, x, n, packet, rows, groups, tile, stride);
+    }
+    return viola_launch_status();
+}
+
+}  // namespace viola
+
+using namespace viola;
+
+extern "C" int viola_comm_pack(const float* x, int64_t n, void* packet, int64_t rows, int64_t groups, int tile, int fp8_dtype,
+                               viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_fp8(fp8_dtype) && n >= 0 && rows >= 0 && groups >= 0 && tile >= 32 && (tile & (tile - 1)) == 0);
+    if (rows == 0 || groups == 0) return 0;
+    VIOLA_CHECK_ARG(packet && (n == 0 || x) && reinterpret_cast<uintptr_t>(packet) % 4 == 0);
+    const int64_t stride = (groups * (tile + 4) + 15) / 16 * 16;
+    VIOLA_CHECK_ARG((rows * groups + 3) / 4 < (1ll << 31));
+    if (fp8_dtype == VIOLA_E4M3) return launch_pack<e4m3_t>(x, n, static_cast<uint8_t*>(packet), rows, groups, tile, stride, stream);
+    return launch_pack<e5m2_t>(x, n, static_cast<uint8_t*>(packet), rows, groups, tile, stride, stream);
+}
+
+extern "C" int viola_comm_unpack(const void* packet, float* out, int64_t n, int64_t rows, int64_t groups, int tile,
+                                 int fp8_dtype, int reduce, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_fp8(fp8_dtype) && n >= 0 && rows >= 0 && groups >= 0 && tile >= 32 && (tile & (tile - 1)) == 0);
+    if (rows == 0 || groups == 0 || n == 0) return 0;
+    VIOLA_CHECK_ARG(packet && out && reinterpret_cast<uintptr_t>(packet) % 4 == 0);
+    VIOLA_CHECK_ARG(n <= (reduce ? 1 : rows) * groups * tile);
+    const int64_t stride = (groups * (tile + 4) + 15) / 16 * 16;
+    const int64_t total = (reduce ? 1 : rows) * groups * tile;
+    const uint8_t* pk = static_cast<const uint8_t*>(packet);
+    if (fp8_dtype == VIOLA_E4M3) hipLaunchKernelGGL(comm_unpack_kernel<e4m3_t>, dim3(grid_for(total)), dim3(256), 0, stream, pk, out, n, rows, groups, tile, stride, reduce);
+    else hipLaunchKernelGGL(comm_unpack_kernel<e5m2_t>, dim3(grid_for(total)), dim3(256), 0, stream, pk, out, n, rows, groups, tile, stride, reduce);
+    return viola_launch_status();
+}
+
+extern "C" int viola_gated_forward(const void* z, void* out, int64_t rows, int64_t h, int dtype, int activation,
+                                   viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_float(dtype) && rows >= 0 && h >= 0 && activation >= VIOLA_SILU && activation <= VIOLA_RELU);
+    if (rows == 0 || h == 0) return 0;
+    VIOLA_CHECK_ARG(z && out);
+    hipLaunchKernelGGL(gated_forward_kernel, dim3(grid_for(rows * h)), dim3(256), 0, stream, z, out, rows, h, dtype, activation);
+    return viola_launch_status();
+}
+
+extern "C" int viola_gated_backward(const void* z, const void* dy, void* dz, int64_t rows, int64_t h, int dtype,
+                                    int activation, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_float(dtype) && rows >= 0 && h >= 0 && activation >= VIOLA_SILU && activation <= VIOLA_RELU);
+    if (rows == 0 || h == 0) return 0;
+    VIOLA_CHECK_ARG(z && dy && dz);
+    hipLaunchKernelGGL(gated_backward_kernel, dim3(grid_for(rows * h)), dim3(256), 0, stream, z, dy, dz, rows, h, dtype, activation);
+    return viola_launch_status();
+}
+
+extern "C" int viola_selftest_fp8(uint64_t* counts, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(counts);
+    hipLaunchKernelGGL(selftest_fp8_kernel, dim3(4096), dim3(256), 0, stream, reinterpret_cast<unsigned long long*>(counts));
+    return viola_launch_status();
+}
+
+extern "C" int viola_selftest_philox(const uint64_t* triples, uint32_t* out, int64_t count, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(count >= 0);
+    if (count == 0) return 0;
+    VIOLA_CHECK_ARG(triples && out);
+    hipLaunchKernelGGL(selftest_philox_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, triples, out, count);
+    return viola_launch_status();
+}
+
+extern "C" int viola_abi_version(void) { return 1; }
+
+extern "C" const char* viola_error_string(int code) {
+    if (code == 0) return "success";
+    if (code == VIOLA_EINVAL) return "invalid argument (nothing launched)";
+    if (code == VIOLA_EUNSUPPORTED) return "unsupported configuration (nothing launched)";
+    return hipGetErrorString(static_cast<hipError_t>(code));
+}

@@ -1,0 +1,291 @@
+// FP8Muon elementwise kernels for gfx950: fused momentum update + e4m3 state codec (1-D tiles and
+// 2-D blocks, nearest or Philox stochastic rounding), weight update, AdamW, copy_scaled.
+// All arithmetic is un-contracted IEEE fp32 (built with -ffp-contract=off) in the order the
+// reference kernels write it. Pointers need only element alignment: accesses are per element,
+// lane-contiguous, so a wavefront still reads and writes whole cache lines.
+#include "common.hpp"
+
+namespace viola {
+
+__device__ __forceinline__ float load_dtype(const void* p, int64_t i, int dtype) {
+    if (dtype == VIOLA_F32) return static_cast<const float*>(p)[i];
+    if (dtype == VIOLA_BF16) return bf16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
+    return (float)static_cast<const _Float16*>(p)[i];
+}
+
+template <bool STOCHASTIC>
+__device__ __forceinline__ void store_rounded(void* p, int64_t i, int dtype, float v, uint64_t element, uint64_t step, uint64_t key) {
+    if (dtype == VIOLA_F32) {
+        static_cast<float*>(p)[i] = v;
+    } else if (dtype == VIOLA_BF16) {
+        if (STOCHASTIC) v = stochastic_bf16(v, element, step, key);
+        static_cast<uint16_t*>(p)[i] = f32_to_bf16_bits(v);
+    } else {
+        if (STOCHASTIC) v = stochastic_fp16(v, element, step, key);
+        static_cast<_Float16*>(p)[i] = (_Float16)v;
+    }
+}
+
+template <bool STOCHASTIC>
+__device__ __forceinline__ uint8_t encode_state(float m, float scale, uint64_t element, uint64_t step, uint64_t key) {
+    const float t = m / scale;
+    float v = t != t ? t : fminf(fmaxf(t, -448.0f), 448.0f);      // NaN (also Inf/Inf) stays NaN
+    if (STOCHASTIC) v = stochastic_e4m3(v, element, step, key);
+    return f32_to_e4m3(v);
+}
+
+// ------------------------------------------------------------------ 1-D tiles: one wavefront per tile
+template <int EPL, bool STOCHASTIC>   // EPL = tile_size / 64 elements per lane
+__global__ __launch_bounds__(256) void momentum_1d_kernel(const void* __restrict__ grad, int grad_dtype,
+                                                           const uint8_t* old_q, const float* old_scale, uint8_t* new_q,
+                                                           float* new_scale, uint16_t* __restrict__ update, int64_t n,
+                                                           int64_t blocks, float beta, float inv_loss_scale, int nesterov,
+                                                           uint64_t step, uint64_t key) {
+    constexpr int TILE = EPL * WAVE;
+    const int64_t b = (int64_t)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (b >= blocks) return;
+    const int lane = threadIdx.x % WAVE;
+    const float scale_old = old_scale[b];
+    const float one_minus = 1.0f - beta;
+    float g[EPL], m[EPL];
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) {
+        const int64_t i = b * TILE + j * WAVE + lane;
+        g[j] = 0.0f;
+        float m0 = 0.0f;
+        if (i < n) {
+            g[j] = load_dtype(grad, i, grad_dtype) * inv_loss_scale;
+            m0 = e4m3_to_f32(old_q[i]) * scale_old;
+        }
+        const float t0 = beta * m0;
+        const float t1 = one_minus * g[j];
+        m[j] = t0 + t1;
+        amax = fmaxf(amax, fabsf(m[j]));
+    }
+    amax = wave_max(amax);
+    const float scale = fmaxf(amax, 1e-30f) / 448.0f;
+    if (lane == 0) new_scale[b] = scale;
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) {
+        const int64_t i = b * TILE + j * WAVE + lane;
+        new_q[i] = encode_state<STOCHASTIC>(m[j], scale, (uint64_t)i, step, key);
+        if (i < n) {
+            float u = m[j];
+            if (nesterov) {
+                const float t0 = one_minus * g[j];
+                const float t1 = beta * m[j];
+                u = t0 + t1;
+            }
+            update[i] = f32_to_bf16_bits(u);
+        }
+    }
+}
+
+// ------------------------------------------------------------------ 2-D blocks: one wavefront per block
+template <bool STOCHASTIC>
+__global__ __launch_bounds__(256) void momentum_2d_kernel(const void* __restrict__ grad, int grad_dtype,
+                                                           const uint8_t* old_q, const float* old_scale, uint8_t* new_q,
+                                                           float* new_scale, uint16_t* __restrict__ update, int64_t planes,
+                                                           int64_t rows, int64_t cols, int tr, int tc, float beta,
+                                                           float inv_loss_scale, int nesterov, uint64_t step, uint64_t key) {
+    const int64_t nr = (rows + tr - 1) / tr, nc = (cols + tc - 1) / tc;
+    const int64_t tile = (int64_t)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (tile >= planes * nr * nc) return;
+    const int lane = threadIdx.x % WAVE;
+    const int64_t plane = tile / (nr * nc), br = tile / nc % nr, bc = tile % nc;
+    const float scale_old = old_scale[tile];
+    const float one_minus = 1.0f - beta;
+    const int size = tr * tc;
+    auto element = [&](int j, int64_t& i, float& g, float& m) -> bool {
+        const int64_t y = br * tr + j / tc, x = bc * tc + j % tc;
+        if (y >= rows || x >= cols) return false;
+        i = (plane * rows + y) * cols + x;
+        g = load_dtype(grad, i, grad_dtype) * inv_loss_scale;
+        const float t0 = beta * (e4m3_to_f32(old_q[i]) * scale_old);
+        const float t1 = one_minus * g;
+        m = t0 + t1;
+        return true;
+    };
+    float amax = 0.0f;
+    for (int j = lane; j < size; j += WAVE) {
+        int64_t i; float g, m;
+        if (element(j, i, g, m)) amax = fmaxf(amax, fabsf(m));
+    }
+    amax = wave_max(amax);
+    const float scale = fmaxf(amax, 1e-30f) / 448.0f;
+    for (int j = lane; j < size; j += WAVE) {
+        int64_t i; float g, m;
+        if (element(j, i, g, m)) {
+            new_q[i] = encode_state<STOCHASTIC>(m, scale, (uint64_t)i, step, key);
+            float u = m;
+            if (nesterov) {
+                const float t0 = one_minus * g;
+                const float t1 = beta * m;
+                u = t0 + t1;
+            }
+            update[i] = f32_to_bf16_bits(u);
+        }
+    }
+    // every lane has finished reading old_scale[tile] (held in a register) before this store
+    if (lane == 0) new_scale[tile] = scale;
+}
+
+// ------------------------------------------------------------------ elementwise updates
+template <bool STOCHASTIC>
+__global__ __launch_bounds__(256) void weight_kernel(void* weight, int weight_dtype, const void* __restrict__ grad,
+                                                      int grad_dtype, int64_t n, float lr, float decay, float update_scale,
+                                                      uint64_t step, uint64_t key, uint64_t offset) {
+    const float keep = 1.0f - lr * decay;
+    const float rate = lr * update_scale;
+    for (int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < n; j += (int64_t)gridDim.x * blockDim.x) {
+        const float t0 = load_dtype(weight, j, weight_dtype) * keep;
+        const float t1 = rate * load_dtype(grad, j, grad_dtype);
+        store_rounded<STOCHASTIC>(weight, j, weight_dtype, t0 - t1, (uint64_t)j + offset, step, key);
+    }
+}
+
+template <bool STOCHASTIC>
+__global__ __launch_bounds__(256) void adam_kernel(void* weight, int weight_dtype, const void* __restrict__ grad,
+                                                    int grad_dtype, void* first, void* second, int state_dtype, int64_t n,
+                                                    float lr, float decay, float b1, float b2, float inv_c1, float inv_c2,
+                                                    float eps, uint64_t step, uint64_t key, uint64_t offset, int adamw,
+                                                    int maximize) {
+    const float one_b1 = 1.0f - b1, one_b2 = 1.0f - b2;
+    const float keep = 1.0f - lr * decay;
+    for (int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < n; j += (int64_t)gridDim.x * blockDim.x) {
+        float w = load_dtype(weight, j, weight_dtype);
+        float g = load_dtype(grad, j, grad_dtype);
+        if (maximize) g = -g;
+        if (!adamw) { const float t = decay * w; g = g + t; }
+        const float m0 = b1 * load_dtype(first, j, state_dtype);
+        const float m1 = one_b1 * g;
+        const float m = m0 + m1;
+        const float v0 = b2 * load_dtype(second, j, state_dtype);
+        const float v1 = (one_b2 * g) * g;
+        const float v = v0 + v1;
+        store_rounded<false>(first, j, state_dtype, m, 0, 0, 0);
+        store_rounded<false>(second, j, state_dtype, v, 0, 0, 0);
+        if (adamw) w = w * keep;
+        const float numerator = lr * (m * inv_c1);
+        const float denominator = sqrtf(v * inv_c2) + eps;
+        store_rounded<STOCHASTIC>(weight, j, weight_dtype, w - numerator / denominator, (uint64_t)j + offset, step, key);
+    }
+}
+
+__global__ __launch_bounds__(256) void copy_scaled_kernel(const void* __restrict__ update, int update_dtype, void* out,
+                                                           int out_dtype, int64_t src, int64_t dst, int64_t count,
+                                                           float scale) {
+    for (int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < count; j += (int64_t)gridDim.x * blockDim.x)
+        store_rounded<false>(out, dst + j, out_dtype, load_dtype(update, src + j, update_dtype) * scale, 0, 0, 0);
+}
+
+__global__ __launch_bounds__(256) void momentum_dequantize_kernel(const uint8_t* __restrict__ q, const float* __restrict__ scale,
+                                                                   float* __restrict__ out, int64_t n, int granularity,
+                                                                   int tile_size, int64_t rows, int64_t cols, int tr, int tc) {
+    const int64_t nr = granularity ? (rows + tr - 1) / tr : 0, nc = granularity ? (cols + tc - 1) / tc : 0;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        int64_t tile;
+        if (granularity == 0) {
+            tile = i / tile_size;
+        } else {
+            const int64_t plane = i / (rows * cols), y = i / cols % rows, x = i % cols;
+            tile = (plane * nr + y / tr) * nc + x / tc;
+        }
+        out[i] = e4m3_to_f32(q[i]) * scale[tile];
+    }
+}
+
+static unsigned grid_for(int64_t n) {
+    const int64_t blocks = (n + 255) / 256;
+    return (unsigned)(blocks < 1 ? 1 : blocks > 65536 * 8 ? 65536 * 8 : blocks);
+}
+
+}  // namespace viola
+
+using namespace viola;
+
+extern "C" int viola_momentum_update(const void* grad, int grad_dtype, const void* old_q, const float* old_scale,
+                                     void* new_q, float* new_scale, void* update, int64_t n, float beta,
+                                     float inv_loss_scale, int nesterov, int granularity, int tile_size, int64_t planes,
+                                     int64_t rows, int64_t cols, int tr, int tc, int rounding, int64_t rounding_step,
+                                     int64_t rounding_key, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_float(grad_dtype) && n >= 0 && (granularity == 0 || granularity == 1));
+    VIOLA_CHECK_ARG(rounding == VIOLA_NEAREST || rounding == VIOLA_STOCHASTIC);
+    if (n == 0) return 0;
+    VIOLA_CHECK_ARG(grad && old_q && old_scale && new_q && new_scale && update);
+    const uint8_t* oq = static_cast<const uint8_t*>(old_q);
+    uint8_t* nq = static_cast<uint8_t*>(new_q);
+    uint16_t* up = static_cast<uint16_t*>(update);
+    const uint64_t step = (uint64_t)rounding_step, key = (uint64_t)rounding_key;
+    if (granularity == 0) {
+        VIOLA_CHECK_ARG(tile_size == 64 || tile_size == 128 || tile_size == 256 || tile_size == 512 || tile_size == 1024);
+        const int64_t blocks = (n + tile_size - 1) / tile_size;
+        const dim3 grid((unsigned)((blocks + 3) / 4));
+#define VIOLA_M1(EPL)                                                                                                        \
+    case EPL * 64:                                                                                                           \
+        if (rounding) hipLaunchKernelGGL((momentum_1d_kernel<EPL, true>), grid, dim3(256), 0, stream, grad, grad_dtype, oq, old_scale, nq, new_scale, up, n, blocks, beta, inv_loss_scale, nesterov, step, key); \
+        else hipLaunchKernelGGL((momentum_1d_kernel<EPL, false>), grid, dim3(256), 0, stream, grad, grad_dtype, oq, old_scale, nq, new_scale, up, n, blocks, beta, inv_loss_scale, nesterov, step, key); \
+        break;
+        switch (tile_size) { VIOLA_M1(1) VIOLA_M1(2) VIOLA_M1(4) VIOLA_M1(8) VIOLA_M1(16) }
+#undef VIOLA_M1
+        return viola_launch_status();
+    }
+    VIOLA_CHECK_ARG(planes > 0 && rows > 0 && cols > 0 && planes * rows * cols == n && tr > 0 && tc > 0 && tr * tc <= 4096);
+    const int64_t tiles = planes * ((rows + tr - 1) / tr) * ((cols + tc - 1) / tc);
+    const dim3 grid((unsigned)((tiles + 3) / 4));
+    if (rounding) hipLaunchKernelGGL((momentum_2d_kernel<true>), grid, dim3(256), 0, stream, grad, grad_dtype, oq, old_scale, nq, new_scale, up, planes, rows, cols, tr, tc, beta, inv_loss_scale, nesterov, step, key);
+    else hipLaunchKernelGGL((momentum_2d_kernel<false>), grid, dim3(256), 0, stream, grad, grad_dtype, oq, old_scale, nq, new_scale, up, planes, rows, cols, tr, tc, beta, inv_loss_scale, nesterov, step, key);
+    return viola_launch_status();
+}
+
+extern "C" int viola_weight_update(void* weight, int weight_dtype, const void* grad, int grad_dtype, int64_t n, float lr,
+                                   float decay, float update_scale, int rounding, int64_t rounding_step,
+                                   int64_t rounding_key, int64_t offset, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_float(weight_dtype) && viola_is_float(grad_dtype) && n >= 0);
+    if (n == 0) return 0;
+    VIOLA_CHECK_ARG(weight && grad);
+    if (rounding && weight_dtype != VIOLA_F32)
+        hipLaunchKernelGGL(weight_kernel<true>, dim3(grid_for(n)), dim3(256), 0, stream, weight, weight_dtype, grad, grad_dtype, n, lr, decay, update_scale, (uint64_t)rounding_step, (uint64_t)rounding_key, (uint64_t)offset);
+    else
+        hipLaunchKernelGGL(weight_kernel<false>, dim3(grid_for(n)), dim3(256), 0, stream, weight, weight_dtype, grad, grad_dtype, n, lr, decay, update_scale, (uint64_t)rounding_step, (uint64_t)rounding_key, (uint64_t)offset);
+    return viola_launch_status();
+}
+
+extern "C" int viola_adam_update(void* weight, int weight_dtype, const void* grad, int grad_dtype, void* first, void* second,
+                                 int state_dtype, int64_t n, float lr, float decay, float b1, float b2, float inv_c1,
+                                 float inv_c2, float eps, int rounding, int64_t rounding_step, int64_t rounding_key,
+                                 int64_t offset, int adamw, int maximize, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_float(weight_dtype) && viola_is_float(grad_dtype) && viola_is_float(state_dtype) && n >= 0);
+    if (n == 0) return 0;
+    VIOLA_CHECK_ARG(weight && grad && first && second);
+    if (rounding && weight_dtype != VIOLA_F32)
+        hipLaunchKernelGGL(adam_kernel<true>, dim3(grid_for(n)), dim3(256), 0, stream, weight, weight_dtype, grad, grad_dtype, first, second, state_dtype, n, lr, decay, b1, b2, inv_c1, inv_c2, eps, (uint64_t)rounding_step, (uint64_t)rounding_key, (uint64_t)offset, adamw, maximize);
+    else
+        hipLaunchKernelGGL(adam_kernel<false>, dim3(grid_for(n)), dim3(256), 0, stream, weight, weight_dtype, grad, grad_dtype, first, second, state_dtype, n, lr, decay, b1, b2, inv_c1, inv_c2, eps, (uint64_t)rounding_step, (uint64_t)rounding_key, (uint64_t)offset, adamw, maximize);
+    return viola_launch_status();
+}
+
+extern "C" int viola_copy_scaled(const void* update, int update_dtype, void* out, int out_dtype, int64_t src, int64_t dst,
+                                 int64_t count, float scale, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_float(update_dtype) && viola_is_float(out_dtype) && src >= 0 && dst >= 0 && count >= 0);
+    if (count == 0) return 0;
+    VIOLA_CHECK_ARG(update && out);
+    hipLaunchKernelGGL(copy_scaled_kernel, dim3(grid_for(count)), dim3(256), 0, stream, update, update_dtype, out, out_dtype, src, dst, count, scale);
+    return viola_launch_status();
+}
+
+extern "C" int viola_momentum_dequantize(const void* q, const float* scale, float* out, int64_t n, int granularity,
+                                         int tile_size, int64_t planes, int64_t rows, int64_t cols, int tr, int tc,
+                                         viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(n >= 0 && (granularity == 0 ? tile_size > 0 : (rows > 0 && cols > 0 && tr > 0 && tc > 0 && planes * rows * cols == n)));
+    if (n == 0) return 0;
+    VIOLA_CHECK_ARG(q && scale && out);
+    hipLaunchKernelGGL(momentum_dequantize_kernel, dim3(grid_for(n)), dim3(256), 0, stream, static_cast<const uint8_t*>(q), scale, out, n, granularity, tile_size, rows, cols, tr, tc);
+    return viola_launch_status();
+}

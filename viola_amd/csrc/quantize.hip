@@ -1,0 +1,452 @@
+// Group-scaled FP8 quantization for gfx950: one coalesced HBM read pass per call, amax by
+// wavefront/LDS reduction, IEEE fp32 division (built with -ffp-contract=off), RNE FP8 encode.
+//
+// Kernels
+//   quantize_rowwise   gr == 1, not transposed: 8 elements per lane, amax over gc/8 lanes.
+//   quantize_tile      gc == 32, gr == 1: 128 x 64 tile through LDS, emits the row-wise layout,
+//                      the quantized transpose, or both from the one read.
+//   quantize_generic   any (gr, gc), transposed or not, optional re-encode from codes+scales:
+//                      one wavefront per group, two passes over the group (second hits cache).
+//   dequantize, fp8 transpose, segmented transposed quantize for the variable-group path.
+#include "common.hpp"
+
+namespace viola {
+
+template <typename TOut>
+__device__ __forceinline__ uint8_t encode_clamped(float v, float s, float limit) {
+    const float t = v / s;
+    const float c = t != t ? t : fminf(fmaxf(t, -limit), limit);
+    return from_f32<TOut>(c).bits;
+}
+
+__device__ __forceinline__ float group_scale(float amax, float limit) { return fmaxf(amax, 1e-30f) / limit; }
+
+// ------------------------------------------------------------------ 8-element chunk loads
+template <typename TIn> struct Chunk8;
+template <> struct Chunk8<bf16_t> {
+    static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[8]) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(p);
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = __uint_as_float(w[i] << 16);
+            v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    }
+};
+template <> struct Chunk8<f16_t> {
+    static __device__ __forceinline__ void load(const f16_t* p, float (&v)[8]) {
+        typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+        const h8 raw = *reinterpret_cast<const h8*>(p);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (float)raw[i];
+    }
+};
+template <> struct Chunk8<float> {
+    static __device__ __forceinline__ void load(const float* p, float (&v)[8]) {
+        const float4 lo = *reinterpret_cast<const float4*>(p);
+        const float4 hi = *reinterpret_cast<const float4*>(p + 4);
+        v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w;
+        v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+    }
+};
+
+template <typename TOut>
+__device__ __forceinline__ uint2 encode8(const float (&v)[8], float s, float limit) {
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        lo |= (uint32_t)encode_clamped<TOut>(v[i], s, limit) << (8 * i);
+        hi |= (uint32_t)encode_clamped<TOut>(v[4 + i], s, limit) << (8 * i);
+    }
+    return make_uint2(lo, hi);
+}
+
+// ------------------------------------------------------------------ row-wise (1, GC)
+// Requires cols % 8 == 0, x aligned to 8 elements, q aligned to 8 bytes.
+template <typename TIn, typename TOut, int GC>
+__global__ __launch_bounds__(256) void quantize_rowwise(const TIn* __restrict__ x, uint8_t* __restrict__ q,
+                                                         float* __restrict__ scale, int64_t rows, int64_t cols,
+                                                         int64_t nc, float limit) {
+    constexpr int LANES = GC / 8;                         // lanes that share one group
+    const int64_t chunks_per_row = nc * LANES;
+    const int64_t chunk = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t row = chunk / chunks_per_row;
+    const int64_t c0 = (chunk % chunks_per_row) * 8;
+    const bool valid = row < rows && c0 < cols;
+    float v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (valid) Chunk8<TIn>::load(x + row * cols + c0, v);
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+    amax = group_max<LANES>(amax);
+    const float s = group_scale(amax, limit);
+    if (valid) {
+        *reinterpret_cast<uint2*>(q + row * cols + c0) = encode8<TOut>(v, s, limit);
+        if ((threadIdx.x & (LANES - 1)) == 0) scale[row * nc + c0 / GC] = s;
+    }
+}
+
+// ------------------------------------------------------------------ 128 x 64 tile, gc = 32
+// ROWWISE: q [rows, cols], scale [rows, ceil(cols/32)].
+// TRANSPOSED: qt [cols, rows], scale_t [cols, ceil(rows/32)], 32-wide groups along rows.
+// VEC: cols % 8 == 0 and x aligned to 8 elements (16-byte loads); otherwise scalar loads.
+constexpr int TILE_R = 128, TILE_C = 64, TILE_LD = TILE_C + 1;
+
+template <typename TIn, bool VEC>
+__device__ __forceinline__ void load_tile(const TIn* __restrict__ x, float* tile, int64_t r0, int64_t c0,
+                                          int64_t rows, int64_t cols) {
+    if constexpr (VEC) {
+#pragma unroll
+        for (int it = 0; it < TILE_R * TILE_C / 8 / 256; ++it) {
+            const int id = it * 256 + threadIdx.x;
+            const int r = id / (TILE_C / 8), ch = id % (TILE_C / 8);
+            float v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (r0 + r < rows && c0 + ch * 8 < cols) Chunk8<TIn>::load(x + (r0 + r) * cols + c0 + ch * 8, v);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) tile[r * TILE_LD + ch * 8 + i] = v[i];
+        }
+    } else {
+        for (int id = threadIdx.x; id < TILE_R * TILE_C; id += 256) {
+            const int r = id / TILE_C, c = id % TILE_C;
+            float v = 0.0f;
+            if (r0 + r < rows && c0 + c < cols) v = to_f32(x[(r0 + r) * cols + c0 + c]);
+            tile[r * TILE_LD + c] = v;
+        }
+    }
+}
+
+// Encode 32 values held by one lane and store them at dst (a run of `count` <= 32 valid bytes).
+template <typename TOut>
+__device__ __forceinline__ void store_group32(const float (&v)[32], float s, float limit, uint8_t* dst, int count,
+                                              bool aligned16) {
+    uint32_t w[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        w[i] = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) w[i] |= (uint32_t)encode_clamped<TOut>(v[4 * i + j], s, limit) << (8 * j);
+    }
+    if (count == 32 && aligned16) {
+        reinterpret_cast<uint4*>(dst)[0] = make_uint4(w[0], w[1], w[2], w[3]);
+        reinterpret_cast<uint4*>(dst)[1] = make_uint4(w[4], w[5], w[6], w[7]);
+    } else {
+        for (int i = 0; i < count; ++i) dst[i] = (uint8_t)(w[i >> 2] >> (8 * (i & 3)));
+    }
+}
+
+template <typename TIn, typename TOut, bool ROWWISE, bool TRANSPOSED, bool VEC>
+__global__ __launch_bounds__(256) void quantize_tile(const TIn* __restrict__ x, uint8_t* __restrict__ q,
+                                                      float* __restrict__ scale, uint8_t* __restrict__ qt,
+                                                      float* __restrict__ scale_t, int64_t rows, int64_t cols,
+                                                      float limit) {
+    __shared__ float tile[TILE_R * TILE_LD];
+    const int64_t r0 = (int64_t)blockIdx.y * TILE_R, c0 = (int64_t)blockIdx.x * TILE_C;
+    load_tile<TIn, VEC>(x, tile, r0, c0, rows, cols);
+    __syncthreads();
+    const int t = threadIdx.x;
+    if constexpr (ROWWISE) {
+        const int r = t % TILE_R, g = t / TILE_R;                       // 128 rows x 2 column groups
+        const int64_t row = r0 + r, col = c0 + g * 32;
+        if (row < rows && col < cols) {
+            float v[32];
+            float amax = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 32; ++i) {
+                v[i] = tile[r * TILE_LD + g * 32 + i];
+                amax = fmaxf(amax, fabsf(v[i]));
+            }
+            const float s = group_scale(amax, limit);
+            const int64_t nc = (cols + 31) / 32;
+            scale[row * nc + col / 32] = s;
+            const int count = (int)(cols - col < 32 ? cols - col : 32);
+            uint8_t* dst = q + row * cols + col;
+            store_group32<TOut>(v, s, limit, dst, count, (reinterpret_cast<uintptr_t>(dst) & 15) == 0);
+        }
+    }
+    if constexpr (TRANSPOSED) {
+        const int c = t % TILE_C, g = t / TILE_C;                       // 64 columns x 4 row groups
+        const int64_t col = c0 + c, row = r0 + g * 32;
+        if (col < cols && row < rows) {
+            float v[32];
+            float amax = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 32; ++i) {
+                v[i] = tile[(g * 32 + i) * TILE_LD + c];
+                amax = fmaxf(amax, fabsf(v[i]));
+            }
+            const float s = group_scale(amax, limit);
+            const int64_t nr = (rows + 31) / 32;
+            scale_t[col * nr + row / 32] = s;
+            const int count = (int)(rows - row < 32 ? rows - row : 32);
+            uint8_t* dst = qt + col * rows + row;
+            store_group32<TOut>(v, s, limit, dst, count, (reinterpret_cast<uintptr_t>(dst) & 15) == 0);
+        }
+    }
+}
+
+// ------------------------------------------------------------------ generic: one wavefront per group
+template <typename TIn, typename TOut, bool ENCODED>
+__global__ __launch_bounds__(256) void quantize_generic(const TIn* __restrict__ x, const float* __restrict__ source_scale,
+                                                         uint8_t* __restrict__ q, float* __restrict__ scale,
+                                                         int64_t rows, int64_t cols, int gr, int gc, int transposed,
+                                                         int source_gr, int source_gc, float limit) {
+    const int64_t out_rows = transposed ? cols : rows, out_cols = transposed ? rows : cols;
+    const int64_t nr = (out_rows + gr - 1) / gr, nc = (out_cols + gc - 1) / gc;
+    const int64_t group = (int64_t)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (group >= nr * nc) return;                                       // whole wavefront leaves together
+    const int lane = threadIdx.x % WAVE;
+    const int64_t gr0 = group / nc * gr, gc0 = group % nc * gc;
+    const int64_t sc = ENCODED ? (cols + source_gc - 1) / source_gc : 0;
+    const int size = gr * gc;
+    auto value = [&](int j, bool& inside) -> float {
+        const int64_t r = gr0 + j / gc, c = gc0 + j % gc;
+        const int64_t xr = transposed ? c : r, xc = transposed ? r : c;
+        inside = r < out_rows && c < out_cols;
+        if (!inside) return 0.0f;
+        float v = to_f32(x[xr * cols + xc]);
+        if constexpr (ENCODED) v *= source_scale[xr / source_gr * sc + xc / source_gc];
+        return v;
+    };
+    float amax = 0.0f;
+    for (int j = lane; j < size; j += WAVE) {
+        bool inside;
+        amax = fmaxf(amax, fabsf(value(j, inside)));
+    }
+    amax = wave_max(amax);
+    const float s = group_scale(amax, limit);
+    if (lane == 0) scale[group] = s;
+    for (int j = lane; j < size; j += WAVE) {
+        bool inside;
+        const float v = value(j, inside);
+        if (inside) q[(gr0 + j / gc) * out_cols + gc0 + j % gc] = encode_clamped<TOut>(v, s, limit);
+    }
+}
+
+// ------------------------------------------------------------------ dequantize
+template <typename TQ>
+__global__ __launch_bounds__(256) void dequantize_kernel(const TQ* __restrict__ q, const float* __restrict__ scale,
+                                                          float* __restrict__ out, int64_t rows, int64_t cols, int gr,
+                                                          int gc) {
+    const int64_t nc = (cols + gc - 1) / gc;
+    const int64_t total = rows * cols;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t r = i / cols, c = i % cols;
+        out[i] = to_f32(q[i]) * scale[r / gr * nc + c / gc];
+    }
+}
+
+// ------------------------------------------------------------------ byte transpose, 64 x 64 tile
+__global__ __launch_bounds__(256) void transpose_bytes(const uint8_t* __restrict__ x, uint8_t* __restrict__ out,
+                                                        int64_t rows, int64_t cols) {
+    __shared__ uint8_t tile[64][64 + 4];
+    const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+    for (int id = threadIdx.x; id < 64 * 64; id += 256) {
+        const int r = id / 64, c = id % 64;
+        tile[r][c] = (r0 + r < rows && c0 + c < cols) ? x[(r0 + r) * cols + c0 + c] : 0;
+    }
+    __syncthreads();
+    for (int id = threadIdx.x; id < 64 * 64; id += 256) {
+        const int c = id / 64, r = id % 64;
+        if (r0 + r < rows && c0 + c < cols) out[(c0 + c) * rows + r0 + r] = tile[r][c];
+    }
+}
+
+// ------------------------------------------------------------------ segmented transposed quantize
+// One block per (64 columns, 32-token slot of the padded token axis). Slot s of group g covers
+// rows offsets[g] + 32*(s - poffsets[g]/32) ...; rows past the group's end are zero.
+template <typename TIn, typename TOut>
+__global__ __launch_bounds__(64) void quantize_transposed_segmented(const TIn* __restrict__ x,
+                                                                     const int64_t* __restrict__ offsets,
+                                                                     const int64_t* __restrict__ poffsets, int groups,
+                                                                     int64_t cols, int64_t t_total,
+                                                                     uint8_t* __restrict__ qt, float* __restrict__ scale_t,
+                                                                     float limit) {
+    const int64_t slot = blockIdx.y;
+    const int64_t col = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    const int64_t token = slot * 32;
+    int g = 0;
+    while (g + 1 < groups && poffsets[g + 1] <= token) ++g;
+    if (col >= cols) return;
+    const int64_t first = offsets[g] + (token - poffsets[g]);
+    const int64_t end = offsets[g + 1];
+    float v[32];
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+        v[i] = first + i < end ? to_f32(x[(first + i) * cols + col]) : 0.0f;
+        amax = fmaxf(amax, fabsf(v[i]));
+    }
+    const float s = group_scale(amax, limit);
+    scale_t[col * (t_total / 32) + slot] = s;
+    uint8_t* dst = qt + col * t_total + token;
+    store_group32<TOut>(v, s, limit, dst, 32, (reinterpret_cast<uintptr_t>(dst) & 15) == 0);
+}
+
+// ------------------------------------------------------------------ host dispatch
+template <typename TIn, typename TOut>
+static int launch_quantize(const void* x, int64_t rows, int64_t cols, void* q, float* scale, int gr, int gc,
+                           float limit, int transposed, hipStream_t stream) {
+    const TIn* xp = static_cast<const TIn*>(x);
+    uint8_t* qp = static_cast<uint8_t*>(q);
+    const bool vec = cols % 8 == 0 && reinterpret_cast<uintptr_t>(x) % (8 * sizeof(TIn)) == 0;
+    if (gr == 1 && !transposed && vec && reinterpret_cast<uintptr_t>(q) % 8 == 0 && gc <= 512) {
+        const int64_t nc = (cols + gc - 1) / gc;
+        const int64_t chunks = rows * nc * (gc / 8);
+        const dim3 grid((unsigned)((chunks + 255) / 256));
+#define VIOLA_ROWWISE(GC) \
+    case GC: hipLaunchKernelGGL((quantize_rowwise<TIn, TOut, GC>), grid, dim3(256), 0, stream, xp, qp, scale, rows, cols, nc, limit); break;
+        switch (gc) {
+            VIOLA_ROWWISE(32) VIOLA_ROWWISE(64) VIOLA_ROWWISE(128) VIOLA_ROWWISE(256) VIOLA_ROWWISE(512)
+            default: return VIOLA_EINVAL;
+        }
+#undef VIOLA_ROWWISE
+        return viola_launch_status();
+    }
+    if (gr == 1 && gc == 32 && transposed) {
+        const dim3 grid((unsigned)((cols + TILE_C - 1) / TILE_C), (unsigned)((rows + TILE_R - 1) / TILE_R));
+        if (vec) hipLaunchKernelGGL((quantize_tile<TIn, TOut, false, true, true>), grid, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit);
+        else hipLaunchKernelGGL((quantize_tile<TIn, TOut, false, true, false>), grid, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit);
+        return viola_launch_status();
+    }
+    const int64_t out_rows = transposed ? cols : rows, out_cols = transposed ? rows : cols;
+    const int64_t ngroups = ((out_rows + gr - 1) / gr) * ((out_cols + gc - 1) / gc);
+    hipLaunchKernelGGL((quantize_generic<TIn, TOut, false>), dim3((unsigned)((ngroups + 3) / 4)), dim3(256), 0, stream,
+                       xp, nullptr, qp, scale, rows, cols, gr, gc, transposed, 1, 32, limit);
+    return viola_launch_status();
+}
+
+template <typename TOut>
+static int dispatch_in(int x_dtype, const void* x, int64_t rows, int64_t cols, void* q, float* scale, int gr, int gc,
+                       float limit, int transposed, hipStream_t stream) {
+    switch (x_dtype) {
+        case VIOLA_F32: return launch_quantize<float, TOut>(x, rows, cols, q, scale, gr, gc, limit, transposed, stream);
+        case VIOLA_BF16: return launch_quantize<bf16_t, TOut>(x, rows, cols, q, scale, gr, gc, limit, transposed, stream);
+        case VIOLA_F16: return launch_quantize<f16_t, TOut>(x, rows, cols, q, scale, gr, gc, limit, transposed, stream);
+        default: return VIOLA_EINVAL;
+    }
+}
+
+template <typename TIn, typename TOut>
+static int launch_reencode(const void* x, const float* source_scale, int64_t rows, int64_t cols, void* q, float* scale,
+                           int gr, int gc, float limit, int transposed, int sgr, int sgc, hipStream_t stream) {
+    const int64_t out_rows = transposed ? cols : rows, out_cols = transposed ? rows : cols;
+    const int64_t ngroups = ((out_rows + gr - 1) / gr) * ((out_cols + gc - 1) / gc);
+    hipLaunchKernelGGL((quantize_generic<TIn, TOut, true>), dim3((unsigned)((ngroups + 3) / 4)), dim3(256), 0, stream,
+                       static_cast<const TIn*>(x), source_scale, static_cast<uint8_t*>(q), scale, rows, cols, gr, gc,
+                       transposed, sgr, sgc, limit);
+    return viola_launch_status();
+}
+
+template <typename TIn, typename TOut>
+static int launch_dual(const void* x, int64_t rows, int64_t cols, void* q, float* scale, void* qt, float* scale_t,
+                       float limit, hipStream_t stream) {
+    const bool vec = cols % 8 == 0 && reinterpret_cast<uintptr_t>(x) % (8 * sizeof(TIn)) == 0;
+    const dim3 grid((unsigned)((cols + TILE_C - 1) / TILE_C), (unsigned)((rows + TILE_R - 1) / TILE_R));
+    const TIn* xp = static_cast<const TIn*>(x);
+    if (vec) hipLaunchKernelGGL((quantize_tile<TIn, TOut, true, true, true>), grid, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale, static_cast<uint8_t*>(qt), scale_t, rows, cols, limit);
+    else hipLaunchKernelGGL((quantize_tile<TIn, TOut, true, true, false>), grid, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale, static_cast<uint8_t*>(qt), scale_t, rows, cols, limit);
+    return viola_launch_status();
+}
+
+template <typename TIn, typename TOut>
+static int launch_segmented(const void* x, int64_t cols, const int64_t* offsets, const int64_t* poffsets, int groups,
+                            int64_t t_total, void* qt, float* scale_t, float limit, hipStream_t stream) {
+    const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)(t_total / 32));
+    hipLaunchKernelGGL((quantize_transposed_segmented<TIn, TOut>), grid, dim3(64), 0, stream, static_cast<const TIn*>(x),
+                       offsets, poffsets, groups, cols, t_total, static_cast<uint8_t*>(qt), scale_t, limit);
+    return viola_launch_status();
+}
+
+static bool pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
+
+}  // namespace viola
+
+using namespace viola;
+
+extern "C" int viola_group_quantize(const void* x, int x_dtype, int64_t rows, int64_t cols, void* q, int q_dtype,
+                                    float* scale, int gr, int gc, float limit, int transposed,
+                                    const float* source_scale, int source_gr, int source_gc, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_fp8(q_dtype) && rows >= 0 && cols >= 0 && pow2(gr) && pow2(gc) && limit > 0.0f);
+    if (rows == 0 || cols == 0) return 0;
+    VIOLA_CHECK_ARG(x && q && scale);
+    if (source_scale) {
+        VIOLA_CHECK_ARG(viola_is_fp8(x_dtype) && source_gr > 0 && source_gc > 0);
+#define VIOLA_RE(TI, TO) return launch_reencode<TI, TO>(x, source_scale, rows, cols, q, scale, gr, gc, limit, transposed, source_gr, source_gc, stream)
+        if (x_dtype == VIOLA_E4M3 && q_dtype == VIOLA_E4M3) VIOLA_RE(e4m3_t, e4m3_t);
+        if (x_dtype == VIOLA_E4M3 && q_dtype == VIOLA_E5M2) VIOLA_RE(e4m3_t, e5m2_t);
+        if (x_dtype == VIOLA_E5M2 && q_dtype == VIOLA_E4M3) VIOLA_RE(e5m2_t, e4m3_t);
+        VIOLA_RE(e5m2_t, e5m2_t);
+#undef VIOLA_RE
+    }
+    VIOLA_CHECK_ARG(viola_is_float(x_dtype));
+    if (q_dtype == VIOLA_E4M3) return dispatch_in<e4m3_t>(x_dtype, x, rows, cols, q, scale, gr, gc, limit, transposed, stream);
+    return dispatch_in<e5m2_t>(x_dtype, x, rows, cols, q, scale, gr, gc, limit, transposed, stream);
+}
+
+extern "C" int viola_group_quantize_dual(const void* x, int x_dtype, int64_t rows, int64_t cols, void* q, float* scale,
+                                         void* qt, float* scale_t, int q_dtype, int gc, float limit,
+                                         viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_fp8(q_dtype) && viola_is_float(x_dtype) && rows >= 0 && cols >= 0 && limit > 0.0f);
+    if (gc != 32) return VIOLA_EUNSUPPORTED;
+    if (rows == 0 || cols == 0) return 0;
+    VIOLA_CHECK_ARG(x && q && scale && qt && scale_t);
+#define VIOLA_DUAL(TI, TO) return launch_dual<TI, TO>(x, rows, cols, q, scale, qt, scale_t, limit, stream)
+    if (q_dtype == VIOLA_E4M3) {
+        if (x_dtype == VIOLA_F32) VIOLA_DUAL(float, e4m3_t);
+        if (x_dtype == VIOLA_BF16) VIOLA_DUAL(bf16_t, e4m3_t);
+        VIOLA_DUAL(f16_t, e4m3_t);
+    }
+    if (x_dtype == VIOLA_F32) VIOLA_DUAL(float, e5m2_t);
+    if (x_dtype == VIOLA_BF16) VIOLA_DUAL(bf16_t, e5m2_t);
+    VIOLA_DUAL(f16_t, e5m2_t);
+#undef VIOLA_DUAL
+}
+
+extern "C" int viola_varlen_quantize_transposed(const void* x, int x_dtype, int64_t rows, int64_t cols,
+                                                const int64_t* offsets, const int64_t* poffsets, int groups,
+                                                int64_t t_total, void* qt, float* scale_t, int q_dtype, float limit,
+                                                viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_fp8(q_dtype) && viola_is_float(x_dtype) && rows >= 0 && cols >= 0 && groups > 0);
+    VIOLA_CHECK_ARG(t_total >= 0 && t_total % 32 == 0 && limit > 0.0f);
+    if (t_total == 0 || cols == 0) return 0;
+    VIOLA_CHECK_ARG(x && offsets && poffsets && qt && scale_t && t_total / 32 <= 65535);
+#define VIOLA_SEG(TI, TO) return launch_segmented<TI, TO>(x, cols, offsets, poffsets, groups, t_total, qt, scale_t, limit, stream)
+    if (q_dtype == VIOLA_E4M3) {
+        if (x_dtype == VIOLA_F32) VIOLA_SEG(float, e4m3_t);
+        if (x_dtype == VIOLA_BF16) VIOLA_SEG(bf16_t, e4m3_t);
+        VIOLA_SEG(f16_t, e4m3_t);
+    }
+    if (x_dtype == VIOLA_F32) VIOLA_SEG(float, e5m2_t);
+    if (x_dtype == VIOLA_BF16) VIOLA_SEG(bf16_t, e5m2_t);
+    VIOLA_SEG(f16_t, e5m2_t);
+#undef VIOLA_SEG
+}
+
+extern "C" int viola_group_dequantize(const void* q, int q_dtype, const float* scale, int64_t rows, int64_t cols, int gr,
+                                      int gc, float* out, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_fp8(q_dtype) && rows >= 0 && cols >= 0 && gr > 0 && gc > 0);
+    if (rows == 0 || cols == 0) return 0;
+    VIOLA_CHECK_ARG(q && scale && out);
+    const int64_t total = rows * cols;
+    const unsigned blocks = (unsigned)((total + 255) / 256 < 65536 * 16 ? (total + 255) / 256 : 65536 * 16);
+    if (q_dtype == VIOLA_E4M3)
+        hipLaunchKernelGGL(dequantize_kernel<e4m3_t>, dim3(blocks), dim3(256), 0, stream, static_cast<const e4m3_t*>(q), scale, out, rows, cols, gr, gc);
+    else
+        hipLaunchKernelGGL(dequantize_kernel<e5m2_t>, dim3(blocks), dim3(256), 0, stream, static_cast<const e5m2_t*>(q), scale, out, rows, cols, gr, gc);
+    return viola_launch_status();
+}
+
+extern "C" int viola_fp8_transpose(const void* x, void* out, int64_t rows, int64_t cols, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(rows >= 0 && cols >= 0);
+    if (rows == 0 || cols == 0) return 0;
+    VIOLA_CHECK_ARG(x && out && (rows + 63) / 64 <= 65535);
+    hipLaunchKernelGGL(transpose_bytes, dim3((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64)), dim3(256), 0, stream,
+                       static_cast<const uint8_t*>(x), static_cast<uint8_t*>(out), rows, cols);
+    return viola_launch_status();
+}

@@ -1,0 +1,103 @@
+"""Group-scaled FP8 quantization and GEMM operators (operator seam of
+viola/nn/_grouped_kernels.py: scale_shape :16, dequantize :44, quantize :127,
+transpose_group :161, transpose :166, gemm :310), each one call into libviola_hip.
+
+FP32 scales only; the reference's `native=True` (E8M0 / MXFP8) variant is not built.
+"""
+
+import torch
+
+from .. import _lib
+from ._linear_kernels import transpose as transpose_payload
+
+
+def scale_shape(shape, group):
+    return tuple(-(-n // g) for n, g in zip(shape, group))
+
+
+def _no_native(native):
+    if native:
+        raise NotImplementedError("MXFP8 (E8M0 scales) is not built in viola_amd; use FP32 group scales")
+
+
+def dequantize(q, scale, group):
+    """fp32 [rows, cols] = float(q) * scale[r // gr, c // gc]."""
+    assert q.is_cuda, "viola_amd kernels run on the GPU only"
+    q = q.contiguous()
+    out = torch.empty(q.shape, device=q.device, dtype=torch.float32)
+    _lib.call("viola_group_dequantize", _lib.ptr(q), _lib.code(q.dtype), _lib.ptr(scale.contiguous()),
+              q.shape[0], q.shape[1], group[0], group[1], _lib.ptr(out))
+    return out
+
+
+def quantize(x, dtype, group, *, native=False, limit=None, transposed=False,
+             source_scale=None, source_group=(1, 32), out=None, scale_out=None):
+    """Group amax quantization of a 2-D tensor; returns (codes, fp32 scales).
+
+    transposed=True yields the quantized transpose (codes [cols, rows]) with the groups laid
+    along the new last dimension, read straight from the floating input. source_scale re-encodes
+    existing codes. out/scale_out let the caller own the outputs (nothing is allocated then).
+    """
+    _no_native(native)
+    assert x.is_cuda and x.dim() == 2, "viola_amd kernels run on the GPU only"
+    x = x.contiguous()
+    shape = tuple(x.shape[::-1]) if transposed else tuple(x.shape)
+    limit = torch.finfo(dtype).max if limit is None else limit
+    q = out if out is not None else torch.empty(shape, device=x.device, dtype=dtype)
+    s = scale_out if scale_out is not None else torch.empty(scale_shape(shape, group), device=x.device, dtype=torch.float32)
+    assert q.is_contiguous() and s.is_contiguous() and tuple(q.shape) == shape and tuple(s.shape) == scale_shape(shape, group)
+    source = source_scale.contiguous() if source_scale is not None else None
+    _lib.call("viola_group_quantize", _lib.ptr(x), _lib.code(x.dtype), x.shape[0], x.shape[1],
+              _lib.ptr(q), _lib.code(q.dtype), _lib.ptr(s), group[0], group[1], float(limit), int(transposed),
+              _lib.ptr(source), source_group[0], source_group[1])
+    return q, s
+
+
+def quantize_dual(x, dtype, group, *, limit=None):
+    """Row-wise codes/scales and the quantized transpose of x from ONE read of x.
+
+    Same values as quantize(x, ...) and quantize(x, ..., transposed=True); 1-D groups of 32 only.
+    Returns (q, s, qt, st).
+    """
+    assert x.is_cuda and x.dim() == 2 and tuple(group) == (1, 32)
+    x = x.contiguous()
+    rows, cols = x.shape
+    limit = torch.finfo(dtype).max if limit is None else limit
+    q = torch.empty((rows, cols), device=x.device, dtype=dtype)
+    s = torch.empty(scale_shape((rows, cols), group), device=x.device, dtype=torch.float32)
+    qt = torch.empty((cols, rows), device=x.device, dtype=dtype)
+    st = torch.empty(scale_shape((cols, rows), group), device=x.device, dtype=torch.float32)
+    _lib.call("viola_group_quantize_dual", _lib.ptr(x), _lib.code(x.dtype), rows, cols, _lib.ptr(q), _lib.ptr(s),
+              _lib.ptr(qt), _lib.ptr(st), _lib.code(dtype), group[1], float(limit))
+    return q, s, qt, st
+
+
+def transpose_group(group):
+    """A 2-D block (>= 32 rows) transposes exactly; a 1-D row group keeps its shape and needs new K groups."""
+    return tuple(group[::-1]) if group[0] >= 32 else tuple(group)
+
+
+def transpose(q, scale, group, *, native=False, limit=None):
+    _no_native(native)
+    if group[0] >= 32:
+        return transpose_payload(q), scale.T.contiguous()
+    return quantize(q, q.dtype, group, limit=limit, transposed=True, source_scale=scale, source_group=group)
+
+
+def gemm(a, b, sa, sb, group_a, group_b, *, out_dtype, native=False, bias=None, autotune=False,
+         accum_dtype="fp32", accum_block_size=0, accum_reduce_dtype="fp32"):
+    """out[m, n] = sum over 32-wide K groups of (a_codes . b_codes^T) * sa * sb (+ bias); a [m, k], b [n, k]."""
+    _no_native(native)
+    if accum_dtype != "fp32" or accum_block_size or accum_reduce_dtype != "fp32":
+        raise NotImplementedError("viola_amd accumulates in FP32 only (blocked FP16 accumulation is not built)")
+    assert a.is_cuda and b.is_cuda and a.shape[1] == b.shape[1]
+    a, b, sa, sb = a.contiguous(), b.contiguous(), sa.contiguous(), sb.contiguous()
+    m, k = a.shape
+    n = b.shape[0]
+    assert tuple(sa.shape) == scale_shape((m, k), group_a) and tuple(sb.shape) == scale_shape((n, k), group_b)
+    out = torch.empty((m, n), device=a.device, dtype=out_dtype)
+    bias_c = bias.contiguous() if bias is not None else None
+    _lib.call("viola_group_gemm", _lib.ptr(a), _lib.code(a.dtype), _lib.ptr(b), _lib.code(b.dtype), _lib.ptr(sa), _lib.ptr(sb),
+              m, n, k, group_a[0], group_a[1], group_b[0], group_b[1],
+              _lib.ptr(bias_c), _lib.code(bias_c.dtype) if bias_c is not None else 0, _lib.ptr(out), _lib.code(out_dtype))
+    return out

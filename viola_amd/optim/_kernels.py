@@ -1,0 +1,78 @@
+"""FP8Muon kernel operators (operator seam of viola/optim/_kernels.py: state_sizes :61, dequantize
+:73, momentum_update :300, copy_scaled :318, weight_update :325, adam_update :331)."""
+
+import math
+
+import torch
+
+from .. import _lib
+
+
+def state_sizes(shape, *, granularity="tile", tile_size=256, block_shape=(16, 16)):
+    """(FP8 payload elements, scale count). 1-D tiles pad the payload; 2-D blocks do not."""
+    n = math.prod(shape)
+    if granularity == "tile":
+        blocks = -(-n // tile_size)
+        return blocks * tile_size, blocks
+    rows, cols = shape[-2:]
+    tr, tc = block_shape
+    return n, math.prod(shape[:-2]) * (-(-rows // tr)) * (-(-cols // tc))
+
+
+def _geometry(n, granularity, tile_size, block_shape, matrix_shape):
+    if granularity == "tile":
+        return 0, int(tile_size), 1, 1, 1, 1, 1
+    rows, cols = matrix_shape[-2:]
+    planes = math.prod(matrix_shape[:-2])
+    assert planes * rows * cols == n
+    return 1, 0, planes, rows, cols, int(block_shape[0]), int(block_shape[1])
+
+
+def dequantize(q, scales, shape, *, granularity="tile", tile_size=256, block_shape=(16, 16)):
+    """Diagnostic: fp32 momentum of `shape` from the FP8 payload and its scales (flat)."""
+    n = math.prod(shape)
+    out = torch.empty(n, device=q.device, dtype=torch.float32)
+    geometry = _geometry(n, granularity, tile_size, block_shape, shape)
+    _lib.call("viola_momentum_dequantize", _lib.ptr(q), _lib.ptr(scales), _lib.ptr(out), n, *geometry)
+    return out
+
+
+def momentum_update(grad, q, scales, next_q, next_scales, out, *, beta, tile_size=256, nesterov=True,
+                    loss_scale=1.0, granularity="tile", block_shape=(16, 16), matrix_shape=None,
+                    rounding="nearest", rounding_step=0, rounding_key=0):
+    """m = beta*deq(q) + (1-beta)*grad/loss_scale; (next_q, next_scales) = e4m3 tiles of m;
+    out = bf16 update (Nesterov or plain). q/next_q and scales/next_scales may alias."""
+    assert grad.is_cuda and out.dtype == torch.bfloat16
+    flat = grad.reshape(-1)
+    n = flat.numel()
+    geometry = _geometry(n, granularity, tile_size, block_shape, matrix_shape)
+    _lib.call("viola_momentum_update", _lib.ptr(flat), _lib.code(flat.dtype), _lib.ptr(q), _lib.ptr(scales),
+              _lib.ptr(next_q), _lib.ptr(next_scales), _lib.ptr(out), n, float(beta), 1.0 / float(loss_scale),
+              int(bool(nesterov)), *geometry, _lib.ROUNDING[rounding], int(rounding_step), int(rounding_key))
+
+
+def copy_scaled(update, partition, src, dst, count, scale):
+    flat = update.contiguous().view(-1)
+    _lib.call("viola_copy_scaled", _lib.ptr(flat), _lib.code(flat.dtype), _lib.ptr(partition), _lib.code(partition.dtype),
+              int(src), int(dst), int(count), float(scale))
+
+
+def weight_update(weight, grad, lr, weight_decay, *, update_scale=1.0, rounding="nearest", step=0, key=0, offset=0):
+    """weight = weight*(1 - lr*wd) - lr*update_scale*grad in fp32, stored in weight's dtype."""
+    assert weight.is_cuda and weight.is_contiguous()
+    flat = grad.reshape(-1)
+    _lib.call("viola_weight_update", _lib.ptr(weight), _lib.code(weight.dtype), _lib.ptr(flat), _lib.code(flat.dtype),
+              weight.numel(), float(lr), float(weight_decay), float(update_scale), _lib.ROUNDING[rounding],
+              int(step), int(key), int(offset))
+
+
+def adam_update(weight, grad, first, second, *, lr, weight_decay, betas, eps, step, rounding="nearest", key=0,
+                offset=0, adamw=True, maximize=False, bias_correction=True):
+    assert weight.is_cuda and weight.is_contiguous() and first.dtype == second.dtype
+    b1, b2 = betas
+    flat = grad.reshape(-1)
+    _lib.call("viola_adam_update", _lib.ptr(weight), _lib.code(weight.dtype), _lib.ptr(flat), _lib.code(flat.dtype),
+              _lib.ptr(first), _lib.ptr(second), _lib.code(first.dtype), weight.numel(), float(lr), float(weight_decay),
+              float(b1), float(b2), 1. / (1. - b1 ** step) if bias_correction else 1.,
+              1. / (1. - b2 ** step) if bias_correction else 1., float(eps), _lib.ROUNDING[rounding],
+              int(step - 1), int(key), int(offset), int(bool(adamw)), int(bool(maximize)))

@@ -1,0 +1,133 @@
+"""FP8Muon: Muon with one e4m3 momentum buffer + FP32 tile scales per matrix, AdamW for vectors
+(viola/optim/muon.py:14-141). Every arithmetic step is a HIP kernel: fused momentum/codec,
+Newton-Schulz GEMM chain, weight update, AdamW."""
+
+import os
+import warnings
+
+import torch
+
+from .matrix import MatrixOptimizer
+from ..precision import _dtype, settings
+from ._kernels import adam_update, momentum_update, state_sizes, weight_update
+from ._orthogonalize import METHODS
+
+_MODES = {"fast": (256, 3), "balanced": (256, 5), "stable": (128, 5)}
+_MASK63 = (1 << 63) - 1
+
+
+def _shape(param, group):
+    """Conv filters flatten to [out, -1]; batched=True keeps the leading dims as independent matrices."""
+    return tuple(param.shape) if group["batched"] else (param.shape[0], param.numel() // param.shape[0])
+
+
+def _use_muon(param, group):
+    return param.ndim >= 2 if group["use_muon"] is None else group["use_muon"]
+
+
+class FP8Muon(MatrixOptimizer):
+    """Matrices use Muon, vectors AdamW; `use_muon=False` on a group forces AdamW (embeddings, heads).
+
+    State per matrix: {"step", "momentum_q" uint8 payload, "momentum_scale" fp32}; per vector:
+    {"step", "exp_avg", "exp_avg_sq"}.
+    """
+
+    def __init__(self, params, lr=1e-3, *, weight_decay=0., momentum=.95, nesterov=True, mode="balanced",
+                 granularity="tile", tile_size=None, block_shape=None, rounding="nearest", rounding_seed=0,
+                 ns_steps=None, ns_method="standard", ns_backend="torch", ns_autotune=True,
+                 adjust_lr_fn="match_rms_adamw", betas=(.9, .95), eps=1e-8, adam_state_dtype="fp32",
+                 skip_nonfinite=False, shard_state=True):
+        tile_default, steps_default = _MODES[mode]
+        policy = settings()
+        defaults = dict(
+            lr=lr, weight_decay=weight_decay, momentum=momentum, nesterov=nesterov, use_muon=None, batched=False,
+            granularity=granularity, tile_size=tile_default if tile_size is None else tile_size,
+            block_shape=(16, 16) if block_shape is None else tuple(block_shape),
+            rounding=rounding, rounding_seed=rounding_seed,
+            ns_steps=steps_default if ns_steps is None else ns_steps, ns_method=ns_method,
+            ns_backend=ns_backend, ns_autotune=ns_autotune, adjust_lr_fn=adjust_lr_fn, betas=betas, eps=eps,
+            adam_state_dtype=_dtype(adam_state_dtype), master_rounding=policy["master_rounding"],
+            master_rounding_seed=policy["master_rounding_seed"])
+        self.observer = None
+        self._workspace = {}
+        super().__init__(params, defaults, shard_state=shard_state, skip_nonfinite=skip_nonfinite)
+
+    def add_param_group(self, group):
+        super().add_param_group(group)
+        group = self.param_groups[-1]
+        assert group["lr"] >= 0 and group["weight_decay"] >= 0
+        assert 0 <= group["momentum"] < 1 and group["ns_steps"] > 0
+        assert group["ns_method"] in METHODS
+        # both backends of the reference ("torch" = torch.compile, "tilelang") map to the HIP GEMM chain
+        assert group["ns_backend"] in ("torch", "tilelang", "hip")
+        assert group["adjust_lr_fn"] in ("original", "match_rms_adamw")
+        assert group["granularity"] in ("tile", "block") and group["rounding"] in ("nearest", "stochastic")
+        assert 0 <= group["rounding_seed"] < (1 << 63)
+        assert group["tile_size"] in (64, 128, 256, 512, 1024)
+        assert len(group["block_shape"]) == 2 and all(v in (8, 16, 32, 64) for v in group["block_shape"])
+        group["adam_state_dtype"] = _dtype(group["adam_state_dtype"])
+        grad_dtype = settings()["gradient_dtype"]
+        ragged = []
+        for param in group["params"]:
+            if grad_dtype is not None:
+                param.grad_dtype = grad_dtype
+            if _use_muon(param, group):
+                assert param.ndim >= 2
+                shape = _shape(param, group)
+                if group["granularity"] == "tile":
+                    partial = shape[-1] % group["tile_size"]
+                else:
+                    partial = shape[-2] % group["block_shape"][0] or shape[-1] % group["block_shape"][1]
+                if partial:
+                    ragged.append(shape)
+        if ragged and int(os.environ.get("RANK", "0")) == 0:
+            warnings.warn(f"FP8Muon: {len(ragged)} matrices have partial {group['granularity']} groups "
+                          f"(e.g. {ragged[:3]}). Original matrix shapes are kept; edge groups use valid elements.",
+                          stacklevel=3)
+
+    def _momentum(self, param, grad, state, group, key):
+        """Advance the FP8 momentum in place and return the bf16 update as a matrix view of the workspace."""
+        shape = _shape(param, group)
+        quant = dict(granularity=group["granularity"], tile_size=group["tile_size"], block_shape=group["block_shape"])
+        if "momentum_q" not in state:
+            payload, scales = state_sizes(shape, **quant)
+            state["momentum_q"] = torch.zeros(payload, device=param.device, dtype=torch.uint8)
+            state["momentum_scale"] = torch.ones(scales, device=param.device, dtype=torch.float32)
+        work = self._workspace.get(param.device)
+        if work is None or work.numel() < param.numel():
+            work = self._workspace[param.device] = torch.empty(param.numel(), device=param.device, dtype=torch.bfloat16)
+        matrix = work[:param.numel()].view(shape)
+        q, scale = state["momentum_q"], state["momentum_scale"]
+        before = (q.clone(), scale.clone()) if self.observer is not None else None
+        momentum_update(grad, q, scale, q, scale, matrix.view(-1), beta=group["momentum"], nesterov=group["nesterov"],
+                        matrix_shape=shape, rounding=group["rounding"], rounding_step=state["step"], rounding_key=key,
+                        **quant)
+        if self.observer is not None:
+            self.observer.momentum(param, grad, *before, q, scale, matrix, group, 1., quant)
+        return matrix
+
+    def _step_local(self, param, grad, state, group, index):
+        key = (group["rounding_seed"] + index * 0x9E3779B97F4A7C15) & _MASK63
+        master_key = (group["master_rounding_seed"] + index * 0x517CC1B727220A95) & _MASK63
+        assert param.is_cuda and not grad.is_sparse
+        assert param.dtype in (torch.float32, torch.bfloat16, torch.float16), \
+            "Bind FP8 modules with viola.optim.bind_optimizer before stepping."
+        state.setdefault("step", 0)
+        if _use_muon(param, group):
+            matrix = self._momentum(param, grad, state, group, key)
+            orthogonalize = METHODS[group["ns_method"]]
+            update = orthogonalize(matrix, steps=group["ns_steps"])
+            if self.observer is not None:
+                self.observer.update(param, update, group, orthogonalize)
+            rows, cols = matrix.shape[-2:]
+            scale = .2 * max(rows, cols) ** .5 if group["adjust_lr_fn"] == "match_rms_adamw" else max(1., rows / cols) ** .5
+            weight_update(param, update, group["lr"], group["weight_decay"], update_scale=scale,
+                          rounding=group["master_rounding"], step=state["step"], key=master_key)
+        else:
+            if "exp_avg" not in state:
+                state["exp_avg"] = torch.zeros_like(param, dtype=group["adam_state_dtype"])
+                state["exp_avg_sq"] = torch.zeros_like(param, dtype=group["adam_state_dtype"])
+            adam_update(param, grad, state["exp_avg"], state["exp_avg_sq"], lr=group["lr"],
+                        weight_decay=group["weight_decay"], betas=group["betas"], eps=group["eps"],
+                        step=state["step"] + 1, rounding=group["master_rounding"], key=master_key)
+        state["step"] += 1
