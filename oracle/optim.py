@@ -196,7 +196,9 @@ def adam_update(weight, grad, first, second, *, lr, weight_decay, betas, eps, st
     v = b2 * second.reshape(-1).float() + ((one - b2) * g) * g
     if adamw:
         w = w * (one - lr * wd)
-    value = w - (lr * (m * inv_c1)) / (torch.sqrt(v * inv_c2) + eps)
+    # numpy's sqrt is correctly rounded; torch's vectorised CPU sqrt is not on every host
+    root = torch.from_numpy(np.sqrt((v * inv_c2).numpy()))
+    value = w - (lr * (m * inv_c1)) / (root + eps)
     element = np.arange(value.numel(), dtype=np.uint64) + np.uint64(offset)
     out = _store(value, weight.dtype, rounding, element, step - 1, key)
     return out.view(weight.shape), m.to(first.dtype).view(first.shape), v.to(second.dtype).view(second.shape)

@@ -1,0 +1,132 @@
+"""GPU parity: grouped-scale FP8 GEMM, gated GEMMs and the variable-group GEMMs vs the CPU oracle."""
+
+import pytest
+import torch
+
+from oracle import grouped as og, linear as ol
+from conftest import rel_l2
+
+pytestmark = pytest.mark.gpu
+E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
+
+
+def _operands(m, k, n, ga, gb, fa, fb, seed=2041):
+    torch.manual_seed(seed)
+    a = (torch.randn(m, k) * torch.exp2(torch.randint(-5, 6, (m, 1)).float())).bfloat16()
+    b = (torch.randn(n, k) * torch.exp2(torch.randint(-5, 6, (n, 1)).float())).bfloat16()
+    return og.quantize(a, fa, ga), og.quantize(b, fb, gb)
+
+
+# shapes and group/format mixes of checks/check_grouped_linear.py:123-126, plus tile-edge and wgrad-like cases
+CASES = [((1, 32), (32, 32), (E4, E4), (65, 96, 128)), ((1, 64), (32, 64), (E5, E4), (96, 65, 64)),
+         ((32, 64), (64, 32), (E4, E5), (64, 160, 96)), ((1, 32), (32, 32), (E5, E4), (65, 4096, 128)),
+         ((1, 32), (1, 32), (E4, E4), (130, 256, 200)), ((1, 32), (32, 32), (E4, E4), (256, 1024, 384)),
+         ((1, 32), (1, 32), (E5, E5), (96, 8192, 64)), ((1, 32), (32, 32), (E4, E4), (1, 32, 1)),
+         ((1, 32), (32, 32), (E4, E4), (129, 48, 257))]
+
+
+@pytest.mark.parametrize("ga,gb,formats,shape", CASES)
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_group_gemm(ga, gb, formats, shape, out_dtype):
+    from viola_amd.nn import _grouped_kernels as g
+    m, k, n = shape
+    (qa, sa), (qb, sb) = _operands(m, k, n, ga, gb, *formats)
+    bias = torch.randn(n)
+    actual = g.gemm(qa.cuda(), qb.cuda(), sa.cuda(), sb.cuda(), ga, gb, out_dtype=out_dtype, bias=bias.cuda())
+    expected = og.gemm(qa, qb, sa, sb, ga, gb, bias=bias, witness=True, out_dtype=torch.float64)
+    assert actual.dtype == out_dtype and torch.isfinite(actual).all()
+    # fp32 out: the reference's own bound (checks/check_grouped_linear.py:41); bf16 out adds half a bf16 ulp
+    assert rel_l2(actual, expected) < (2e-5 if out_dtype == torch.float32 else 3e-3)
+    for _ in range(2):                                                        # bit-identical on repeat (:43-46)
+        again = g.gemm(qa.cuda(), qb.cuda(), sa.cuda(), sb.cuda(), ga, gb, out_dtype=out_dtype, bias=bias.cuda())
+        assert torch.equal(again, actual)
+    nobias = g.gemm(qa.cuda(), qb.cuda(), sa.cuda(), sb.cuda(), ga, gb, out_dtype=torch.float32)
+    assert rel_l2(nobias, og.gemm(qa, qb, sa, sb, ga, gb, witness=True, out_dtype=torch.float64)) < 2e-5
+
+
+def test_group_gemm_special_structure():
+    """Identity-like operands make the expected value exact: catches a transposed operand or a wrong scale index."""
+    from viola_amd.nn import _grouped_kernels as g
+    m = n = k = 128
+    a = torch.eye(m, k) * torch.arange(1, m + 1).float()[:, None]
+    b = torch.randn(n, k).bfloat16().float()
+    qa, sa = og.quantize(a, E4, (1, 32))
+    qb, sb = og.quantize(b, E4, (32, 32))
+    out = g.gemm(qa.cuda(), qb.cuda(), sa.cuda(), sb.cuda(), (1, 32), (32, 32), out_dtype=torch.float32).cpu()
+    expect = og.dequantize(qa, sa, (1, 32)) @ og.dequantize(qb, sb, (32, 32)).T
+    assert torch.allclose(out, expect, rtol=1e-6, atol=0)
+    assert not torch.allclose(out, expect.T, rtol=1e-3, atol=0)
+
+
+class _Layer:
+    """The attributes the gated GEMM wrapper reads from a Linear."""
+    _grouped_scaling, _native_scaling = True, False
+    input_group_shape, weight_group_shape = (1, 32), (32, 32)
+
+
+@pytest.mark.parametrize("activation", ["silu", "gelu", "relu"])
+@pytest.mark.parametrize("m,h,k", [(66, 160, 128), (130, 64, 96), (64, 40, 64)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_gated_gemm_forward_backward(activation, m, h, k, dtype):
+    from viola_amd.nn import _mlp_kernels as mk
+    gw = (32, 32) if h % 32 == 0 else (1, 32)
+    layer = _Layer()
+    layer.weight_group_shape = gw
+    (qa, sa), (qb, sb) = _operands(m, k, 2 * h, (1, 32), gw, E4, E4, seed=131)
+    bias = torch.randn(2 * h).to(dtype)
+    out, aux, _ = mk.gemm(qa.cuda(), qb.cuda(), sa.cuda(), sb.cuda(), layer=layer, out_dtype=dtype, bias=bias.cuda(),
+                          activation=activation, save=True)
+    z = og.gemm(qa, qb, sa, sb, (1, 32), gw, bias=bias.float()).to(dtype)
+    assert rel_l2(aux, z) < 4e-3
+    expect = ol.gated_forward(aux.cpu()[:, :h], aux.cpu()[:, h:], activation).to(dtype)     # from the saved g, u
+    assert rel_l2(out, expect) < 4e-3
+    nosave, aux2, _ = mk.gemm(qa.cuda(), qb.cuda(), sa.cuda(), sb.cuda(), layer=layer, out_dtype=dtype, bias=bias.cuda(),
+                              activation=activation, save=False)
+    assert aux2.numel() == 0 and torch.equal(nosave, out)
+    # backward: d = a2 . w2^T with w2 [h, k2]
+    k2 = 96
+    (qg, sg), (qw, sw) = _operands(m, k2, h, (1, 32), (32, 32), E4, E4, seed=17)
+    dz, _, _ = mk.gemm(qg.cuda(), qw.cuda(), sg.cuda(), sw.cuda(), layer=layer, out_dtype=dtype, backward=True,
+                       activation=activation, aux=aux, group_a=(1, 32), group_b=(32, 32))
+    d = og.gemm(qg, qw, sg, sw, (1, 32), (32, 32)).to(dtype)
+    dg, du = ol.gated_backward(d, aux.cpu()[:, :h], aux.cpu()[:, h:], activation)
+    assert dz.shape == (m, 2 * h) and rel_l2(dz, torch.cat([dg, du], 1).to(dtype)) < 6e-3
+
+
+@pytest.mark.parametrize("activation", ["silu", "gelu", "relu"])
+def test_gated_elementwise(activation):
+    from viola_amd.nn._gated_kernels import GatedActivation
+    torch.manual_seed(3)
+    z = torch.randn(5, 33, 2 * 72).bfloat16().cuda().requires_grad_()
+    out = GatedActivation.apply(z, activation, False)
+    dy = torch.randn_like(out)
+    out.backward(dy)
+    g, u = z.detach().cpu()[..., :72], z.detach().cpu()[..., 72:]
+    assert rel_l2(out, ol.gated_forward(g, u, activation).bfloat16()) < 3e-3
+    dg, du = ol.gated_backward(dy.cpu(), g, u, activation)
+    assert rel_l2(z.grad, torch.cat([dg, du], -1).bfloat16()) < 4e-3
+
+
+@pytest.mark.parametrize("counts", [[130, 0, 3, 64, 1, 200], [5], [0, 0, 7]])
+def test_varlen_group_gemm_and_wgrad(counts):
+    from viola_amd.nn import _varlen as v
+    groups, k, n = len(counts), 128, 96
+    total = sum(counts)
+    torch.manual_seed(5)
+    x = torch.randn(total, k).bfloat16()
+    dy = torch.randn(total, n).bfloat16()
+    w = torch.randn(groups, n, k) / 11
+    qw = torch.stack([og.quantize(w[g], E4, (32, 32))[0] for g in range(groups)])
+    sw = torch.stack([og.quantize(w[g], E4, (32, 32))[1] for g in range(groups)])
+    wreal = [og.dequantize(qw[g], sw[g], (32, 32)) for g in range(groups)]
+    expect = ol.varlen_linear(x, wreal, counts, dy, grad_dtype=torch.float32)
+    xg = x.cuda().requires_grad_()
+    wparam = torch.nn.Parameter(qw.cuda())
+    wparam.grad_dtype = torch.float32
+    y = v.grouped_linear(xg, wparam, sw.cuda(), counts)
+    y.backward(dy.cuda())
+    assert rel_l2(y, expect["y"]) < 3e-3 and rel_l2(xg.grad, expect["dx"]) < 3e-3
+    assert wparam.grad.shape == (groups, n, k) and rel_l2(wparam.grad, expect["dw"]) < 2e-5
+    for g, c in enumerate(counts):
+        if c == 0:
+            assert wparam.grad[g].count_nonzero() == 0

@@ -1,0 +1,225 @@
+"""GPU parity: FP8Muon kernels (momentum codec, Philox SR, weight / AdamW updates, copy_scaled) vs the CPU oracle.
+FP8 payloads, scales and fp32 results are compared bit for bit."""
+
+import itertools
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import optim as oo
+
+pytestmark = pytest.mark.gpu
+
+
+def _k():
+    from viola_amd.optim import _kernels
+    return _kernels
+
+
+def test_philox_known_answers_on_device():
+    from viola_amd import _lib
+    triples = [(0, 0, 0), (0xffffffffffffffff,) * 3, (0x85a308d3243f6a88, 0x0370734413198a2e, 0x299f31d0a4093822)]
+    rng = np.random.default_rng(0)
+    extra = rng.integers(0, 2 ** 63, size=(200, 3), dtype=np.uint64)
+    table = np.concatenate([np.array(triples, dtype=np.uint64), extra])
+    dev = torch.from_numpy(table.view(np.int64).copy()).cuda()
+    out = torch.zeros(len(table), dtype=torch.int32, device="cuda")
+    _lib.call("viola_selftest_philox", _lib.ptr(dev), _lib.ptr(out), len(table))
+    got = out.cpu().numpy().view(np.uint32)
+    assert got[:3].tolist() == [0x6627e8d5, 0x408f276d, 0xd16cfe09]          # Random123 kat_vectors
+    expect = np.array([oo.philox(np.array([e], dtype=np.uint64), int(s), int(k))[0] for e, s, k in table], dtype=np.uint32)
+    assert np.array_equal(got, expect)
+
+
+CONFIGS = [("tile", b) for b in (64, 128, 256, 512, 1024)] + [("block", t) for t in ((8, 8), (8, 32), (16, 16), (16, 32), (32, 32), (64, 64))]
+
+
+@pytest.mark.parametrize("granularity,size", CONFIGS)
+@pytest.mark.parametrize("shape", [(17, 31), (2, 33, 67)])
+@pytest.mark.parametrize("rounding", ["nearest", "stochastic"])
+def test_momentum_update_bit_exact(granularity, size, shape, rounding):
+    """The sweep of checks/quantization.py:83-112 (tile sizes, block shapes, ragged shapes, unaligned buffers,
+    in-place state), held to bit equality with the oracle instead of the reference's rtol 2e-6."""
+    k = _k()
+    torch.manual_seed(79)
+    quant = dict(granularity=granularity, tile_size=size if granularity == "tile" else 256,
+                 block_shape=size if granularity == "block" else (16, 16))
+    qn, sn = k.state_sizes(shape, **quant)
+    assert (qn, sn) == oo.state_sizes(shape, **quant)
+    n = math.prod(shape)
+    q = torch.zeros(qn + 1, dtype=torch.uint8, device="cuda")[1:]            # element-aligned views only
+    scale = torch.ones(sn + 1, device="cuda")[1:]
+    u = torch.empty(n + 1, dtype=torch.bfloat16, device="cuda")[1:]
+    rq, rs = torch.zeros(qn, dtype=torch.uint8), torch.ones(sn)
+    for step in range(6):
+        g = torch.randn(n + 1)[1:] * (1e-8 if step < 2 else 1.)
+        gd = torch.empty(n + 1, device="cuda")[1:].copy_(g)
+        nesterov = step % 2 == 0
+        k.momentum_update(gd, q, scale, q, scale, u, beta=.95, matrix_shape=shape, nesterov=nesterov,
+                          rounding=rounding, rounding_step=step, rounding_key=123, **quant)
+        rq, rs, ru = oo.momentum_update(g, rq, rs, beta=.95, shape=shape, nesterov=nesterov, rounding=rounding,
+                                        rounding_step=step, rounding_key=123, **quant)
+        assert torch.equal(scale.cpu(), rs), f"scales differ at step {step}"
+        assert torch.equal(q.cpu(), rq), f"payload differs at step {step}"
+        assert torch.equal(u.cpu().view(torch.int16), ru.view(torch.int16)), f"update differs at step {step}"
+        assert torch.equal(k.dequantize(q, scale, shape, **quant).cpu(), oo.dequantize(rq, rs, shape, **quant))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("tile_size,n", [(128, 13), (256, 257), (512, 1537), (256, 8192)])
+def test_momentum_out_of_place_loss_scale(dtype, tile_size, n):
+    """checks/numerics.py:18-49: separate next buffers, fp16 gradients with loss scaling."""
+    k = _k()
+    torch.manual_seed(42)
+    blocks = -(-n // tile_size)
+    q, scales = torch.zeros(blocks * tile_size, dtype=torch.uint8, device="cuda"), torch.ones(blocks, device="cuda")
+    nq, ns_ = torch.empty_like(q), torch.empty_like(scales)
+    out = torch.empty(n, dtype=torch.bfloat16, device="cuda")
+    rq, rs = q.cpu(), scales.cpu()
+    loss_scale = 32.0 if dtype == torch.float16 else 1.0
+    for step in range(4):
+        grad = torch.randn(n).to(dtype)
+        k.momentum_update(grad.cuda(), q, scales, nq, ns_, out, beta=.95, tile_size=tile_size, nesterov=step % 2 == 0,
+                          loss_scale=loss_scale)
+        rq, rs, ru = oo.momentum_update(grad, rq, rs, beta=.95, shape=(n,), tile_size=tile_size, nesterov=step % 2 == 0,
+                                        loss_scale=loss_scale)
+        assert torch.equal(nq.cpu(), rq) and torch.equal(ns_.cpu(), rs) and torch.equal(out.cpu().view(torch.int16), ru.view(torch.int16))
+        q, nq, scales, ns_ = nq, q, ns_, scales
+    zero = torch.zeros(n, device="cuda", dtype=dtype)
+    q.zero_(); scales.fill_(1)
+    k.momentum_update(zero, q, scales, nq, ns_, out, beta=.95, tile_size=tile_size)
+    assert nq.count_nonzero() == 0 and out.count_nonzero() == 0                # zero stays zero (numerics.py:51-55)
+
+
+def test_stochastic_rounding_statistics_and_replay():
+    """checks/quantization.py:114-153 on the device."""
+    k = _k()
+    n = 256 * 1024
+    g = torch.full((n,), 1 + .27 * .125, device="cuda")
+    g[::256] = 448
+    q, scales = torch.zeros(n, dtype=torch.uint8, device="cuda"), torch.ones(n // 256, device="cuda")
+    out = torch.empty(n, dtype=torch.bfloat16, device="cuda")
+
+    def draw(step=7, key=42):
+        q.zero_(); scales.fill_(1)
+        k.momentum_update(g, q, scales, q, scales, out, beta=0., rounding="stochastic", rounding_step=step,
+                          rounding_key=key, nesterov=False)
+        return q.clone()
+
+    rng_state = torch.cuda.get_rng_state()
+    first = draw()
+    assert torch.equal(first, draw()) and not torch.equal(first, draw(step=8)) and not torch.equal(first, draw(key=43))
+    assert torch.equal(rng_state, torch.cuda.get_rng_state())
+    values = first.view(torch.float8_e4m3fn).float().view(-1, 256)[:, 1:]
+    assert ((values == 1.) | (values == 1.125)).all()
+    assert abs((values == 1.125).float().mean().item() - .27) < .005
+    table = torch.arange(127, dtype=torch.uint8).view(torch.float8_e4m3fn).float().cuda()
+    mids = (table[:-1] * .7 + table[1:] * .3).repeat(1024)
+    g2 = torch.cat((mids, -mids, table.repeat(1024)))
+    g2[::256] = 448
+    qn, sn = k.state_sizes(g2.shape)
+    q2, s2 = torch.zeros(qn, dtype=torch.uint8, device="cuda"), torch.ones(sn, device="cuda")
+    o2 = torch.empty(g2.numel(), dtype=torch.bfloat16, device="cuda")
+    torch.cuda.synchronize()
+    allocated = torch.cuda.memory_allocated()
+    torch.cuda.reset_peak_memory_stats()
+    k.momentum_update(g2, q2, s2, q2, s2, o2, beta=0., rounding="stochastic", nesterov=False)
+    torch.cuda.synchronize()
+    assert torch.cuda.max_memory_allocated() - allocated == 0                  # kernels allocate nothing (:155-161)
+    actual = k.dequantize(q2, s2, g2.shape)
+    idx = torch.searchsorted(table, g2.abs()).clamp_max(126)
+    lower, upper = table[(idx - 1).clamp_min(0)], table[idx]
+    assert ((actual.abs() == lower) | (actual.abs() == upper)).all()
+    assert ((actual.sign() == g2.sign()) | (actual == 0)).all()
+
+
+DTYPES = (torch.float32, torch.bfloat16, torch.float16)
+
+
+@pytest.mark.parametrize("wdtype,gdtype", list(itertools.product(DTYPES, repeat=2)))
+def test_weight_and_adam_bit_exact(wdtype, gdtype):
+    """The dtype sweep of checks/precision_kernels.py:26-46 on unaligned views; bit equality with the oracle."""
+    k = _k()
+    torch.manual_seed(107)
+    w = (torch.randn(1030) * .1).to(wdtype)[1:1026]
+    g = (torch.randn(1030) * .01).to(gdtype)[1:1026]
+    wd = (torch.zeros(1030, device="cuda", dtype=wdtype))[1:1026].copy_(w)
+    gd = (torch.zeros(1030, device="cuda", dtype=gdtype))[1:1026].copy_(g)
+    k.weight_update(wd, gd, .001, .01, update_scale=6.4)
+    ref = oo.weight_update(w, g, .001, .01, update_scale=6.4)
+    assert torch.equal(wd.cpu().view(torch.uint8), ref.contiguous().view(torch.uint8))
+    for sdtype in DTYPES:
+        m, v = torch.zeros(1025, device="cuda", dtype=sdtype), torch.zeros(1025, device="cuda", dtype=sdtype)
+        rm, rv, rw = m.cpu(), v.cpu(), ref
+        for step in range(1, 4):
+            k.adam_update(wd, gd, m, v, lr=.001, weight_decay=.01, betas=(.9, .95), eps=1e-8, step=step)
+            rw, rm, rv = oo.adam_update(rw, g, rm, rv, lr=.001, weight_decay=.01, betas=(.9, .95), eps=1e-8, step=step)
+            assert torch.equal(m.cpu().view(torch.uint8), rm.contiguous().view(torch.uint8))
+            assert torch.equal(v.cpu().view(torch.uint8), rv.contiguous().view(torch.uint8))
+            assert torch.equal(wd.cpu().view(torch.uint8), rw.contiguous().view(torch.uint8)), (sdtype, step)
+        ref = rw
+
+
+def test_adam_variants():
+    k = _k()
+    torch.manual_seed(1)
+    w, g = torch.randn(300), torch.randn(300)
+    for adamw, maximize, bias_correction in itertools.product((True, False), repeat=3):
+        wd, m, v = w.cuda(), torch.zeros(300, device="cuda"), torch.zeros(300, device="cuda")
+        k.adam_update(wd, g.cuda(), m, v, lr=.01, weight_decay=.1, betas=(.9, .999), eps=1e-8, step=3, adamw=adamw,
+                      maximize=maximize, bias_correction=bias_correction)
+        rw, rm, rv = oo.adam_update(w, g, torch.zeros(300), torch.zeros(300), lr=.01, weight_decay=.1, betas=(.9, .999),
+                                    eps=1e-8, step=3, adamw=adamw, maximize=maximize, bias_correction=bias_correction)
+        assert torch.equal(wd.cpu(), rw) and torch.equal(m.cpu(), rm) and torch.equal(v.cpu(), rv)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_stochastic_master_rounding(dtype):
+    """checks/precision_kernels.py:48-65: 25 % of sub-ulp updates survive; a split call with `offset` replays exactly."""
+    k = _k()
+    n = 131072
+    spacing = 2. ** (-8 if dtype == torch.bfloat16 else -11)
+    w = torch.ones(n, device="cuda", dtype=dtype)
+    g = torch.ones(n, device="cuda")
+    k.weight_update(w, g, spacing / 4, 0., rounding="stochastic", step=17, key=29)
+    assert abs((w != 1).float().mean().item() - .25) < .005
+    ref = oo.weight_update(torch.ones(n, dtype=dtype), torch.ones(n), spacing / 4, 0., rounding="stochastic", step=17, key=29)
+    assert torch.equal(w.cpu(), ref)
+    replay = torch.ones_like(w)
+    cut = 13001
+    k.weight_update(replay[:cut], g[:cut], spacing / 4, 0., rounding="stochastic", step=17, key=29)
+    k.weight_update(replay[cut:], g[cut:], spacing / 4, 0., rounding="stochastic", step=17, key=29, offset=cut)
+    assert torch.equal(w, replay)
+    m, v = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+    w2 = torch.ones(n, device="cuda", dtype=dtype)
+    k.adam_update(w2, g * 1e-3, m, v, lr=1e-4, weight_decay=0., betas=(.9, .95), eps=1e-8, step=1, rounding="stochastic", key=5)
+    rw, _, _ = oo.adam_update(torch.ones(n, dtype=dtype), torch.ones(n) * 1e-3, torch.zeros(n), torch.zeros(n), lr=1e-4,
+                              weight_decay=0., betas=(.9, .95), eps=1e-8, step=1, rounding="stochastic", key=5)
+    assert torch.equal(w2.cpu(), rw)
+
+
+def test_copy_scaled():
+    k = _k()
+    matrix = torch.randn(17, 31).bfloat16().T
+    partition = torch.zeros(257, device="cuda")
+    k.copy_scaled(matrix.cuda(), partition, 11, 3, 251, 3.2)
+    assert torch.equal(partition.cpu(), oo.copy_scaled(matrix, torch.zeros(257), 11, 3, 251, 3.2))   # numerics.py:74-77
+
+
+def test_full_size_momentum_properties():
+    """DiT-XL qkv-sized state: replay determinism, payload/scales consistent with the bf16 update it emitted."""
+    k = _k()
+    torch.manual_seed(3)
+    n = 3456 * 1152
+    g = (torch.randn(n, device="cuda") * 1e-3)
+    q, s = torch.zeros(n, dtype=torch.uint8, device="cuda"), torch.ones(n // 256, device="cuda")
+    u = torch.empty(n, dtype=torch.bfloat16, device="cuda")
+    k.momentum_update(g, q, s, q, s, u, beta=.95, tile_size=256, nesterov=False)
+    m = k.dequantize(q, s, (n,))
+    assert ((m - u.float()).norm() / u.float().norm()).item() < .04
+    assert q.view(torch.float8_e4m3fn).float().abs().view(-1, 256).amax(1).eq(448).all()
+    q2, s2 = torch.zeros_like(q), torch.ones_like(s)
+    k.momentum_update(g, q2, s2, q2, s2, u, beta=.95, tile_size=256, nesterov=False)
+    assert torch.equal(q, q2) and torch.equal(s, s2)

@@ -1,0 +1,144 @@
+"""GPU parity: group quantize / dequantize / transpose through the C ABI vs the CPU oracle, bit-exact."""
+
+import pytest
+import torch
+
+from oracle import grouped as og
+from conftest import rel_l2
+
+pytestmark = pytest.mark.gpu
+E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
+
+
+def _gpu():
+    from viola_amd.nn import _grouped_kernels as g
+    return g
+
+
+def _input(shape, dtype, seed=2041):
+    torch.manual_seed(seed)
+    x = torch.randn(*shape) * torch.exp2(torch.randint(-5, 6, (shape[0], 1)).float())
+    return x.to(dtype)
+
+
+def _same(q, s, rq, rs):
+    assert q.dtype == rq.dtype and tuple(q.shape) == tuple(rq.shape) and tuple(s.shape) == tuple(rs.shape)
+    assert torch.equal(s.cpu(), rs), "scales differ"
+    assert torch.equal(q.cpu().view(torch.uint8), rq.view(torch.uint8)), "codes differ"
+
+
+def test_hardware_fp8_conversions_vs_software():
+    """Exhaustive: every fp32 bit pattern in range through v_cvt_pk_{fp8,bf8}_f32, all 256 codes back."""
+    from viola_amd import _lib
+    counts = torch.zeros(4, dtype=torch.int64, device="cuda")
+    _lib.call("viola_selftest_fp8", _lib.ptr(counts))
+    torch.cuda.synchronize()
+    print("hw-vs-sw mismatches [e4m3 enc, e5m2 enc, e4m3 dec, e5m2 dec]:", counts.tolist())
+    assert counts[2:].tolist() == [0, 0]
+
+
+def test_software_codecs_all_codes():
+    """dequantize of every code with unit scale == torch's decode; quantize of every finite value is the identity."""
+    g = _gpu()
+    for dtype in (E4, E5):
+        codes = torch.arange(256, dtype=torch.uint8).view(dtype).reshape(8, 32)
+        out = g.dequantize(codes.cuda(), torch.ones(8, 1, device="cuda"), (1, 32)).cpu()
+        ref = codes.float()
+        assert torch.equal(out.isnan(), ref.isnan()) and torch.equal(out.nan_to_num(1.0, 2.0, 3.0), ref.nan_to_num(1.0, 2.0, 3.0))
+        finite = ref.flatten()[ref.flatten().isfinite()]
+        x = finite.repeat(2)[:256 + 64].reshape(-1, 32).contiguous()
+        x[:, 0] = torch.finfo(dtype).max                                     # unit scale in every row tile
+        q, s = g.quantize(x.cuda(), dtype, (1, 32))
+        assert torch.equal(s.cpu(), torch.ones_like(s.cpu())) and torch.equal(q.float().cpu(), x)
+
+
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("fp8", [E4, E5])
+@pytest.mark.parametrize("group,shape", [((1, 32), (65, 96)), ((1, 32), (256, 1024)), ((1, 64), (96, 136)), ((1, 128), (33, 256)),
+                                          ((32, 32), (96, 128)), ((32, 32), (70, 45)), ((32, 64), (64, 160)), ((64, 32), (130, 96)),
+                                          ((1, 32), (7, 33)), ((1, 512), (9, 1024))])
+def test_quantize_rowwise_and_blocks(in_dtype, fp8, group, shape):
+    g = _gpu()
+    x = _input(shape, in_dtype)
+    q, s = g.quantize(x.cuda(), fp8, group)
+    _same(q, s, *og.quantize(x, fp8, group))
+    deq = g.dequantize(q, s, group)
+    assert torch.equal(deq.cpu(), og.dequantize(q.cpu(), s.cpu(), group))
+
+
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("fp8", [E4, E5])
+@pytest.mark.parametrize("group,shape", [((1, 32), (65, 96)), ((1, 32), (300, 200)), ((1, 32), (128, 64)), ((1, 32), (31, 7)),
+                                          ((32, 32), (96, 70)), ((1, 64), (96, 65)), ((64, 32), (64, 160))])
+def test_quantize_transposed(in_dtype, fp8, group, shape):
+    g = _gpu()
+    x = _input(shape, in_dtype, seed=7)
+    q, s = g.quantize(x.cuda(), fp8, group, transposed=True)
+    _same(q, s, *og.quantize(x, fp8, group, transposed=True))
+
+
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(65, 128), (128, 64), (300, 200), (1, 32), (129, 72), (8192, 1024)])
+def test_quantize_dual_equals_two_passes(in_dtype, shape):
+    g = _gpu()
+    x = _input(shape, in_dtype, seed=11)
+    q, s, qt, st = g.quantize_dual(x.cuda(), E4, (1, 32))
+    _same(q, s, *og.quantize(x, E4, (1, 32)))
+    _same(qt, st, *og.quantize(x, E4, (1, 32), transposed=True))
+
+
+def test_quantize_limit_and_out_arguments():
+    g = _gpu()
+    x = _input((64, 96), torch.float32, seed=3)
+    q, s = g.quantize(x.cuda(), E4, (32, 32), limit=8.0)
+    _same(q, s, *og.quantize(x, E4, (32, 32), limit=8.0))
+    out = torch.empty((64, 96), device="cuda", dtype=E4)
+    scale_out = torch.empty((2, 3), device="cuda")
+    q2, s2 = g.quantize(x.cuda(), E4, (32, 32), out=out, scale_out=scale_out)
+    assert q2 is out and s2 is scale_out
+    _same(out, scale_out, *og.quantize(x, E4, (32, 32)))
+
+
+def test_quantize_nonfinite_and_zero():
+    g = _gpu()
+    x = torch.ones(4, 64)
+    x[0, 3], x[1, 40], x[2] = float("nan"), float("inf"), 0.0
+    for transposed in (False, True):
+        q, s = g.quantize(x.cuda(), E4, (1, 32), transposed=transposed)
+        rq, rs = og.quantize(x, E4, (1, 32), transposed=transposed)
+        assert torch.equal(s.cpu(), rs)
+        a, b = q.float().cpu(), rq.float()
+        assert torch.equal(a.isnan(), b.isnan()) and torch.equal(a.nan_to_num(9.0), b.nan_to_num(9.0))
+    q, s = g.quantize(torch.zeros(0, 32, device="cuda"), E4, (1, 32))
+    assert q.numel() == 0 and s.numel() == 0
+
+
+@pytest.mark.parametrize("group", [(32, 32), (1, 32), (64, 32)])
+def test_transpose_of_codes(group):
+    g = _gpu()
+    w = _input((96, 160), torch.float32, seed=5)
+    q, s = og.quantize(w, E4, group)
+    qt, st = g.transpose(q.cuda(), s.cuda(), group)
+    _same(qt, st, *og.transpose(q, s, group))
+    from viola_amd.nn._linear_kernels import transpose
+    raw = torch.randint(0, 255, (70, 45), dtype=torch.uint8).view(E4)
+    assert torch.equal(transpose(raw.cuda()).cpu().view(torch.uint8), raw.view(torch.uint8).T)
+
+
+def test_full_size_properties():
+    """C2-sized inputs: properties that need no CPU oracle at that size."""
+    g = _gpu()
+    torch.manual_seed(1)
+    dy = (torch.randn(8192, 4096) * 1e-2).bfloat16().cuda()
+    q, s, qt, st = g.quantize_dual(dy, E4, (1, 32))
+    assert q.float().abs().reshape(8192, 128, 32).amax(2).eq(448).all()          # every tile reaches the limit
+    assert qt.float().abs().reshape(4096, 256, 32).amax(2).eq(448).all()
+    assert rel_l2(g.dequantize(q, s, (1, 32)), dy.float()) < 0.04
+    assert rel_l2(g.dequantize(qt, st, (1, 32)).T, dy.float()) < 0.04
+    q1, s1 = g.quantize(dy, E4, (1, 32))
+    q2, s2 = g.quantize(dy, E4, (1, 32), transposed=True)
+    assert torch.equal(q1.view(torch.uint8), q.view(torch.uint8)) and torch.equal(s1, s)
+    assert torch.equal(q2.view(torch.uint8), qt.view(torch.uint8)) and torch.equal(s2, st)
+    # idempotence: quantizing the dequantized tensor reproduces codes and scales
+    q3, s3 = g.quantize(g.dequantize(q, s, (1, 32)), E4, (1, 32))
+    assert torch.equal(q3.view(torch.uint8), q.view(torch.uint8)) and torch.equal(s3, s)
