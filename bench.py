@@ -1,0 +1,198 @@
+"""Headline benchmark on ONE MI355X: viola.nn.Linear FP8 forward+backward at 8192 x 1024 -> 4096
+(e4m3, FP32 tile/block scales, bf16 outputs) in TFLOP/s, with the FP8Muon step time on the DiT-XL
+parameter set, the wire codec and quantizer bandwidths, a roofline object for the dominant kernel
+(the grouped-scale FP8 GEMM) and the CPU oracle timed on this host's cores.
+
+    python bench.py --gpus 1 --steps 20 --warmup 3
+
+A step is one `y = layer(x); y.backward(dy)` including every quantize / transpose launch, inputs
+resident in HBM. TFLOP/s = 6*M*K*N / t (the reference's definition, checks/benchmark_linear.py:165).
+"""
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+M, K, N = 8192, 1024, 4096
+PEAK = {"fp8_tflops": 5000.0, "bf16_tflops": 2500.0, "hbm_gbs": 8000.0}
+
+
+def timed(fn, steps, warmup):
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    begin = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - begin) * 1e3
+    return max(start.elapsed_time(end), 0.0) / steps, wall / steps
+
+
+def kernel_breakdown(fn, steps):
+    """Second, instrumented pass: HIP events around every C-ABI call on the stream it is launched on."""
+    import torch
+    from viola_amd import _lib
+    _lib.timeline = []
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    rows, _lib.timeline = _lib.timeline, None
+    table = {}
+    for name, start, end in rows:
+        table.setdefault(name, []).append(start.elapsed_time(end))
+    return {name: dict(launches_per_step=len(v) / steps, avg_ms=sum(v) / len(v)) for name, v in table.items()}
+
+
+def linear_case():
+    import torch
+    import viola_amd
+    torch.manual_seed(20261125)
+    viola_amd.set_gradient_dtype("bf16")
+    layer = viola_amd.nn.Linear(K, N, device="cuda", dtype=torch.bfloat16, scaling="grouped", forward_dtype="e4m3",
+                                backward_dtype="e4m3", mode="memory", weight_dtype="fp8")
+    viola_amd.precision._settings["gradient_dtype"] = None
+    x = torch.randn(M, K).bfloat16().cuda().requires_grad_()
+    dy = (torch.randn(M, N) * 1e-2).bfloat16().cuda()
+
+    def step():
+        x.grad = layer.weight.grad = layer.bias.grad = None
+        layer(x).backward(dy)
+
+    return layer, x, dy, step
+
+
+def muon_case(method="standard", rounding="nearest", blocks=28, d=1152):
+    """DiT-XL-shaped parameter set: per block qkv [3d, d], proj [d, d], fc1 [4d, d], fc2 [d, 4d] + vectors."""
+    import torch
+    import viola_amd
+    torch.manual_seed(7)
+    params = []
+    for _ in range(blocks):
+        for shape in ((3 * d, d), (d, d), (4 * d, d), (d, 4 * d), (3 * d,), (d,), (4 * d,), (d,), (d,), (d,)):
+            p = torch.nn.Parameter(torch.randn(*shape, device="cuda") * .02)
+            p.grad = torch.randn_like(p) * 1e-3
+            params.append(p)
+    opt = viola_amd.optim.FP8Muon(params, lr=1e-3, weight_decay=.01, mode="balanced", tile_size=256, ns_method=method,
+                                  rounding=rounding, rounding_seed=42, adjust_lr_fn="match_rms_adamw")
+    elements = sum(p.numel() for p in params if p.ndim >= 2)
+    return opt, params, elements
+
+
+def cpu_baseline():
+    """The oracle's Linear forward+backward (dequantized-FP32 matmuls) on this host's cores, one full C2 step."""
+    import torch
+    from oracle import grouped as og, linear as ol
+    torch.manual_seed(20261125)
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    x = torch.randn(M, K).bfloat16()
+    dy = (torch.randn(M, N) * 1e-2).bfloat16()
+    w = torch.empty(N, K).uniform_(-1 / 32, 1 / 32)
+    qw, sw = og.quantize(w, torch.float8_e4m3fn, (32, 32))
+    w_real = og.dequantize(qw, sw, (32, 32))
+    times = []
+    for _ in range(3):
+        begin = time.perf_counter()
+        ol.linear(x, w_real, torch.zeros(N), dy)
+        times.append(time.perf_counter() - begin)
+    best = statistics.median(times[1:])
+    return dict(value=6 * M * K * N / best / 1e12, unit="TFLOP/s", cores=cores, kind="port",
+                sample=f"one full {M}x{K}->{N} forward+backward per run, median of 2 after 1 warm-up "
+                       f"({best * 1e3:.0f} ms per step)")
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=20)
+    parser.add_argument("--warmup", type=int, default=3)
+    parser.add_argument("--skip-cpu", action="store_true", help="leave out the CPU baseline leg")
+    parser.add_argument("--skip-muon", action="store_true", help="leave out the FP8Muon / codec legs")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    import torch
+    from viola_amd import _lib
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    _lib.library()
+
+    layer, x, dy, step = linear_case()
+    ms, wall_ms = timed(step, args.steps, args.warmup)
+    flops = 6 * M * K * N
+    value = flops / (ms * 1e-3) / 1e12
+    breakdown = kernel_breakdown(step, args.steps)
+    gemm = breakdown["viola_group_gemm"]
+    gemm_tflops = 2 * M * K * N / (gemm["avg_ms"] * 1e-3) / 1e12
+    roofline = dict(bound="mfma", kernel="group_gemm_kernel (viola_group_gemm: fwd, dgrad, wgrad)",
+                    achieved=gemm_tflops, peak=PEAK["fp8_tflops"], unit="TFLOP/s", frac=gemm_tflops / PEAK["fp8_tflops"],
+                    avg_launch_ms=gemm["avg_ms"], traffic=None)
+    quant = {}
+    if "viola_group_quantize_dual" in breakdown:
+        # X [M, K] and dY [M, N] each once per step: 4.25 B per element (bf16 in, two FP8 layouts + scales out)
+        per_step = 4.25 * (M * K + M * N) / 2
+        q = breakdown["viola_group_quantize_dual"]
+        quant = dict(kernel="quantize_tile (row-wise + transposed, one read)", avg_ms=q["avg_ms"],
+                     gbs=per_step / (q["avg_ms"] * 1e-3) / 1e9, frac_hbm=per_step / (q["avg_ms"] * 1e-3) / 1e9 / PEAK["hbm_gbs"])
+
+    extra = {}
+    if not args.skip_muon:
+        for method in ("standard", "gram"):
+            opt, params, elements = muon_case(method)
+            step_ms, step_wall = timed(opt.step, 5, 3)
+            b = kernel_breakdown(opt.step, 2)
+            ns_flops = 0.0
+            for p in params:
+                if p.ndim >= 2:
+                    m_, n_ = min(p.shape), max(p.shape)
+                    if method == "standard":
+                        ns_flops += 5 * (4 * m_ * m_ * n_ + 2 * m_ ** 3)
+                    else:
+                        ns_flops += 5 * 6 * m_ ** 3 if m_ == n_ else 8 * m_ * m_ * n_ + 28 * m_ ** 3
+            ns_ms = b["viola_ns_gemm"]["avg_ms"] * b["viola_ns_gemm"]["launches_per_step"]
+            mom = b["viola_momentum_update"]
+            extra[f"muon_{method}"] = dict(step_ms=step_ms, step_wall_ms=step_wall, muon_elements=elements,
+                                           ns_gemm_ms=ns_ms, ns_tflops=ns_flops / (ns_ms * 1e-3) / 1e12,
+                                           ns_frac_bf16_peak=ns_flops / (ns_ms * 1e-3) / 1e12 / PEAK["bf16_tflops"],
+                                           momentum_gbs=8.03 * elements / (mom["avg_ms"] * mom["launches_per_step"] * 1e-3) / 1e9,
+                                           launches_per_step=sum(v["launches_per_step"] for v in b.values()))
+            del opt, params
+            torch.cuda.empty_cache()
+        from viola_amd.distributed import _fp8_kernels as codec, packet_bytes
+        n = 6553600
+        bucket = torch.randn(n, device="cuda") * 1e-3
+        packet = torch.empty((1, packet_bytes(n // 256, 256)), dtype=torch.uint8, device="cuda")
+        out = torch.empty_like(bucket)
+        pack_ms, _ = timed(lambda: codec.pack(bucket, packet, 256, torch.float8_e4m3fn), 50, 5)
+        unpack_ms, _ = timed(lambda: codec.unpack(packet, out, 256, torch.float8_e4m3fn), 50, 5)
+        extra["comm_codec"] = dict(bucket_elements=n, pack_ms=pack_ms, unpack_ms=unpack_ms,
+                                   pack_gbs=5.016 * n / (pack_ms * 1e-3) / 1e9, unpack_gbs=5.016 * n / (unpack_ms * 1e-3) / 1e9)
+
+    result = {
+        "metric": "FP8 Linear fwd+bwd TFLOPS (8192x1024->4096) + FP8Muon step ms; % of roofline",
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "wall_ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "e4m3 operands, fp32 accumulate", "data": "synthetic",
+        "config": {"workload": "viola.nn.Linear(1024, 4096, scaling='grouped', e4m3/e4m3, fp8 weight storage, mode='memory') "
+                               "forward+backward on 8192 tokens, bf16 activations and gradients"},
+        "frac_of_fp8_peak": value / PEAK["fp8_tflops"],
+        "roofline": roofline, "quantize": quant, "kernels": breakdown, **extra,
+    }
+    if not args.skip_cpu:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

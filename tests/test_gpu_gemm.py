@@ -10,10 +10,10 @@ pytestmark = pytest.mark.gpu
 E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
 
 
-def _operands(m, k, n, ga, gb, fa, fb, seed=2041):
+def _operands(m, k, n, ga, gb, fa, fb, seed=2041, spread=5):
     torch.manual_seed(seed)
-    a = (torch.randn(m, k) * torch.exp2(torch.randint(-5, 6, (m, 1)).float())).bfloat16()
-    b = (torch.randn(n, k) * torch.exp2(torch.randint(-5, 6, (n, 1)).float())).bfloat16()
+    a = (torch.randn(m, k) * torch.exp2(torch.randint(-spread, spread + 1, (m, 1)).float())).bfloat16()
+    b = (torch.randn(n, k) * torch.exp2(torch.randint(-spread, spread + 1, (n, 1)).float())).bfloat16()
     return og.quantize(a, fa, ga), og.quantize(b, fb, gb)
 
 
@@ -72,7 +72,8 @@ def test_gated_gemm_forward_backward(activation, m, h, k, dtype):
     gw = (32, 32) if h % 32 == 0 else (1, 32)
     layer = _Layer()
     layer.weight_group_shape = gw
-    (qa, sa), (qb, sb) = _operands(m, k, 2 * h, (1, 32), gw, E4, E4, seed=131)
+    spread = 5 if dtype == torch.bfloat16 else 1                              # keep g*u inside fp16's range
+    (qa, sa), (qb, sb) = _operands(m, k, 2 * h, (1, 32), gw, E4, E4, seed=131, spread=spread)
     bias = torch.randn(2 * h).to(dtype)
     out, aux, _ = mk.gemm(qa.cuda(), qb.cuda(), sa.cuda(), sb.cuda(), layer=layer, out_dtype=dtype, bias=bias.cuda(),
                           activation=activation, save=True)
@@ -85,7 +86,7 @@ def test_gated_gemm_forward_backward(activation, m, h, k, dtype):
     assert aux2.numel() == 0 and torch.equal(nosave, out)
     # backward: d = a2 . w2^T with w2 [h, k2]
     k2 = 96
-    (qg, sg), (qw, sw) = _operands(m, k2, h, (1, 32), (32, 32), E4, E4, seed=17)
+    (qg, sg), (qw, sw) = _operands(m, k2, h, (1, 32), (32, 32), E4, E4, seed=17, spread=spread)
     dz, _, _ = mk.gemm(qg.cuda(), qw.cuda(), sg.cuda(), sw.cuda(), layer=layer, out_dtype=dtype, backward=True,
                        activation=activation, aux=aux, group_a=(1, 32), group_b=(32, 32))
     d = og.gemm(qg, qw, sg, sw, (1, 32), (32, 32)).to(dtype)

@@ -77,10 +77,20 @@ def stream():
     return torch.cuda.current_stream().cuda_stream
 
 
+timeline = None   # when a list, every call appends (name, start_event, end_event) recorded on the current stream
+
+
 def call(name, *args):
     """Invoke one entry point on the current stream; non-zero status raises."""
     lib = library()
-    status = getattr(lib, name)(*args, stream())
+    if timeline is not None:
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        status = getattr(lib, name)(*args, stream())
+        end.record()
+        timeline.append((name, start, end))
+    else:
+        status = getattr(lib, name)(*args, stream())
     if status:
         raise RuntimeError(f"{name} failed: {lib.viola_error_string(status).decode()} (status {status})")
 
