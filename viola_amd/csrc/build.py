@@ -17,7 +17,7 @@ ARCH = "gfx950"
 # scale with an explicit fmaf.
 COMMON = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17", "-ffp-contract=off", "-fno-fast-math",
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
-SOURCES = ["quantize.hip", "gemm.hip", "ns.hip", "optim.hip", "misc.hip"]
+SOURCES = ["quantize.hip", "gemm.hip", "gemm_fast.hip", "ns.hip", "optim.hip", "misc.hip"]
 
 
 def hipcc():
@@ -46,7 +46,7 @@ def build(verbose=True):
             print(message, file=sys.stderr)
         return obj
 
-    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
+    with ThreadPoolExecutor(max_workers=min(6, len(SOURCES))) as pool:
         objects = list(pool.map(compile_one, SOURCES))
     link = [compiler, f"--offload-arch={ARCH}", "-shared", "-fPIC", *map(str, objects), "-o", str(LIBRARY)]
     result = subprocess.run(link, capture_output=True, text=True)

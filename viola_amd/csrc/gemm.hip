@@ -17,29 +17,11 @@
 // One kernel template serves: the plain GEMM, the gated-MLP forward (two 64-row panels of b, gate
 // and up, sharing a; epilogue act(g)*u), the gated-MLP backward (epilogue reads g,u and writes
 // [d*u*act'(g), d*act(g)]), the variable-group row-range GEMM and the variable-group wgrad.
-#include "common.hpp"
+#include "gemm_args.hpp"
 
 namespace viola {
 
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-
-constexpr int BM = 128, BN = 128, BK = 64, LDK = BK + 8, KG = BK / 32;
-enum { MODE_PLAIN = 0, MODE_GATED_FWD = 1, MODE_GATED_BWD = 2 };
-
-struct GemmArgs {
-    const uint8_t* a; const uint8_t* b; const float* sa; const float* sb;
-    const void* bias; void* out; void* aux;
-    int64_t m, n, k;              // n: rows of one b panel (h for the gated modes)
-    int64_t lda, ldb;             // bytes between rows of a / b
-    int64_t ldsa, ldsb;           // floats between rows of sa / sb
-    int64_t ldo;                  // elements between rows of out
-    int ar, br, ak_shift, bk_shift;
-    int activation;
-    // variable-group row ranges (grid.y walks the tiles of all groups)
-    const int64_t* offsets; int groups; int64_t b_group_stride, sb_group_stride;
-    // variable-group K ranges (grid.z = group): k range [koffsets[g], koffsets[g+1])
-    const int64_t* koffsets; int64_t out_group_stride;
-};
+constexpr int BK = 64, LDK = BK + 8, KG = BK / 32;
 
 template <bool A_BF8, bool B_BF8>
 __device__ __forceinline__ f32x16 mfma32(long x, long y, f32x16 c) {
@@ -323,24 +305,25 @@ static void launch_formats(const GemmArgs& p, int a_dtype, int b_dtype, int bias
 }
 
 template <int MODE, typename TO>
-static void launch_paths(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, bool rowscale, bool vec, dim3 grid,
-                         hipStream_t stream) {
-    if (rowscale) {
-        if (vec) launch_formats<MODE, true, true, TO>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
-        else launch_formats<MODE, true, false, TO>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
-    } else {
-        if (vec) launch_formats<MODE, false, true, TO>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
-        else launch_formats<MODE, false, false, TO>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
-    }
+static void launch_paths(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, bool rowscale, dim3 grid, hipStream_t stream) {
+    // the generic kernel is only built with guarded byte loads; aligned problems take the fast kernel
+    if (rowscale) launch_formats<MODE, true, false, TO>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
+    else launch_formats<MODE, false, false, TO>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
 }
 
 template <int MODE>
 static int launch_out(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, bool rowscale, bool vec,
                       dim3 grid, hipStream_t stream) {
+    const int64_t b_rows = MODE == MODE_GATED_FWD ? 2 * p.n : p.n;
+    // the fast kernel addresses operands and scales with 31-bit byte offsets
+    const bool small = b_rows * p.ldb < (1ll << 31) && (int64_t)BM * p.lda < (1ll << 31) &&
+                       (p.m + p.ar - 1) / p.ar * p.ldsa * 4 < (1ll << 31) && (b_rows + p.br - 1) / p.br * p.ldsb * 4 < (1ll << 31);
+    if (vec && small)
+        return launch_group_gemm_fast(p, MODE, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
     switch (out_dtype) {
-        case VIOLA_F32: launch_paths<MODE, float>(p, a_dtype, b_dtype, bias_dtype, rowscale, vec, grid, stream); break;
-        case VIOLA_BF16: launch_paths<MODE, bf16_t>(p, a_dtype, b_dtype, bias_dtype, rowscale, vec, grid, stream); break;
-        case VIOLA_F16: launch_paths<MODE, f16_t>(p, a_dtype, b_dtype, bias_dtype, rowscale, vec, grid, stream); break;
+        case VIOLA_F32: launch_paths<MODE, float>(p, a_dtype, b_dtype, bias_dtype, rowscale, grid, stream); break;
+        case VIOLA_BF16: launch_paths<MODE, bf16_t>(p, a_dtype, b_dtype, bias_dtype, rowscale, grid, stream); break;
+        case VIOLA_F16: launch_paths<MODE, f16_t>(p, a_dtype, b_dtype, bias_dtype, rowscale, grid, stream); break;
         default: return VIOLA_EINVAL;
     }
     return viola_launch_status();

@@ -1,0 +1,35 @@
+// Shared between the generic and the fast grouped-scale FP8 GEMM translation units.
+#pragma once
+#include "common.hpp"
+
+namespace viola {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 128, BN = 128;                                 // output tile of both kernels
+enum { MODE_PLAIN = 0, MODE_GATED_FWD = 1, MODE_GATED_BWD = 2 };
+
+struct GemmArgs {
+    const uint8_t* a; const uint8_t* b; const float* sa; const float* sb;
+    const void* bias; void* out; void* aux;
+    int64_t m, n, k;              // n: rows of one b panel (h for the gated modes)
+    int64_t lda, ldb;             // bytes between rows of a / b
+    int64_t ldsa, ldsb;           // floats between rows of sa / sb
+    int64_t ldo;                  // elements between rows of out
+    int ar, br, ak_shift, bk_shift;
+    int activation;
+    // variable-group row ranges (grid.y walks the tiles of all groups)
+    const int64_t* offsets; int groups; int64_t b_group_stride, sb_group_stride;
+    // variable-group K ranges (grid.z = group): k range [koffsets[g], koffsets[g+1])
+    const int64_t* koffsets; int64_t out_group_stride;
+    // fast kernel only: 1-D grid of tiles_m * tiles_n output tiles (rounded up to a multiple of 8) walked in an
+    // XCD-aware order; tiles_m == 0 keeps the plain (blockIdx.x, blockIdx.y) = (n tile, m tile) mapping
+    int tiles_m, tiles_n;
+};
+
+
+// Fast path (16-byte aligned operands, k ranges multiples of 16). Defined in gemm_fast.hip.
+int launch_group_gemm_fast(const GemmArgs& p, int mode, int a_dtype, int b_dtype, int bias_dtype, int out_dtype,
+                           bool rowscale, dim3 grid, hipStream_t stream);
+
+}  // namespace viola
