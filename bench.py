@@ -22,6 +22,11 @@ sys.path.insert(0, str(ROOT))
 
 M, K, N = 8192, 1024, 4096
 PEAK = {"fp8_tflops": 5000.0, "bf16_tflops": 2500.0, "hbm_gbs": 8000.0}
+# L2<->fabric bytes per grouped-scale GEMM launch, mean of the step's three launches (fwd, dgrad, wgrad), from two
+# `rocprofv3 --pmc` runs of `bench.py --skip-cpu --skip-muon --steps 5 --calibrate` (FETCH_SIZE, then WRITE_SIZE, KiB per
+# dispatch), each scaled by the same counter's reading for the 256 MiB copy_scaled_kernel launch (factors 2.00 and 1.00):
+# fetch (2 * 76.5 + 113.6) / 3 MB, write (2 * 41.9 + 8.4) / 3 MB. The algorithmic figure is 65 MB per launch.
+GEMM_TRAFFIC_BYTES = 88.9e6 + 30.7e6
 
 
 def timed(fn, steps, warmup):
@@ -120,6 +125,9 @@ def main():
     parser.add_argument("--warmup", type=int, default=3)
     parser.add_argument("--skip-cpu", action="store_true", help="leave out the CPU baseline leg")
     parser.add_argument("--skip-muon", action="store_true", help="leave out the FP8Muon / codec legs")
+    parser.add_argument("--calibrate", action="store_true",
+                        help="also launch copy_scaled_kernel once over 64 Mi floats (256 MiB read, 256 MiB written): "
+                             "the known-size kernel that FETCH_SIZE / WRITE_SIZE readings are scaled by")
     args = parser.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -135,9 +143,9 @@ def main():
     breakdown = kernel_breakdown(step, args.steps)
     gemm = breakdown["viola_group_gemm"]
     gemm_tflops = 2 * M * K * N / (gemm["avg_ms"] * 1e-3) / 1e12
-    roofline = dict(bound="mfma", kernel="group_gemm_kernel (viola_group_gemm: fwd, dgrad, wgrad)",
+    roofline = dict(bound="mfma", kernel="group_gemm_fast (viola_group_gemm: fwd, dgrad, wgrad)",
                     achieved=gemm_tflops, peak=PEAK["fp8_tflops"], unit="TFLOP/s", frac=gemm_tflops / PEAK["fp8_tflops"],
-                    avg_launch_ms=gemm["avg_ms"], traffic=None)
+                    avg_launch_ms=gemm["avg_ms"], traffic=GEMM_TRAFFIC_BYTES)
     quant = {}
     if "viola_group_quantize_dual" in breakdown:
         # X [M, K] and dY [M, N] each once per step: 4.25 B per element (bf16 in, two FP8 layouts + scales out)
@@ -178,6 +186,13 @@ def main():
         unpack_ms, _ = timed(lambda: codec.unpack(packet, out, 256, torch.float8_e4m3fn), 50, 5)
         extra["comm_codec"] = dict(bucket_elements=n, pack_ms=pack_ms, unpack_ms=unpack_ms,
                                    pack_gbs=5.016 * n / (pack_ms * 1e-3) / 1e9, unpack_gbs=5.016 * n / (unpack_ms * 1e-3) / 1e9)
+
+    if args.calibrate:
+        from viola_amd.optim import _kernels as ok
+        src = torch.ones(1 << 26, device="cuda")
+        dst = torch.empty_like(src)
+        ok.copy_scaled(src, dst, 0, 0, src.numel(), 1.0)
+        torch.cuda.synchronize()
 
     result = {
         "metric": "FP8 Linear fwd+bwd TFLOPS (8192x1024->4096) + FP8Muon step ms; % of roofline",
