@@ -35,6 +35,7 @@ class MatrixOptimizer(torch.optim.Optimizer):
             self.step_was_skipped = True
             return loss
         index = 0
+        work = []
         for group in self.param_groups:
             stable = group.get("viola_parameter_indices")
             for local, param in enumerate(group["params"]):
@@ -42,8 +43,14 @@ class MatrixOptimizer(torch.optim.Optimizer):
                 index += 1
                 if param.grad is None:          # no decay, no state advance for a missing gradient
                     continue
-                self._step_local(param, param.grad, self.state[param], group, position)
+                work.append((param, param.grad, self.state[param], group, position))
+        self._step_all(work)
         return loss
+
+    def _step_all(self, work):
+        """All (parameter, gradient, state, group, index) of one step; subclasses may batch equal shapes."""
+        for item in work:
+            self._step_local(*item)
 
     # Optimizer.load_state_dict casts floating state tensors to the parameter's dtype, which would
     # destroy the raw uint8 FP8 payload / fp32 scales / bf16 moments. Tensors are therefore set

@@ -85,18 +85,20 @@ class FP8Muon(MatrixOptimizer):
                           f"(e.g. {ragged[:3]}). Original matrix shapes are kept; edge groups use valid elements.",
                           stacklevel=3)
 
-    def _momentum(self, param, grad, state, group, key):
-        """Advance the FP8 momentum in place and return the bf16 update as a matrix view of the workspace."""
+    def _momentum(self, param, grad, state, group, key, out=None):
+        """Advance the FP8 momentum in place and return the bf16 update as a matrix view of the workspace
+        (or of `out`, a flat bf16 buffer of the parameter's size)."""
         shape = _shape(param, group)
         quant = dict(granularity=group["granularity"], tile_size=group["tile_size"], block_shape=group["block_shape"])
         if "momentum_q" not in state:
             payload, scales = state_sizes(shape, **quant)
             state["momentum_q"] = torch.zeros(payload, device=param.device, dtype=torch.uint8)
             state["momentum_scale"] = torch.ones(scales, device=param.device, dtype=torch.float32)
-        work = self._workspace.get(param.device)
-        if work is None or work.numel() < param.numel():
-            work = self._workspace[param.device] = torch.empty(param.numel(), device=param.device, dtype=torch.bfloat16)
-        matrix = work[:param.numel()].view(shape)
+        if out is None:
+            out = self._workspace.get(param.device)
+            if out is None or out.numel() < param.numel():
+                out = self._workspace[param.device] = torch.empty(param.numel(), device=param.device, dtype=torch.bfloat16)
+        matrix = out[:param.numel()].view(shape)
         q, scale = state["momentum_q"], state["momentum_scale"]
         before = (q.clone(), scale.clone()) if self.observer is not None else None
         momentum_update(grad, q, scale, q, scale, matrix.view(-1), beta=group["momentum"], nesterov=group["nesterov"],
@@ -105,6 +107,53 @@ class FP8Muon(MatrixOptimizer):
         if self.observer is not None:
             self.observer.momentum(param, grad, *before, q, scale, matrix, group, 1., quant)
         return matrix
+
+    # Equal-shaped matrices of one step go through Newton-Schulz as ONE batched GEMM chain: every matrix of
+    # the batch sees exactly the arithmetic it would see alone, and the launches fill the GPU.
+    _BATCH_ELEMENTS = 1 << 28
+
+    def _step_all(self, work):
+        if self.observer is not None:
+            return super()._step_all(work)
+        buckets = {}
+        for item in work:
+            param, grad, state, group, index = item
+            if not _use_muon(param, group):
+                self._step_local(*item)
+                continue
+            shape = _shape(param, group)
+            key = (shape, param.device, group["ns_method"], group["ns_steps"])
+            bucket = buckets.setdefault(key, [])
+            bucket.append(item)
+            if (len(bucket) + 1) * param.numel() > self._BATCH_ELEMENTS:
+                self._step_bucket(buckets.pop(key))
+        for bucket in buckets.values():
+            self._step_bucket(bucket)
+
+    def _step_bucket(self, bucket):
+        param, _, _, group, _ = bucket[0]
+        shape = _shape(param, group)
+        count = param.numel()
+        work = self._workspace.get(param.device)
+        if work is None or work.numel() < len(bucket) * count:
+            work = self._workspace[param.device] = torch.empty(len(bucket) * count, device=param.device, dtype=torch.bfloat16)
+        keys = []
+        for slot, (param, grad, state, group, index) in enumerate(bucket):
+            assert param.is_cuda and not grad.is_sparse
+            assert param.dtype in (torch.float32, torch.bfloat16, torch.float16), \
+                "Bind FP8 modules with viola.optim.bind_optimizer before stepping."
+            state.setdefault("step", 0)
+            key = (group["rounding_seed"] + index * 0x9E3779B97F4A7C15) & _MASK63
+            self._momentum(param, grad, state, group, key, out=work[slot * count:(slot + 1) * count])
+        stacked = work[:len(bucket) * count].view(len(bucket), -1, *shape[-2:])
+        updates = METHODS[group["ns_method"]](stacked, steps=group["ns_steps"]).reshape(len(bucket), count)
+        rows, cols = shape[-2:]
+        for slot, (param, grad, state, group, index) in enumerate(bucket):
+            master_key = (group["master_rounding_seed"] + index * 0x517CC1B727220A95) & _MASK63
+            scale = .2 * max(rows, cols) ** .5 if group["adjust_lr_fn"] == "match_rms_adamw" else max(1., rows / cols) ** .5
+            weight_update(param, updates[slot], group["lr"], group["weight_decay"], update_scale=scale,
+                          rounding=group["master_rounding"], step=state["step"], key=master_key)
+            state["step"] += 1
 
     def _step_local(self, param, grad, state, group, index):
         key = (group["rounding_seed"] + index * 0x9E3779B97F4A7C15) & _MASK63
