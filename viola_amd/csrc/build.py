@@ -17,7 +17,7 @@ ARCH = "gfx950"
 # scale with an explicit fmaf.
 COMMON = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17", "-ffp-contract=off", "-fno-fast-math",
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
-SOURCES = ["quantize.hip", "gemm.hip", "gemm_fast.hip", "ns.hip", "optim.hip", "misc.hip"]
+SOURCES = ["quantize.hip", "gemm.hip", "gemm_fast.hip", "ns.hip", "ns_fast.hip", "optim.hip", "misc.hip"]
 
 
 def hipcc():
@@ -31,12 +31,17 @@ def _filter(text):
     return "\n".join(line for line in text.splitlines() if "is not a recognized feature for this target" not in line)
 
 
-def build(verbose=True):
+def build(verbose=True, incremental=False):
+    """Compile every source and link. incremental=True (a development convenience) reuses objects that
+    are newer than their source and every header."""
     compiler = hipcc()
     objects = []
+    newest_header = max(h.stat().st_mtime for h in HERE.glob("*.hpp"))
 
     def compile_one(name):
         obj = HERE / (name.rsplit(".", 1)[0] + ".o")
+        if incremental and obj.exists() and obj.stat().st_mtime > newest_header and obj.stat().st_mtime > (HERE / name).stat().st_mtime:
+            return obj
         cmd = [compiler, *COMMON, "-c", str(HERE / name), "-o", str(obj)]
         result = subprocess.run(cmd, capture_output=True, text=True)
         message = _filter(result.stdout + result.stderr)
@@ -56,4 +61,4 @@ def build(verbose=True):
 
 
 if __name__ == "__main__":
-    print(build())
+    print(build(incremental="--incremental" in sys.argv))

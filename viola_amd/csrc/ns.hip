@@ -6,7 +6,7 @@
 // GEMM the b matrix is the MFMA "A" operand so a lane owns one output row m and runs of four
 // consecutive n. b may be given as [n, k] (transpose_b) or [k, n]; the latter is transposed on
 // its way into LDS.
-#include "common.hpp"
+#include "ns_args.hpp"
 
 namespace viola {
 
@@ -275,6 +275,11 @@ extern "C" int viola_ns_gemm(const void* a, const void* bmat, const void* residu
     VIOLA_CHECK_ARG(batch >= 0 && m >= 0 && n >= 0 && k >= 0);
     if (batch == 0 || m == 0 || n == 0) return 0;
     VIOLA_CHECK_ARG(out && (k == 0 || (a && bmat)) && (epilogue == 0 || residual));
+    if (k > 0) {
+        NsArgs fast{static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(bmat), static_cast<const uint16_t*>(residual),
+                    static_cast<uint16_t*>(out), static_cast<uint16_t*>(out_diag), batch, m, n, k, add_diag, 0, 0, 0};
+        if (launch_ns_gemm_fast(fast, dtype == VIOLA_BF16, !transpose_b, epilogue, stream)) return viola_launch_status();
+    }
     const int64_t gx = (n + NBN - 1) / NBN, gy = (m + NBM - 1) / NBM;
     VIOLA_CHECK_ARG(gy <= 65535 && batch <= 65535);
     const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch);

@@ -1,0 +1,23 @@
+// Arguments of the tiled Newton-Schulz GEMM (ns_fast.hip), shared with the entry point in ns.hip.
+#pragma once
+#include "common.hpp"
+
+namespace viola {
+
+struct NsArgs {
+    const uint16_t* a;          // [batch, m, k]
+    const uint16_t* b;          // [batch, n, k], or [batch, k, n] when b_kn
+    const uint16_t* residual;   // [batch, m, n] or null
+    uint16_t* out;              // [batch, m, n]
+    uint16_t* out_diag;         // second copy with add_diag on the diagonal, or null
+    int64_t batch, m, n, k;
+    float add_diag;
+    int tiles_m, tiles_n;
+    int64_t tiles;              // batch * tiles_m * tiles_n
+};
+
+// Launches the tiled kernel when the shape qualifies (16-byte aligned rows, k and n multiples of 8,
+// one matrix below 2 GiB); returns false without launching otherwise.
+bool launch_ns_gemm_fast(const NsArgs& args, bool is_bf16, bool b_kn, int epilogue, hipStream_t stream);
+
+}  // namespace viola

@@ -1,0 +1,242 @@
+// Tiled Newton-Schulz GEMM for gfx950: batched out[b] = a[b] . b[b]^T (b as [n, k]) or a[b] . b[b] (b as
+// [k, n]) in bf16 / fp16 on v_mfma_f32_32x32x16, fp32 accumulation, with the chain's epilogues.
+//
+// Block: 256 threads = 2 x 2 wavefronts, each owning WM x WN accumulators of 32 x 32 (192 x 192 tiles
+// for the 1152-multiples of transformer blocks, 128 x 128 otherwise), two blocks per CU so one block's
+// barrier and LDS traffic hide behind the other's MFMAs.
+//   * global -> registers (raw buffer loads, out-of-range lanes read zero: no tail branches) -> LDS,
+//     32 k per stage, two stages; the loads of chunk c+2 are in flight during the math of chunk c.
+//   * k-contiguous operands ([m, k] and [n, k]) sit in LDS as rows of 32 + 8 elements and are read with
+//     ds_read_b128; an [k, n] operand keeps its layout (rows of BN + 32 elements) and is transposed on
+//     the way out of LDS by ds_read_b64_tr_b16, which hands lane i of each 16-lane group the four k
+//     values of column i.
+//   * the b matrix is the MFMA "A" source, so a lane owns one output row m and runs of four
+//     consecutive n: 8-byte stores, per-row residual loads.
+//   * work order: the 1-D grid is cut into eight contiguous ranges, one per XCD (blockIdx % 8), and
+//     inside a range tiles walk n fastest, so the tiles that share an a panel meet in one L2.
+#include "ns_args.hpp"
+
+namespace viola {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int SBK = 32;             // k per LDS stage
+constexpr int SLDK = SBK + 8;       // row stride (elements) of a k-contiguous tile: 80 bytes
+constexpr uint32_t NS_OUTSIDE = 0x80000000u;
+
+template <bool IS_BF16>
+__device__ __forceinline__ f32x16 ns_mfma(uint4 x, uint4 y, f32x16 c) {
+    if constexpr (IS_BF16) return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, x), __builtin_bit_cast(bf16x8, y), c, 0, 0, 0);
+    else return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, x), __builtin_bit_cast(f16x8, y), c, 0, 0, 0);
+}
+template <bool IS_BF16> __device__ __forceinline__ float ns_widen(uint16_t bits) {
+    if constexpr (IS_BF16) return bf16_bits_to_f32(bits);
+    else { _Float16 h; __builtin_memcpy(&h, &bits, 2); return (float)h; }
+}
+template <bool IS_BF16> __device__ __forceinline__ uint16_t ns_narrow(float v) {
+    if constexpr (IS_BF16) return f32_to_bf16_bits(v);
+    else { _Float16 h = (_Float16)v; uint16_t bits; __builtin_memcpy(&bits, &h, 2); return bits; }
+}
+
+template <bool IS_BF16, bool B_KN, int EPILOGUE, int WM, int WN>
+__global__ __launch_bounds__(256, 2) void ns_gemm_fast(NsArgs p) {
+    constexpr int BM = 64 * WM, BN = 64 * WN;
+    constexpr int LDN = BN + 32;                                     // row stride of a [k, n] tile
+    constexpr int A_EL = BM * SLDK, B_EL = B_KN ? SBK * LDN : BN * SLDK;
+    constexpr int NCH = BN / 8;                                      // 16-byte chunks per [k, n] row
+    __shared__ __attribute__((aligned(16))) uint16_t lds[2][A_EL + B_EL];
+
+    const int64_t per_xcd = (p.tiles + 7) / 8;
+    const int64_t seq = blockIdx.x / 8;
+    const int64_t work = (int64_t)(blockIdx.x % 8) * per_xcd + seq;
+    if (work >= p.tiles) return;
+    const int tn = (int)(work % p.tiles_n);
+    const int tm = (int)((work / p.tiles_n) % p.tiles_m);
+    const int64_t bz = work / ((int64_t)p.tiles_n * p.tiles_m);
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    const int64_t m = p.m, n = p.n, k = p.k;
+
+    const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+    const int wm = wave / 2, wn = wave % 2, l32 = lane % 32, lhi = lane / 32;
+
+    const uint16_t* abase = p.a + bz * m * k;
+    const uint16_t* bbase = p.b + bz * n * k;
+    const __amdgpu_buffer_rsrc_t res_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(abase), 0, 0x7fffffff, 0x00020000);
+    const __amdgpu_buffer_rsrc_t res_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(bbase), 0, 0x7fffffff, 0x00020000);
+
+    // per-thread byte offsets of the 16-byte pieces it moves per chunk (k0 = 0), and their k position
+    uint32_t a_off[WM], b_off[WN];
+    int a_k[WM], b_k[WN];
+    int a_lds[WM], b_lds[WN];
+#pragma unroll
+    for (int it = 0; it < WM; ++it) {
+        const int id = it * 256 + tid, lr = id / 4, c = id % 4;
+        const int64_t row = m0 + lr;
+        a_off[it] = row < m ? (uint32_t)((row * k + c * 8) * 2) : NS_OUTSIDE;
+        a_k[it] = c * 8;
+        a_lds[it] = lr * SLDK + c * 8;
+    }
+#pragma unroll
+    for (int it = 0; it < WN; ++it) {
+        const int id = it * 256 + tid;
+        if constexpr (B_KN) {
+            const int kr = id / NCH, cn = id % NCH;
+            const int64_t col = n0 + cn * 8;
+            b_off[it] = col < n ? (uint32_t)(((int64_t)kr * n + col) * 2) : NS_OUTSIDE;
+            b_k[it] = kr;
+            b_lds[it] = A_EL + kr * LDN + cn * 8;
+        } else {
+            const int lr = id / 4, c = id % 4;
+            const int64_t row = n0 + lr;
+            b_off[it] = row < n ? (uint32_t)((row * k + c * 8) * 2) : NS_OUTSIDE;
+            b_k[it] = c * 8;
+            b_lds[it] = A_EL + lr * SLDK + c * 8;
+        }
+    }
+
+    u32x4 ra[WM], rb[WN];
+    auto fetch = [&](int64_t k0) {
+        const uint32_t a_step = (uint32_t)(k0 * 2);
+        const uint32_t b_step = B_KN ? (uint32_t)(k0 * n * 2) : (uint32_t)(k0 * 2);
+#pragma unroll
+        for (int it = 0; it < WM; ++it) {
+            const bool inside = k0 + a_k[it] < k;
+            ra[it] = __builtin_amdgcn_raw_buffer_load_b128(res_a, inside ? (int)(a_off[it] + a_step) : (int)NS_OUTSIDE, 0, 0);
+        }
+#pragma unroll
+        for (int it = 0; it < WN; ++it) {
+            const bool inside = k0 + b_k[it] < k;
+            rb[it] = __builtin_amdgcn_raw_buffer_load_b128(res_b, inside ? (int)(b_off[it] + b_step) : (int)NS_OUTSIDE, 0, 0);
+        }
+    };
+    auto stash = [&](int s) {
+#pragma unroll
+        for (int it = 0; it < WM; ++it) *reinterpret_cast<u32x4*>(&lds[s][a_lds[it]]) = ra[it];
+#pragma unroll
+        for (int it = 0; it < WN; ++it) *reinterpret_cast<u32x4*>(&lds[s][b_lds[it]]) = rb[it];
+    };
+
+    // fragment addresses (elements) inside a stage
+    const int a_frag = (wm * 32 * WM + l32) * SLDK + lhi * 8;
+    const int b_frag = B_KN ? A_EL + (lhi * 8 + ((lane & 15) >> 2)) * LDN + wn * 32 * WN + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)
+                            : A_EL + (wn * 32 * WN + l32) * SLDK + lhi * 8;
+
+    f32x16 acc[WN][WM];
+#pragma unroll
+    for (int i = 0; i < WN; ++i)
+#pragma unroll
+        for (int j = 0; j < WM; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    auto compute = [&](int s) {
+#pragma unroll
+        for (int ks = 0; ks < SBK / 16; ++ks) {
+            uint4 opa[WM], opb[WN];
+#pragma unroll
+            for (int i = 0; i < WN; ++i) {
+                if constexpr (B_KN) {
+                    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+                    const uint16_t* at = &lds[s][b_frag + ks * 16 * LDN + i * 32];
+                    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)at);
+                    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at + 4 * LDN));
+                    const uint2 l2 = __builtin_bit_cast(uint2, lo), h2 = __builtin_bit_cast(uint2, hi);
+                    opb[i] = make_uint4(l2.x, l2.y, h2.x, h2.y);
+                } else {
+                    opb[i] = *reinterpret_cast<const uint4*>(&lds[s][b_frag + i * 32 * SLDK + ks * 16]);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < WM; ++j) opa[j] = *reinterpret_cast<const uint4*>(&lds[s][a_frag + j * 32 * SLDK + ks * 16]);
+#pragma unroll
+            for (int i = 0; i < WN; ++i)
+#pragma unroll
+                for (int j = 0; j < WM; ++j) acc[i][j] = ns_mfma<IS_BF16>(opb[i], opa[j], acc[i][j]);
+        }
+    };
+
+    const int64_t chunks = (k + SBK - 1) / SBK;
+    fetch(0);
+    stash(0);
+    fetch(SBK);
+    __syncthreads();
+    for (int64_t c = 0; c < chunks; ++c) {
+        const int s = (int)(c & 1);
+        stash(s ^ 1);                       // chunk c+1 (zeros past the end)
+        fetch((c + 2) * SBK);
+        compute(s);
+        __syncthreads();
+    }
+
+    const uint16_t* residual = EPILOGUE ? p.residual + bz * m * n : nullptr;
+    uint16_t* out = p.out + bz * m * n;
+    uint16_t* out_diag = p.out_diag ? p.out_diag + bz * m * n : nullptr;
+#pragma unroll
+    for (int j = 0; j < WM; ++j) {
+        const int64_t row = m0 + wm * 32 * WM + j * 32 + l32;
+        if (row >= m) continue;
+#pragma unroll
+        for (int i = 0; i < WN; ++i) {
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const int64_t col = n0 + wn * 32 * WN + i * 32 + r4 * 8 + lhi * 4;
+                if (col >= n) continue;                               // n is a multiple of 8: whole quads
+                uint16_t res[4] = {0, 0, 0, 0}, o[4], od[4];
+                if (EPILOGUE) {
+                    const uint2 raw = *reinterpret_cast<const uint2*>(residual + row * n + col);
+                    res[0] = (uint16_t)raw.x; res[1] = (uint16_t)(raw.x >> 16); res[2] = (uint16_t)raw.y; res[3] = (uint16_t)(raw.y >> 16);
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float value = ns_widen<IS_BF16>(ns_narrow<IS_BF16>(acc[i][j][r4 * 4 + e]));
+                    if (EPILOGUE == 1) value = -4.7750f * ns_widen<IS_BF16>(res[e]) + 2.0315f * value;
+                    if (EPILOGUE == 2) value = value + 3.4445f * ns_widen<IS_BF16>(res[e]);
+                    const uint16_t bits = ns_narrow<IS_BF16>(value);
+                    o[e] = bits;
+                    od[e] = col + e == row ? ns_narrow<IS_BF16>(ns_widen<IS_BF16>(bits) + p.add_diag) : bits;
+                }
+                *reinterpret_cast<uint2*>(out + row * n + col) = make_uint2((uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16));
+                if (out_diag) *reinterpret_cast<uint2*>(out_diag + row * n + col) = make_uint2((uint32_t)od[0] | ((uint32_t)od[1] << 16), (uint32_t)od[2] | ((uint32_t)od[3] << 16));
+            }
+        }
+    }
+}
+
+template <bool IS_BF16, bool B_KN, int WM, int WN>
+static void launch_tiles(NsArgs p, int epilogue, hipStream_t stream) {
+    constexpr int BM = 64 * WM, BN = 64 * WN;
+    p.tiles_m = (int)((p.m + BM - 1) / BM);
+    p.tiles_n = (int)((p.n + BN - 1) / BN);
+    p.tiles = p.batch * p.tiles_m * p.tiles_n;
+    const unsigned grid = (unsigned)((p.tiles + 7) / 8 * 8);
+    if (epilogue == 0) hipLaunchKernelGGL((ns_gemm_fast<IS_BF16, B_KN, 0, WM, WN>), dim3(grid), dim3(256), 0, stream, p);
+    else if (epilogue == 1) hipLaunchKernelGGL((ns_gemm_fast<IS_BF16, B_KN, 1, WM, WN>), dim3(grid), dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL((ns_gemm_fast<IS_BF16, B_KN, 2, WM, WN>), dim3(grid), dim3(256), 0, stream, p);
+}
+
+template <bool IS_BF16, bool B_KN>
+static void launch_shape(const NsArgs& p, int epilogue, hipStream_t stream) {
+    // 192-wide tiles move a third less operand data per flop; take them unless their padding costs more
+    // than that (1152 = 6 x 192 and its multiples fit exactly)
+    auto area = [&](int64_t t) { return ((p.m + t - 1) / t) * ((p.n + t - 1) / t) * t * t; };
+    if (area(192) * 20 <= area(128) * 21) launch_tiles<IS_BF16, B_KN, 3, 3>(p, epilogue, stream);
+    else launch_tiles<IS_BF16, B_KN, 2, 2>(p, epilogue, stream);
+}
+
+bool launch_ns_gemm_fast(const NsArgs& p, bool is_bf16, bool b_kn, int epilogue, hipStream_t stream) {
+    auto aligned = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+    if (p.k % 8 || p.n % 8 || p.k == 0) return false;
+    if (!aligned(p.a) || !aligned(p.b) || !aligned(p.out) || !aligned(p.residual) || !aligned(p.out_diag)) return false;
+    const int64_t limit = (1ll << 31) - 65536;
+    if (p.m * p.k * 2 >= limit || p.n * p.k * 2 >= limit) return false;
+    if (p.batch * ((p.m + 127) / 128) * ((p.n + 127) / 128) >= (1ll << 31) - 8) return false;
+    if (is_bf16) { if (b_kn) launch_shape<true, true>(p, epilogue, stream); else launch_shape<true, false>(p, epilogue, stream); }
+    else { if (b_kn) launch_shape<false, true>(p, epilogue, stream); else launch_shape<false, false>(p, epilogue, stream); }
+    return true;
+}
+
+}  // namespace viola
