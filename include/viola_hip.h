@@ -153,10 +153,12 @@ int viola_momentum_dequantize(const void* q, const float* scale, float* out, int
  * then epilogue 0: nothing; 1: -4.7750*residual + 2.0315*value; 2: value + 3.4445*residual; rounded
  * to dtype. a [batch, m, k]; bmat [batch, n, k] if transpose_b else [batch, k, n]; dtype bf16 or f16.
  * out_diag (nullable) receives a second copy of the result with add_diag added to its diagonal after
- * rounding (Q = Z + 3.4445 I, viola/optim/_orthogonalize.py:45-47). */
+ * rounding (Q = Z + 3.4445 I, viola/optim/_orthogonalize.py:45-47). transpose_out = 1 stores out and
+ * out_diag as [batch, n, m] (the un-transposition of a tall matrix at the end of the chain,
+ * viola/optim/_orthogonalize.py:20-21,52-53); residual stays [batch, m, n]. */
 int viola_ns_gemm(const void* a, const void* bmat, const void* residual, void* out, int dtype,
                   int transpose_b, int epilogue, int64_t batch, int64_t m, int64_t n, int64_t k,
-                  float add_diag, void* out_diag, viola_stream_t stream);
+                  float add_diag, void* out_diag, int transpose_out, viola_stream_t stream);
 
 /* viola/optim/_orthogonalize.py:12-16 / _orthogonalize_kernels.py:80-84: x = dtype(matrix), optionally
  * transposed so rows <= cols, divided by (Frobenius norm + 1e-7), all in the working dtype.

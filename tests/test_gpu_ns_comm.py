@@ -14,7 +14,7 @@ E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("batch,m,n,k", [(1, 64, 64, 256), (2, 130, 72, 96), (1, 256, 384, 128), (3, 33, 47, 65)])
+@pytest.mark.parametrize("batch,m,n,k", [(1, 64, 64, 256), (2, 130, 72, 96), (1, 256, 384, 128), (3, 33, 47, 65), (2, 384, 576, 200)])
 @pytest.mark.parametrize("transpose_b,epilogue", [(True, 0), (False, 0), (False, 1), (True, 1), (False, 2)])
 def test_ns_gemm_contract(dtype, batch, m, n, k, transpose_b, epilogue):
     """One chain GEMM against its contract: fp32 accumulate -> round -> fp32 epilogue -> round."""
@@ -29,7 +29,10 @@ def test_ns_gemm_contract(dtype, batch, m, n, k, transpose_b, epilogue):
     # identical except where a different fp32 summation order flips the final rounding (one ulp of the output dtype)
     ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
     diff = (out.cpu().float() - ref.float()).abs()
-    bound = 4 * ulp * ref.float().abs() + 1e-4 * ref.float().abs().max()      # second term: cancellation near zero
+    # second term: the rounded product may flip by one ulp before the epilogue scales it (by 2.0315 at most),
+    # which is not small next to a result that cancels towards zero
+    product = ons.matmul(a, b, transpose_b=transpose_b).float().abs()
+    bound = 4 * ulp * ref.float().abs() + 2.1 * ulp * product + 1e-4 * ref.float().abs().max()
     assert (diff <= bound).all()
     assert rel_l2(out, ref) < (2e-3 if dtype == torch.bfloat16 else 3e-4)
     assert (diff == 0).float().mean() > .9
@@ -39,6 +42,40 @@ def test_ns_gemm_contract(dtype, batch, m, n, k, transpose_b, epilogue):
         expect = out.clone()
         expect.diagonal(dim1=-2, dim2=-1).add_(3.4445)
         assert torch.equal(q, expect)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("batch,m,k", [(2, 384, 200), (1, 576, 96), (3, 200, 72), (1, 1152, 64)])
+@pytest.mark.parametrize("epilogue", [0, 1])
+def test_ns_gram_product_is_mirrored(dtype, batch, m, k, epilogue):
+    """a . a^T (same buffer for both operands) computes the upper tiles only and mirrors them: the result
+    must equal the product taken with b as a separate copy of a, and be exactly symmetric."""
+    from viola_amd.optim import _orthogonalize_kernels as nk
+    torch.manual_seed(21)
+    a = (torch.randn(batch, m, k) / math.sqrt(k)).to(dtype).cuda()
+    r = nk._matmul(a, a, transpose_b=True)
+    residual = r if epilogue else None
+    same = nk._matmul(a, a, transpose_b=True, residual=residual, epilogue=epilogue, add_diag=3.4445 if epilogue else None)
+    other = nk._matmul(a, a.clone(), transpose_b=True, residual=residual, epilogue=epilogue, add_diag=3.4445 if epilogue else None)
+    for x, y in zip(same if epilogue else (same,), other if epilogue else (other,)):
+        assert torch.equal(x, y)
+        assert torch.equal(x, x.mT)
+    ref = ons.matmul(a.cpu(), a.cpu(), transpose_b=True, residual=residual.cpu() if epilogue else None, epilogue=epilogue)
+    assert rel_l2(same[0] if epilogue else same, ref) < (2e-3 if dtype == torch.bfloat16 else 3e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("batch,m,n,k", [(2, 192, 384, 192), (1, 130, 72, 96), (2, 64, 200, 136), (1, 33, 47, 65)])
+@pytest.mark.parametrize("transpose_b,epilogue", [(False, 2), (False, 0), (True, 0)])
+def test_ns_gemm_transposed_output(dtype, batch, m, n, k, transpose_b, epilogue):
+    from viola_amd.optim import _orthogonalize_kernels as nk
+    torch.manual_seed(22)
+    a = (torch.randn(batch, m, k) / math.sqrt(k)).to(dtype).cuda()
+    b = (torch.randn(batch, n, k) if transpose_b else torch.randn(batch, k, n)).to(dtype).cuda()
+    residual = torch.randn(batch, m, n).to(dtype).cuda() if epilogue else None
+    plain = nk._matmul(a, b, transpose_b=transpose_b, residual=residual, epilogue=epilogue)
+    flipped = nk._matmul(a, b, transpose_b=transpose_b, residual=residual, epilogue=epilogue, transpose_out=True)
+    assert flipped.shape == (batch, n, m) and torch.equal(flipped, plain.mT.contiguous())
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

@@ -37,7 +37,7 @@ template <bool IS_BF16, bool TRANSPOSE_B, int EPILOGUE, bool VEC>
 __global__ __launch_bounds__(256, 2) void ns_gemm_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b,
                                                           const uint16_t* __restrict__ residual, uint16_t* __restrict__ out,
                                                           uint16_t* __restrict__ out_diag, int64_t m, int64_t n, int64_t k,
-                                                          float add_diag) {
+                                                          float add_diag, int transpose_out) {
     __shared__ __attribute__((aligned(16))) uint16_t lds_a[2][NBM * NLD];
     __shared__ __attribute__((aligned(16))) uint16_t lds_b[2][NBN * NLD];
     const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
@@ -158,7 +158,13 @@ __global__ __launch_bounds__(256, 2) void ns_gemm_kernel(const uint16_t* __restr
                     o[e] = bits;
                     od[e] = col + e == row ? f32_to_half<IS_BF16>(half_to_f32<IS_BF16>(bits) + add_diag) : bits;
                 }
-                if (full) {
+                if (transpose_out) {
+                    for (int e = 0; e < 4; ++e)
+                        if (col + e < n) {
+                            out[(col + e) * m + row] = o[e];
+                            if (out_diag) out_diag[(col + e) * m + row] = od[e];
+                        }
+                } else if (full) {
                     *reinterpret_cast<uint2*>(out + row * n + col) = make_uint2((uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16));
                     if (out_diag) *reinterpret_cast<uint2*>(out_diag + row * n + col) = make_uint2((uint32_t)od[0] | ((uint32_t)od[1] << 16), (uint32_t)od[2] | ((uint32_t)od[3] << 16));
                 } else {
@@ -240,15 +246,15 @@ __global__ __launch_bounds__(256) void ns_scale_kernel(const TIn* __restrict__ i
 
 template <bool IS_BF16, bool TRANSPOSE_B, bool VEC>
 static int launch_ns(const void* a, const void* b, const void* residual, void* out, void* out_diag, int epilogue, dim3 grid,
-                     int64_t m, int64_t n, int64_t k, float add_diag, hipStream_t stream) {
+                     int64_t m, int64_t n, int64_t k, float add_diag, int transpose_out, hipStream_t stream) {
     const uint16_t* ap = static_cast<const uint16_t*>(a);
     const uint16_t* bp = static_cast<const uint16_t*>(b);
     const uint16_t* rp = static_cast<const uint16_t*>(residual);
     uint16_t* op = static_cast<uint16_t*>(out);
     uint16_t* dp = static_cast<uint16_t*>(out_diag);
-    if (epilogue == 0) hipLaunchKernelGGL((ns_gemm_kernel<IS_BF16, TRANSPOSE_B, 0, VEC>), grid, dim3(256), 0, stream, ap, bp, rp, op, dp, m, n, k, add_diag);
-    else if (epilogue == 1) hipLaunchKernelGGL((ns_gemm_kernel<IS_BF16, TRANSPOSE_B, 1, VEC>), grid, dim3(256), 0, stream, ap, bp, rp, op, dp, m, n, k, add_diag);
-    else hipLaunchKernelGGL((ns_gemm_kernel<IS_BF16, TRANSPOSE_B, 2, VEC>), grid, dim3(256), 0, stream, ap, bp, rp, op, dp, m, n, k, add_diag);
+    if (epilogue == 0) hipLaunchKernelGGL((ns_gemm_kernel<IS_BF16, TRANSPOSE_B, 0, VEC>), grid, dim3(256), 0, stream, ap, bp, rp, op, dp, m, n, k, add_diag, transpose_out);
+    else if (epilogue == 1) hipLaunchKernelGGL((ns_gemm_kernel<IS_BF16, TRANSPOSE_B, 1, VEC>), grid, dim3(256), 0, stream, ap, bp, rp, op, dp, m, n, k, add_diag, transpose_out);
+    else hipLaunchKernelGGL((ns_gemm_kernel<IS_BF16, TRANSPOSE_B, 2, VEC>), grid, dim3(256), 0, stream, ap, bp, rp, op, dp, m, n, k, add_diag, transpose_out);
     return viola_launch_status();
 }
 
@@ -269,7 +275,7 @@ using namespace viola;
 
 extern "C" int viola_ns_gemm(const void* a, const void* bmat, const void* residual, void* out, int dtype, int transpose_b,
                              int epilogue, int64_t batch, int64_t m, int64_t n, int64_t k, float add_diag, void* out_diag,
-                             viola_stream_t stream_) {
+                             int transpose_out, viola_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     VIOLA_CHECK_ARG((dtype == VIOLA_BF16 || dtype == VIOLA_F16) && epilogue >= 0 && epilogue <= 2);
     VIOLA_CHECK_ARG(batch >= 0 && m >= 0 && n >= 0 && k >= 0);
@@ -277,7 +283,8 @@ extern "C" int viola_ns_gemm(const void* a, const void* bmat, const void* residu
     VIOLA_CHECK_ARG(out && (k == 0 || (a && bmat)) && (epilogue == 0 || residual));
     if (k > 0) {
         NsArgs fast{static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(bmat), static_cast<const uint16_t*>(residual),
-                    static_cast<uint16_t*>(out), static_cast<uint16_t*>(out_diag), batch, m, n, k, add_diag, 0, 0, 0};
+                    static_cast<uint16_t*>(out), static_cast<uint16_t*>(out_diag), batch, m, n, k, add_diag, transpose_out,
+                    transpose_b && a == bmat && m == n, 0, 0, 0};
         if (launch_ns_gemm_fast(fast, dtype == VIOLA_BF16, !transpose_b, epilogue, stream)) return viola_launch_status();
     }
     const int64_t gx = (n + NBN - 1) / NBN, gy = (m + NBM - 1) / NBM;
@@ -285,7 +292,7 @@ extern "C" int viola_ns_gemm(const void* a, const void* bmat, const void* residu
     const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch);
     auto al = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
     const bool vec = k % 8 == 0 && n % 8 == 0 && al(a) && al(bmat) && al(out) && (!residual || al(residual)) && (!out_diag || al(out_diag));
-#define VIOLA_NS(BF, TB, V) return launch_ns<BF, TB, V>(a, bmat, residual, out, out_diag, epilogue, grid, m, n, k, add_diag, stream)
+#define VIOLA_NS(BF, TB, V) return launch_ns<BF, TB, V>(a, bmat, residual, out, out_diag, epilogue, grid, m, n, k, add_diag, transpose_out, stream)
     if (dtype == VIOLA_BF16) {
         if (transpose_b) { if (vec) VIOLA_NS(true, true, true); VIOLA_NS(true, true, false); }
         if (vec) VIOLA_NS(true, false, true);

@@ -12,6 +12,8 @@ struct NsArgs {
     uint16_t* out_diag;         // second copy with add_diag on the diagonal, or null
     int64_t batch, m, n, k;
     float add_diag;
+    int transpose_out;          // store out (and out_diag) as [batch, n, m]
+    int symmetric;              // b == a, m == n: compute tiles with tn >= tm only and mirror them
     int tiles_m, tiles_n;
     int64_t tiles;              // batch * tiles_m * tiles_n
 };

@@ -12,6 +12,8 @@
 //     values of column i.
 //   * the b matrix is the MFMA "A" source, so a lane owns one output row m and runs of four
 //     consecutive n: 8-byte stores, per-row residual loads.
+//   * a Gram-type product (b == a, square output) computes only the tiles on and above the diagonal and
+//     stores each off-diagonal tile a second time transposed; transpose_out stores [n, m] only.
 //   * work order: the 1-D grid is cut into eight contiguous ranges, one per XCD (blockIdx % 8), and
 //     inside a range tiles walk n fastest, so the tiles that share an a panel meet in one L2.
 #include "ns_args.hpp"
@@ -54,9 +56,22 @@ __global__ __launch_bounds__(256, 2) void ns_gemm_fast(NsArgs p) {
     const int64_t seq = blockIdx.x / 8;
     const int64_t work = (int64_t)(blockIdx.x % 8) * per_xcd + seq;
     if (work >= p.tiles) return;
-    const int tn = (int)(work % p.tiles_n);
-    const int tm = (int)((work / p.tiles_n) % p.tiles_m);
-    const int64_t bz = work / ((int64_t)p.tiles_n * p.tiles_m);
+    int tm, tn;
+    int64_t bz;
+    if (p.symmetric) {
+        // upper triangle of the tile grid, row by row: row tm holds tiles_n - tm tiles
+        const int64_t upper = (int64_t)p.tiles_n * (p.tiles_n + 1) / 2;
+        bz = work / upper;
+        int rest = (int)(work % upper);
+        tm = 0;
+        while (rest >= p.tiles_n - tm) { rest -= p.tiles_n - tm; ++tm; }
+        tn = tm + rest;
+    } else {
+        tn = (int)(work % p.tiles_n);
+        tm = (int)((work / p.tiles_n) % p.tiles_m);
+        bz = work / ((int64_t)p.tiles_n * p.tiles_m);
+    }
+    const bool mirror = p.symmetric && tn != tm;
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
     const int64_t m = p.m, n = p.n, k = p.k;
 
@@ -199,8 +214,19 @@ __global__ __launch_bounds__(256, 2) void ns_gemm_fast(NsArgs p) {
                     o[e] = bits;
                     od[e] = col + e == row ? ns_narrow<IS_BF16>(ns_widen<IS_BF16>(bits) + p.add_diag) : bits;
                 }
-                *reinterpret_cast<uint2*>(out + row * n + col) = make_uint2((uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16));
-                if (out_diag) *reinterpret_cast<uint2*>(out_diag + row * n + col) = make_uint2((uint32_t)od[0] | ((uint32_t)od[1] << 16), (uint32_t)od[2] | ((uint32_t)od[3] << 16));
+                if (!p.transpose_out) {
+                    *reinterpret_cast<uint2*>(out + row * n + col) = make_uint2((uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16));
+                    if (out_diag) *reinterpret_cast<uint2*>(out_diag + row * n + col) = make_uint2((uint32_t)od[0] | ((uint32_t)od[1] << 16), (uint32_t)od[2] | ((uint32_t)od[3] << 16));
+                }
+                if (p.transpose_out || mirror) {
+                    // [n, m] placement: 32 lanes hold 32 consecutive m of one n, so each 2-byte store
+                    // instruction still fills 64-byte segments
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        out[(col + e) * m + row] = o[e];
+                        if (out_diag) out_diag[(col + e) * m + row] = od[e];
+                    }
+                }
             }
         }
     }
@@ -211,7 +237,7 @@ static void launch_tiles(NsArgs p, int epilogue, hipStream_t stream) {
     constexpr int BM = 64 * WM, BN = 64 * WN;
     p.tiles_m = (int)((p.m + BM - 1) / BM);
     p.tiles_n = (int)((p.n + BN - 1) / BN);
-    p.tiles = p.batch * p.tiles_m * p.tiles_n;
+    p.tiles = p.batch * (p.symmetric ? (int64_t)p.tiles_n * (p.tiles_n + 1) / 2 : (int64_t)p.tiles_m * p.tiles_n);
     const unsigned grid = (unsigned)((p.tiles + 7) / 8 * 8);
     if (epilogue == 0) hipLaunchKernelGGL((ns_gemm_fast<IS_BF16, B_KN, 0, WM, WN>), dim3(grid), dim3(256), 0, stream, p);
     else if (epilogue == 1) hipLaunchKernelGGL((ns_gemm_fast<IS_BF16, B_KN, 1, WM, WN>), dim3(grid), dim3(256), 0, stream, p);

@@ -12,14 +12,15 @@ from .. import _lib
 A_COEFF = 3.4445
 
 
-def _matmul(a, b, *, transpose_b=False, residual=None, epilogue=0, add_diag=None):
-    """One chain GEMM. With add_diag, also returns a copy of the result with add_diag on its diagonal."""
+def _matmul(a, b, *, transpose_b=False, residual=None, epilogue=0, add_diag=None, transpose_out=False):
+    """One chain GEMM. With add_diag, also returns a copy of the result with add_diag on its diagonal;
+    transpose_out stores the result as [batch, n, m]."""
     batch, m, k = a.shape
     n = b.shape[-2] if transpose_b else b.shape[-1]
-    out = a.new_empty((batch, m, n))
-    second = a.new_empty((batch, m, n)) if add_diag is not None else None
+    out = a.new_empty((batch, n, m) if transpose_out else (batch, m, n))
+    second = a.new_empty(out.shape) if add_diag is not None else None
     _lib.call("viola_ns_gemm", _lib.ptr(a), _lib.ptr(b), _lib.ptr(residual), _lib.ptr(out), _lib.code(a.dtype),
-              int(transpose_b), epilogue, batch, m, n, k, float(add_diag or 0.0), _lib.ptr(second))
+              int(transpose_b), epilogue, batch, m, n, k, float(add_diag or 0.0), _lib.ptr(second), int(transpose_out))
     return out if add_diag is None else (out, second)
 
 
@@ -40,14 +41,13 @@ def run(matrix, steps, method):
     dtype = torch.bfloat16 if method == "standard" else torch.float16
     x = prepare(matrix.contiguous().reshape(-1, shape[-2], shape[-1]), dtype)
     if method == "standard" or x.shape[-2] == x.shape[-1]:
-        for _ in range(steps):
+        for step in range(steps):
             r = _matmul(x, x, transpose_b=True)
             z = _matmul(r, r, transpose_b=True, residual=r, epilogue=1)      # r is symmetric: r r = r r^T
-            x = _matmul(z, x, residual=x, epilogue=2)
+            x = _matmul(z, x, residual=x, epilogue=2, transpose_out=tall and step == steps - 1)
     else:
-        for length in (min(steps, 2), max(steps - 2, 0)):
-            if not length:
-                continue
+        segments = [length for length in (min(steps, 2), max(steps - 2, 0)) if length]
+        for index, length in enumerate(segments):
             r = _matmul(x, x, transpose_b=True)
             q = None
             for i in range(length):
@@ -60,9 +60,7 @@ def run(matrix, steps, method):
                 if i + 1 < length:
                     rz = _matmul(z, r, residual=r, epilogue=2)
                     r = _matmul(z, rz, residual=rz, epilogue=2)
-            x = _matmul(q, x)
-    if tall:
-        x = x.mT
+            x = _matmul(q, x, transpose_out=tall and index == len(segments) - 1)
     return x.reshape(shape)
 
 
