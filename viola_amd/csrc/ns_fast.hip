@@ -4,12 +4,17 @@
 // Block: 256 threads = 2 x 2 wavefronts, each owning WM x WN accumulators of 32 x 32 (192 x 192 tiles
 // for the 1152-multiples of transformer blocks, 128 x 128 otherwise), two blocks per CU so one block's
 // barrier and LDS traffic hide behind the other's MFMAs.
-//   * global -> registers (raw buffer loads, out-of-range lanes read zero: no tail branches) -> LDS,
-//     32 k per stage, two stages; the loads of chunk c+2 are in flight during the math of chunk c.
-//   * k-contiguous operands ([m, k] and [n, k]) sit in LDS as rows of 32 + 8 elements and are read with
-//     ds_read_b128; an [k, n] operand keeps its layout (rows of BN + 32 elements) and is transposed on
-//     the way out of LDS by ds_read_b64_tr_b16, which hands lane i of each 16-lane group the four k
-//     values of column i.
+//   * global -> LDS directly (buffer_load_dwordx4 ... lds: no staging registers, no ds_write; lanes
+//     past the matrix read zero, so there are no tail branches), 32 k per stage, a ring of three
+//     stages: the loads of chunk c+2 are in flight during the math of chunk c, one barrier per chunk.
+//     A direct load puts lane l's 16 bytes at base + 16 l, so the tile layout is chosen on the global
+//     side: which (row, k piece) a lane fetches.
+//   * k-contiguous operands ([m, k] and [n, k]) are rows of 4 x 16 bytes with piece c of row r stored in
+//     slot c ^ ((r >> 2) & 3): the 16 rows a ds_read_b128 group touches fall in 16 different bank
+//     groups. An [k, n] operand keeps its layout (rows of BN elements, 16-byte units XOR-swizzled by
+//     the row so four consecutive k rows start 64 bytes apart in bank space) and is transposed on the
+//     way out of LDS by ds_read_b64_tr_b16, which hands lane i of each 16-lane group the four k values
+//     of column i.
 //   * the b matrix is the MFMA "A" source, so a lane owns one output row m and runs of four
 //     consecutive n: 8-byte stores, per-row residual loads.
 //   * a Gram-type product (b == a, square output) computes only the tiles on and above the diagonal and
@@ -24,10 +29,11 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 
 constexpr int SBK = 32;             // k per LDS stage
-constexpr int SLDK = SBK + 8;       // row stride (elements) of a k-contiguous tile: 80 bytes
+constexpr int STAGES = 3;
 constexpr uint32_t NS_OUTSIDE = 0x80000000u;
 
 template <bool IS_BF16>
@@ -44,13 +50,26 @@ template <bool IS_BF16> __device__ __forceinline__ uint16_t ns_narrow(float v) {
     else { _Float16 h = (_Float16)v; uint16_t bits; __builtin_memcpy(&bits, &h, 2); return bits; }
 }
 
+// 64 lanes x 16 bytes from a raw buffer straight into LDS at lds_addr + 16 * lane. The compiler is
+// not told that this touches LDS (it would drain every outstanding load before each LDS read); the
+// kernel orders it against its LDS reads with s_waitcnt vmcnt + barrier itself.
+__device__ __forceinline__ void load_to_lds(i32x4 rsrc, uint32_t lds_addr, uint32_t voffset, uint32_t soffset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+}
+__device__ __forceinline__ i32x4 make_rsrc(const void* base) {
+    const uint64_t address = reinterpret_cast<uint64_t>(base);
+    i32x4 r = {__builtin_amdgcn_readfirstlane((int)(uint32_t)address), __builtin_amdgcn_readfirstlane((int)(uint32_t)(address >> 32)),
+               0x7fffffff, 0x00020000};
+    return r;
+}
+
 template <bool IS_BF16, bool B_KN, int EPILOGUE, int WM, int WN>
 __global__ __launch_bounds__(256, 2) void ns_gemm_fast(NsArgs p) {
     constexpr int BM = 64 * WM, BN = 64 * WN;
-    constexpr int LDN = BN + 32;                                     // row stride of a [k, n] tile
-    constexpr int A_EL = BM * SLDK, B_EL = B_KN ? SBK * LDN : BN * SLDK;
-    constexpr int NCH = BN / 8;                                      // 16-byte chunks per [k, n] row
-    __shared__ __attribute__((aligned(16))) uint16_t lds[2][A_EL + B_EL];
+    constexpr int A_EL = BM * SBK, B_EL = BN * SBK, STAGE_EL = A_EL + B_EL;
+    constexpr int NCH = BN / 8;                                      // 16-byte units per [k, n] row
+    __shared__ __attribute__((aligned(1024))) uint16_t lds[STAGES * STAGE_EL];
 
     const int64_t per_xcd = (p.tiles + 7) / 8;
     const int64_t seq = blockIdx.x / 8;
@@ -71,74 +90,70 @@ __global__ __launch_bounds__(256, 2) void ns_gemm_fast(NsArgs p) {
         tm = (int)((work / p.tiles_n) % p.tiles_m);
         bz = work / ((int64_t)p.tiles_n * p.tiles_m);
     }
+    // the tile coordinates come out of 64-bit divisions the compiler carries in vector registers; pin them
+    // to scalars so everything derived from them (buffer resources, LDS bases) is wave-uniform
+    tm = __builtin_amdgcn_readfirstlane(tm);
+    tn = __builtin_amdgcn_readfirstlane(tn);
+    bz = __builtin_amdgcn_readfirstlane((int)bz);
     const bool mirror = p.symmetric && tn != tm;
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
     const int64_t m = p.m, n = p.n, k = p.k;
 
-    const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+    const int tid = threadIdx.x, lane = tid % WAVE;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
     const int wm = wave / 2, wn = wave % 2, l32 = lane % 32, lhi = lane / 32;
 
-    const uint16_t* abase = p.a + bz * m * k;
-    const uint16_t* bbase = p.b + bz * n * k;
-    const __amdgpu_buffer_rsrc_t res_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(abase), 0, 0x7fffffff, 0x00020000);
-    const __amdgpu_buffer_rsrc_t res_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(bbase), 0, 0x7fffffff, 0x00020000);
+    const i32x4 res_a = make_rsrc(p.a + bz * m * k);
+    const i32x4 res_b = make_rsrc(p.b + bz * n * k);
 
-    // per-thread byte offsets of the 16-byte pieces it moves per chunk (k0 = 0), and their k position
+    // Load plan: instruction `it` of this wave fills LDS units (16 bytes) [it * 256 + wave * 64, +64);
+    // per thread: the global byte offset (k0 = 0) of the piece that belongs in its unit, and its k position.
     uint32_t a_off[WM], b_off[WN];
     int a_k[WM], b_k[WN];
-    int a_lds[WM], b_lds[WN];
 #pragma unroll
     for (int it = 0; it < WM; ++it) {
-        const int id = it * 256 + tid, lr = id / 4, c = id % 4;
+        const int u = it * 256 + tid, lr = u >> 2, c = (u & 3) ^ ((lr >> 2) & 3);
         const int64_t row = m0 + lr;
         a_off[it] = row < m ? (uint32_t)((row * k + c * 8) * 2) : NS_OUTSIDE;
         a_k[it] = c * 8;
-        a_lds[it] = lr * SLDK + c * 8;
     }
 #pragma unroll
     for (int it = 0; it < WN; ++it) {
-        const int id = it * 256 + tid;
+        const int u = it * 256 + tid;
         if constexpr (B_KN) {
-            const int kr = id / NCH, cn = id % NCH;
-            const int64_t col = n0 + cn * 8;
+            const int kr = u / NCH, pos = u % NCH;
+            const int unit = pos ^ (BN % 128 == 0 ? (kr & 3) * 4 : ((kr >> 1) & 1) * 4);
+            const int64_t col = n0 + unit * 8;
             b_off[it] = col < n ? (uint32_t)(((int64_t)kr * n + col) * 2) : NS_OUTSIDE;
             b_k[it] = kr;
-            b_lds[it] = A_EL + kr * LDN + cn * 8;
         } else {
-            const int lr = id / 4, c = id % 4;
+            const int lr = u >> 2, c = (u & 3) ^ ((lr >> 2) & 3);
             const int64_t row = n0 + lr;
             b_off[it] = row < n ? (uint32_t)((row * k + c * 8) * 2) : NS_OUTSIDE;
             b_k[it] = c * 8;
-            b_lds[it] = A_EL + lr * SLDK + c * 8;
         }
     }
-
-    u32x4 ra[WM], rb[WN];
-    auto fetch = [&](int64_t k0) {
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t*)lds;
+    const uint32_t wave_units = (uint32_t)wave * 64 * 16;             // byte offset of this wave's 64 units
+    auto issue = [&](int64_t k0, int stage) {
         const uint32_t a_step = (uint32_t)(k0 * 2);
         const uint32_t b_step = B_KN ? (uint32_t)(k0 * n * 2) : (uint32_t)(k0 * 2);
+        const uint32_t base = lds_base + (uint32_t)stage * STAGE_EL * 2 + wave_units;
 #pragma unroll
-        for (int it = 0; it < WM; ++it) {
-            const bool inside = k0 + a_k[it] < k;
-            ra[it] = __builtin_amdgcn_raw_buffer_load_b128(res_a, inside ? (int)(a_off[it] + a_step) : (int)NS_OUTSIDE, 0, 0);
-        }
+        for (int it = 0; it < WM; ++it)
+            load_to_lds(res_a, base + it * 4096, k0 + a_k[it] < k ? a_off[it] : NS_OUTSIDE, a_step);
 #pragma unroll
-        for (int it = 0; it < WN; ++it) {
-            const bool inside = k0 + b_k[it] < k;
-            rb[it] = __builtin_amdgcn_raw_buffer_load_b128(res_b, inside ? (int)(b_off[it] + b_step) : (int)NS_OUTSIDE, 0, 0);
-        }
-    };
-    auto stash = [&](int s) {
-#pragma unroll
-        for (int it = 0; it < WM; ++it) *reinterpret_cast<u32x4*>(&lds[s][a_lds[it]]) = ra[it];
-#pragma unroll
-        for (int it = 0; it < WN; ++it) *reinterpret_cast<u32x4*>(&lds[s][b_lds[it]]) = rb[it];
+        for (int it = 0; it < WN; ++it)
+            load_to_lds(res_b, base + A_EL * 2 + it * 4096, k0 + b_k[it] < k ? b_off[it] : NS_OUTSIDE, b_step);
     };
 
     // fragment addresses (elements) inside a stage
-    const int a_frag = (wm * 32 * WM + l32) * SLDK + lhi * 8;
-    const int b_frag = B_KN ? A_EL + (lhi * 8 + ((lane & 15) >> 2)) * LDN + wn * 32 * WN + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)
-                            : A_EL + (wn * 32 * WN + l32) * SLDK + lhi * 8;
+    const int sw = (l32 >> 2) & 3;
+    const int a_frag = (wm * 32 * WM + l32) * SBK + ((lhi ^ sw) * 8);                  // k half ks: ^ (ks * 16)
+    const int kn_row = lhi * 8 + ((lane & 15) >> 2);                                   // + ks * 16 (+ 4 for the upper half)
+    const int kn_unit = (wn * 4 * WN + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1)) ^ (BN % 128 == 0 ? (kn_row & 3) * 4 : ((kn_row >> 1) & 1) * 4);
+    const int b_frag = B_KN ? A_EL + kn_row * BN + kn_unit * 8 + 4 * (lane & 1)
+                            : A_EL + (wn * 32 * WN + l32) * SBK + ((lhi ^ sw) * 8);
 
     f32x16 acc[WN][WM];
 #pragma unroll
@@ -148,25 +163,28 @@ __global__ __launch_bounds__(256, 2) void ns_gemm_fast(NsArgs p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    auto compute = [&](int s) {
+    auto compute = [&](const uint16_t* stage) {
 #pragma unroll
         for (int ks = 0; ks < SBK / 16; ++ks) {
             uint4 opa[WM], opb[WN];
 #pragma unroll
             for (int i = 0; i < WN; ++i) {
                 if constexpr (B_KN) {
-                    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-                    const uint16_t* at = &lds[s][b_frag + ks * 16 * LDN + i * 32];
+                    // i * 32 columns = 4 units further along the row: the swizzle only touches bits the
+                    // lane's own term already fixed modulo 8 units when 4 i stays below 8, so add it before
+                    // the XOR would be wrong; the unit index is rebuilt instead
+                    const int unit = ((wn * 4 * WN + i * 4 + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1)) ^ (BN % 128 == 0 ? (kn_row & 3) * 4 : ((kn_row >> 1) & 1) * 4));
+                    const uint16_t* at = stage + A_EL + (kn_row + ks * 16) * BN + unit * 8 + 4 * (lane & 1);
                     const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)at);
-                    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at + 4 * LDN));
+                    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at + 4 * BN));
                     const uint2 l2 = __builtin_bit_cast(uint2, lo), h2 = __builtin_bit_cast(uint2, hi);
                     opb[i] = make_uint4(l2.x, l2.y, h2.x, h2.y);
                 } else {
-                    opb[i] = *reinterpret_cast<const uint4*>(&lds[s][b_frag + i * 32 * SLDK + ks * 16]);
+                    opb[i] = *reinterpret_cast<const uint4*>(stage + ((b_frag + i * 32 * SBK) ^ (ks * 16)));
                 }
             }
 #pragma unroll
-            for (int j = 0; j < WM; ++j) opa[j] = *reinterpret_cast<const uint4*>(&lds[s][a_frag + j * 32 * SLDK + ks * 16]);
+            for (int j = 0; j < WM; ++j) opa[j] = *reinterpret_cast<const uint4*>(stage + ((a_frag + j * 32 * SBK) ^ (ks * 16)));
 #pragma unroll
             for (int i = 0; i < WN; ++i)
 #pragma unroll
@@ -175,17 +193,19 @@ __global__ __launch_bounds__(256, 2) void ns_gemm_fast(NsArgs p) {
     };
 
     const int64_t chunks = (k + SBK - 1) / SBK;
-    fetch(0);
-    stash(0);
-    fetch(SBK);
-    __syncthreads();
+    issue(0, 0);
+    issue(SBK, 1);
+    int cur = 0, fill = 2;
     for (int64_t c = 0; c < chunks; ++c) {
-        const int s = (int)(c & 1);
-        stash(s ^ 1);                       // chunk c+1 (zeros past the end)
-        fetch((c + 2) * SBK);
-        compute(s);
-        __syncthreads();
+        // all loads but the newest chunk's have landed: chunk c is in LDS for this wave ...
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (WM + WN));
+        __syncthreads();                    // ... and for every wave; stage `fill` was last read in chunk c-1
+        issue((c + 2) * SBK, fill);         // past the end: zeros into a stage nobody reads
+        compute(lds + cur * STAGE_EL);
+        cur = cur == STAGES - 1 ? 0 : cur + 1;
+        fill = fill == STAGES - 1 ? 0 : fill + 1;
     }
+    __builtin_amdgcn_s_waitcnt(0x0F70);     // drain the trailing loads before the LDS allocation is released
 
     const uint16_t* residual = EPILOGUE ? p.residual + bz * m * n : nullptr;
     uint16_t* out = p.out + bz * m * n;
