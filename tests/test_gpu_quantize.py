@@ -87,6 +87,42 @@ def test_quantize_dual_equals_two_passes(in_dtype, shape):
     _same(qt, st, *og.quantize(x, E4, (1, 32), transposed=True))
 
 
+@pytest.mark.parametrize("fp8", [E4, E5])
+@pytest.mark.parametrize("limit", [None, 240.0])
+def test_quantize_rounding_ties_over_all_magnitudes(fp8, limit):
+    """The kernels replace v / s by a reciprocal and two FMAs where that is provably the same quotient.
+    Values sitting exactly on FP8 rounding ties (where a one-ulp error in the quotient flips the code),
+    groups from 1e-36 to 1e30 in magnitude (tiny scales fall back to true division) and groups with
+    NaN / Inf members must all give the oracle's codes and scales."""
+    g = _gpu()
+    torch.manual_seed(77)
+    rows, cols = 512, 256
+    top = torch.finfo(fp8).max if limit is None else limit
+    amax = torch.exp(torch.empty(rows, cols // 32, 1).uniform_(-83., 69.))               # 1e-36 .. 1e30
+    scale = amax.clamp_min(1e-30) / top
+    mant = 3 if fp8 == E4 else 2
+    k = torch.randint(2 ** mant, 2 ** (mant + 1), (rows, cols // 32, 32)).float()
+    j = torch.randint(-12 if fp8 == E4 else -19, 7 if fp8 == E4 else 14, (rows, cols // 32, 32)).float()
+    tie = (k + .5) / 2 ** mant * torch.exp2(j)
+    x = scale * tie * torch.where(torch.rand_like(tie) < .5, -1., 1.)
+    x = torch.where(x.abs() > amax, amax, x)
+    x[..., 0] = amax[..., 0]
+    x = x.reshape(rows, cols).contiguous()
+    x[5, 40] = float("nan")
+    x[6, 70] = float("inf")
+    x[7, 100:132] = 0
+    x[9, ::3] = -0.0
+    for transposed in (False, True):
+        q, sc = g.quantize(x.cuda(), fp8, (1, 32), limit=limit, transposed=transposed)
+        rq, rs = og.quantize(x, fp8, (1, 32), limit=limit, transposed=transposed)
+        _same(q, sc, rq, rs)
+    q, sc, qt, st = g.quantize_dual(x.cuda(), fp8, (1, 32), limit=limit)
+    _same(q, sc, *og.quantize(x, fp8, (1, 32), limit=limit))
+    _same(qt, st, *og.quantize(x, fp8, (1, 32), limit=limit, transposed=True))
+    q, sc = g.quantize(x.cuda(), fp8, (32, 32), limit=limit)
+    _same(q, sc, *og.quantize(x, fp8, (32, 32), limit=limit))
+
+
 def test_quantize_limit_and_out_arguments():
     g = _gpu()
     x = _input((64, 96), torch.float32, seed=3)

@@ -118,6 +118,49 @@ template <typename T> struct fp8_traits;
 template <> struct fp8_traits<e4m3_t> { static constexpr float max = 448.0f; };
 template <> struct fp8_traits<e5m2_t> { static constexpr float max = 57344.0f; };
 
+// ------------------------------------------------------------------ many quotients by one divisor
+// v / s for values that share the divisor s (a quantization group), bit for bit the IEEE quotient at
+// three operations per value instead of a full division: with r = RN(1/s), t0 = RN(v r) and the exact
+// residual e = v - s t0 (one FMA), RN(t0 + e r) is the correctly rounded v / s (Markstein). The argument
+// needs the residual to be exact, which fails when it underflows (tiny s), when s has an all-ones
+// significand (then RN(1/s) is not close enough), and for non-finite operands; `fast` is false in those
+// cases and the caller divides. `poison` is any value that is NaN iff the group holds a NaN or an Inf
+// (see poison_of).
+struct SharedDivisor {
+    float s, r;
+    bool fast;
+    __device__ __forceinline__ SharedDivisor(float divisor, float poison) : s(divisor) {
+        const uint32_t bits = __float_as_uint(divisor);
+        r = 1.0f / divisor;
+        fast = divisor >= 0x1p-80f && bits < 0x7f800000u && (bits & 0x7fffffu) != 0x7fffffu && poison == poison;
+    }
+    __device__ __forceinline__ float quotient(float v) const {
+        const float t0 = v * r;
+        const float e = -fmaf(t0, s, -v);        // this order of signs keeps -0 / s = -0
+        return fmaf(e, r, t0);
+    }
+};
+__device__ __forceinline__ float poison_of(float acc, float v) { return fmaf(v, 0.0f, acc); }
+
+// Four values -> four FP8 codes in one word with the gfx950 converters. They agree with f32_to_e4m3 /
+// f32_to_e5m2 (torch's casts) on every input that is not NaN; NaN comes out as 0xff / 0xfe instead of
+// 0x7f | sign, so callers use them only on groups without NaN.
+template <typename T> __device__ __forceinline__ uint32_t hw_encode4(float a, float b, float c, float d);
+template <> __device__ __forceinline__ uint32_t hw_encode4<e4m3_t>(float a, float b, float c, float d) {
+    int w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
+}
+template <> __device__ __forceinline__ uint32_t hw_encode4<e5m2_t>(float a, float b, float c, float d) {
+    int w = __builtin_amdgcn_cvt_pk_bf8_f32(a, b, 0, false);
+    return (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(c, d, w, true);
+}
+// clamp(v / s, +-limit) -> code, four at a time, for a group whose divisor took the fast path
+template <typename T>
+__device__ __forceinline__ uint32_t fast_encode4(const SharedDivisor& d, float limit, float a, float b, float c, float e) {
+    return hw_encode4<T>(__builtin_amdgcn_fmed3f(d.quotient(a), -limit, limit), __builtin_amdgcn_fmed3f(d.quotient(b), -limit, limit),
+                         __builtin_amdgcn_fmed3f(d.quotient(c), -limit, limit), __builtin_amdgcn_fmed3f(d.quotient(e), -limit, limit));
+}
+
 // ------------------------------------------------------------------ wavefront reductions
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll

@@ -52,7 +52,8 @@ template <> struct Chunk8<float> {
 };
 
 template <typename TOut>
-__device__ __forceinline__ uint2 encode8(const float (&v)[8], float s, float limit) {
+__device__ __forceinline__ uint2 encode8(const float (&v)[8], float s, float limit, const SharedDivisor& d) {
+    if (d.fast) return make_uint2(fast_encode4<TOut>(d, limit, v[0], v[1], v[2], v[3]), fast_encode4<TOut>(d, limit, v[4], v[5], v[6], v[7]));
     uint32_t lo = 0, hi = 0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -76,13 +77,19 @@ __global__ __launch_bounds__(256) void quantize_rowwise(const TIn* __restrict__ 
     const bool valid = row < rows && c0 < cols;
     float v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     if (valid) Chunk8<TIn>::load(x + row * cols + c0, v);
-    float amax = 0.0f;
+    float amax = 0.0f, poison = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+    for (int i = 0; i < 8; ++i) {
+        amax = fmaxf(amax, fabsf(v[i]));
+        poison = poison_of(poison, v[i]);
+    }
     amax = group_max<LANES>(amax);
+#pragma unroll
+    for (int offset = LANES / 2; offset > 0; offset >>= 1) poison += __shfl_xor(poison, offset, WAVE);
     const float s = group_scale(amax, limit);
+    const SharedDivisor divisor(s, poison);
     if (valid) {
-        *reinterpret_cast<uint2*>(q + row * cols + c0) = encode8<TOut>(v, s, limit);
+        *reinterpret_cast<uint2*>(q + row * cols + c0) = encode8<TOut>(v, s, limit, divisor);
         if ((threadIdx.x & (LANES - 1)) == 0) scale[row * nc + c0 / GC] = s;
     }
 }
@@ -118,14 +125,20 @@ __device__ __forceinline__ void load_tile(const TIn* __restrict__ x, float* tile
 
 // Encode 32 values held by one lane and store them at dst (a run of `count` <= 32 valid bytes).
 template <typename TOut>
-__device__ __forceinline__ void store_group32(const float (&v)[32], float s, float limit, uint8_t* dst, int count,
+__device__ __forceinline__ void store_group32(const float (&v)[32], float s, float poison, float limit, uint8_t* dst, int count,
                                               bool aligned16) {
     uint32_t w[8];
+    const SharedDivisor divisor(s, poison);
+    if (divisor.fast) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        w[i] = 0;
+        for (int i = 0; i < 8; ++i) w[i] = fast_encode4<TOut>(divisor, limit, v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
+    } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) w[i] |= (uint32_t)encode_clamped<TOut>(v[4 * i + j], s, limit) << (8 * j);
+        for (int i = 0; i < 8; ++i) {
+            w[i] = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) w[i] |= (uint32_t)encode_clamped<TOut>(v[4 * i + j], s, limit) << (8 * j);
+        }
     }
     if (count == 32 && aligned16) {
         reinterpret_cast<uint4*>(dst)[0] = make_uint4(w[0], w[1], w[2], w[3]);
@@ -150,18 +163,19 @@ __global__ __launch_bounds__(256) void quantize_tile(const TIn* __restrict__ x, 
         const int64_t row = r0 + r, col = c0 + g * 32;
         if (row < rows && col < cols) {
             float v[32];
-            float amax = 0.0f;
+            float amax = 0.0f, poison = 0.0f;
 #pragma unroll
             for (int i = 0; i < 32; ++i) {
                 v[i] = tile[r * TILE_LD + g * 32 + i];
                 amax = fmaxf(amax, fabsf(v[i]));
+                poison = poison_of(poison, v[i]);
             }
             const float s = group_scale(amax, limit);
             const int64_t nc = (cols + 31) / 32;
             scale[row * nc + col / 32] = s;
             const int count = (int)(cols - col < 32 ? cols - col : 32);
             uint8_t* dst = q + row * cols + col;
-            store_group32<TOut>(v, s, limit, dst, count, (reinterpret_cast<uintptr_t>(dst) & 15) == 0);
+            store_group32<TOut>(v, s, poison, limit, dst, count, (reinterpret_cast<uintptr_t>(dst) & 15) == 0);
         }
     }
     if constexpr (TRANSPOSED) {
@@ -169,18 +183,19 @@ __global__ __launch_bounds__(256) void quantize_tile(const TIn* __restrict__ x, 
         const int64_t col = c0 + c, row = r0 + g * 32;
         if (col < cols && row < rows) {
             float v[32];
-            float amax = 0.0f;
+            float amax = 0.0f, poison = 0.0f;
 #pragma unroll
             for (int i = 0; i < 32; ++i) {
                 v[i] = tile[(g * 32 + i) * TILE_LD + c];
                 amax = fmaxf(amax, fabsf(v[i]));
+                poison = poison_of(poison, v[i]);
             }
             const float s = group_scale(amax, limit);
             const int64_t nr = (rows + 31) / 32;
             scale_t[col * nr + row / 32] = s;
             const int count = (int)(rows - row < 32 ? rows - row : 32);
             uint8_t* dst = qt + col * rows + row;
-            store_group32<TOut>(v, s, limit, dst, count, (reinterpret_cast<uintptr_t>(dst) & 15) == 0);
+            store_group32<TOut>(v, s, poison, limit, dst, count, (reinterpret_cast<uintptr_t>(dst) & 15) == 0);
         }
     }
 }
@@ -271,16 +286,17 @@ __global__ __launch_bounds__(64) void quantize_transposed_segmented(const TIn* _
     const int64_t first = offsets[g] + (token - poffsets[g]);
     const int64_t end = offsets[g + 1];
     float v[32];
-    float amax = 0.0f;
+    float amax = 0.0f, poison = 0.0f;
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
         v[i] = first + i < end ? to_f32(x[(first + i) * cols + col]) : 0.0f;
         amax = fmaxf(amax, fabsf(v[i]));
+        poison = poison_of(poison, v[i]);
     }
     const float s = group_scale(amax, limit);
     scale_t[col * (t_total / 32) + slot] = s;
     uint8_t* dst = qt + col * t_total + token;
-    store_group32<TOut>(v, s, limit, dst, 32, (reinterpret_cast<uintptr_t>(dst) & 15) == 0);
+    store_group32<TOut>(v, s, poison, limit, dst, 32, (reinterpret_cast<uintptr_t>(dst) & 15) == 0);
 }
 
 // ------------------------------------------------------------------ host dispatch
