@@ -34,10 +34,14 @@ struct e5m2_t { uint8_t bits; };
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits) { return __uint_as_float(bits << 16); }
 
 // Round-to-nearest-even, NaN -> quiet NaN with the sign dropped (the rule of PyTorch's cast).
-__device__ __forceinline__ uint16_t f32_to_bf16_bits(float x) {
-    uint32_t u = __float_as_uint(x);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;
-    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+// v_cvt_pk_bf16_f32: round to nearest even, identical to the usual add-0x7fff arithmetic on every input
+// that is not NaN (checked over all 2^32 patterns); a NaN keeps its sign and top payload bits.
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float x) { return __builtin_bit_cast(uint16_t, (__bf16)x); }
+__device__ __forceinline__ uint32_t f32_to_bf16x2_bits(float lo, float hi) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t pair = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2_t));
 }
 
 // ------------------------------------------------------------------ FP8 (OCP) codecs

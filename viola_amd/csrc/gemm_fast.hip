@@ -60,8 +60,7 @@ template <> struct Quad<float> {
 };
 template <> struct Quad<bf16_t> {
     static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[4]) {
-        *reinterpret_cast<uint2*>(p) = make_uint2((uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16),
-                                                  (uint32_t)f32_to_bf16_bits(v[2]) | ((uint32_t)f32_to_bf16_bits(v[3]) << 16));
+        *reinterpret_cast<uint2*>(p) = make_uint2(f32_to_bf16x2_bits(v[0], v[1]), f32_to_bf16x2_bits(v[2], v[3]));
     }
     static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[4]) {
         const uint2 t = *reinterpret_cast<const uint2*>(p);
