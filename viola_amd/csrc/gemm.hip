@@ -317,7 +317,8 @@ static int launch_out(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtyp
     const int64_t b_rows = MODE == MODE_GATED_FWD ? 2 * p.n : p.n;
     // the fast kernel addresses operands and scales with 31-bit byte offsets
     const bool small = b_rows * p.ldb < (1ll << 31) && (int64_t)BM * p.lda < (1ll << 31) &&
-                       (p.m + p.ar - 1) / p.ar * p.ldsa * 4 < (1ll << 31) && (b_rows + p.br - 1) / p.br * p.ldsb * 4 < (1ll << 31);
+                       (p.m + p.ar - 1) / p.ar * p.ldsa * 4 < (1ll << 31) && (b_rows + p.br - 1) / p.br * p.ldsb * 4 < (1ll << 31) &&
+                       p.ak_shift == 5 && p.bk_shift == 5;         // and stages the scales of 8 consecutive 32-wide K groups at once
     if (vec && small)
         return launch_group_gemm_fast(p, MODE, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
     switch (out_dtype) {

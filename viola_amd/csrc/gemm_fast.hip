@@ -1,26 +1,54 @@
 // Fast path of the grouped-scale FP8 GEMM for gfx950 (see gemm.hip for the contract and the operand
 // orientation). Requires 16-byte aligned operand rows and k ranges that are multiples of 16.
 //
-// Block: 512 threads = 8 wavefronts (two per SIMD), tile 128 (m) x 128 (b rows) x 128 (k), two LDS
-// stages, one block per CU. A wavefront owns two 32 x 32 sub-tiles (64 m x 32 n; gated forward: 32 m x
-// 32 gate + 32 up columns).
-//   * global -> registers -> LDS, next chunk's loads issued before the math of the current chunk;
-//     per thread two 16-byte loads per operand, eight lanes cover one 128-byte row segment.
-//   * LDS rows are 128 + 16 bytes. Inside each 32-byte K group the two middle 8-byte pieces are swapped,
-//     so the 8 codes a lane needs for both k halves of a group (k = 16*ks + 8*(lane/32)) are adjacent
-//     and one ds_read_b128 fetches them; the 144-byte stride spreads 8 consecutive rows over all banks.
-//   * math: per K group 2 x v_mfma_f32_32x32x16 per sub-tile into a fresh accumulator set, then
-//     total += acc * (sa * sb), one FMA per output element. Two accumulator sets alternate: the FMAs
-//     that fold group g are issued between the MFMAs of group g+1, so the matrix pipe and the VALU
-//     run together inside one wavefront as well as across the two wavefronts of a SIMD. The operands
-//     of group g+1 are read from LDS before the MFMAs of group g.
+// Block: 256 threads = 2 x 2 wavefronts, tile 128 (m) x 128 (b rows), 64 k per LDS stage; a wavefront owns
+// 2 x 2 sub-tiles of 32 x 32. Two blocks share a CU, so one block's prologue, barrier and output stores
+// run under the other block's math.
+//   * global -> LDS directly (buffer_load ... lds, no staging registers, lanes past the k range read
+//     zero), a ring of three stages: the loads of chunk c+2 fly during the math of chunk c, one barrier
+//     per chunk. Operand rows are 4 x 16 bytes, piece u = 2 * (K group) + half stored in slot
+//     u ^ ((row >> 2) & 3), which spreads the 16 rows of a ds_read_b128 group over all banks. A lane
+//     takes 16 consecutive bytes of a 32-byte K group (half = lane / 32): the first 8 feed the first
+//     MFMA of the group, the last 8 the second -- a and b use the same split, so every product meets its
+//     partner. The scales come in blocks of 8 K groups (32 bytes per row, so a scale row's cache
+//     line is touched once per 256 k) and are rearranged in LDS to [group][row].
+//   * math per (K group, sub-tile): 2 x v_mfma_f32_32x32x16 into one of two 16-register accumulators,
+//     then total += acc * (sa * sb), one FMA per output element, issued between the MFMAs of the next
+//     sub-tile so the matrix pipe and the VALU run together inside a wavefront as well as across the
+//     two wavefronts of a SIMD. The last fold of a chunk rides into the next chunk (uniform b scales;
+//     with row-wise b scales, which live in registers per chunk, that fold stays in its own chunk).
 //   * epilogue stores runs of four consecutive n as one 8- or 16-byte store.
 #include "gemm_args.hpp"
 
 namespace viola {
 
-constexpr int FBK = 128, FKG = FBK / 32, FLD = FBK + 16;          // LDS row stride: 16 bytes of padding per row
-constexpr int FTHREADS = 512;
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int FBK = 64, FKG = FBK / 32;                           // k bytes and K groups per LDS stage
+constexpr int FTHREADS = 256, FSTAGES = 3;
+constexpr int F_TILE = BM * FBK;                                  // bytes of one operand tile
+constexpr int F_STAGE = 2 * F_TILE;
+// Scales travel in blocks of 8 K groups (4 chunks): 32 bytes per row and operand, fetched as two 16-byte pieces
+// ("raw", piece = 4 groups of one row) and then rearranged in LDS to [group][row] floats, double-buffered.
+constexpr int F_SGROUPS = 8, F_SCHUNKS = F_SGROUPS / FKG;
+constexpr int F_SBLOCK = F_SGROUPS * BM * 4;                      // bytes of one operand's scale block
+constexpr int F_RAW = FSTAGES * F_STAGE;                          // raw a block, raw b block
+constexpr int F_SCALE = F_RAW + 2 * F_SBLOCK;                     // [buffer][operand][group][row]
+constexpr int F_LDS = F_SCALE + 4 * F_SBLOCK;
+
+// 64 lanes x 16 (or 4) bytes from a raw buffer straight into LDS at lds_addr + 16 (4) * lane. The compiler
+// is not told that these touch LDS (it would drain every outstanding load before each LDS read); the kernel
+// orders them against its LDS reads with s_waitcnt vmcnt + barrier itself.
+__device__ __forceinline__ void load16_to_lds(i32x4 rsrc, uint32_t lds_addr, uint32_t voffset, uint32_t soffset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+}
+__device__ __forceinline__ i32x4 raw_resource(const void* base, int64_t bytes = 0x7fffffff) {
+    const uint64_t address = reinterpret_cast<uint64_t>(base);
+    i32x4 r = {__builtin_amdgcn_readfirstlane((int)(uint32_t)address), __builtin_amdgcn_readfirstlane((int)(uint32_t)(address >> 32)),
+               __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000};
+    return r;
+}
 
 template <bool A_BF8, bool B_BF8>
 __device__ __forceinline__ f32x16 mfma32(long x, long y, f32x16 c) {
@@ -80,24 +108,24 @@ template <> struct Quad<f16_t> {
     }
 };
 
-template <int S> struct Stage { static constexpr int value = S; };
-
 template <typename TO> __device__ __forceinline__ float rounded(float v) { return to_f32(from_f32<TO>(v)); }
 
-template <int MODE, bool A_BF8, bool B_BF8, bool B_ROWSCALE, typename TO>
+// TN: 32-column sub-tiles per wave; TN = 1 halves the tile to 128 x 64 for problems with too few 128 x 128 tiles to
+// give every CU two blocks (plain mode only).
+template <int MODE, bool A_BF8, bool B_BF8, bool B_ROWSCALE, typename TO, int TN>
 __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int bias_dtype) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds_a[2][BM * FLD];
-    __shared__ __attribute__((aligned(16))) uint8_t lds_b[2][BN * FLD];
-    __shared__ __attribute__((aligned(16))) float lds_sa[2][FKG][BM];
-    __shared__ __attribute__((aligned(16))) float lds_sb[2][FKG][BN];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[F_LDS];
 
-    // wave grid and sub-tiles per wave: plain / gated backward 2 (m) x 4 (n) waves of 2 x 1 sub-tiles;
-    // gated forward 4 (m) x 2 (n) waves of 1 x 2 sub-tiles (gate and up columns of the same n in one lane)
+    // wave grid 2 (m) x 2 (n), 2 x 2 sub-tiles each. Plain / gated backward: sub-tile i of wave wn covers b rows
+    // 64 wn + 32 i. Gated forward: the tile's b rows are 64 gate rows then the 64 up rows of the same n, and
+    // i = 0 / 1 is the gate / up sub-tile of columns 32 wn .. 32 wn + 31, so one lane holds g and u of the same n.
     constexpr bool GATED = MODE == MODE_GATED_FWD;
-    constexpr int TM = GATED ? 1 : 2, TN = GATED ? 2 : 1, WN = GATED ? 2 : 4;
-    constexpr int PANEL = GATED ? BN / 2 : BN;
-    const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
-    const int wm = wave / WN, wn = wave % WN;
+    constexpr int TM = 2;
+    constexpr int PANEL = GATED ? BN / 2 : 64 * TN;
+    static_assert(!GATED || TN == 2, "gated forward pairs a gate and an up sub-tile");
+    const int tid = threadIdx.x, lane = tid % WAVE;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+    const int wm = wave / 2, wn = wave % 2;
     const int l32 = lane % 32, lhi = lane / 32;
 
     // ---- which problem / tile (uniform per block)
@@ -149,85 +177,77 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
         else bn = n_begin + r;
         return bn < b_rows_total ? bn : b_rows_total - 1;
     };
+    auto a_global_row = [&](int r) -> int64_t {                               // rows past the end repeat the last row
+        const int64_t am = m_begin + r;
+        return am < m_end ? am : m_end - 1;
+    };
 
-    // ---- per-thread constants: global offsets of its two 16-byte chunks per operand, LDS slots
-    const int lrow = tid / 8, chunk = tid % 8;                               // rows lrow + 64*it, 16-byte chunk of the 128-byte row
+    // ---- load plan. Instruction `it` of this wave fills 16-byte LDS units [it * 256 + wave * 64, +64) of an operand
+    // tile: unit U = 4 * row + slot holds piece (slot ^ ((row >> 2) & 3)) of the row's 64 k bytes.
+    const i32x4 res_a = raw_resource(p.a + m_begin * p.lda + k_begin);
+    const i32x4 res_b = raw_resource(bptr + k_begin);
+    // scale buffers carry their true size: a 16-byte piece may reach past the last row, and must then read zero
+    const i32x4 res_sa = raw_resource(p.sa, (p.m + p.ar - 1) / p.ar * p.ldsa * 4);
+    const i32x4 res_sb = raw_resource(sbptr, (b_rows_total + p.br - 1) / p.br * p.ldsb * 4);
+    constexpr uint32_t OUTSIDE = 0x80000000u;
     uint32_t goff_a[2], goff_b[2];
-    const uint8_t* abase = p.a + m_begin * p.lda + k_begin;
+    int piece_k[2];
 #pragma unroll
     for (int it = 0; it < 2; ++it) {
-        const int r = lrow + 64 * it;
-        int64_t am = m_begin + r;
-        am = am < m_end ? am : m_end - 1;
-        goff_a[it] = (uint32_t)((am - m_begin) * p.lda + chunk * 16);
-        goff_b[it] = (uint32_t)(b_global_row(r) * p.ldb + chunk * 16);       // relative to bptr + k offset (row span < 4 GiB)
+        const int unit = it * 256 + tid, r = unit >> 2, piece = (unit & 3) ^ ((r >> 2) & 3);
+        goff_a[it] = (uint32_t)((a_global_row(r) - m_begin) * p.lda + piece * 16);
+        goff_b[it] = (uint32_t)(b_global_row(r) * p.ldb + piece * 16);        // relative to bptr + k_begin (row span < 2 GiB)
+        piece_k[it] = piece * 16;
     }
-    const uint8_t* bbase = bptr + k_begin;
-    // global bytes [16c, 16c+16) of a row are the pieces (ks = c % 2, half 0) and (ks, half 1) of K group c / 2; in LDS
-    // a group is laid out [ks0 h0][ks1 h0][ks0 h1][ks1 h1]
-    const int wslot = lrow * FLD + (chunk / 2) * 32 + (chunk % 2) * 8;       // second piece 16 bytes further; + 64*it*FLD
-    // scale staging: thread owns tile row srow and K group sgroup of each chunk (512 = 4 groups x 128 rows)
-    const int srow = tid % BM, sgroup = tid / BM;
-    uint32_t sa_off, sb_off;                                                 // byte offsets of this thread's scale rows
-    {
-        int64_t am = m_begin + srow;
-        am = am < m_end ? am : m_end - 1;
-        sa_off = (uint32_t)(am / p.ar * p.ldsa * 4);
-        sb_off = (uint32_t)(b_global_row(srow) / p.br * p.ldsb * 4);
-    }
-    // MFMA operand reads: 16 bytes = both k halves of one K group for row l32 (+32 per sub-tile), quarter pair lhi
-    auto a_sub = [&](int j) -> int { return (wm * TM + j) * 32; };
-    auto b_sub = [&](int i) -> int { return GATED ? i * PANEL + wn * 32 : wn * 32; };
-    const int rd_a = (a_sub(0) + l32) * FLD + lhi * 16;
-    const int rd_b = (b_sub(0) + l32) * FLD + lhi * 16;
-
-    // Two register staging sets: the loads of chunk c+2 are issued while chunk c+1 is still in flight, so every
-    // chunk has a whole iteration of math to arrive before it is written to LDS.
-    // Raw buffer loads: 32-bit per-lane offset + uniform chunk offset, no per-load address arithmetic.
-    // (a chunk offset k0 enters as the scalar offset)
-    const __amdgpu_buffer_rsrc_t res_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(abase), 0, 0x7fffffff, 0x00020000);
-    const __amdgpu_buffer_rsrc_t res_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(bbase), 0, 0x7fffffff, 0x00020000);
-    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-    auto load16 = [&](const __amdgpu_buffer_rsrc_t& res, uint32_t voffset, int32_t soffset) -> uint4 {
-        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(res, (int)voffset, soffset, 0);
-        return make_uint4(v[0], v[1], v[2], v[3]);
-    };
-    uint4 ra[2][2], rb[2][2];
-    float rsa[2], rsb[2];
-    // Branch-free: a lane whose 16 bytes lie past the end of the k range (or a chunk past the last one) loads from
-    // an offset outside the buffer, which returns zeros without touching memory. No control flow around the loads,
-    // so the compiler's wait counters stay exact and the newest loads remain in flight across the LDS writes.
-    const __amdgpu_buffer_rsrc_t res_sa = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.sa), 0, 0x7fffffff, 0x00020000);
-    const __amdgpu_buffer_rsrc_t res_sb = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(sbptr), 0, 0x7fffffff, 0x00020000);
-    constexpr uint32_t OUTSIDE = 0x80000000u;
+    constexpr int B_LOADS = TN;                                              // 64 b rows per load instruction
+    // scales: per block of 8 K groups the thread fetches groups 4 shalf .. 4 shalf + 3 of tile row srow
+    const int srow = tid % BM, shalf = tid / BM;
+    const uint32_t sa_off = (uint32_t)(a_global_row(srow) / p.ar * p.ldsa * 4 + ((k_begin >> 5) + shalf * 4) * 4);
+    const uint32_t sb_off = (uint32_t)(b_global_row(srow) / p.br * p.ldsb * 4 + ((k_begin >> 5) + shalf * 4) * 4);
     const int64_t k_len = k_end - k_begin;
+    const int groups_total = (int)((k_len + 31) / 32);
     const int64_t chunks = (k_len + FBK - 1) / FBK;
-    auto fetch = [&](int64_t c, int set) {                                    // set is a compile-time constant at every call
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
+    auto issue = [&](int64_t c, int stage) {
         const int64_t k0 = c * FBK;                                          // relative to k_begin
-        const bool inside = k0 + chunk * 16 < k_len;
+        const uint32_t base = lds_base + (uint32_t)stage * F_STAGE + (uint32_t)wave * 1024;
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
-            ra[set][it] = load16(res_a, inside ? goff_a[it] : OUTSIDE, (int32_t)k0);
-            rb[set][it] = load16(res_b, inside ? goff_b[it] : OUTSIDE, (int32_t)k0);
+            const bool inside = k0 + piece_k[it] < k_len;
+            load16_to_lds(res_a, base + it * 4096, inside ? goff_a[it] : OUTSIDE, (uint32_t)k0);
+            if (it < B_LOADS) load16_to_lds(res_b, base + F_TILE + it * 4096, inside ? goff_b[it] : OUTSIDE, (uint32_t)k0);
         }
-        const int64_t kk = k_begin + k0 + sgroup * 32;
-        const bool group_inside = k0 + sgroup * 32 < k_len;
-        rsa[set] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(res_sa, group_inside ? (int)(sa_off + (uint32_t)(kk >> p.ak_shift) * 4) : (int)OUTSIDE, 0, 0));
-        rsb[set] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(res_sb, group_inside ? (int)(sb_off + (uint32_t)(kk >> p.bk_shift) * 4) : (int)OUTSIDE, 0, 0));
     };
-    auto stash = [&](int s, int set) {
+    // scale block `block` (K groups 8 block .. 8 block + 7 of the k range) -> raw area, one 16-byte piece per thread
+    // and operand; a piece wholly past the k range is not fetched
+    auto issue_scales = [&](int64_t block) {
+        const bool inside = block * F_SGROUPS + shalf * 4 < groups_total;
+        const uint32_t at = lds_base + F_RAW + (uint32_t)wave * 1024;
+        load16_to_lds(res_sa, at, inside ? sa_off : OUTSIDE, (uint32_t)(block * F_SGROUPS * 4));
+        load16_to_lds(res_sb, at + F_SBLOCK, inside ? sb_off : OUTSIDE, (uint32_t)(block * F_SGROUPS * 4));
+    };
+    // raw area -> [group][row] floats of scale buffer `block & 1`; groups past the k range become zero (their
+    // products are zero too, and a neighbouring row's value must not meet them)
+    auto arrange_scales = [&](int64_t block) {
+        const float4 va = *reinterpret_cast<const float4*>(lds + F_RAW + tid * 16);
+        const float4 vb = *reinterpret_cast<const float4*>(lds + F_RAW + F_SBLOCK + tid * 16);
+        float* ta = reinterpret_cast<float*>(lds + F_SCALE + (block & 1) * 2 * F_SBLOCK);
+        float* tb = ta + F_SBLOCK / 4;
+        const int left = groups_total - (int)(block * F_SGROUPS + shalf * 4);
+        const float a4[4] = {va.x, va.y, va.z, va.w}, b4[4] = {vb.x, vb.y, vb.z, vb.w};
 #pragma unroll
-        for (int it = 0; it < 2; ++it) {
-            uint8_t* da = &lds_a[s][wslot + it * 64 * FLD];
-            *reinterpret_cast<uint2*>(da) = make_uint2(ra[set][it].x, ra[set][it].y);
-            *reinterpret_cast<uint2*>(da + 16) = make_uint2(ra[set][it].z, ra[set][it].w);
-            uint8_t* db = &lds_b[s][wslot + it * 64 * FLD];
-            *reinterpret_cast<uint2*>(db) = make_uint2(rb[set][it].x, rb[set][it].y);
-            *reinterpret_cast<uint2*>(db + 16) = make_uint2(rb[set][it].z, rb[set][it].w);
+        for (int q = 0; q < 4; ++q) {
+            ta[(shalf * 4 + q) * BM + srow] = q < left ? a4[q] : 0.0f;
+            tb[(shalf * 4 + q) * BM + srow] = q < left ? b4[q] : 0.0f;
         }
-        lds_sa[s][sgroup][srow] = rsa[set];
-        lds_sb[s][sgroup][srow] = rsb[set];
     };
+
+    // ---- MFMA operand reads: 16 bytes = this lane's half (lhi) of K group kg for row l32 of a sub-tile
+    auto a_sub = [&](int j) -> int { return (wm * TM + j) * 32; };
+    auto b_sub = [&](int i) -> int { return GATED ? i * PANEL + wn * 32 : (wn * TN + i) * 32; };
+    const int sw = (l32 >> 2) & 3;
+    const int rd_a = (a_sub(0) + l32) * FBK + ((lhi ^ sw) * 16);             // K group 1: ^ 32
+    const int rd_b = (b_sub(0) + l32) * FBK + ((lhi ^ sw) * 16);
 
     f32x16 total[TN][TM];                                                    // [b sub-tile i][a sub-tile j]
 #pragma unroll
@@ -237,122 +257,108 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
 #pragma unroll
             for (int r = 0; r < 16; ++r) total[i][j][r] = 0.0f;
 
-    fetch(0, 0);
-    stash(0, 0);
-    fetch(1, 0);                                                             // chunk 1 in flight in set 0
-    __syncthreads();
-
-    // Software pipeline state, carried across chunks: operands of the group about to be multiplied, the accumulators
-    // of the group multiplied last (not yet folded) and its scale products.
-    struct Ops { uint4 a[TM], b[TN]; };                                      // x,y: ks 0, z,w: ks 1
-    Ops ops[2];                                                              // [parity of the K group]
-    f32x16 acc[2][TN][TM];
-    float sc[2][TN][TM];                                                     // uniform b scales: sa * sb per sub-tile
-    float sa_p[2][TM];                                                       // row-scaled b: sa only, sb read per fold
-    auto read_ops = [&](int s, int kg, Ops& o) {
-#pragma unroll
-        for (int j = 0; j < TM; ++j) o.a[j] = *reinterpret_cast<const uint4*>(&lds_a[s][rd_a + kg * 32 + j * 32 * FLD]);
-#pragma unroll
-        for (int i = 0; i < TN; ++i) o.b[i] = *reinterpret_cast<const uint4*>(&lds_b[s][rd_b + kg * 32 + (b_sub(i) - b_sub(0)) * FLD]);
-    };
-    auto as_long = [](uint32_t lo, uint32_t hi) -> long { return (long)(((uint64_t)hi << 32) | lo); };
-    // Fold accumulator set `set` (group kg of stage s) into the totals; `part` of `parts` slices so that it can be
-    // spread between MFMAs.
-    auto fold = [&](int set, int s, int kg, int part, int parts) {
-        const int per = TN * TM * 16 / parts;
-#pragma unroll
-        for (int e = part * per; e < (part + 1) * per; ++e) {
-            const int i = e / (TM * 16), j = e / 16 % TM, r = e % 16;
-            if constexpr (!B_ROWSCALE) {
-                total[i][j][r] = fmaf(acc[set][i][j][r], sc[set][i][j], total[i][j][r]);
-            } else {
-                const float sbv = lds_sb[s][kg][b_sub(i) + (r / 4) * 8 + lhi * 4 + r % 4];
-                total[i][j][r] = fmaf(acc[set][i][j][r], sa_p[set][j] * sbv, total[i][j][r]);
-            }
-        }
-    };
-    // One chunk of math on LDS stage S (compile time). Group g: read ops(g+1); MFMAs(g) into set g&1 with the fold of
-    // group g-1 (set (g-1)&1) spread between them.
-    // The last group of a chunk is folded during the first MFMAs of the next chunk (the very first fold adds zeros).
-    // With row-wise b scales the fold reads them from the LDS stage that other wavefronts may already be refilling,
-    // so there each chunk folds its own last group.
+    // Two 16-register accumulators alternate between consecutive (K group, sub-tile) units; `pending` is the unit whose
+    // MFMAs were issued last and whose fold is still to come (across chunk boundaries when CARRY).
     constexpr bool CARRY = !B_ROWSCALE;
+    f32x16 acc[2];
+    float pending_scale = 0.0f;                                              // sa * sb of the pending unit (uniform b scales)
 #pragma unroll
-    for (int i = 0; i < TN; ++i)
-#pragma unroll
-        for (int j = 0; j < TM; ++j) {
-            sc[1][i][j] = 0.0f;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[1][i][j][r] = 0.0f;
-        }
-    auto compute = [&](auto stage_tag) {
-        constexpr int S = decltype(stage_tag)::value;
+    for (int r = 0; r < 16; ++r) acc[0][r] = acc[1][r] = 0.0f;
+    auto as_long = [](uint32_t lo, uint32_t hi) -> long { return (long)(((uint64_t)hi << 32) | lo); };
+
+    auto compute = [&](int stage, int64_t c) {
+        const uint8_t* tile_a = lds + stage * F_STAGE;
+        const uint8_t* tile_b = tile_a + F_TILE;
+        const float* scale_a = reinterpret_cast<const float*>(lds + F_SCALE + ((c / F_SCHUNKS) & 1) * 2 * F_SBLOCK) + (c % F_SCHUNKS) * FKG * BM;
+        const float* scale_b = scale_a + F_SBLOCK / 4;
+        uint4 opa[FKG][TM], opb[FKG][TN];
+        float sa_l[FKG][TM], sb_u[FKG][TN];
+        float4 sb_q[FKG][TN][4];                                             // row-wise b scales of the lane's 16 columns
 #pragma unroll
         for (int kg = 0; kg < FKG; ++kg) {
-            const int set = kg & 1;
-            if (kg + 1 < FKG) read_ops(S, kg + 1, ops[(kg + 1) & 1]);
-            const Ops& cur = ops[kg & 1];
-            float sc_new[TN][TM];
 #pragma unroll
-            for (int j = 0; j < TM; ++j) {
-                const float sa_l = lds_sa[S][kg][a_sub(j) + l32];
-                if constexpr (B_ROWSCALE) sa_p[set][j] = sa_l;
-                else {
+            for (int j = 0; j < TM; ++j) opa[kg][j] = *reinterpret_cast<const uint4*>(tile_a + ((rd_a + j * 32 * FBK) ^ (kg * 32)));
 #pragma unroll
-                    for (int i = 0; i < TN; ++i) sc_new[i][j] = sa_l * lds_sb[S][kg][b_sub(i)];
-                }
-            }
-            const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-            int step = 0;
+            for (int i = 0; i < TN; ++i) opb[kg][i] = *reinterpret_cast<const uint4*>(tile_b + ((rd_b + (b_sub(i) - b_sub(0)) * FBK) ^ (kg * 32)));
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-                for (int i = 0; i < TN; ++i)
-#pragma unroll
-                    for (int j = 0; j < TM; ++j) {
-                        const long x = ks == 0 ? as_long(cur.b[i].x, cur.b[i].y) : as_long(cur.b[i].z, cur.b[i].w);
-                        const long y = ks == 0 ? as_long(cur.a[j].x, cur.a[j].y) : as_long(cur.a[j].z, cur.a[j].w);
-                        acc[set][i][j] = mfma32<A_BF8, B_BF8>(x, y, ks == 0 ? zero : acc[set][i][j]);
-                        // a quarter of the previous group's fold after each MFMA
-                        if (CARRY || kg > 0) fold(set ^ 1, S, kg - 1, step, 4);
-                        ++step;
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
+            for (int j = 0; j < TM; ++j) sa_l[kg][j] = scale_a[kg * BM + a_sub(j) + l32];
             if constexpr (!B_ROWSCALE) {
 #pragma unroll
+                for (int i = 0; i < TN; ++i) sb_u[kg][i] = scale_b[kg * BM + b_sub(i)];
+            } else {
+#pragma unroll
                 for (int i = 0; i < TN; ++i)
 #pragma unroll
-                    for (int j = 0; j < TM; ++j) sc[set][i][j] = sc_new[i][j];
+                    for (int r4 = 0; r4 < 4; ++r4)
+                        sb_q[kg][i][r4] = *reinterpret_cast<const float4*>(&scale_b[kg * BM + b_sub(i) + r4 * 8 + lhi * 4]);
             }
+        }
+        // fold half `h` (registers 8h .. 8h+7) of accumulator `buf` into total[i][j]
+        auto fold_half = [&](int buf, int i, int j, int kg, int h, float scale) {
 #pragma unroll
-            for (int i = 0; i < TN; ++i)
+            for (int r = 8 * h; r < 8 * h + 8; ++r) {
+                if constexpr (!B_ROWSCALE) {
+                    total[i][j][r] = fmaf(acc[buf][r], scale, total[i][j][r]);
+                } else {
+                    const float4 q = sb_q[kg][i][r / 4];
+                    const float sbv = r % 4 == 0 ? q.x : r % 4 == 1 ? q.y : r % 4 == 2 ? q.z : q.w;
+                    total[i][j][r] = fmaf(acc[buf][r], scale * sbv, total[i][j][r]);
+                }
+            }
+        };
+        const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-                for (int j = 0; j < TM; ++j) asm volatile("" : "+v"(total[i][j]));
+        for (int unit = 0; unit < FKG * TN * TM; ++unit) {
+            const int kg = unit / (TN * TM), i = unit / TM % TN, j = unit % TM, buf = unit & 1;
+            // the unit before this one (the last unit of the previous chunk for unit 0)
+            const int prev = (unit + FKG * TN * TM - 1) % (FKG * TN * TM);
+            const int pkg = prev / (TN * TM), pi = prev / TM % TN, pj = prev % TM;
+            const bool fold_prev = unit > 0 || CARRY;
+            const float prev_scale = B_ROWSCALE ? (unit > 0 ? sa_l[pkg][pj] : 0.0f) : pending_scale;
+            acc[buf] = mfma32<A_BF8, B_BF8>(as_long(opb[kg][i].x, opb[kg][i].y), as_long(opa[kg][j].x, opa[kg][j].y), zero);
+            if (fold_prev) fold_half(buf ^ 1, pi, pj, pkg, 0, prev_scale);
+            __builtin_amdgcn_sched_barrier(0);
+            acc[buf] = mfma32<A_BF8, B_BF8>(as_long(opb[kg][i].z, opb[kg][i].w), as_long(opa[kg][j].z, opa[kg][j].w), acc[buf]);
+            if (fold_prev) fold_half(buf ^ 1, pi, pj, pkg, 1, prev_scale);
+            if constexpr (!B_ROWSCALE) pending_scale = sa_l[kg][j] * sb_u[kg][i];
+            asm volatile("" : "+v"(total[pi][pj]));
+            __builtin_amdgcn_sched_barrier(0);
         }
         if constexpr (!CARRY) {
-            fold((FKG - 1) & 1, S, FKG - 1, 0, 1);
-#pragma unroll
-            for (int i = 0; i < TN; ++i)
-#pragma unroll
-                for (int j = 0; j < TM; ++j) asm volatile("" : "+v"(total[i][j]));
+            constexpr int last = FKG * TN * TM - 1;
+            fold_half(last & 1, last / TM % TN, last % TM, last / (TN * TM), 0, sa_l[last / (TN * TM)][last % TM]);
+            fold_half(last & 1, last / TM % TN, last % TM, last / (TN * TM), 1, sa_l[last / (TN * TM)][last % TM]);
         }
     };
-    // Straight-line steady state: no control flow between the loads, the math and the LDS writes. An odd chunk count
-    // runs one extra all-zero chunk.
-    read_ops(0, 0, ops[0]);
-    for (int64_t c = 0; c < chunks; c += 2) {
-        fetch(c + 2, 1);                                                     // set 1 <- chunk c+2; set 0 holds chunk c+1
-        compute(Stage<0>{});
-        stash(1, 0);
-        __syncthreads();
-        read_ops(1, 0, ops[0]);
-        fetch(c + 3, 0);                                                     // set 0 <- chunk c+3; set 1 holds chunk c+2
-        compute(Stage<1>{});
-        stash(0, 1);
-        __syncthreads();
-        read_ops(0, 0, ops[0]);
+
+    // Per chunk: wait for its loads, one barrier, refill the stage read last, math. Every fourth chunk also fetches
+    // the next scale block (first chunk of a block) or rearranges it (last chunk of the block before).
+    issue_scales(0);
+    issue(0, 0);
+    issue(1, 1);
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * (2 + B_LOADS)));               // scale block 0 is in LDS
+    __syncthreads();
+    arrange_scales(0);
+    int cur = 0, fill = 2;
+    for (int64_t c = 0; c < chunks; ++c) {
+        // all loads but the newest chunk's (and the scale pieces issued with it) have landed: chunk c is in LDS for
+        // this wave ...
+        if (c % F_SCHUNKS == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 + B_LOADS + 2));
+        else __builtin_amdgcn_s_waitcnt(0x0F70 | (2 + B_LOADS));
+        __syncthreads();                    // ... and for every wave; stage `fill` was last read in chunk c-1
+        issue(c + 2, fill);                 // past the end: zeros into a stage nobody reads
+        if (c % F_SCHUNKS == 0) issue_scales(c / F_SCHUNKS + 1);
+        if (c % F_SCHUNKS == F_SCHUNKS - 1) arrange_scales(c / F_SCHUNKS + 1);
+        compute(cur, c);
+        cur = cur == FSTAGES - 1 ? 0 : cur + 1;
+        fill = fill == FSTAGES - 1 ? 0 : fill + 1;
     }
-    if constexpr (CARRY) fold((FKG - 1) & 1, 0, FKG - 1, 0, 1);
+    __builtin_amdgcn_s_waitcnt(0x0F70);     // drain the trailing loads before the LDS allocation is released
+    if constexpr (CARRY) {
+        constexpr int last = FKG * TN * TM - 1;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) total[last / TM % TN][last % TM][r] = fmaf(acc[last & 1][r], pending_scale, total[last / TM % TN][last % TM][r]);
+    }
 
     // ---- epilogue: for sub-tiles (i, j) the lane holds row m = 32*j + l32 and, per register quad r4, columns
     // n = 8*r4 + 4*lhi + 0..3
@@ -364,8 +370,10 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
         const int64_t mrow = m_begin + a_sub(j) + l32;
         if (mrow >= m_end) continue;
 #pragma unroll
+        for (int i = 0; i < (GATED ? 1 : TN); ++i)
+#pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
-            const int64_t ncol = n_begin + wn * 32 + r4 * 8 + lhi * 4;
+            const int64_t ncol = n_begin + (GATED ? wn * 32 : b_sub(i)) + r4 * 8 + lhi * 4;
             if (ncol >= p.n) continue;
             const bool full = ncol + 3 < p.n;
             if constexpr (GATED) {
@@ -401,7 +409,7 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
             } else {
                 float v[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = total[0][j][r4 * 4 + e];
+                for (int e = 0; e < 4; ++e) v[e] = total[i][j][r4 * 4 + e];
                 if constexpr (MODE == MODE_PLAIN) {
                     if (p.bias) {
 #pragma unroll
@@ -448,21 +456,21 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
 }
 
 #ifndef VIOLA_GEMM_PROBE   // a probe build instantiates single kernels itself
-template <int MODE, bool B_ROWSCALE, typename TO>
+template <int MODE, bool B_ROWSCALE, typename TO, int TN>
 static void launch_formats(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, dim3 grid, hipStream_t stream) {
     const bool a5 = a_dtype == VIOLA_E5M2, b5 = b_dtype == VIOLA_E5M2;
-    if (!a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE, false, false, B_ROWSCALE, TO>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else if (a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE, true, false, B_ROWSCALE, TO>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else if (!a5 && b5) hipLaunchKernelGGL((group_gemm_fast<MODE, false, true, B_ROWSCALE, TO>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else hipLaunchKernelGGL((group_gemm_fast<MODE, true, true, B_ROWSCALE, TO>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    if (!a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE, false, false, B_ROWSCALE, TO, TN>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    else if (a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE, true, false, B_ROWSCALE, TO, TN>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    else if (!a5 && b5) hipLaunchKernelGGL((group_gemm_fast<MODE, false, true, B_ROWSCALE, TO, TN>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    else hipLaunchKernelGGL((group_gemm_fast<MODE, true, true, B_ROWSCALE, TO, TN>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
 }
 
-template <int MODE>
+template <int MODE, int TN>
 static int launch_mode(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, bool rowscale, dim3 grid,
                        hipStream_t stream) {
-#define VIOLA_FAST(TO)                                                                       \
-    if (rowscale) launch_formats<MODE, true, TO>(p, a_dtype, b_dtype, bias_dtype, grid, stream); \
-    else launch_formats<MODE, false, TO>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
+#define VIOLA_FAST(TO)                                                                           \
+    if (rowscale) launch_formats<MODE, true, TO, TN>(p, a_dtype, b_dtype, bias_dtype, grid, stream); \
+    else launch_formats<MODE, false, TO, TN>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
     switch (out_dtype) {
         case VIOLA_F32: VIOLA_FAST(float) break;
         case VIOLA_BF16: VIOLA_FAST(bf16_t) break;
@@ -476,14 +484,18 @@ static int launch_mode(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dty
 int launch_group_gemm_fast(const GemmArgs& args, int mode, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, bool rowscale,
                            dim3 grid, hipStream_t stream) {
     GemmArgs p = args;
+    // Two blocks fit a CU: with fewer than 512 tiles of 128 x 128, halve the tile in n so that all 256 CUs get two.
+    const bool narrow = mode == MODE_PLAIN && (int64_t)grid.x * grid.y * grid.z < 512 && p.n > 64;
+    if (narrow) grid.x = (unsigned)((p.n + 63) / 64);
     if (!p.offsets && (int64_t)grid.x * grid.y < (1 << 30)) {
         p.tiles_n = (int)grid.x;
         p.tiles_m = (int)grid.y;
         grid = dim3((grid.x * grid.y + 7) / 8 * 8, 1, grid.z);
     }
-    if (mode == MODE_PLAIN) return launch_mode<MODE_PLAIN>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
-    if (mode == MODE_GATED_FWD) return launch_mode<MODE_GATED_FWD>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
-    return launch_mode<MODE_GATED_BWD>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
+    if (narrow) return launch_mode<MODE_PLAIN, 1>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
+    if (mode == MODE_PLAIN) return launch_mode<MODE_PLAIN, 2>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
+    if (mode == MODE_GATED_FWD) return launch_mode<MODE_GATED_FWD, 2>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
+    return launch_mode<MODE_GATED_BWD, 2>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
 }
 #endif
 
