@@ -200,6 +200,90 @@ __global__ __launch_bounds__(256) void quantize_tile(const TIn* __restrict__ x, 
     }
 }
 
+// ------------------------------------------------------------------ 16-bit inputs: both layouts per wavefront
+// A wavefront owns 32 rows x 64 columns. Lane l loads 16 bytes (8 elements) of rows l/8 + 8i, quantizes them for
+// the row-wise layout straight from registers (a 32-column group is four neighbouring lanes), and parks the raw
+// 16 bytes in a wave-private LDS tile. ds_read_b64_tr_b16 then hands every lane the 32 rows of ONE column, four at
+// a time, which is exactly a group of the transposed layout. The LDS tile holds 2-byte values (rows of 64 + 32
+// elements: four consecutive rows start 64 bytes apart in bank space), so LDS moves 12 instructions per 32
+// elements instead of one per element and layout. No block-level synchronisation.
+template <typename TIn> __device__ __forceinline__ float widen16(uint32_t bits);
+template <> __device__ __forceinline__ float widen16<bf16_t>(uint32_t bits) { return __uint_as_float(bits << 16); }
+template <> __device__ __forceinline__ float widen16<f16_t>(uint32_t bits) {
+    const uint16_t b = (uint16_t)bits;
+    return (float)__builtin_bit_cast(_Float16, b);
+}
+
+template <typename TIn, typename TOut, bool ROWWISE>
+__global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x, uint8_t* __restrict__ q,
+                                                        float* __restrict__ scale, uint8_t* __restrict__ qt,
+                                                        float* __restrict__ scale_t, int64_t rows, int64_t cols,
+                                                        float limit) {
+    constexpr int LD = 64 + 32;
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    __shared__ __attribute__((aligned(16))) uint16_t park[4][32 * LD];
+    const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+    const int64_t r0 = (int64_t)blockIdx.y * 128 + wave * 32, c0 = (int64_t)blockIdx.x * 64;
+    if (r0 >= rows) return;                                                  // whole wavefront leaves together
+    uint16_t* mine = park[wave];
+    const int lr = lane / 8, ch = lane % 8;
+    const int64_t nc = (cols + 31) / 32;
+    const int64_t col8 = c0 + ch * 8;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int64_t row = r0 + lr + 8 * i;
+        const bool inside = row < rows && col8 < cols;                       // cols is a multiple of 8
+        uint4 raw = make_uint4(0, 0, 0, 0);
+        if (inside) raw = *reinterpret_cast<const uint4*>(x + row * cols + col8);
+        *reinterpret_cast<uint4*>(&mine[(lr + 8 * i) * LD + ch * 8]) = raw;
+        if constexpr (ROWWISE) {
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+            float v[8];
+            float amax = 0.0f, poison = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                v[e] = widen16<TIn>(e % 2 ? w[e / 2] >> 16 : w[e / 2] & 0xffffu);
+                amax = fmaxf(amax, fabsf(v[e]));
+                poison = poison_of(poison, v[e]);
+            }
+            amax = group_max<4>(amax);
+            poison += __shfl_xor(poison, 1, WAVE);
+            poison += __shfl_xor(poison, 2, WAVE);
+            const float s = group_scale(amax, limit);
+            const SharedDivisor divisor(s, poison);
+            if (inside) {
+                *reinterpret_cast<uint2*>(q + row * cols + col8) = encode8<TOut>(v, s, limit, divisor);
+                if (ch % 4 == 0) scale[row * nc + col8 / 32] = s;
+            }
+        }
+    }
+    // column lane % 16 of the 16-column strip lane / 16: rows 4t .. 4t+3 per read
+    const int64_t col = c0 + lane;
+    const int strip = (lane / 16) * 16, sub = lane & 15;
+    const uint16_t* at = &mine[(sub >> 2) * LD + strip + 4 * (sub & 3)];
+    float v[32];
+    float amax = 0.0f, poison = 0.0f;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        const s16x4 four = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at + 4 * t * LD));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            v[4 * t + e] = widen16<TIn>((uint16_t)four[e]);
+            amax = fmaxf(amax, fabsf(v[4 * t + e]));
+            poison = poison_of(poison, v[4 * t + e]);
+        }
+    }
+    if (col < cols) {
+        const float s = group_scale(amax, limit);
+        const int64_t nr = (rows + 31) / 32;
+        scale_t[col * nr + r0 / 32] = s;
+        const int count = (int)(rows - r0 < 32 ? rows - r0 : 32);
+        uint8_t* dst = qt + col * rows + r0;
+        store_group32<TOut>(v, s, poison, limit, dst, count, (reinterpret_cast<uintptr_t>(dst) & 15) == 0);
+    }
+}
+
 // ------------------------------------------------------------------ generic: one wavefront per group
 template <typename TIn, typename TOut, bool ENCODED>
 __global__ __launch_bounds__(256) void quantize_generic(const TIn* __restrict__ x, const float* __restrict__ source_scale,
@@ -319,6 +403,13 @@ static int launch_quantize(const void* x, int64_t rows, int64_t cols, void* q, f
 #undef VIOLA_ROWWISE
         return viola_launch_status();
     }
+    if constexpr (sizeof(TIn) == 2) {
+        if (gr == 1 && gc == 32 && transposed && vec) {
+            const dim3 grid16((unsigned)((cols + 63) / 64), (unsigned)((rows + 127) / 128));
+            hipLaunchKernelGGL((quantize_dual16<TIn, TOut, false>), grid16, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit);
+            return viola_launch_status();
+        }
+    }
     if (gr == 1 && gc == 32 && transposed) {
         const dim3 grid((unsigned)((cols + TILE_C - 1) / TILE_C), (unsigned)((rows + TILE_R - 1) / TILE_R));
         if (vec) hipLaunchKernelGGL((quantize_tile<TIn, TOut, false, true, true>), grid, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit);
@@ -360,6 +451,14 @@ static int launch_dual(const void* x, int64_t rows, int64_t cols, void* q, float
     const bool vec = cols % 8 == 0 && reinterpret_cast<uintptr_t>(x) % (8 * sizeof(TIn)) == 0;
     const dim3 grid((unsigned)((cols + TILE_C - 1) / TILE_C), (unsigned)((rows + TILE_R - 1) / TILE_R));
     const TIn* xp = static_cast<const TIn*>(x);
+    if constexpr (sizeof(TIn) == 2) {
+        if (vec && reinterpret_cast<uintptr_t>(q) % 8 == 0) {
+            const dim3 grid16((unsigned)((cols + 63) / 64), (unsigned)((rows + 127) / 128));
+            hipLaunchKernelGGL((quantize_dual16<TIn, TOut, true>), grid16, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale,
+                               static_cast<uint8_t*>(qt), scale_t, rows, cols, limit);
+            return viola_launch_status();
+        }
+    }
     if (vec) hipLaunchKernelGGL((quantize_tile<TIn, TOut, true, true, true>), grid, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale, static_cast<uint8_t*>(qt), scale_t, rows, cols, limit);
     else hipLaunchKernelGGL((quantize_tile<TIn, TOut, true, true, false>), grid, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale, static_cast<uint8_t*>(qt), scale_t, rows, cols, limit);
     return viola_launch_status();
