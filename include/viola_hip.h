@@ -52,7 +52,14 @@ int viola_group_quantize(const void* x, int x_dtype, int64_t rows, int64_t cols,
  * viola_group_quantize (viola/nn/_grouped_linear.py:21,46-47 and :73,92 make those two calls). */
 int viola_group_quantize_dual(const void* x, int x_dtype, int64_t rows, int64_t cols,
                               void* q, float* scale, void* qt, float* scale_t, int q_dtype, int gc,
-                              float limit, viola_stream_t stream);
+                              float limit, float* column_partial, viola_stream_t stream);
+
+/* column_partial (nullable) of viola_group_quantize_dual receives [ceil(rows/32), cols] fp32 sums of x over
+ * each 32-row group, taken from the same read; viola_column_reduce adds the parts in a fixed order:
+ * out[c] = sum_p partial[p][c], stored as out_dtype. Together they are the bias gradient dy.sum(0)
+ * (viola/nn/_grouped_linear.py:101) without a second pass over dy. */
+int viola_column_reduce(const float* partial, int64_t parts, int64_t cols, void* out, int out_dtype,
+                        viola_stream_t stream);
 
 /* viola/nn/_grouped_kernels.py:44-50 `dequantize` (decode_kernel :24-41): out = f32(q) * scale[r/gr, c/gc]. */
 int viola_group_dequantize(const void* q, int q_dtype, const float* scale, int64_t rows, int64_t cols,

@@ -123,6 +123,26 @@ def test_quantize_rounding_ties_over_all_magnitudes(fp8, limit):
     _same(q, sc, *og.quantize(x, fp8, (32, 32), limit=limit))
 
 
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(65, 128), (300, 200), (129, 72), (8192, 1024), (32, 64)])
+def test_quantize_dual_column_sums(in_dtype, shape):
+    """x.sum(0) from the quantizer's own read: fp32 accumulation in a fixed order, same codes as without it."""
+    g = _gpu()
+    x = _input(shape, in_dtype, seed=13)
+    plain = g.quantize_dual(x.cuda(), E4, (1, 32))
+    for out_dtype in (torch.float32, in_dtype):
+        *codes, total = g.quantize_dual(x.cuda(), E4, (1, 32), column_sum_dtype=out_dtype)
+        for a, b in zip(codes, plain):
+            assert torch.equal(a.view(torch.uint8) if a.dtype == E4 else a, b.view(torch.uint8) if b.dtype == E4 else b)
+        ref = x.double().sum(0)
+        assert total.dtype == out_dtype and total.shape == (shape[1],)
+        # fp32 partial sums: error well below one rounding of the widest term per 32 rows
+        bound = x.double().abs().sum(0) * 2.0 ** -22 + (ref.abs() * torch.finfo(out_dtype).eps)
+        assert ((total.cpu().double() - ref).abs() <= bound + 1e-30).all()
+    again = g.quantize_dual(x.cuda(), E4, (1, 32), column_sum_dtype=torch.float32)[-1]
+    assert torch.equal(again, g.quantize_dual(x.cuda(), E4, (1, 32), column_sum_dtype=torch.float32)[-1])    # deterministic
+
+
 def test_quantize_limit_and_out_arguments():
     g = _gpu()
     x = _input((64, 96), torch.float32, seed=3)

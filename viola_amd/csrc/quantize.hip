@@ -152,7 +152,7 @@ template <typename TIn, typename TOut, bool ROWWISE, bool TRANSPOSED, bool VEC>
 __global__ __launch_bounds__(256) void quantize_tile(const TIn* __restrict__ x, uint8_t* __restrict__ q,
                                                       float* __restrict__ scale, uint8_t* __restrict__ qt,
                                                       float* __restrict__ scale_t, int64_t rows, int64_t cols,
-                                                      float limit) {
+                                                      float limit, float* __restrict__ column_partial) {
     __shared__ float tile[TILE_R * TILE_LD];
     const int64_t r0 = (int64_t)blockIdx.y * TILE_R, c0 = (int64_t)blockIdx.x * TILE_C;
     load_tile<TIn, VEC>(x, tile, r0, c0, rows, cols);
@@ -193,6 +193,12 @@ __global__ __launch_bounds__(256) void quantize_tile(const TIn* __restrict__ x, 
             const float s = group_scale(amax, limit);
             const int64_t nr = (rows + 31) / 32;
             scale_t[col * nr + row / 32] = s;
+            if (column_partial) {
+                float sum = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 32; ++i) sum += v[i];
+                column_partial[(row / 32) * cols + col] = sum;
+            }
             const int count = (int)(rows - row < 32 ? rows - row : 32);
             uint8_t* dst = qt + col * rows + row;
             store_group32<TOut>(v, s, poison, limit, dst, count, (reinterpret_cast<uintptr_t>(dst) & 15) == 0);
@@ -218,7 +224,7 @@ template <typename TIn, typename TOut, bool ROWWISE>
 __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x, uint8_t* __restrict__ q,
                                                         float* __restrict__ scale, uint8_t* __restrict__ qt,
                                                         float* __restrict__ scale_t, int64_t rows, int64_t cols,
-                                                        float limit) {
+                                                        float limit, float* __restrict__ column_partial) {
     constexpr int LD = 64 + 32;
     typedef short s16x4 __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
@@ -278,9 +284,48 @@ __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x
         const float s = group_scale(amax, limit);
         const int64_t nr = (rows + 31) / 32;
         scale_t[col * nr + r0 / 32] = s;
+        if (column_partial) {
+            float sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 32; ++i) sum += v[i];
+            column_partial[(r0 / 32) * cols + col] = sum;
+        }
         const int count = (int)(rows - r0 < 32 ? rows - r0 : 32);
         uint8_t* dst = qt + col * rows + r0;
         store_group32<TOut>(v, s, poison, limit, dst, count, (reinterpret_cast<uintptr_t>(dst) & 15) == 0);
+    }
+}
+
+// ------------------------------------------------------------------ column sums from 32-row partials
+// out[c] = sum over p of partial[p][c] in a fixed order: 8 threads per column each add a contiguous eighth of the
+// parts in ascending order (loads issued eight at a time), then the eighths are added in order.
+template <typename TO>
+__global__ __launch_bounds__(256) void column_reduce_kernel(const float* __restrict__ partial, int64_t parts, int64_t cols,
+                                                             TO* __restrict__ out) {
+    __shared__ float piece[8][32];
+    const int c = threadIdx.x % 32, slice = threadIdx.x / 32;
+    const int64_t col = (int64_t)blockIdx.x * 32 + c;
+    const int64_t per = (parts + 7) / 8;
+    const int64_t begin = slice * per, end = begin + per < parts ? begin + per : parts;
+    float sum = 0.0f;
+    if (col < cols) {
+        int64_t part = begin;
+        for (; part + 8 <= end; part += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = partial[(part + u) * cols + col];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) sum += v[u];
+        }
+        for (; part < end; ++part) sum += partial[part * cols + col];
+    }
+    piece[slice][c] = sum;
+    __syncthreads();
+    if (slice == 0 && col < cols) {
+        float total = piece[0][c];
+#pragma unroll
+        for (int u = 1; u < 8; ++u) total += piece[u][c];
+        out[col] = from_f32<TO>(total);
     }
 }
 
@@ -406,14 +451,14 @@ static int launch_quantize(const void* x, int64_t rows, int64_t cols, void* q, f
     if constexpr (sizeof(TIn) == 2) {
         if (gr == 1 && gc == 32 && transposed && vec) {
             const dim3 grid16((unsigned)((cols + 63) / 64), (unsigned)((rows + 127) / 128));
-            hipLaunchKernelGGL((quantize_dual16<TIn, TOut, false>), grid16, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit);
+            hipLaunchKernelGGL((quantize_dual16<TIn, TOut, false>), grid16, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit, nullptr);
             return viola_launch_status();
         }
     }
     if (gr == 1 && gc == 32 && transposed) {
         const dim3 grid((unsigned)((cols + TILE_C - 1) / TILE_C), (unsigned)((rows + TILE_R - 1) / TILE_R));
-        if (vec) hipLaunchKernelGGL((quantize_tile<TIn, TOut, false, true, true>), grid, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit);
-        else hipLaunchKernelGGL((quantize_tile<TIn, TOut, false, true, false>), grid, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit);
+        if (vec) hipLaunchKernelGGL((quantize_tile<TIn, TOut, false, true, true>), grid, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit, nullptr);
+        else hipLaunchKernelGGL((quantize_tile<TIn, TOut, false, true, false>), grid, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit, nullptr);
         return viola_launch_status();
     }
     const int64_t out_rows = transposed ? cols : rows, out_cols = transposed ? rows : cols;
@@ -447,7 +492,7 @@ static int launch_reencode(const void* x, const float* source_scale, int64_t row
 
 template <typename TIn, typename TOut>
 static int launch_dual(const void* x, int64_t rows, int64_t cols, void* q, float* scale, void* qt, float* scale_t,
-                       float limit, hipStream_t stream) {
+                       float limit, float* column_partial, hipStream_t stream) {
     const bool vec = cols % 8 == 0 && reinterpret_cast<uintptr_t>(x) % (8 * sizeof(TIn)) == 0;
     const dim3 grid((unsigned)((cols + TILE_C - 1) / TILE_C), (unsigned)((rows + TILE_R - 1) / TILE_R));
     const TIn* xp = static_cast<const TIn*>(x);
@@ -455,12 +500,12 @@ static int launch_dual(const void* x, int64_t rows, int64_t cols, void* q, float
         if (vec && reinterpret_cast<uintptr_t>(q) % 8 == 0) {
             const dim3 grid16((unsigned)((cols + 63) / 64), (unsigned)((rows + 127) / 128));
             hipLaunchKernelGGL((quantize_dual16<TIn, TOut, true>), grid16, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale,
-                               static_cast<uint8_t*>(qt), scale_t, rows, cols, limit);
+                               static_cast<uint8_t*>(qt), scale_t, rows, cols, limit, column_partial);
             return viola_launch_status();
         }
     }
-    if (vec) hipLaunchKernelGGL((quantize_tile<TIn, TOut, true, true, true>), grid, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale, static_cast<uint8_t*>(qt), scale_t, rows, cols, limit);
-    else hipLaunchKernelGGL((quantize_tile<TIn, TOut, true, true, false>), grid, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale, static_cast<uint8_t*>(qt), scale_t, rows, cols, limit);
+    if (vec) hipLaunchKernelGGL((quantize_tile<TIn, TOut, true, true, true>), grid, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale, static_cast<uint8_t*>(qt), scale_t, rows, cols, limit, column_partial);
+    else hipLaunchKernelGGL((quantize_tile<TIn, TOut, true, true, false>), grid, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale, static_cast<uint8_t*>(qt), scale_t, rows, cols, limit, column_partial);
     return viola_launch_status();
 }
 
@@ -502,13 +547,13 @@ extern "C" int viola_group_quantize(const void* x, int x_dtype, int64_t rows, in
 
 extern "C" int viola_group_quantize_dual(const void* x, int x_dtype, int64_t rows, int64_t cols, void* q, float* scale,
                                          void* qt, float* scale_t, int q_dtype, int gc, float limit,
-                                         viola_stream_t stream_) {
+                                         float* column_partial, viola_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     VIOLA_CHECK_ARG(viola_is_fp8(q_dtype) && viola_is_float(x_dtype) && rows >= 0 && cols >= 0 && limit > 0.0f);
     if (gc != 32) return VIOLA_EUNSUPPORTED;
     if (rows == 0 || cols == 0) return 0;
     VIOLA_CHECK_ARG(x && q && scale && qt && scale_t);
-#define VIOLA_DUAL(TI, TO) return launch_dual<TI, TO>(x, rows, cols, q, scale, qt, scale_t, limit, stream)
+#define VIOLA_DUAL(TI, TO) return launch_dual<TI, TO>(x, rows, cols, q, scale, qt, scale_t, limit, column_partial, stream)
     if (q_dtype == VIOLA_E4M3) {
         if (x_dtype == VIOLA_F32) VIOLA_DUAL(float, e4m3_t);
         if (x_dtype == VIOLA_BF16) VIOLA_DUAL(bf16_t, e4m3_t);
@@ -518,6 +563,19 @@ extern "C" int viola_group_quantize_dual(const void* x, int x_dtype, int64_t row
     if (x_dtype == VIOLA_BF16) VIOLA_DUAL(bf16_t, e5m2_t);
     VIOLA_DUAL(f16_t, e5m2_t);
 #undef VIOLA_DUAL
+}
+
+extern "C" int viola_column_reduce(const float* partial, int64_t parts, int64_t cols, void* out, int out_dtype,
+                                   viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_float(out_dtype) && parts >= 0 && cols >= 0);
+    if (cols == 0) return 0;
+    VIOLA_CHECK_ARG(out && (parts == 0 || partial));
+    const dim3 grid((unsigned)((cols + 31) / 32));
+    if (out_dtype == VIOLA_F32) hipLaunchKernelGGL(column_reduce_kernel<float>, grid, dim3(256), 0, stream, partial, parts, cols, static_cast<float*>(out));
+    else if (out_dtype == VIOLA_BF16) hipLaunchKernelGGL(column_reduce_kernel<bf16_t>, grid, dim3(256), 0, stream, partial, parts, cols, static_cast<bf16_t*>(out));
+    else hipLaunchKernelGGL(column_reduce_kernel<f16_t>, grid, dim3(256), 0, stream, partial, parts, cols, static_cast<f16_t*>(out));
+    return viola_launch_status();
 }
 
 extern "C" int viola_varlen_quantize_transposed(const void* x, int x_dtype, int64_t rows, int64_t cols,

@@ -53,11 +53,12 @@ def quantize(x, dtype, group, *, native=False, limit=None, transposed=False,
     return q, s
 
 
-def quantize_dual(x, dtype, group, *, limit=None):
+def quantize_dual(x, dtype, group, *, limit=None, column_sum_dtype=None):
     """Row-wise codes/scales and the quantized transpose of x from ONE read of x.
 
     Same values as quantize(x, ...) and quantize(x, ..., transposed=True); 1-D groups of 32 only.
-    Returns (q, s, qt, st).
+    Returns (q, s, qt, st), plus x.sum(0) in column_sum_dtype (fp32 accumulation, from the same read)
+    when that is given.
     """
     assert x.is_cuda and x.dim() == 2 and tuple(group) == (1, 32)
     x = x.contiguous()
@@ -67,9 +68,15 @@ def quantize_dual(x, dtype, group, *, limit=None):
     s = torch.empty(scale_shape((rows, cols), group), device=x.device, dtype=torch.float32)
     qt = torch.empty((cols, rows), device=x.device, dtype=dtype)
     st = torch.empty(scale_shape((cols, rows), group), device=x.device, dtype=torch.float32)
+    parts = -(-rows // 32)
+    partial = torch.empty((parts, cols), device=x.device, dtype=torch.float32) if column_sum_dtype is not None else None
     _lib.call("viola_group_quantize_dual", _lib.ptr(x), _lib.code(x.dtype), rows, cols, _lib.ptr(q), _lib.ptr(s),
-              _lib.ptr(qt), _lib.ptr(st), _lib.code(dtype), group[1], float(limit))
-    return q, s, qt, st
+              _lib.ptr(qt), _lib.ptr(st), _lib.code(dtype), group[1], float(limit), _lib.ptr(partial))
+    if column_sum_dtype is None:
+        return q, s, qt, st
+    total = torch.empty(cols, device=x.device, dtype=column_sum_dtype)
+    _lib.call("viola_column_reduce", _lib.ptr(partial), parts, cols, _lib.ptr(total), _lib.code(column_sum_dtype))
+    return q, s, qt, st, total
 
 
 def transpose_group(group):

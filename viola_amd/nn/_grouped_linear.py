@@ -78,9 +78,13 @@ def backward_core(record, tensors, dy, needs, *, gated=None, aux=None):
     limit = layer._group_limit(gg, bwd)
     weight_limit = layer._group_limit(gw, fp8, weight=True)
     qg = sg = gt = sgt = None
-    if needs[0] and needs[1] and _one_d32(gg):
-        qg, sg, gt, sgt = kernels.quantize_dual(dy, bwd, gg, limit=limit)
     dx = dw = db = None
+    if needs[0] and needs[1] and _one_d32(gg):
+        if needs[2] and dy.shape[0] > 0:
+            # the bias gradient rides on the quantizer's read of dy
+            qg, sg, gt, sgt, db = kernels.quantize_dual(dy, bwd, gg, limit=limit, column_sum_dtype=record.bias_grad_dtype)
+        else:
+            qg, sg, gt, sgt = kernels.quantize_dual(dy, bwd, gg, limit=limit)
     for op in ((1, 0) if gated else (0, 1)):
         if op == 0 and needs[0]:
             if qg is None:
@@ -108,7 +112,7 @@ def backward_core(record, tensors, dy, needs, *, gated=None, aux=None):
                 xt, sxt = kernels.quantize(saved_x, fp8, gx, limit=record.input_limit, transposed=True)
             dw = layer._group_gemm(gt, xt, sgt, sxt, gg, gx, out_dtype=record.weight_grad_dtype)
             gt = sgt = xt = sxt = None
-    if needs[2]:
+    if needs[2] and db is None:
         db = dy.sum(0, dtype=record.bias_grad_dtype)
     return dx, dw, db
 
