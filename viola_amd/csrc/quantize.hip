@@ -381,18 +381,46 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const TQ* __restrict__ 
 }
 
 // ------------------------------------------------------------------ byte transpose, 64 x 64 tile
+// WORDS: rows and cols multiples of 4 and both pointers 4-byte aligned. A thread then owns a 4 x 4 byte block: four
+// 4-byte loads (16 lanes cover 64 contiguous bytes of a row), a 4 x 4 transpose with byte permutes, the four words
+// handed over through LDS so that the stores are again 64 contiguous bytes per 16 lanes.
+template <bool WORDS>
 __global__ __launch_bounds__(256) void transpose_bytes(const uint8_t* __restrict__ x, uint8_t* __restrict__ out,
                                                         int64_t rows, int64_t cols) {
-    __shared__ uint8_t tile[64][64 + 4];
     const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
-    for (int id = threadIdx.x; id < 64 * 64; id += 256) {
-        const int r = id / 64, c = id % 64;
-        tile[r][c] = (r0 + r < rows && c0 + c < cols) ? x[(r0 + r) * cols + c0 + c] : 0;
-    }
-    __syncthreads();
-    for (int id = threadIdx.x; id < 64 * 64; id += 256) {
-        const int c = id / 64, r = id % 64;
-        if (r0 + r < rows && c0 + c < cols) out[(c0 + c) * rows + r0 + r] = tile[r][c];
+    if constexpr (WORDS) {
+        __shared__ uint32_t tile[64][17];
+        const int b = threadIdx.x % 16, a = threadIdx.x / 16;               // block of rows 4a.., cols 4b..
+        uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (r0 + 4 * a + i < rows && c0 + 4 * b < cols) w[i] = *reinterpret_cast<const uint32_t*>(x + (r0 + 4 * a + i) * cols + c0 + 4 * b);
+        // t[j] = byte j of w[0..3]
+        const uint32_t lo01 = __builtin_amdgcn_perm(w[1], w[0], 0x05010400u);   // w0.b0 w1.b0 w0.b1 w1.b1
+        const uint32_t hi01 = __builtin_amdgcn_perm(w[1], w[0], 0x07030602u);   // w0.b2 w1.b2 w0.b3 w1.b3
+        const uint32_t lo23 = __builtin_amdgcn_perm(w[3], w[2], 0x05010400u);
+        const uint32_t hi23 = __builtin_amdgcn_perm(w[3], w[2], 0x07030602u);
+        tile[4 * b + 0][a] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);    // bytes 0,1 of lo01 then of lo23
+        tile[4 * b + 1][a] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+        tile[4 * b + 2][a] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+        tile[4 * b + 3][a] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = threadIdx.x / 16 + 16 * i, ra = threadIdx.x % 16;
+            if (c0 + c < cols && r0 + 4 * ra < rows) *reinterpret_cast<uint32_t*>(out + (c0 + c) * rows + r0 + 4 * ra) = tile[c][ra];
+        }
+    } else {
+        __shared__ uint8_t tile[64][64 + 4];
+        for (int id = threadIdx.x; id < 64 * 64; id += 256) {
+            const int r = id / 64, c = id % 64;
+            tile[r][c] = (r0 + r < rows && c0 + c < cols) ? x[(r0 + r) * cols + c0 + c] : 0;
+        }
+        __syncthreads();
+        for (int id = threadIdx.x; id < 64 * 64; id += 256) {
+            const int c = id / 64, r = id % 64;
+            if (r0 + r < rows && c0 + c < cols) out[(c0 + c) * rows + r0 + r] = tile[r][c];
+        }
     }
 }
 
@@ -619,7 +647,9 @@ extern "C" int viola_fp8_transpose(const void* x, void* out, int64_t rows, int64
     VIOLA_CHECK_ARG(rows >= 0 && cols >= 0);
     if (rows == 0 || cols == 0) return 0;
     VIOLA_CHECK_ARG(x && out && (rows + 63) / 64 <= 65535);
-    hipLaunchKernelGGL(transpose_bytes, dim3((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64)), dim3(256), 0, stream,
-                       static_cast<const uint8_t*>(x), static_cast<uint8_t*>(out), rows, cols);
+    const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64));
+    const bool words = rows % 4 == 0 && cols % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 4 == 0;
+    if (words) hipLaunchKernelGGL(transpose_bytes<true>, grid, dim3(256), 0, stream, static_cast<const uint8_t*>(x), static_cast<uint8_t*>(out), rows, cols);
+    else hipLaunchKernelGGL(transpose_bytes<false>, grid, dim3(256), 0, stream, static_cast<const uint8_t*>(x), static_cast<uint8_t*>(out), rows, cols);
     return viola_launch_status();
 }
