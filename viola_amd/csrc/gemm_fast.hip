@@ -257,13 +257,13 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
 #pragma unroll
             for (int r = 0; r < 16; ++r) total[i][j][r] = 0.0f;
 
-    // Two 16-register accumulators alternate between consecutive (K group, sub-tile) units; `pending` is the unit whose
-    // MFMAs were issued last and whose fold is still to come (across chunk boundaries when CARRY).
+    // Four 16-register accumulators: two receive the MFMAs of the current pair of (K group, sub-tile) units while the
+    // two of the pair before are folded into the totals (across chunk boundaries when CARRY).
     constexpr bool CARRY = !B_ROWSCALE;
-    f32x16 acc[2];
-    float pending_scale = 0.0f;                                              // sa * sb of the pending unit (uniform b scales)
+    f32x16 acc[4];
+    float pending_scale[2] = {0.0f, 0.0f};                                   // sa * sb of the pending pair (uniform b scales)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[0][r] = acc[1][r] = 0.0f;
+    for (int r = 0; r < 16; ++r) acc[0][r] = acc[1][r] = acc[2][r] = acc[3][r] = 0.0f;
     auto as_long = [](uint32_t lo, uint32_t hi) -> long { return (long)(((uint64_t)hi << 32) | lo); };
 
     auto compute = [&](int stage, int64_t c) {
@@ -307,27 +307,47 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
             }
         };
         const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        // Units go in pairs: the four MFMAs of a pair alternate between its two accumulators, so an MFMA never waits
+        // for the one issued just before it, and a quarter of the previous pair's fold follows each of them.
+        constexpr int UNITS = FKG * TN * TM, PAIRS = UNITS / 2;
 #pragma unroll
-        for (int unit = 0; unit < FKG * TN * TM; ++unit) {
-            const int kg = unit / (TN * TM), i = unit / TM % TN, j = unit % TM, buf = unit & 1;
-            // the unit before this one (the last unit of the previous chunk for unit 0)
-            const int prev = (unit + FKG * TN * TM - 1) % (FKG * TN * TM);
-            const int pkg = prev / (TN * TM), pi = prev / TM % TN, pj = prev % TM;
-            const bool fold_prev = unit > 0 || CARRY;
-            const float prev_scale = B_ROWSCALE ? (unit > 0 ? sa_l[pkg][pj] : 0.0f) : pending_scale;
-            acc[buf] = mfma32<A_BF8, B_BF8>(as_long(opb[kg][i].x, opb[kg][i].y), as_long(opa[kg][j].x, opa[kg][j].y), zero);
-            if (fold_prev) fold_half(buf ^ 1, pi, pj, pkg, 0, prev_scale);
-            __builtin_amdgcn_sched_barrier(0);
-            acc[buf] = mfma32<A_BF8, B_BF8>(as_long(opb[kg][i].z, opb[kg][i].w), as_long(opa[kg][j].z, opa[kg][j].w), acc[buf]);
-            if (fold_prev) fold_half(buf ^ 1, pi, pj, pkg, 1, prev_scale);
-            if constexpr (!B_ROWSCALE) pending_scale = sa_l[kg][j] * sb_u[kg][i];
-            asm volatile("" : "+v"(total[pi][pj]));
-            __builtin_amdgcn_sched_barrier(0);
+        for (int pair = 0; pair < PAIRS; ++pair) {
+            const int base = (pair & 1) * 2, other = base ^ 2;
+            const int before = (pair + PAIRS - 1) % PAIRS;                   // the pair folded now (last of the chunk before for pair 0)
+            const bool fold_prev = pair > 0 || CARRY;
+            int kg[2], ti[2], tj[2], pkg[2], pi[2], pj[2];
+            float prev_scale[2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int unit = 2 * pair + h, prev = 2 * before + h;
+                kg[h] = unit / (TN * TM); ti[h] = unit / TM % TN; tj[h] = unit % TM;
+                pkg[h] = prev / (TN * TM); pi[h] = prev / TM % TN; pj[h] = prev % TM;
+                prev_scale[h] = B_ROWSCALE ? (pair > 0 ? sa_l[pkg[h]][pj[h]] : 0.0f) : pending_scale[h];
+            }
+#pragma unroll
+            for (int step = 0; step < 4; ++step) {
+                const int h = step & 1, ks = step >> 1;
+                const uint4 ob = opb[kg[h]][ti[h]], oa = opa[kg[h]][tj[h]];
+                if (ks == 0) acc[base + h] = mfma32<A_BF8, B_BF8>(as_long(ob.x, ob.y), as_long(oa.x, oa.y), zero);
+                else acc[base + h] = mfma32<A_BF8, B_BF8>(as_long(ob.z, ob.w), as_long(oa.z, oa.w), acc[base + h]);
+                if (fold_prev) fold_half(other + (step >> 1), pi[step >> 1], pj[step >> 1], pkg[step >> 1], step & 1, prev_scale[step >> 1]);
+                asm volatile("" : "+v"(total[pi[step >> 1]][pj[step >> 1]]));
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if constexpr (!B_ROWSCALE) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h) pending_scale[h] = sa_l[kg[h]][tj[h]] * sb_u[kg[h]][ti[h]];
+            }
         }
         if constexpr (!CARRY) {
-            constexpr int last = FKG * TN * TM - 1;
-            fold_half(last & 1, last / TM % TN, last % TM, last / (TN * TM), 0, sa_l[last / (TN * TM)][last % TM]);
-            fold_half(last & 1, last / TM % TN, last % TM, last / (TN * TM), 1, sa_l[last / (TN * TM)][last % TM]);
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                constexpr int last_pair = PAIRS - 1;
+                const int unit = 2 * last_pair + h;
+                const int lkg = unit / (TN * TM), li = unit / TM % TN, lj = unit % TM;
+                fold_half((last_pair & 1) * 2 + h, li, lj, lkg, 0, sa_l[lkg][lj]);
+                fold_half((last_pair & 1) * 2 + h, li, lj, lkg, 1, sa_l[lkg][lj]);
+            }
         }
     };
 
@@ -355,9 +375,13 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);     // drain the trailing loads before the LDS allocation is released
     if constexpr (CARRY) {
-        constexpr int last = FKG * TN * TM - 1;
+        constexpr int UNITS = FKG * TN * TM, last_pair = UNITS / 2 - 1;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) total[last / TM % TN][last % TM][r] = fmaf(acc[last & 1][r], pending_scale, total[last / TM % TN][last % TM][r]);
+        for (int h = 0; h < 2; ++h) {
+            const int unit = 2 * last_pair + h, li = unit / TM % TN, lj = unit % TM;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) total[li][lj][r] = fmaf(acc[(last_pair & 1) * 2 + h][r], pending_scale[h], total[li][lj][r]);
+        }
     }
 
     // ---- epilogue: for sub-tiles (i, j) the lane holds row m = 32*j + l32 and, per register quad r4, columns
