@@ -6,6 +6,7 @@
 // GEMM the b matrix is the MFMA "A" operand so a lane owns one output row m and runs of four
 // consecutive n. b may be given as [n, k] (transpose_b) or [k, n]; the latter is transposed on
 // its way into LDS.
+#include <type_traits>
 #include "ns_args.hpp"
 
 namespace viola {
@@ -244,6 +245,149 @@ __global__ __launch_bounds__(256) void ns_scale_kernel(const TIn* __restrict__ i
     }
 }
 
+// ------------------------------------------------------------------ normalisation, 16-byte accesses
+// The same values as the kernels above for 16-bit inputs whose extents allow 8-element accesses. The division by
+// the one denominator of a matrix takes the shared-divisor route (exact quotient from a reciprocal and two FMAs)
+// whenever the denominator allows it.
+__device__ __forceinline__ float ns_denominator(const float* __restrict__ workspace, int64_t bz, bool is_bf16, float* shared) {
+    if (threadIdx.x < WAVE) {
+        float sum = 0.0f;
+        for (int i = threadIdx.x; i < PARTS; i += WAVE) sum += workspace[bz * PARTS + i];
+        sum = wave_sum(sum);
+        if (threadIdx.x == 0) {
+            if (is_bf16) {
+                const float norm = half_to_f32<true>(f32_to_half<true>(sqrtf(sum)));
+                *shared = half_to_f32<true>(f32_to_half<true>(norm + 1e-7f));
+            } else {
+                const float norm = half_to_f32<false>(f32_to_half<false>(sqrtf(sum)));
+                *shared = half_to_f32<false>(f32_to_half<false>(norm + 1e-7f));
+            }
+        }
+    }
+    __syncthreads();
+    return *shared;
+}
+
+template <typename TIn, bool IS_BF16> __device__ __forceinline__ float ns_working(uint32_t raw16) {
+    // a 16-bit input value converted to the working dtype and widened
+    float v;
+    if constexpr (sizeof(TIn) == 2 && std::is_same<TIn, bf16_t>::value) v = __uint_as_float(raw16 << 16);
+    else { const uint16_t b = (uint16_t)raw16; v = (float)__builtin_bit_cast(_Float16, b); }
+    return half_to_f32<IS_BF16>(f32_to_half<IS_BF16>(v));
+}
+
+template <typename TIn, bool IS_BF16>
+__global__ __launch_bounds__(256) void ns_sumsq16_kernel(const TIn* __restrict__ in, float* __restrict__ workspace, int64_t count) {
+    const int64_t bz = blockIdx.y;
+    const uint4* src = reinterpret_cast<const uint4*>(in + bz * count);
+    const int64_t octets = count / 8;
+    const int64_t per = (octets + PARTS - 1) / PARTS;
+    const int64_t begin = (int64_t)blockIdx.x * per;
+    const int64_t end = begin + per < octets ? begin + per : octets;
+    float sum = 0.0f;
+    for (int64_t i = begin + threadIdx.x; i < end; i += 256) {
+        const uint4 raw = src[i];
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float v = ns_working<TIn, IS_BF16>(e % 2 ? w[e / 2] >> 16 : w[e / 2] & 0xffffu);
+            sum += v * v;
+        }
+    }
+    __shared__ float partial[4];
+    sum = wave_sum(sum);
+    if (threadIdx.x % WAVE == 0) partial[threadIdx.x / WAVE] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) workspace[bz * PARTS + blockIdx.x] = (partial[0] + partial[1]) + (partial[2] + partial[3]);
+}
+
+template <bool IS_BF16>
+__device__ __forceinline__ uint32_t ns_scaled(float v, float denom, const SharedDivisor& d) {
+    return f32_to_half<IS_BF16>(d.fast ? d.quotient(v) : v / denom);
+}
+
+template <typename TIn, bool IS_BF16>
+__global__ __launch_bounds__(256) void ns_scale16_kernel(const TIn* __restrict__ in, uint16_t* __restrict__ out,
+                                                          const float* __restrict__ workspace, int64_t count) {
+    __shared__ float denom_s;
+    const int64_t bz = blockIdx.y;
+    const float denom = ns_denominator(workspace, bz, IS_BF16, &denom_s);
+    const SharedDivisor divisor(denom, 0.0f);
+    const uint4* src = reinterpret_cast<const uint4*>(in + bz * count);
+    uint4* dst = reinterpret_cast<uint4*>(out + bz * count);
+    const int64_t octets = count / 8;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < octets; i += (int64_t)gridDim.x * 256) {
+        const uint4 raw = src[i];
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float lo = ns_working<TIn, IS_BF16>(w[e] & 0xffffu), hi = ns_working<TIn, IS_BF16>(w[e] >> 16);
+            // a non-finite value keeps the plain division (the quotient route assumes finite operands)
+            const bool plain = !(fabsf(lo) < INFINITY) || !(fabsf(hi) < INFINITY);
+            const SharedDivisor use = plain ? SharedDivisor(denom, __uint_as_float(0x7fc00000u)) : divisor;
+            o[e] = ns_scaled<IS_BF16>(lo, denom, use) | (ns_scaled<IS_BF16>(hi, denom, use) << 16);
+        }
+        dst[i] = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+}
+
+// Transposed: a wavefront parks 32 rows x 64 columns of raw 16-bit values in LDS and reads them back with
+// ds_read_b64_tr_b16, so each lane ends up with the 32 rows of one column = 64 contiguous bytes of the output.
+template <typename TIn, bool IS_BF16>
+__global__ __launch_bounds__(256) void ns_scale16_transposed_kernel(const TIn* __restrict__ in, uint16_t* __restrict__ out,
+                                                                     const float* __restrict__ workspace, int64_t rows,
+                                                                     int64_t cols) {
+    constexpr int LD = 64 + 32;
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    __shared__ __attribute__((aligned(16))) uint16_t park[4][32 * LD];
+    __shared__ float denom_s;
+    const int64_t bz = blockIdx.z;
+    const float denom = ns_denominator(workspace, bz, IS_BF16, &denom_s);
+    const SharedDivisor divisor(denom, 0.0f);
+    const TIn* src = in + bz * rows * cols;
+    uint16_t* dst = out + bz * rows * cols;
+    const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+    const int64_t r0 = (int64_t)blockIdx.y * 128 + wave * 32, c0 = (int64_t)blockIdx.x * 64;
+    if (r0 >= rows) return;
+    uint16_t* mine = park[wave];
+    const int lr = lane / 8, ch = lane % 8;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int64_t row = r0 + lr + 8 * i, col8 = c0 + ch * 8;
+        uint4 raw = make_uint4(0, 0, 0, 0);
+        if (row < rows && col8 < cols) raw = *reinterpret_cast<const uint4*>(src + row * cols + col8);
+        *reinterpret_cast<uint4*>(&mine[(lr + 8 * i) * LD + ch * 8]) = raw;
+    }
+    const int64_t col = c0 + lane;
+    const int strip = (lane / 16) * 16, sub = lane & 15;
+    const uint16_t* at = &mine[(sub >> 2) * LD + strip + 4 * (sub & 3)];
+    uint32_t o[16];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        const s16x4 four = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at + 4 * t * LD));
+        uint32_t h[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float v = ns_working<TIn, IS_BF16>((uint16_t)four[e]);
+            const bool plain = !(fabsf(v) < INFINITY);
+            h[e] = f32_to_half<IS_BF16>(divisor.fast && !plain ? divisor.quotient(v) : v / denom);
+        }
+        o[2 * t] = h[0] | (h[1] << 16);
+        o[2 * t + 1] = h[2] | (h[3] << 16);
+    }
+    if (col < cols) {
+        uint16_t* row_out = dst + col * rows + r0;
+        if (r0 + 32 <= rows && (reinterpret_cast<uintptr_t>(row_out) & 15) == 0) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) reinterpret_cast<uint4*>(row_out)[k] = make_uint4(o[4 * k], o[4 * k + 1], o[4 * k + 2], o[4 * k + 3]);
+        } else {
+            for (int e = 0; e < 32 && r0 + e < rows; ++e) row_out[e] = (uint16_t)(o[e / 2] >> (16 * (e % 2)));
+        }
+    }
+}
+
 template <bool IS_BF16, bool TRANSPOSE_B, bool VEC>
 static int launch_ns(const void* a, const void* b, const void* residual, void* out, void* out_diag, int epilogue, dim3 grid,
                      int64_t m, int64_t n, int64_t k, float add_diag, int transpose_out, hipStream_t stream) {
@@ -262,6 +406,21 @@ template <typename TIn, bool IS_BF16>
 static int launch_prepare(const void* in, void* out, int64_t batch, int64_t rows, int64_t cols, float* workspace,
                           hipStream_t stream) {
     const TIn* src = static_cast<const TIn*>(in);
+    if constexpr (sizeof(TIn) == 2) {
+        const bool aligned = reinterpret_cast<uintptr_t>(in) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+        if (aligned && cols % 8 == 0 && (rows * cols) % 8 == 0 && (rows + 127) / 128 <= 65535) {
+            hipLaunchKernelGGL((ns_sumsq16_kernel<TIn, IS_BF16>), dim3(PARTS, (unsigned)batch), dim3(256), 0, stream, src, workspace, rows * cols);
+            if (rows > cols) {
+                const dim3 tgrid((unsigned)((cols + 63) / 64), (unsigned)((rows + 127) / 128), (unsigned)batch);
+                hipLaunchKernelGGL((ns_scale16_transposed_kernel<TIn, IS_BF16>), tgrid, dim3(256), 0, stream, src, static_cast<uint16_t*>(out), workspace, rows, cols);
+            } else {
+                const int64_t octets = rows * cols / 8;
+                const unsigned bx = (unsigned)(octets / 256 / 4 < 1 ? 1 : octets / 256 / 4 > 4096 ? 4096 : octets / 256 / 4);
+                hipLaunchKernelGGL((ns_scale16_kernel<TIn, IS_BF16>), dim3(bx, (unsigned)batch), dim3(256), 0, stream, src, static_cast<uint16_t*>(out), workspace, rows * cols);
+            }
+            return viola_launch_status();
+        }
+    }
     hipLaunchKernelGGL((ns_sumsq_kernel<TIn, IS_BF16>), dim3(PARTS, (unsigned)batch), dim3(256), 0, stream, src, workspace, rows * cols);
     const dim3 grid((unsigned)((cols + 31) / 32), (unsigned)((rows + 31) / 32), (unsigned)batch);
     if (rows > cols) hipLaunchKernelGGL((ns_scale_kernel<TIn, IS_BF16, true>), grid, dim3(256), 0, stream, src, static_cast<uint16_t*>(out), workspace, rows, cols);

@@ -39,10 +39,10 @@ template <int EPL, bool STOCHASTIC>   // EPL = tile_size / 64 elements per lane
 __global__ __launch_bounds__(256) void momentum_1d_kernel(const void* __restrict__ grad, int grad_dtype,
                                                            const uint8_t* old_q, const float* old_scale, uint8_t* new_q,
                                                            float* new_scale, uint16_t* __restrict__ update, int64_t n,
-                                                           int64_t blocks, float beta, float inv_loss_scale, int nesterov,
-                                                           uint64_t step, uint64_t key) {
+                                                           int64_t first_block, int64_t blocks, float beta,
+                                                           float inv_loss_scale, int nesterov, uint64_t step, uint64_t key) {
     constexpr int TILE = EPL * WAVE;
-    const int64_t b = (int64_t)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    const int64_t b = first_block + (int64_t)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
     if (b >= blocks) return;
     const int lane = threadIdx.x % WAVE;
     const float scale_old = old_scale[b];
@@ -79,6 +79,93 @@ __global__ __launch_bounds__(256) void momentum_1d_kernel(const void* __restrict
             }
             update[i] = f32_to_bf16_bits(u);
         }
+    }
+}
+
+// Same tile, same arithmetic, four consecutive elements per lane: 16-byte gradient loads, the four state codes as
+// one word through the hardware decoder, 8-byte update stores. Needs the gradient aligned to four elements, the
+// state to 4 bytes and the update to 8 bytes; only whole tiles inside n (the host sends a ragged last tile to the
+// kernel above). The quotient m / scale takes the shared-divisor route when the tile allows it.
+template <typename TG> __device__ __forceinline__ void load_quad(const TG* p, float (&v)[4]);
+template <> __device__ __forceinline__ void load_quad<float>(const float* p, float (&v)[4]) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+template <> __device__ __forceinline__ void load_quad<bf16_t>(const bf16_t* p, float (&v)[4]) {
+    const uint2 t = *reinterpret_cast<const uint2*>(p);
+    v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+    v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+}
+template <> __device__ __forceinline__ void load_quad<f16_t>(const f16_t* p, float (&v)[4]) {
+    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+    const h4 t = *reinterpret_cast<const h4*>(p);
+    v[0] = (float)t[0]; v[1] = (float)t[1]; v[2] = (float)t[2]; v[3] = (float)t[3];
+}
+
+template <typename TG, int EPL, bool STOCHASTIC>
+__global__ __launch_bounds__(256) void momentum_1d_quads(const TG* __restrict__ grad, const uint8_t* old_q,
+                                                          const float* old_scale, uint8_t* new_q, float* new_scale,
+                                                          uint16_t* __restrict__ update, int64_t blocks, float beta,
+                                                          float inv_loss_scale, int nesterov, uint64_t step, uint64_t key) {
+    constexpr int TILE = EPL * WAVE, QUADS = EPL / 4;
+    const int64_t b = (int64_t)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (b >= blocks) return;
+    const int lane = threadIdx.x % WAVE;
+    const float scale_old = old_scale[b];
+    const float one_minus = 1.0f - beta;
+    float g[QUADS][4], m[QUADS][4];
+    float amax = 0.0f, poison = 0.0f;
+#pragma unroll
+    for (int c = 0; c < QUADS; ++c) {
+        const int64_t i = b * TILE + (c * WAVE + lane) * 4;
+        load_quad<TG>(grad + i, g[c]);
+        const int codes = *reinterpret_cast<const int*>(old_q + i);
+        const float m0[4] = {__builtin_amdgcn_cvt_f32_fp8(codes, 0), __builtin_amdgcn_cvt_f32_fp8(codes, 1),
+                             __builtin_amdgcn_cvt_f32_fp8(codes, 2), __builtin_amdgcn_cvt_f32_fp8(codes, 3)};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            g[c][e] = g[c][e] * inv_loss_scale;
+            const float t0 = beta * (m0[e] * scale_old);
+            const float t1 = one_minus * g[c][e];
+            m[c][e] = t0 + t1;
+            amax = fmaxf(amax, fabsf(m[c][e]));
+            poison = poison_of(poison, m[c][e]);
+        }
+    }
+    amax = wave_max(amax);
+    const bool any_bad = __builtin_amdgcn_ballot_w64(poison != poison) != 0;
+    const float scale = fmaxf(amax, 1e-30f) / 448.0f;
+    if (lane == 0) new_scale[b] = scale;
+    const SharedDivisor divisor(scale, any_bad ? __uint_as_float(0x7fc00000u) : 0.0f);
+#pragma unroll
+    for (int c = 0; c < QUADS; ++c) {
+        const int64_t i = b * TILE + (c * WAVE + lane) * 4;
+        uint32_t word;
+        if (divisor.fast) {
+            float t[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                t[e] = __builtin_amdgcn_fmed3f(divisor.quotient(m[c][e]), -448.0f, 448.0f);
+                if (STOCHASTIC) t[e] = stochastic_e4m3(t[e], (uint64_t)(i + e), step, key);
+            }
+            word = hw_encode4<e4m3_t>(t[0], t[1], t[2], t[3]);
+        } else {
+            word = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) word |= (uint32_t)encode_state<STOCHASTIC>(m[c][e], scale, (uint64_t)(i + e), step, key) << (8 * e);
+        }
+        *reinterpret_cast<uint32_t*>(new_q + i) = word;
+        float u[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            u[e] = m[c][e];
+            if (nesterov) {
+                const float t0 = one_minus * g[c][e];
+                const float t1 = beta * m[c][e];
+                u[e] = t0 + t1;
+            }
+        }
+        *reinterpret_cast<uint2*>(update + i) = make_uint2(f32_to_bf16x2_bits(u[0], u[1]), f32_to_bf16x2_bits(u[2], u[3]));
     }
 }
 
@@ -142,6 +229,23 @@ __global__ __launch_bounds__(256) void weight_kernel(void* weight, int weight_dt
         const float t0 = load_dtype(weight, j, weight_dtype) * keep;
         const float t1 = rate * load_dtype(grad, j, grad_dtype);
         store_rounded<STOCHASTIC>(weight, j, weight_dtype, t0 - t1, (uint64_t)j + offset, step, key);
+    }
+}
+
+// fp32 weights, four per thread (16-byte accesses); same arithmetic as weight_kernel. quads = n / 4 whole quads, the
+// host sends the last n % 4 elements through weight_kernel.
+template <typename TG>
+__global__ __launch_bounds__(256) void weight_quads_kernel(float* weight, const TG* __restrict__ grad, int64_t quads, float lr,
+                                                            float decay, float update_scale) {
+    const float keep = 1.0f - lr * decay;
+    const float rate = lr * update_scale;
+    for (int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < quads; j += (int64_t)gridDim.x * blockDim.x) {
+        float4 w = reinterpret_cast<const float4*>(weight)[j];
+        float g[4];
+        load_quad<TG>(grad + 4 * j, g);
+        const float t0[4] = {w.x * keep, w.y * keep, w.z * keep, w.w * keep};
+        const float t1[4] = {rate * g[0], rate * g[1], rate * g[2], rate * g[3]};
+        reinterpret_cast<float4*>(weight)[j] = make_float4(t0[0] - t1[0], t0[1] - t1[1], t0[2] - t1[2], t0[3] - t1[3]);
     }
 }
 
@@ -222,14 +326,37 @@ extern "C" int viola_momentum_update(const void* grad, int grad_dtype, const voi
     if (granularity == 0) {
         VIOLA_CHECK_ARG(tile_size == 64 || tile_size == 128 || tile_size == 256 || tile_size == 512 || tile_size == 1024);
         const int64_t blocks = (n + tile_size - 1) / tile_size;
-        const dim3 grid((unsigned)((blocks + 3) / 4));
+        // whole tiles go four elements per lane when the pointers allow it; the ragged last tile (and everything,
+        // for small tiles or odd alignment) one element per lane
+        const int64_t whole = n / tile_size;
+        const size_t grad_bytes = grad_dtype == VIOLA_F32 ? 4 : 2;
+        const bool quads = tile_size >= 256 && whole > 0 && reinterpret_cast<uintptr_t>(grad) % (4 * grad_bytes) == 0 &&
+                           reinterpret_cast<uintptr_t>(old_q) % 4 == 0 && reinterpret_cast<uintptr_t>(new_q) % 4 == 0 &&
+                           reinterpret_cast<uintptr_t>(update) % 8 == 0;
+        const int64_t first = quads ? whole : 0;
+        if (quads) {
+            const dim3 qgrid((unsigned)((whole + 3) / 4));
+#define VIOLA_MQ(TG, EPL)                                                                                                   \
+    if (rounding) hipLaunchKernelGGL((momentum_1d_quads<TG, EPL, true>), qgrid, dim3(256), 0, stream, static_cast<const TG*>(grad), oq, old_scale, nq, new_scale, up, whole, beta, inv_loss_scale, nesterov, step, key); \
+    else hipLaunchKernelGGL((momentum_1d_quads<TG, EPL, false>), qgrid, dim3(256), 0, stream, static_cast<const TG*>(grad), oq, old_scale, nq, new_scale, up, whole, beta, inv_loss_scale, nesterov, step, key);
+#define VIOLA_MQT(EPL)                                                          \
+    if (grad_dtype == VIOLA_F32) { VIOLA_MQ(float, EPL) }                        \
+    else if (grad_dtype == VIOLA_BF16) { VIOLA_MQ(bf16_t, EPL) }                 \
+    else { VIOLA_MQ(f16_t, EPL) }
+            if (tile_size == 256) { VIOLA_MQT(4) } else if (tile_size == 512) { VIOLA_MQT(8) } else { VIOLA_MQT(16) }
+#undef VIOLA_MQT
+#undef VIOLA_MQ
+        }
+        if (first < blocks) {
+            const dim3 grid((unsigned)((blocks - first + 3) / 4));
 #define VIOLA_M1(EPL)                                                                                                        \
     case EPL * 64:                                                                                                           \
-        if (rounding) hipLaunchKernelGGL((momentum_1d_kernel<EPL, true>), grid, dim3(256), 0, stream, grad, grad_dtype, oq, old_scale, nq, new_scale, up, n, blocks, beta, inv_loss_scale, nesterov, step, key); \
-        else hipLaunchKernelGGL((momentum_1d_kernel<EPL, false>), grid, dim3(256), 0, stream, grad, grad_dtype, oq, old_scale, nq, new_scale, up, n, blocks, beta, inv_loss_scale, nesterov, step, key); \
+        if (rounding) hipLaunchKernelGGL((momentum_1d_kernel<EPL, true>), grid, dim3(256), 0, stream, grad, grad_dtype, oq, old_scale, nq, new_scale, up, n, first, blocks, beta, inv_loss_scale, nesterov, step, key); \
+        else hipLaunchKernelGGL((momentum_1d_kernel<EPL, false>), grid, dim3(256), 0, stream, grad, grad_dtype, oq, old_scale, nq, new_scale, up, n, first, blocks, beta, inv_loss_scale, nesterov, step, key); \
         break;
-        switch (tile_size) { VIOLA_M1(1) VIOLA_M1(2) VIOLA_M1(4) VIOLA_M1(8) VIOLA_M1(16) }
+            switch (tile_size) { VIOLA_M1(1) VIOLA_M1(2) VIOLA_M1(4) VIOLA_M1(8) VIOLA_M1(16) }
 #undef VIOLA_M1
+        }
         return viola_launch_status();
     }
     VIOLA_CHECK_ARG(planes > 0 && rows > 0 && cols > 0 && planes * rows * cols == n && tr > 0 && tc > 0 && tr * tc <= 4096);
@@ -247,6 +374,19 @@ extern "C" int viola_weight_update(void* weight, int weight_dtype, const void* g
     VIOLA_CHECK_ARG(viola_is_float(weight_dtype) && viola_is_float(grad_dtype) && n >= 0);
     if (n == 0) return 0;
     VIOLA_CHECK_ARG(weight && grad);
+    const size_t grad_bytes = grad_dtype == VIOLA_F32 ? 4 : 2;
+    if (weight_dtype == VIOLA_F32 && n >= 4 && reinterpret_cast<uintptr_t>(weight) % 16 == 0 &&
+        reinterpret_cast<uintptr_t>(grad) % (4 * grad_bytes) == 0) {
+        const int64_t quads = n / 4, rest = n % 4;
+        float* wp = static_cast<float*>(weight);
+        if (grad_dtype == VIOLA_F32) hipLaunchKernelGGL(weight_quads_kernel<float>, dim3(grid_for(quads)), dim3(256), 0, stream, wp, static_cast<const float*>(grad), quads, lr, decay, update_scale);
+        else if (grad_dtype == VIOLA_BF16) hipLaunchKernelGGL(weight_quads_kernel<bf16_t>, dim3(grid_for(quads)), dim3(256), 0, stream, wp, static_cast<const bf16_t*>(grad), quads, lr, decay, update_scale);
+        else hipLaunchKernelGGL(weight_quads_kernel<f16_t>, dim3(grid_for(quads)), dim3(256), 0, stream, wp, static_cast<const f16_t*>(grad), quads, lr, decay, update_scale);
+        if (rest)
+            hipLaunchKernelGGL(weight_kernel<false>, dim3(1), dim3(256), 0, stream, wp + 4 * quads, weight_dtype,
+                               static_cast<const uint8_t*>(grad) + 4 * quads * grad_bytes, grad_dtype, rest, lr, decay, update_scale, 0ull, 0ull, 0ull);
+        return viola_launch_status();
+    }
     if (rounding && weight_dtype != VIOLA_F32)
         hipLaunchKernelGGL(weight_kernel<true>, dim3(grid_for(n)), dim3(256), 0, stream, weight, weight_dtype, grad, grad_dtype, n, lr, decay, update_scale, (uint64_t)rounding_step, (uint64_t)rounding_key, (uint64_t)offset);
     else
