@@ -210,6 +210,53 @@ __global__ __launch_bounds__(256, 2) void ns_gemm_fast(NsArgs p) {
     const uint16_t* residual = EPILOGUE ? p.residual + bz * m * n : nullptr;
     uint16_t* out = p.out + bz * m * n;
     uint16_t* out_diag = p.out_diag ? p.out_diag + bz * m * n : nullptr;
+    if (!p.transpose_out && !mirror) {
+        // Row-major output: the accumulators hold one row per lane in runs of four columns, which as stores would touch
+        // 32 cache lines per instruction. Each wavefront instead parks its rounded products, 32 rows at a time, in LDS
+        // (the stage ring is free now) and picks them up as 16-byte pieces along the rows, so that the residual loads,
+        // the epilogue arithmetic and the stores all run on 8 consecutive columns of one row.
+        constexpr int WCOLS = 32 * WN, PLD = WCOLS + 8, PIECES = WCOLS / 8;   // parked row: 16 bytes of padding
+        static_assert(4 * 32 * PLD * 2 <= (int)sizeof(lds), "parking area fits in the stage ring");
+        __syncthreads();                                                  // every wave has left the ring
+        uint16_t* park = lds + wave * 32 * PLD;
+#pragma unroll
+        for (int j = 0; j < WM; ++j) {
+#pragma unroll
+            for (int i = 0; i < WN; ++i)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    uint32_t h[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) h[e] = ns_narrow<IS_BF16>(acc[i][j][r4 * 4 + e]);
+                    *reinterpret_cast<uint2*>(&park[l32 * PLD + i * 32 + r4 * 8 + lhi * 4]) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+                }
+#pragma unroll
+            for (int it = 0; it < 32 * PIECES / WAVE; ++it) {
+                const int id = it * WAVE + lane, pr = id / PIECES, pc = id % PIECES;
+                const int64_t row = m0 + wm * 32 * WM + j * 32 + pr, col = n0 + wn * WCOLS + pc * 8;
+                const uint4 raw = *reinterpret_cast<const uint4*>(&park[pr * PLD + pc * 8]);
+                if (row >= m || col >= n) continue;                       // n is a multiple of 8: whole pieces
+                uint4 res = make_uint4(0, 0, 0, 0);
+                if (EPILOGUE) res = *reinterpret_cast<const uint4*>(residual + row * n + col);
+                const uint32_t pw[4] = {raw.x, raw.y, raw.z, raw.w}, rw[4] = {res.x, res.y, res.z, res.w};
+                uint32_t o[4], od[4];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    float value = ns_widen<IS_BF16>((uint16_t)(pw[e / 2] >> (16 * (e % 2))));
+                    const float r = ns_widen<IS_BF16>((uint16_t)(rw[e / 2] >> (16 * (e % 2))));
+                    if (EPILOGUE == 1) value = -4.7750f * r + 2.0315f * value;
+                    if (EPILOGUE == 2) value = value + 3.4445f * r;
+                    const uint32_t bits = ns_narrow<IS_BF16>(value);
+                    const uint32_t dbits = col + e == row ? ns_narrow<IS_BF16>(ns_widen<IS_BF16>((uint16_t)bits) + p.add_diag) : bits;
+                    if (e % 2 == 0) { o[e / 2] = bits; od[e / 2] = dbits; }
+                    else { o[e / 2] |= bits << 16; od[e / 2] |= dbits << 16; }
+                }
+                *reinterpret_cast<uint4*>(out + row * n + col) = make_uint4(o[0], o[1], o[2], o[3]);
+                if (out_diag) *reinterpret_cast<uint4*>(out_diag + row * n + col) = make_uint4(od[0], od[1], od[2], od[3]);
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < WM; ++j) {
         const int64_t row = m0 + wm * 32 * WM + j * 32 + l32;
