@@ -389,6 +389,50 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
     TO* out = reinterpret_cast<TO*>(outptr);
     const bool vec_out = p.ldo % 4 == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
     const bool vec_aux = p.n % 4 == 0 && (reinterpret_cast<uintptr_t>(p.aux) & 15) == 0;
+    if constexpr (MODE == MODE_PLAIN) {
+        // Row-major output: as stores, "one row per lane, four columns" would touch 32 cache lines per instruction. When
+        // rows of out are 16-byte aligned, each wavefront parks its finished values, 32 rows at a time, in LDS (the
+        // stage ring is free now) and stores them as 16-byte pieces along the rows instead.
+        constexpr int PER = 16 / (int)sizeof(TO);                            // values per piece
+        constexpr int WCOLS = 32 * TN, PLD = WCOLS + PER, PIECES = WCOLS / PER;
+        static_assert(4 * 32 * PLD * (int)sizeof(TO) <= F_RAW, "parking area fits in the stage ring");
+        if ((p.ldo * sizeof(TO)) % 16 == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+            __syncthreads();                                                 // every wave has left the ring
+            TO* park = reinterpret_cast<TO*>(lds) + wave * 32 * PLD;
+            const int64_t ncol0 = n_begin + wn * WCOLS;
+#pragma unroll
+            for (int j = 0; j < TM; ++j) {
+#pragma unroll
+                for (int i = 0; i < TN; ++i)
+#pragma unroll
+                    for (int r4 = 0; r4 < 4; ++r4) {
+                        float v[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            v[e] = total[i][j][r4 * 4 + e];
+                            const int64_t ncol = ncol0 + i * 32 + r4 * 8 + lhi * 4 + e;
+                            if (p.bias && ncol < p.n) v[e] += load_bias(p.bias, ncol, bias_dtype);
+                        }
+                        Quad<TO>::store(&park[l32 * PLD + i * 32 + r4 * 8 + lhi * 4], v);
+                    }
+#pragma unroll
+                for (int it = 0; it < 32 * PIECES / WAVE; ++it) {
+                    const int id = it * WAVE + lane, pr = id / PIECES, pc = id % PIECES;
+                    const int64_t mrow = m_begin + a_sub(j) + pr, ncol = ncol0 + pc * PER;
+                    const uint4 piece = *reinterpret_cast<const uint4*>(&park[pr * PLD + pc * PER]);
+                    if (mrow >= m_end || ncol >= p.n) continue;
+                    if (ncol + PER <= p.n) {
+                        *reinterpret_cast<uint4*>(out + mrow * p.ldo + ncol) = piece;
+                    } else {
+                        const TO* values = reinterpret_cast<const TO*>(&piece);
+                        for (int e = 0; e < PER; ++e)
+                            if (ncol + e < p.n) out[mrow * p.ldo + ncol + e] = values[e];
+                    }
+                }
+            }
+            return;
+        }
+    }
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
         const int64_t mrow = m_begin + a_sub(j) + l32;
