@@ -228,71 +228,126 @@ __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x
     constexpr int LD = 64 + 32;
     typedef short s16x4 __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     __shared__ __attribute__((aligned(16))) uint16_t park[4][32 * LD];
     const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
-    const int64_t r0 = (int64_t)blockIdx.y * 128 + wave * 32, c0 = (int64_t)blockIdx.x * 64;
-    if (r0 >= rows) return;                                                  // whole wavefront leaves together
     uint16_t* mine = park[wave];
     const int lr = lane / 8, ch = lane % 8;
     const int64_t nc = (cols + 31) / 32;
+    // a block walks tiles of 128 rows x 64 columns (column tiles fastest) with the grid's stride: the wavefronts stay
+    // resident, so the SIMDs keep several of them in flight instead of waiting for new workgroups to be dispatched
+    const int64_t tiles_x = (cols + 63) / 64, tiles = tiles_x * ((rows + 127) / 128);
+    for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+    const int64_t r0 = tile / tiles_x * 128 + wave * 32, c0 = tile % tiles_x * 64;
+    if (r0 >= rows) continue;                                                // whole wavefront skips together
     const int64_t col8 = c0 + ch * 8;
+
+    // all four loads first, without control flow: a raw buffer over the wavefront's 32 rows returns zero past its end
+    const int64_t span = (rows - r0 < 32 ? rows - r0 : 32) * cols * 2;
+    const __amdgpu_buffer_rsrc_t res = __builtin_amdgcn_make_buffer_rsrc(const_cast<TIn*>(x + r0 * cols), 0, (int)span, 0x00020000);
+    u32x4 raw[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int64_t row = r0 + lr + 8 * i;
-        const bool inside = row < rows && col8 < cols;                       // cols is a multiple of 8
-        uint4 raw = make_uint4(0, 0, 0, 0);
-        if (inside) raw = *reinterpret_cast<const uint4*>(x + row * cols + col8);
-        *reinterpret_cast<uint4*>(&mine[(lr + 8 * i) * LD + ch * 8]) = raw;
-        if constexpr (ROWWISE) {
-            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-            float v[8];
+    for (int i = 0; i < 4; ++i)
+        raw[i] = __builtin_amdgcn_raw_buffer_load_b128(res, col8 < cols ? (int)(((lr + 8 * i) * cols + col8) * 2) : (int)0x80000000u, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(&mine[(lr + 8 * i) * LD + ch * 8]) = raw[i];
+
+    // row-wise groups: four lanes x 8 values
+    float vr[4][8], s_row[4];
+    bool fast = true;
+    SharedDivisor d_row[4] = {SharedDivisor(1.0f, 0.0f), SharedDivisor(1.0f, 0.0f), SharedDivisor(1.0f, 0.0f), SharedDivisor(1.0f, 0.0f)};
+    if constexpr (ROWWISE) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
             float amax = 0.0f, poison = 0.0f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                v[e] = widen16<TIn>(e % 2 ? w[e / 2] >> 16 : w[e / 2] & 0xffffu);
-                amax = fmaxf(amax, fabsf(v[e]));
-                poison = poison_of(poison, v[e]);
+                vr[i][e] = widen16<TIn>(e % 2 ? raw[i][e / 2] >> 16 : raw[i][e / 2] & 0xffffu);
+                amax = fmaxf(amax, fabsf(vr[i][e]));
+                poison = poison_of(poison, vr[i][e]);
             }
             amax = group_max<4>(amax);
             poison += __shfl_xor(poison, 1, WAVE);
             poison += __shfl_xor(poison, 2, WAVE);
-            const float s = group_scale(amax, limit);
-            const SharedDivisor divisor(s, poison);
-            if (inside) {
-                *reinterpret_cast<uint2*>(q + row * cols + col8) = encode8<TOut>(v, s, limit, divisor);
-                if (ch % 4 == 0) scale[row * nc + col8 / 32] = s;
-            }
+            s_row[i] = group_scale(amax, limit);
+            d_row[i] = SharedDivisor(s_row[i], poison);
+            fast = fast && d_row[i].fast;
         }
     }
-    // column lane % 16 of the 16-column strip lane / 16: rows 4t .. 4t+3 per read
+    // transposed groups: column lane % 16 of the 16-column strip lane / 16, rows 4t .. 4t+3 per read
     const int64_t col = c0 + lane;
     const int strip = (lane / 16) * 16, sub = lane & 15;
     const uint16_t* at = &mine[(sub >> 2) * LD + strip + 4 * (sub & 3)];
-    float v[32];
+    float vc[32];
     float amax = 0.0f, poison = 0.0f;
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
         const s16x4 four = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at + 4 * t * LD));
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            v[4 * t + e] = widen16<TIn>((uint16_t)four[e]);
-            amax = fmaxf(amax, fabsf(v[4 * t + e]));
-            poison = poison_of(poison, v[4 * t + e]);
+            vc[4 * t + e] = widen16<TIn>((uint16_t)four[e]);
+            amax = fmaxf(amax, fabsf(vc[4 * t + e]));
+            poison = poison_of(poison, vc[4 * t + e]);
+        }
+    }
+    const float s_col = group_scale(amax, limit);
+    const SharedDivisor d_col(s_col, poison);
+    fast = fast && d_col.fast;
+
+    // one decision per wavefront: the common case runs without a single divergent branch
+    uint2 row_codes[4];
+    uint32_t col_codes[8];
+    if (__builtin_amdgcn_ballot_w64(!fast) == 0) {
+        if constexpr (ROWWISE) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                row_codes[i] = make_uint2(fast_encode4<TOut>(d_row[i], limit, vr[i][0], vr[i][1], vr[i][2], vr[i][3]),
+                                          fast_encode4<TOut>(d_row[i], limit, vr[i][4], vr[i][5], vr[i][6], vr[i][7]));
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) col_codes[k] = fast_encode4<TOut>(d_col, limit, vc[4 * k], vc[4 * k + 1], vc[4 * k + 2], vc[4 * k + 3]);
+    } else {
+        const SharedDivisor exact(1.0f, __uint_as_float(0x7fc00000u));       // fast == false: true division, software encoder
+        if constexpr (ROWWISE) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) row_codes[i] = encode8<TOut>(vr[i], s_row[i], limit, exact);
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            col_codes[k] = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) col_codes[k] |= (uint32_t)encode_clamped<TOut>(vc[4 * k + e], s_col, limit) << (8 * e);
+        }
+    }
+
+    if constexpr (ROWWISE) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int64_t row = r0 + lr + 8 * i;
+            if (row < rows && col8 < cols) {
+                *reinterpret_cast<uint2*>(q + row * cols + col8) = row_codes[i];
+                if (ch % 4 == 0) scale[row * nc + col8 / 32] = s_row[i];
+            }
         }
     }
     if (col < cols) {
-        const float s = group_scale(amax, limit);
         const int64_t nr = (rows + 31) / 32;
-        scale_t[col * nr + r0 / 32] = s;
+        scale_t[col * nr + r0 / 32] = s_col;
         if (column_partial) {
             float sum = 0.0f;
 #pragma unroll
-            for (int i = 0; i < 32; ++i) sum += v[i];
+            for (int i = 0; i < 32; ++i) sum += vc[i];
             column_partial[(r0 / 32) * cols + col] = sum;
         }
-        const int count = (int)(rows - r0 < 32 ? rows - r0 : 32);
         uint8_t* dst = qt + col * rows + r0;
-        store_group32<TOut>(v, s, poison, limit, dst, count, (reinterpret_cast<uintptr_t>(dst) & 15) == 0);
+        if (rows - r0 >= 32 && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+            reinterpret_cast<uint4*>(dst)[0] = make_uint4(col_codes[0], col_codes[1], col_codes[2], col_codes[3]);
+            reinterpret_cast<uint4*>(dst)[1] = make_uint4(col_codes[4], col_codes[5], col_codes[6], col_codes[7]);
+        } else {
+            const int count = (int)(rows - r0 < 32 ? rows - r0 : 32);
+            for (int i = 0; i < count; ++i) dst[i] = (uint8_t)(col_codes[i >> 2] >> (8 * (i & 3)));
+        }
+    }
     }
 }
 
@@ -478,7 +533,8 @@ static int launch_quantize(const void* x, int64_t rows, int64_t cols, void* q, f
     }
     if constexpr (sizeof(TIn) == 2) {
         if (gr == 1 && gc == 32 && transposed && vec) {
-            const dim3 grid16((unsigned)((cols + 63) / 64), (unsigned)((rows + 127) / 128));
+            const int64_t tiles16 = ((cols + 63) / 64) * ((rows + 127) / 128);
+            const dim3 grid16((unsigned)(tiles16 < 256 * 6 ? tiles16 : 256 * 6));
             hipLaunchKernelGGL((quantize_dual16<TIn, TOut, false>), grid16, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit, nullptr);
             return viola_launch_status();
         }
@@ -526,7 +582,8 @@ static int launch_dual(const void* x, int64_t rows, int64_t cols, void* q, float
     const TIn* xp = static_cast<const TIn*>(x);
     if constexpr (sizeof(TIn) == 2) {
         if (vec && reinterpret_cast<uintptr_t>(q) % 8 == 0) {
-            const dim3 grid16((unsigned)((cols + 63) / 64), (unsigned)((rows + 127) / 128));
+            const int64_t tiles16 = ((cols + 63) / 64) * ((rows + 127) / 128);
+            const dim3 grid16((unsigned)(tiles16 < 256 * 6 ? tiles16 : 256 * 6));
             hipLaunchKernelGGL((quantize_dual16<TIn, TOut, true>), grid16, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale,
                                static_cast<uint8_t*>(qt), scale_t, rows, cols, limit, column_partial);
             return viola_launch_status();
