@@ -400,6 +400,22 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
             __syncthreads();                                                 // every wave has left the ring
             TO* park = reinterpret_cast<TO*>(lds) + wave * 32 * PLD;
             const int64_t ncol0 = n_begin + wn * WCOLS;
+            // the tile's bias as fp32 in the (now idle) raw scale area: one global load per column, not per element
+            float4 bias_q[TN][4];
+            if (p.bias) {
+                float* bias_lds = reinterpret_cast<float*>(lds + F_RAW);
+                if (tid < 64 * TN) bias_lds[tid] = n_begin + tid < p.n ? load_bias(p.bias, n_begin + tid, bias_dtype) : 0.0f;
+                __syncthreads();
+#pragma unroll
+                for (int i = 0; i < TN; ++i)
+#pragma unroll
+                    for (int r4 = 0; r4 < 4; ++r4) bias_q[i][r4] = *reinterpret_cast<const float4*>(&bias_lds[wn * WCOLS + i * 32 + r4 * 8 + lhi * 4]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < TN; ++i)
+#pragma unroll
+                    for (int r4 = 0; r4 < 4; ++r4) bias_q[i][r4] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            }
 #pragma unroll
             for (int j = 0; j < TM; ++j) {
 #pragma unroll
@@ -407,12 +423,9 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
 #pragma unroll
                     for (int r4 = 0; r4 < 4; ++r4) {
                         float v[4];
+                        const float bq[4] = {bias_q[i][r4].x, bias_q[i][r4].y, bias_q[i][r4].z, bias_q[i][r4].w};
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            v[e] = total[i][j][r4 * 4 + e];
-                            const int64_t ncol = ncol0 + i * 32 + r4 * 8 + lhi * 4 + e;
-                            if (p.bias && ncol < p.n) v[e] += load_bias(p.bias, ncol, bias_dtype);
-                        }
+                        for (int e = 0; e < 4; ++e) v[e] = total[i][j][r4 * 4 + e] + bq[e];
                         Quad<TO>::store(&park[l32 * PLD + i * 32 + r4 * 8 + lhi * 4], v);
                     }
 #pragma unroll
