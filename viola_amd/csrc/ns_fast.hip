@@ -1,16 +1,17 @@
 // Tiled Newton-Schulz GEMM for gfx950: batched out[b] = a[b] . b[b]^T (b as [n, k]) or a[b] . b[b] (b as
 // [k, n]) in bf16 / fp16 on v_mfma_f32_32x32x16, fp32 accumulation, with the chain's epilogues.
 //
-// Block: 256 threads = 2 x 2 wavefronts, each owning WM x WN accumulators of 32 x 32 (192 x 192 tiles
-// for the 1152-multiples of transformer blocks, 128 x 128 otherwise), two blocks per CU so one block's
-// barrier and LDS traffic hide behind the other's MFMAs.
+// Block: WAVES_M x WAVES_N wavefronts, each owning WM x WN accumulators of 32 x 32. Three shapes are built:
+// 2 x 2 waves of 3 x 3 (192 x 192 tiles for the 1152-multiples of transformer blocks) or of 2 x 2 (128 x 128), two
+// blocks per CU so one block's barrier and LDS traffic hide behind the other's MFMAs; and 4 x 2 waves of 3 x 3
+// (384 x 192, 64 k per stage, one block per CU) for large non-symmetric products.
 //   * global -> LDS directly (buffer_load_dwordx4 ... lds: no staging registers, no ds_write; lanes
-//     past the matrix read zero, so there are no tail branches), 32 k per stage, a ring of three
-//     stages: the loads of chunk c+2 are in flight during the math of chunk c, one barrier per chunk.
+//     past the matrix read zero, so there are no tail branches), a ring of STAGES stages of SBK k: the
+//     loads of the next STAGES - 1 chunks are in flight during the math of a chunk, one barrier per chunk.
 //     A direct load puts lane l's 16 bytes at base + 16 l, so the tile layout is chosen on the global
 //     side: which (row, k piece) a lane fetches.
-//   * k-contiguous operands ([m, k] and [n, k]) are rows of 4 x 16 bytes with piece c of row r stored in
-//     slot c ^ ((r >> 2) & 3): the 16 rows a ds_read_b128 group touches fall in 16 different bank
+//   * k-contiguous operands ([m, k] and [n, k]) are rows of 4 (or 8) x 16 bytes with piece c of row r stored in
+//     slot c ^ ((r >> 2) & 3) (or c ^ ((r >> 1) & 7)): the 16 rows a ds_read_b128 group touches fall in 16 different bank
 //     groups. An [k, n] operand keeps its layout (rows of BN elements, 16-byte units XOR-swizzled by
 //     the row so four consecutive k rows start 64 bytes apart in bank space) and is transposed on the
 //     way out of LDS by ds_read_b64_tr_b16, which hands lane i of each 16-lane group the four k values
@@ -32,8 +33,6 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 
-constexpr int SBK = 32;             // k per LDS stage
-constexpr int STAGES = 3;
 constexpr uint32_t NS_OUTSIDE = 0x80000000u;
 
 template <bool IS_BF16>
@@ -64,12 +63,23 @@ __device__ __forceinline__ i32x4 make_rsrc(const void* base) {
     return r;
 }
 
-template <bool IS_BF16, bool B_KN, int EPILOGUE, int WM, int WN>
-__global__ __launch_bounds__(256, 2) void ns_gemm_fast(NsArgs p) {
-    constexpr int BM = 64 * WM, BN = 64 * WN;
+// Shape: WAVES_M x WAVES_N wavefronts of WM x WN accumulators; SBK k per stage, STAGES stages (loads run
+// STAGES - 1 chunks ahead). Small: 2 x 2 waves, 32 k, 3 stages, two blocks per CU. Big: 4 x 2 waves of 3 x 3
+// (384 x 192), 64 k (whole 128-byte lines per row and load), 2 stages, one block per CU.
+template <int WAVES_M, int WAVES_N> struct NsThreads { static constexpr int value = 64 * WAVES_M * WAVES_N; };
+
+template <bool IS_BF16, bool B_KN, int EPILOGUE, int WM, int WN, int WAVES_M, int WAVES_N, int SBK, int STAGES>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void ns_gemm_fast(NsArgs p) {
+    constexpr int THREADS = 64 * WAVES_M * WAVES_N;
+    constexpr int BM = 32 * WM * WAVES_M, BN = 32 * WN * WAVES_N;
     constexpr int A_EL = BM * SBK, B_EL = BN * SBK, STAGE_EL = A_EL + B_EL;
     constexpr int NCH = BN / 8;                                      // 16-byte units per [k, n] row
+    constexpr int UPR = SBK / 8;                                     // 16-byte units per k-contiguous row
+    constexpr int A_LOADS = BM * UPR / THREADS, B_LOADS = BN * UPR / THREADS;   // = SBK * NCH / THREADS for [k, n]
+    static_assert(BM * UPR % THREADS == 0 && BN * UPR % THREADS == 0, "whole load instructions");
     __shared__ __attribute__((aligned(1024))) uint16_t lds[STAGES * STAGE_EL];
+    // slot of piece c in row r: c ^ swz(r); 16 consecutive rows reading the same piece then cover all 16 bank groups
+    auto swz = [](int r) -> int { return UPR == 4 ? (r >> 2) & 3 : (r >> 1) & 7; };
 
     const int64_t per_xcd = (p.tiles + 7) / 8;
     const int64_t seq = blockIdx.x / 8;
@@ -101,25 +111,25 @@ __global__ __launch_bounds__(256, 2) void ns_gemm_fast(NsArgs p) {
 
     const int tid = threadIdx.x, lane = tid % WAVE;
     const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
-    const int wm = wave / 2, wn = wave % 2, l32 = lane % 32, lhi = lane / 32;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N, l32 = lane % 32, lhi = lane / 32;
 
     const i32x4 res_a = make_rsrc(p.a + bz * m * k);
     const i32x4 res_b = make_rsrc(p.b + bz * n * k);
 
-    // Load plan: instruction `it` of this wave fills LDS units (16 bytes) [it * 256 + wave * 64, +64);
+    // Load plan: instruction `it` of this wave fills LDS units (16 bytes) [it * THREADS + wave * 64, +64);
     // per thread: the global byte offset (k0 = 0) of the piece that belongs in its unit, and its k position.
-    uint32_t a_off[WM], b_off[WN];
-    int a_k[WM], b_k[WN];
+    uint32_t a_off[A_LOADS], b_off[B_LOADS];
+    int a_k[A_LOADS], b_k[B_LOADS];
 #pragma unroll
-    for (int it = 0; it < WM; ++it) {
-        const int u = it * 256 + tid, lr = u >> 2, c = (u & 3) ^ ((lr >> 2) & 3);
+    for (int it = 0; it < A_LOADS; ++it) {
+        const int u = it * THREADS + tid, lr = u / UPR, c = (u % UPR) ^ swz(lr);
         const int64_t row = m0 + lr;
         a_off[it] = row < m ? (uint32_t)((row * k + c * 8) * 2) : NS_OUTSIDE;
         a_k[it] = c * 8;
     }
 #pragma unroll
-    for (int it = 0; it < WN; ++it) {
-        const int u = it * 256 + tid;
+    for (int it = 0; it < B_LOADS; ++it) {
+        const int u = it * THREADS + tid;
         if constexpr (B_KN) {
             const int kr = u / NCH, pos = u % NCH;
             const int unit = pos ^ (BN % 128 == 0 ? (kr & 3) * 4 : ((kr >> 1) & 1) * 4);
@@ -127,7 +137,7 @@ __global__ __launch_bounds__(256, 2) void ns_gemm_fast(NsArgs p) {
             b_off[it] = col < n ? (uint32_t)(((int64_t)kr * n + col) * 2) : NS_OUTSIDE;
             b_k[it] = kr;
         } else {
-            const int lr = u >> 2, c = (u & 3) ^ ((lr >> 2) & 3);
+            const int lr = u / UPR, c = (u % UPR) ^ swz(lr);
             const int64_t row = n0 + lr;
             b_off[it] = row < n ? (uint32_t)((row * k + c * 8) * 2) : NS_OUTSIDE;
             b_k[it] = c * 8;
@@ -140,15 +150,15 @@ __global__ __launch_bounds__(256, 2) void ns_gemm_fast(NsArgs p) {
         const uint32_t b_step = B_KN ? (uint32_t)(k0 * n * 2) : (uint32_t)(k0 * 2);
         const uint32_t base = lds_base + (uint32_t)stage * STAGE_EL * 2 + wave_units;
 #pragma unroll
-        for (int it = 0; it < WM; ++it)
-            load_to_lds(res_a, base + it * 4096, k0 + a_k[it] < k ? a_off[it] : NS_OUTSIDE, a_step);
+        for (int it = 0; it < A_LOADS; ++it)
+            load_to_lds(res_a, base + it * THREADS * 16, k0 + a_k[it] < k ? a_off[it] : NS_OUTSIDE, a_step);
 #pragma unroll
-        for (int it = 0; it < WN; ++it)
-            load_to_lds(res_b, base + A_EL * 2 + it * 4096, k0 + b_k[it] < k ? b_off[it] : NS_OUTSIDE, b_step);
+        for (int it = 0; it < B_LOADS; ++it)
+            load_to_lds(res_b, base + A_EL * 2 + it * THREADS * 16, k0 + b_k[it] < k ? b_off[it] : NS_OUTSIDE, b_step);
     };
 
     // fragment addresses (elements) inside a stage
-    const int sw = (l32 >> 2) & 3;
+    const int sw = swz(l32);
     const int a_frag = (wm * 32 * WM + l32) * SBK + ((lhi ^ sw) * 8);                  // k half ks: ^ (ks * 16)
     const int kn_row = lhi * 8 + ((lane & 15) >> 2);                                   // + ks * 16 (+ 4 for the upper half)
     const int kn_unit = (wn * 4 * WN + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1)) ^ (BN % 128 == 0 ? (kn_row & 3) * 4 : ((kn_row >> 1) & 1) * 4);
@@ -193,14 +203,15 @@ __global__ __launch_bounds__(256, 2) void ns_gemm_fast(NsArgs p) {
     };
 
     const int64_t chunks = (k + SBK - 1) / SBK;
-    issue(0, 0);
-    issue(SBK, 1);
-    int cur = 0, fill = 2;
+    constexpr int AHEAD = STAGES - 1;                                   // chunks in flight beyond the one being multiplied
+#pragma unroll
+    for (int c = 0; c < AHEAD; ++c) issue((int64_t)c * SBK, c);
+    int cur = 0, fill = AHEAD;
     for (int64_t c = 0; c < chunks; ++c) {
-        // all loads but the newest chunk's have landed: chunk c is in LDS for this wave ...
-        __builtin_amdgcn_s_waitcnt(0x0F70 | (WM + WN));
+        // all loads but those of the newest AHEAD - 1 chunks have landed: chunk c is in LDS for this wave ...
+        __builtin_amdgcn_s_waitcnt(0x0F70 | ((AHEAD - 1) * (A_LOADS + B_LOADS)));
         __syncthreads();                    // ... and for every wave; stage `fill` was last read in chunk c-1
-        issue((c + 2) * SBK, fill);         // past the end: zeros into a stage nobody reads
+        issue((c + AHEAD) * SBK, fill);     // past the end: zeros into a stage nobody reads
         compute(lds + cur * STAGE_EL);
         cur = cur == STAGES - 1 ? 0 : cur + 1;
         fill = fill == STAGES - 1 ? 0 : fill + 1;
@@ -216,7 +227,7 @@ __global__ __launch_bounds__(256, 2) void ns_gemm_fast(NsArgs p) {
         // (the stage ring is free now) and picks them up as 16-byte pieces along the rows, so that the residual loads,
         // the epilogue arithmetic and the stores all run on 8 consecutive columns of one row.
         constexpr int WCOLS = 32 * WN, PLD = WCOLS + 8, PIECES = WCOLS / 8;   // parked row: 16 bytes of padding
-        static_assert(4 * 32 * PLD * 2 <= (int)sizeof(lds), "parking area fits in the stage ring");
+        static_assert(WAVES_M * WAVES_N * 32 * PLD * 2 <= (int)sizeof(lds), "parking area fits in the stage ring");
         __syncthreads();                                                  // every wave has left the ring
         uint16_t* park = lds + wave * 32 * PLD;
 #pragma unroll
@@ -299,25 +310,31 @@ __global__ __launch_bounds__(256, 2) void ns_gemm_fast(NsArgs p) {
     }
 }
 
-template <bool IS_BF16, bool B_KN, int WM, int WN>
+template <bool IS_BF16, bool B_KN, int WM, int WN, int WAVES_M, int WAVES_N, int SBK, int STAGES>
 static void launch_tiles(NsArgs p, int epilogue, hipStream_t stream) {
-    constexpr int BM = 64 * WM, BN = 64 * WN;
+    constexpr int BM = 32 * WM * WAVES_M, BN = 32 * WN * WAVES_N, THREADS = 64 * WAVES_M * WAVES_N;
     p.tiles_m = (int)((p.m + BM - 1) / BM);
     p.tiles_n = (int)((p.n + BN - 1) / BN);
     p.tiles = p.batch * (p.symmetric ? (int64_t)p.tiles_n * (p.tiles_n + 1) / 2 : (int64_t)p.tiles_m * p.tiles_n);
     const unsigned grid = (unsigned)((p.tiles + 7) / 8 * 8);
-    if (epilogue == 0) hipLaunchKernelGGL((ns_gemm_fast<IS_BF16, B_KN, 0, WM, WN>), dim3(grid), dim3(256), 0, stream, p);
-    else if (epilogue == 1) hipLaunchKernelGGL((ns_gemm_fast<IS_BF16, B_KN, 1, WM, WN>), dim3(grid), dim3(256), 0, stream, p);
-    else hipLaunchKernelGGL((ns_gemm_fast<IS_BF16, B_KN, 2, WM, WN>), dim3(grid), dim3(256), 0, stream, p);
+    if (epilogue == 0) hipLaunchKernelGGL((ns_gemm_fast<IS_BF16, B_KN, 0, WM, WN, WAVES_M, WAVES_N, SBK, STAGES>), dim3(grid), dim3(THREADS), 0, stream, p);
+    else if (epilogue == 1) hipLaunchKernelGGL((ns_gemm_fast<IS_BF16, B_KN, 1, WM, WN, WAVES_M, WAVES_N, SBK, STAGES>), dim3(grid), dim3(THREADS), 0, stream, p);
+    else hipLaunchKernelGGL((ns_gemm_fast<IS_BF16, B_KN, 2, WM, WN, WAVES_M, WAVES_N, SBK, STAGES>), dim3(grid), dim3(THREADS), 0, stream, p);
 }
 
 template <bool IS_BF16, bool B_KN>
 static void launch_shape(const NsArgs& p, int epilogue, hipStream_t stream) {
     // 192-wide tiles move a third less operand data per flop; take them unless their padding costs more
     // than that (1152 = 6 x 192 and its multiples fit exactly)
-    auto area = [&](int64_t t) { return ((p.m + t - 1) / t) * ((p.n + t - 1) / t) * t * t; };
-    if (area(192) * 20 <= area(128) * 21) launch_tiles<IS_BF16, B_KN, 3, 3>(p, epilogue, stream);
-    else launch_tiles<IS_BF16, B_KN, 2, 2>(p, epilogue, stream);
+    auto area = [&](int64_t tm, int64_t tn) { return ((p.m + tm - 1) / tm) * ((p.n + tn - 1) / tn) * tm * tn; };
+    const bool wide = area(192, 192) * 20 <= area(128, 128) * 21;
+    // 384 x 192 blocks with whole-line loads when they fit as well as the 192s and still give every CU a few tiles
+    // (a Gram product keeps square tiles for its mirrored stores)
+    const bool big = wide && !p.symmetric && area(384, 192) <= area(192, 192) &&
+                     p.batch * ((p.m + 383) / 384) * ((p.n + 191) / 192) >= 3 * 256;
+    if (big) launch_tiles<IS_BF16, B_KN, 3, 3, 4, 2, 64, 2>(p, epilogue, stream);
+    else if (wide) launch_tiles<IS_BF16, B_KN, 3, 3, 2, 2, 32, 3>(p, epilogue, stream);
+    else launch_tiles<IS_BF16, B_KN, 2, 2, 2, 2, 32, 3>(p, epilogue, stream);
 }
 
 bool launch_ns_gemm_fast(const NsArgs& p, bool is_bf16, bool b_kn, int epilogue, hipStream_t stream) {
