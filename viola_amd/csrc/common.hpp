@@ -135,8 +135,12 @@ struct SharedDivisor {
     bool fast;
     __device__ __forceinline__ SharedDivisor(float divisor, float poison) : s(divisor) {
         const uint32_t bits = __float_as_uint(divisor);
-        r = 1.0f / divisor;
-        fast = divisor >= 0x1p-80f && bits < 0x7f800000u && (bits & 0x7fffffu) != 0x7fffffu && poison == poison;
+        // 2^-80 <= s < 2^126, significand not all ones, no NaN/Inf in the group
+        fast = bits >= (47u << 23) && bits < (253u << 23) && (bits & 0x7fffffu) != 0x7fffffu && poison == poison;
+        // One Newton step on the hardware reciprocal (1 ulp) is the correctly rounded 1/s for every s in that domain:
+        // checked over all of them on the device.
+        const float y0 = __builtin_amdgcn_rcpf(divisor);
+        r = fmaf(fmaf(-divisor, y0, 1.0f), y0, y0);
     }
     __device__ __forceinline__ float quotient(float v) const {
         const float t0 = v * r;
@@ -144,6 +148,17 @@ struct SharedDivisor {
         return fmaf(e, r, t0);
     }
 };
+// amax / limit for the group scale. For the two FP8 maxima the reciprocal route is exact for every amax >= 1e-30
+// (checked over all floats on the device); any other limit divides.
+__device__ __forceinline__ float scale_of(float amax, float limit) {
+    const float a = fmaxf(amax, 1e-30f);
+    if ((limit == 448.0f || limit == 57344.0f) && a < __uint_as_float(0x7f800000u)) {        // an infinite amax divides
+        const float r = limit == 448.0f ? 1.0f / 448.0f : 1.0f / 57344.0f;
+        const float t0 = a * r;
+        return fmaf(-fmaf(t0, limit, -a), r, t0);
+    }
+    return a / limit;
+}
 __device__ __forceinline__ float poison_of(float acc, float v) { return fmaf(v, 0.0f, acc); }
 
 // Four values -> four FP8 codes in one word with the gfx950 converters. They agree with f32_to_e4m3 /

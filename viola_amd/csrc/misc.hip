@@ -20,7 +20,7 @@ __global__ __launch_bounds__(256) void comm_pack_kernel(const float* __restrict_
         amax = fmaxf(amax, v != v ? __uint_as_float(0x7f800000u) : fabsf(v));
     }
     amax = group_max<LANES>(amax);
-    const float s = fmaxf(amax, 1e-30f) / fp8_traits<TQ>::max;
+    const float s = scale_of(amax, fp8_traits<TQ>::max);
     uint8_t* codes = packet + row * stride + group * tile;
     for (int i = sub; i < tile; i += LANES) {
         const float v = base + i < n ? x[base + i] : 0.0f;
@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256) void comm_pack256_kernel(const float* __restri
 #pragma unroll
     for (int i = 0; i < 4; ++i) amax = fmaxf(amax, v[i] != v[i] ? __uint_as_float(0x7f800000u) : fabsf(v[i]));
     amax = wave_max(amax);
-    const float s = fmaxf(amax, 1e-30f) / fp8_traits<TQ>::max;
+    const float s = scale_of(amax, fp8_traits<TQ>::max);
     uint32_t w = 0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) w |= (uint32_t)from_f32<TQ>(v[i] / s).bits << (8 * i);

@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256) void momentum_1d_kernel(const void* __restrict
         amax = fmaxf(amax, fabsf(m[j]));
     }
     amax = wave_max(amax);
-    const float scale = fmaxf(amax, 1e-30f) / 448.0f;
+    const float scale = scale_of(amax, 448.0f);
     if (lane == 0) new_scale[b] = scale;
 #pragma unroll
     for (int j = 0; j < EPL; ++j) {
@@ -134,7 +134,7 @@ __global__ __launch_bounds__(256) void momentum_1d_quads(const TG* __restrict__ 
     }
     amax = wave_max(amax);
     const bool any_bad = __builtin_amdgcn_ballot_w64(poison != poison) != 0;
-    const float scale = fmaxf(amax, 1e-30f) / 448.0f;
+    const float scale = scale_of(amax, 448.0f);
     if (lane == 0) new_scale[b] = scale;
     const SharedDivisor divisor(scale, any_bad ? __uint_as_float(0x7fc00000u) : 0.0f);
 #pragma unroll
@@ -200,7 +200,7 @@ __global__ __launch_bounds__(256) void momentum_2d_kernel(const void* __restrict
         if (element(j, i, g, m)) amax = fmaxf(amax, fabsf(m));
     }
     amax = wave_max(amax);
-    const float scale = fmaxf(amax, 1e-30f) / 448.0f;
+    const float scale = scale_of(amax, 448.0f);
     for (int j = lane; j < size; j += WAVE) {
         int64_t i; float g, m;
         if (element(j, i, g, m)) {

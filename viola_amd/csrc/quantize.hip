@@ -19,7 +19,7 @@ __device__ __forceinline__ uint8_t encode_clamped(float v, float s, float limit)
     return from_f32<TOut>(c).bits;
 }
 
-__device__ __forceinline__ float group_scale(float amax, float limit) { return fmaxf(amax, 1e-30f) / limit; }
+__device__ __forceinline__ float group_scale(float amax, float limit) { return scale_of(amax, limit); }
 
 // ------------------------------------------------------------------ 8-element chunk loads
 template <typename TIn> struct Chunk8;
