@@ -1,0 +1,163 @@
+"""GPU checks at the full sizes of the named configurations, where the CPU oracle would take minutes: the HIP path is
+held to size-independent properties (exact ones where the arithmetic gives them) and to a plain fp32 GPU matmul of
+the dequantized operands, a library routine whose only difference from the contract is fp32 summation order."""
+
+import math
+
+import pytest
+import torch
+
+from conftest import rel_l2
+
+pytestmark = pytest.mark.gpu
+E4 = torch.float8_e4m3fn
+
+
+def _quantized(rows, cols, group, seed):
+    from viola_amd.nn import _grouped_kernels as g
+    torch.manual_seed(seed)
+    x = (torch.randn(rows, cols, device="cuda") * torch.exp2(torch.randint(-3, 4, (rows, 1), device="cuda").float())).bfloat16()
+    q, s = g.quantize(x, E4, group)
+    return x, q, s
+
+
+@pytest.mark.parametrize("name,m,k,n,gb", [("forward", 8192, 1024, 4096, (32, 32)), ("dgrad", 8192, 4096, 1024, (32, 32)),
+                                          ("wgrad", 4096, 8192, 1024, (1, 32))])
+def test_linear_gemms_at_8192x1024x4096(name, m, k, n, gb):
+    from viola_amd.nn import _grouped_kernels as g
+    _, qa, sa = _quantized(m, k, (1, 32), 1)
+    _, qb, sb = _quantized(n, k, gb, 2)
+    out = g.gemm(qa, qb, sa, sb, (1, 32), gb, out_dtype=torch.float32)
+    reference = g.dequantize(qa, sa, (1, 32)) @ g.dequantize(qb, sb, gb).T
+    assert rel_l2(out, reference) < 2e-5
+    # exact: scaling every a scale by a power of two scales the result by it
+    assert torch.equal(g.gemm(qa, qb, sa * 4, sb, (1, 32), gb, out_dtype=torch.float32), out * 4)
+    # exact: rows of a are independent, so permuting them permutes the output rows
+    perm = torch.randperm(m, device="cuda")
+    assert torch.equal(g.gemm(qa[perm].contiguous(), qb, sa[perm].contiguous(), sb, (1, 32), gb, out_dtype=torch.float32), out[perm])
+    # bf16 output is the rounded fp32 output, bias added before the rounding
+    bias = torch.randn(n, device="cuda")
+    assert torch.equal(g.gemm(qa, qb, sa, sb, (1, 32), gb, out_dtype=torch.bfloat16, bias=bias), (out + bias).bfloat16())
+
+
+def test_linear_module_at_8192x1024x4096():
+    import viola_amd
+    viola_amd.set_gradient_dtype("bf16")
+    try:
+        torch.manual_seed(3)
+        layer = viola_amd.nn.Linear(1024, 4096, device="cuda", dtype=torch.bfloat16, scaling="grouped", forward_dtype="e4m3",
+                                    backward_dtype="e4m3", mode="memory", weight_dtype="fp8")
+    finally:
+        viola_amd.precision._settings["gradient_dtype"] = None
+    from viola_amd.nn import _grouped_kernels as g
+    x = torch.randn(8192, 1024, device="cuda").bfloat16().requires_grad_()
+    dy = (torch.randn(8192, 4096, device="cuda") * 1e-2).bfloat16()
+    y = layer(x)
+    y.backward(dy)
+    w = g.dequantize(layer.weight.detach(), layer.weight_scale, (32, 32))
+    xq = g.dequantize(*g.quantize(x.detach(), E4, (1, 32)), (1, 32))
+    gq = g.dequantize(*g.quantize(dy, E4, (1, 32)), (1, 32))
+    assert rel_l2(y, (xq @ w.T + layer.bias.float()).bfloat16()) < 3e-3
+    assert rel_l2(x.grad, (gq @ w).bfloat16()) < 3e-3
+    xt = g.dequantize(*g.quantize(x.detach(), E4, (1, 32), transposed=True), (1, 32))
+    gt = g.dequantize(*g.quantize(dy, E4, (1, 32), transposed=True), (1, 32))
+    assert rel_l2(layer.weight.grad, (gt @ xt.T).bfloat16()) < 3e-3
+    assert rel_l2(layer.bias.grad, dy.float().sum(0).bfloat16()) < 3e-3
+
+
+def test_gated_mlp_gemms_at_16384x4096x11008():
+    from viola_amd.nn import _grouped_kernels as g, _mlp_kernels as mk
+    m, d, h = 16384, 4096, 11008
+    _, qx, sx = _quantized(m, d, (1, 32), 4)
+    torch.manual_seed(5)
+    w = torch.empty(2 * h, d, device="cuda").uniform_(-1 / 64, 1 / 64)
+    qw, sw = g.quantize(w, E4, (32, 32))
+    del w
+    import types
+    recipe = types.SimpleNamespace(_native_scaling=False, _grouped_scaling=True, input_group_shape=(1, 32), weight_group_shape=(32, 32))
+    out, aux, _ = mk.gemm(qx, qw, sx, sw, layer=recipe, out_dtype=torch.bfloat16, activation="silu", save=True)
+    assert out.shape == (m, h) and aux.shape == (m, 2 * h)
+    rows = torch.arange(0, m, 61, device="cuda")                              # a 269-row sample keeps the fp32 reference small
+    z = g.dequantize(qx[rows].contiguous(), sx[rows].contiguous(), (1, 32)) @ g.dequantize(qw, sw, (32, 32)).T
+    assert rel_l2(aux[rows], z.bfloat16()) < 3e-3
+    gate, up = aux[rows, :h].float(), aux[rows, h:].float()
+    assert rel_l2(out[rows], (torch.nn.functional.silu(gate) * up).bfloat16()) < 3e-3
+    # the fused forward equals the plain GEMM followed by the elementwise kernel
+    plain = g.gemm(qx, qw, sx, sw, (1, 32), (32, 32), out_dtype=torch.bfloat16)
+    assert torch.equal(plain, aux)
+
+
+def test_variable_groups_at_16x32768x4096x1024():
+    from viola_amd.nn import _varlen as v, _grouped_kernels as g
+    groups, k, n, total = 16, 4096, 1024, 32768
+    generator = torch.Generator().manual_seed(6)
+    counts = torch.bincount(torch.multinomial(torch.ones(groups) / groups, total, replacement=True, generator=generator), minlength=groups)
+    counts[3] += counts[5] - 3
+    counts[5] = 3
+    counts[7] += counts[9]
+    counts[9] = 0
+    counts = counts.tolist()
+    assert sum(counts) == total
+    torch.manual_seed(7)
+    x = torch.randn(total, k, device="cuda").bfloat16().requires_grad_()
+    dy = torch.randn(total, n, device="cuda").bfloat16()
+    experts = v.GroupedExperts(groups, k, n, device="cuda")
+    y = experts(x, counts)
+    y.backward(dy)
+    w = experts.dequantize_weight()
+    xq = g.dequantize(*g.quantize(x.detach(), E4, (1, 32)), (1, 32))
+    gq = g.dequantize(*g.quantize(dy, E4, (1, 32)), (1, 32))
+    start = 0
+    for group, count in enumerate(counts):
+        rows = slice(start, start + count)
+        if count:
+            assert rel_l2(y[rows], (xq[rows] @ w[group].T).bfloat16()) < 3e-3, group
+            assert rel_l2(x.grad[rows], (gq[rows] @ w[group]).bfloat16()) < 3e-3, group
+        else:
+            assert experts.weight.grad[group].count_nonzero() == 0
+        start += count
+    # weight gradient of one full and one tiny group against the quantized transposes
+    for group in (0, 5):
+        begin = sum(counts[:group])
+        rows = slice(begin, begin + counts[group])
+        xt = g.dequantize(*g.quantize(x.detach()[rows].contiguous(), E4, (1, 32), transposed=True), (1, 32))
+        gt = g.dequantize(*g.quantize(dy[rows].contiguous(), E4, (1, 32), transposed=True), (1, 32))
+        assert rel_l2(experts.weight.grad[group], gt @ xt.T) < 3e-3, group
+
+
+@pytest.mark.parametrize("method", ["standard", "gram"])
+def test_newton_schulz_batched_equals_single_at_ditxl_shapes(method):
+    from viola_amd.optim._orthogonalize import METHODS
+    torch.manual_seed(8)
+    for shape in ((3456, 1152), (1152, 1152), (1152, 4608)):
+        batch = torch.randn(3, *shape, device="cuda").bfloat16()
+        together = METHODS[method](batch, steps=5)
+        for i in range(3):
+            assert torch.equal(METHODS[method](batch[i:i + 1].clone(), steps=5)[0], together[i]), (shape, i)
+        sigma = torch.linalg.svdvals(together[0].float())
+        # a square Gaussian matrix has singular values arbitrarily close to zero, which five steps do not lift
+        assert sigma.max() < 1.3 and (shape[0] == shape[1] or sigma.min() > .3), (shape, float(sigma.min()), float(sigma.max()))
+
+
+def test_fp8muon_step_at_ditxl_block():
+    """One transformer block of the DiT-XL set: the batched step equals stepping each parameter in its own optimizer."""
+    import viola_amd
+    d = 1152
+    shapes = ((3 * d, d), (d, d), (4 * d, d), (d, 4 * d), (d,), (3 * d,))
+
+    def build(seed):
+        torch.manual_seed(seed)
+        params = [torch.nn.Parameter(torch.randn(*s, device="cuda") * .02) for s in shapes for _ in range(2)]
+        for p in params:
+            p.grad = torch.randn_like(p) * 1e-3
+        return params
+
+    together = build(9)
+    viola_amd.optim.FP8Muon(together, lr=1e-3, weight_decay=.01, adjust_lr_fn="match_rms_adamw").step()
+    alone = build(9)
+    for index, p in enumerate(alone):
+        opt = viola_amd.optim.FP8Muon([{"params": [p], "viola_parameter_indices": [index]}], lr=1e-3, weight_decay=.01,
+                                      adjust_lr_fn="match_rms_adamw")
+        opt.step()
+    for a, b in zip(together, alone):
+        assert torch.equal(a, b)
