@@ -65,8 +65,9 @@ int viola_column_reduce(const float* partial, int64_t parts, int64_t cols, void*
 int viola_group_dequantize(const void* q, int q_dtype, const float* scale, int64_t rows, int64_t cols,
                            int gr, int gc, float* out, viola_stream_t stream);
 
-/* viola/nn/_linear_kernels.py:107-121,253-257 `transpose`: byte-matrix transpose, out [cols, rows]. */
-int viola_fp8_transpose(const void* x, void* out, int64_t rows, int64_t cols, viola_stream_t stream);
+/* viola/nn/_linear_kernels.py:107-121,253-257 `transpose`: byte-matrix transpose, x [batch, rows, cols] ->
+ * out [batch, cols, rows] (the reference transposes one matrix per call; batch > 1 serves stacked expert weights). */
+int viola_fp8_transpose(const void* x, void* out, int64_t batch, int64_t rows, int64_t cols, viola_stream_t stream);
 
 /* ---------------------------------------------------------------- grouped-scale FP8 GEMM
  * viola/nn/_grouped_kernels.py:310-328 `gemm` (gemm_kernel :195-293).
@@ -112,7 +113,10 @@ int viola_varlen_wgrad_gemm(const void* at, int a_dtype, const void* bt, int b_d
  * counted from the group's own first row; padding columns get zero codes and scale 1e-30/limit. */
 int viola_varlen_quantize_transposed(const void* x, int x_dtype, int64_t rows, int64_t cols,
                                      const int64_t* offsets, const int64_t* poffsets, int groups, int64_t t_total,
-                                     void* qt, float* scale_t, int q_dtype, float limit, viola_stream_t stream);
+                                     void* qt, float* scale_t, int q_dtype, float limit,
+                                     void* q, float* scale, viola_stream_t stream);
+/* q / scale (both or neither; 16-bit x with cols a multiple of 8, else VIOLA_EUNSUPPORTED): the plain row-wise
+ * (1, 32) quantization of x, q [rows, cols] and scale [rows, ceil(cols/32)], written from the same read. */
 
 /* ---------------------------------------------------------------- gated activations (elementwise)
  * viola/nn/_gated_kernels.py:16-36 forward_kernel: out[r, c] = act(z[r, c]) * z[r, c + h].

@@ -131,3 +131,26 @@ def test_varlen_group_gemm_and_wgrad(counts):
     for g, c in enumerate(counts):
         if c == 0:
             assert wparam.grad[g].count_nonzero() == 0
+
+
+@pytest.mark.parametrize("counts", [[130, 0, 3, 64, 1, 200], [31, 33]])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_varlen_segmented_quantizer_rowwise_byproduct(counts, dtype):
+    """The segmented transposed quantizer can emit the plain row-wise codes from the same read: both outputs must be the
+    ones the separate kernels give."""
+    from viola_amd.nn import _varlen as v, _grouped_kernels as g
+    torch.manual_seed(12)
+    x = (torch.randn(sum(counts), 136) * 3).to(dtype).cuda()
+    offsets, padded, offsets_dev, padded_dev = v._offsets(counts, x.device)
+    qt, st = v.quantize_transposed_segmented(x, E4, offsets_dev, padded_dev, len(counts), padded[-1])
+    qt2, st2, q, s = v.quantize_transposed_segmented(x, E4, offsets_dev, padded_dev, len(counts), padded[-1], rowwise=True)
+    rq, rs = g.quantize(x, E4, (1, 32))
+    assert torch.equal(qt.view(torch.uint8), qt2.view(torch.uint8)) and torch.equal(st, st2)
+    assert torch.equal(q.view(torch.uint8), rq.view(torch.uint8)) and torch.equal(s, rs)
+    # against the oracle, group by group: the transposed block of a group is the quantized transpose of its rows
+    for group, count in enumerate(counts):
+        if count:
+            oq, os_ = og.quantize(x[offsets[group]:offsets[group + 1]].cpu(), E4, (1, 32), transposed=True)
+            got = qt[:, padded[group]:padded[group] + count].cpu().view(torch.uint8)
+            assert torch.equal(got, oq.view(torch.uint8))
+            assert torch.equal(st[:, padded[group] // 32:padded[group] // 32 + (count + 31) // 32].cpu(), os_)

@@ -23,12 +23,12 @@ _SIGNATURES = {
     "viola_group_quantize_dual": [_p, _i, _l, _l, _p, _p, _p, _p, _i, _i, _f, _p, _p],
     "viola_column_reduce": [_p, _l, _l, _p, _i, _p],
     "viola_group_dequantize": [_p, _i, _p, _l, _l, _i, _i, _p, _p],
-    "viola_fp8_transpose": [_p, _p, _l, _l, _p],
+    "viola_fp8_transpose": [_p, _p, _l, _l, _l, _p],
     "viola_group_gemm": [_p, _i, _p, _i, _p, _p, _l, _l, _l, _i, _i, _i, _i, _p, _i, _p, _i, _p],
     "viola_gated_gemm": [_p, _i, _p, _i, _p, _p, _l, _l, _l, _i, _i, _i, _i, _p, _i, _p, _p, _i, _i, _i, _p],
     "viola_varlen_group_gemm": [_p, _i, _p, _i, _p, _p, _p, _i, _l, _l, _l, _i, _i, _i, _i, _l, _l, _p, _i, _p],
     "viola_varlen_wgrad_gemm": [_p, _i, _p, _i, _p, _p, _p, _i, _l, _l, _l, _p, _i, _p],
-    "viola_varlen_quantize_transposed": [_p, _i, _l, _l, _p, _p, _i, _l, _p, _p, _i, _f, _p],
+    "viola_varlen_quantize_transposed": [_p, _i, _l, _l, _p, _p, _i, _l, _p, _p, _i, _f, _p, _p, _p],
     "viola_gated_forward": [_p, _p, _l, _l, _i, _i, _p],
     "viola_gated_backward": [_p, _p, _p, _l, _l, _i, _i, _p],
     "viola_momentum_update": [_p, _i, _p, _p, _p, _p, _p, _l, _f, _f, _i, _i, _i, _l, _l, _l, _i, _i, _i, _l, _l, _p],

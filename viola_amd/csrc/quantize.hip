@@ -443,6 +443,8 @@ template <bool WORDS>
 __global__ __launch_bounds__(256) void transpose_bytes(const uint8_t* __restrict__ x, uint8_t* __restrict__ out,
                                                         int64_t rows, int64_t cols) {
     const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+    x += (int64_t)blockIdx.z * rows * cols;
+    out += (int64_t)blockIdx.z * rows * cols;
     if constexpr (WORDS) {
         __shared__ uint32_t tile[64][17];
         const int b = threadIdx.x % 16, a = threadIdx.x / 16;               // block of rows 4a.., cols 4b..
@@ -509,6 +511,90 @@ __global__ __launch_bounds__(64) void quantize_transposed_segmented(const TIn* _
     scale_t[col * (t_total / 32) + slot] = s;
     uint8_t* dst = qt + col * t_total + token;
     store_group32<TOut>(v, s, poison, limit, dst, 32, (reinterpret_cast<uintptr_t>(dst) & 15) == 0);
+}
+
+// 16-bit inputs: the same wavefront tile as quantize_dual16 over one 32-token slot x 64 columns, with the slot's rows
+// taken from its group (rows past the group's end read as zero) and, optionally, the row-wise layout of the valid rows
+// written in the same pass (q [rows, cols], scale [rows, ceil(cols/32)] in the unpadded row order).
+template <typename TIn, typename TOut, bool ROWWISE>
+__global__ __launch_bounds__(256) void quantize_segmented16(const TIn* __restrict__ x, const int64_t* __restrict__ offsets,
+                                                             const int64_t* __restrict__ poffsets, int groups, int64_t cols,
+                                                             int64_t t_total, uint8_t* __restrict__ qt, float* __restrict__ scale_t,
+                                                             uint8_t* __restrict__ q, float* __restrict__ scale, float limit) {
+    constexpr int LD = 64 + 32;
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    __shared__ __attribute__((aligned(16))) uint16_t park[4][32 * LD];
+    const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+    uint16_t* mine = park[wave];
+    const int lr = lane / 8, ch = lane % 8;
+    const int64_t nc = (cols + 31) / 32;
+    const int64_t tiles_x = (cols + 63) / 64, slots = t_total / 32;
+    const int64_t work = ((int64_t)blockIdx.x * 4 + wave);                    // one (slot, column tile) per wavefront
+    if (work >= slots * tiles_x) return;
+    const int64_t slot = work / tiles_x, c0 = work % tiles_x * 64;
+    const int64_t token = slot * 32;
+    int g = 0;
+    while (g + 1 < groups && poffsets[g + 1] <= token) ++g;
+    const int64_t first = offsets[g] + (token - poffsets[g]);
+    const int64_t left = offsets[g + 1] - first;                               // valid rows of this slot (may be <= 0)
+    const int valid = (int)(left < 0 ? 0 : left > 32 ? 32 : left);
+    const int64_t col8 = c0 + ch * 8;
+
+    const __amdgpu_buffer_rsrc_t res = __builtin_amdgcn_make_buffer_rsrc(const_cast<TIn*>(x + first * cols), 0, (int)(valid * cols * 2), 0x00020000);
+    u32x4 raw[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        raw[i] = __builtin_amdgcn_raw_buffer_load_b128(res, col8 < cols ? (int)(((lr + 8 * i) * cols + col8) * 2) : (int)0x80000000u, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(&mine[(lr + 8 * i) * LD + ch * 8]) = raw[i];
+
+    if constexpr (ROWWISE) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float v[8];
+            float amax = 0.0f, poison = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                v[e] = widen16<TIn>(e % 2 ? raw[i][e / 2] >> 16 : raw[i][e / 2] & 0xffffu);
+                amax = fmaxf(amax, fabsf(v[e]));
+                poison = poison_of(poison, v[e]);
+            }
+            amax = group_max<4>(amax);
+            poison += __shfl_xor(poison, 1, WAVE);
+            poison += __shfl_xor(poison, 2, WAVE);
+            const float s = group_scale(amax, limit);
+            const SharedDivisor divisor(s, poison);
+            const uint2 codes = encode8<TOut>(v, s, limit, divisor);
+            const int r = lr + 8 * i;
+            if (r < valid && col8 < cols) {
+                *reinterpret_cast<uint2*>(q + (first + r) * cols + col8) = codes;
+                if (ch % 4 == 0) scale[(first + r) * nc + col8 / 32] = s;
+            }
+        }
+    }
+    const int64_t col = c0 + lane;
+    const int strip = (lane / 16) * 16, sub = lane & 15;
+    const uint16_t* at = &mine[(sub >> 2) * LD + strip + 4 * (sub & 3)];
+    float vc[32];
+    float amax = 0.0f, poison = 0.0f;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        const s16x4 four = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at + 4 * t * LD));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            vc[4 * t + e] = widen16<TIn>((uint16_t)four[e]);
+            amax = fmaxf(amax, fabsf(vc[4 * t + e]));
+            poison = poison_of(poison, vc[4 * t + e]);
+        }
+    }
+    if (col < cols) {
+        const float s = group_scale(amax, limit);
+        scale_t[col * slots + slot] = s;
+        uint8_t* dst = qt + col * t_total + token;
+        store_group32<TOut>(vc, s, poison, limit, dst, 32, (reinterpret_cast<uintptr_t>(dst) & 15) == 0);
+    }
 }
 
 // ------------------------------------------------------------------ host dispatch
@@ -596,7 +682,18 @@ static int launch_dual(const void* x, int64_t rows, int64_t cols, void* q, float
 
 template <typename TIn, typename TOut>
 static int launch_segmented(const void* x, int64_t cols, const int64_t* offsets, const int64_t* poffsets, int groups,
-                            int64_t t_total, void* qt, float* scale_t, float limit, hipStream_t stream) {
+                            int64_t t_total, void* qt, float* scale_t, void* q, float* scale, float limit, hipStream_t stream) {
+    if constexpr (sizeof(TIn) == 2) {
+        const bool aligned = cols % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && (!q || reinterpret_cast<uintptr_t>(q) % 8 == 0);
+        const int64_t waves = (t_total / 32) * ((cols + 63) / 64);
+        if (aligned && (waves + 3) / 4 < (1ll << 31)) {
+            const dim3 grid16((unsigned)((waves + 3) / 4));
+            if (q) hipLaunchKernelGGL((quantize_segmented16<TIn, TOut, true>), grid16, dim3(256), 0, stream, static_cast<const TIn*>(x), offsets, poffsets, groups, cols, t_total, static_cast<uint8_t*>(qt), scale_t, static_cast<uint8_t*>(q), scale, limit);
+            else hipLaunchKernelGGL((quantize_segmented16<TIn, TOut, false>), grid16, dim3(256), 0, stream, static_cast<const TIn*>(x), offsets, poffsets, groups, cols, t_total, static_cast<uint8_t*>(qt), scale_t, nullptr, nullptr, limit);
+            return viola_launch_status();
+        }
+    }
+    if (q) return VIOLA_EUNSUPPORTED;                                      // the row-wise by-product needs the 16-bit aligned path
     const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)(t_total / 32));
     hipLaunchKernelGGL((quantize_transposed_segmented<TIn, TOut>), grid, dim3(64), 0, stream, static_cast<const TIn*>(x),
                        offsets, poffsets, groups, cols, t_total, static_cast<uint8_t*>(qt), scale_t, limit);
@@ -666,13 +763,13 @@ extern "C" int viola_column_reduce(const float* partial, int64_t parts, int64_t 
 extern "C" int viola_varlen_quantize_transposed(const void* x, int x_dtype, int64_t rows, int64_t cols,
                                                 const int64_t* offsets, const int64_t* poffsets, int groups,
                                                 int64_t t_total, void* qt, float* scale_t, int q_dtype, float limit,
-                                                viola_stream_t stream_) {
+                                                void* q, float* scale, viola_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     VIOLA_CHECK_ARG(viola_is_fp8(q_dtype) && viola_is_float(x_dtype) && rows >= 0 && cols >= 0 && groups > 0);
     VIOLA_CHECK_ARG(t_total >= 0 && t_total % 32 == 0 && limit > 0.0f);
     if (t_total == 0 || cols == 0) return 0;
-    VIOLA_CHECK_ARG(x && offsets && poffsets && qt && scale_t && t_total / 32 <= 65535);
-#define VIOLA_SEG(TI, TO) return launch_segmented<TI, TO>(x, cols, offsets, poffsets, groups, t_total, qt, scale_t, limit, stream)
+    VIOLA_CHECK_ARG(x && offsets && poffsets && qt && scale_t && t_total / 32 <= 65535 && (!q == !scale));
+#define VIOLA_SEG(TI, TO) return launch_segmented<TI, TO>(x, cols, offsets, poffsets, groups, t_total, qt, scale_t, q, scale, limit, stream)
     if (q_dtype == VIOLA_E4M3) {
         if (x_dtype == VIOLA_F32) VIOLA_SEG(float, e4m3_t);
         if (x_dtype == VIOLA_BF16) VIOLA_SEG(bf16_t, e4m3_t);
@@ -699,12 +796,12 @@ extern "C" int viola_group_dequantize(const void* q, int q_dtype, const float* s
     return viola_launch_status();
 }
 
-extern "C" int viola_fp8_transpose(const void* x, void* out, int64_t rows, int64_t cols, viola_stream_t stream_) {
+extern "C" int viola_fp8_transpose(const void* x, void* out, int64_t batch, int64_t rows, int64_t cols, viola_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    VIOLA_CHECK_ARG(rows >= 0 && cols >= 0);
-    if (rows == 0 || cols == 0) return 0;
-    VIOLA_CHECK_ARG(x && out && (rows + 63) / 64 <= 65535);
-    const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64));
+    VIOLA_CHECK_ARG(batch >= 0 && rows >= 0 && cols >= 0);
+    if (batch == 0 || rows == 0 || cols == 0) return 0;
+    VIOLA_CHECK_ARG(x && out && (rows + 63) / 64 <= 65535 && batch <= 65535);
+    const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64), (unsigned)batch);
     const bool words = rows % 4 == 0 && cols % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 4 == 0;
     if (words) hipLaunchKernelGGL(transpose_bytes<true>, grid, dim3(256), 0, stream, static_cast<const uint8_t*>(x), static_cast<uint8_t*>(out), rows, cols);
     else hipLaunchKernelGGL(transpose_bytes<false>, grid, dim3(256), 0, stream, static_cast<const uint8_t*>(x), static_cast<uint8_t*>(out), rows, cols);

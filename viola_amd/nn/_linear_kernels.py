@@ -7,10 +7,10 @@ from .. import _lib
 
 
 def transpose(x, out=None):
-    """FP8 code matrix [rows, cols] -> [cols, rows], one HIP launch."""
-    assert x.is_cuda and x.dim() == 2 and x.element_size() == 1
+    """FP8 code matrix [rows, cols] -> [cols, rows] (or a stack [batch, rows, cols] -> [batch, cols, rows]), one HIP launch."""
+    assert x.is_cuda and x.dim() in (2, 3) and x.element_size() == 1
     x = x.contiguous()
     if out is None:
-        out = torch.empty(x.shape[::-1], device=x.device, dtype=x.dtype)
-    _lib.call("viola_fp8_transpose", _lib.ptr(x), _lib.ptr(out), x.shape[0], x.shape[1])
+        out = torch.empty((*x.shape[:-2], x.shape[-1], x.shape[-2]), device=x.device, dtype=x.dtype)
+    _lib.call("viola_fp8_transpose", _lib.ptr(x), _lib.ptr(out), x.shape[0] if x.dim() == 3 else 1, x.shape[-2], x.shape[-1])
     return out

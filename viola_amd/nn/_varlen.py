@@ -44,15 +44,23 @@ def varlen_gemm(a, b, sa, sb, offsets_dev, *, out_dtype):
     return out
 
 
-def quantize_transposed_segmented(x, dtype, offsets_dev, padded_dev, groups, t_total):
-    """Per-group quantized transpose of x [M, C]: codes [C, t_total], scales [C, t_total/32]."""
+def quantize_transposed_segmented(x, dtype, offsets_dev, padded_dev, groups, t_total, *, rowwise=False):
+    """Per-group quantized transpose of x [M, C]: codes [C, t_total], scales [C, t_total/32]. With rowwise, also the
+    plain (1, 32) row-wise codes and scales of x from the same read: returns (qt, st, q, s)."""
     rows, cols = x.shape
     qt = torch.empty((cols, t_total), device=x.device, dtype=dtype)
     st = torch.empty((cols, t_total // 32), device=x.device, dtype=torch.float32)
+    fused = rowwise and x.element_size() == 2 and cols % 8 == 0 and x.data_ptr() % 16 == 0
+    q = torch.empty((rows, cols), device=x.device, dtype=dtype) if fused else None
+    s = torch.empty((rows, -(-cols // 32)), device=x.device, dtype=torch.float32) if fused else None
     _lib.call("viola_varlen_quantize_transposed", _lib.ptr(x), _lib.code(x.dtype), rows, cols, _lib.ptr(offsets_dev),
               _lib.ptr(padded_dev), groups, t_total, _lib.ptr(qt), _lib.ptr(st), _lib.code(dtype),
-              float(torch.finfo(dtype).max))
-    return qt, st
+              float(torch.finfo(dtype).max), _lib.ptr(q), _lib.ptr(s))
+    if not rowwise:
+        return qt, st
+    if not fused:
+        q, s = kernels.quantize(x, dtype, GX)
+    return qt, st, q, s
 
 
 def varlen_wgrad(gt, xt, sgt, sxt, padded_dev, groups, *, out_dtype):
@@ -72,13 +80,13 @@ class _VarlenLinear(torch.autograd.Function):
         groups = weight.shape[0]
         offsets, padded, offsets_dev, padded_dev = _offsets(counts, x.device)
         assert offsets[-1] == x.shape[0] and len(offsets) == groups + 1
-        qx, sx = kernels.quantize(x, fp8, GX)
-        y = varlen_gemm(qx, weight, sx, weight_scale, offsets_dev, out_dtype=x.dtype)
         need_w = ctx.needs_input_grad[1]
-        if need_w:
-            xt, sxt = quantize_transposed_segmented(x, fp8, offsets_dev, padded_dev, groups, padded[-1])
+        if need_w and x.shape[0]:
+            xt, sxt, qx, sx = quantize_transposed_segmented(x, fp8, offsets_dev, padded_dev, groups, padded[-1], rowwise=True)
         else:
+            qx, sx = kernels.quantize(x, fp8, GX)
             xt = sxt = x.new_empty(0)
+        y = varlen_gemm(qx, weight, sx, weight_scale, offsets_dev, out_dtype=x.dtype)
         ctx.save_for_backward(xt, sxt, weight, weight_scale, offsets_dev, padded_dev)
         ctx.meta = (groups, padded[-1], bwd_fp8, grad_dtype, x.dtype)
         return y
@@ -89,13 +97,18 @@ class _VarlenLinear(torch.autograd.Function):
         groups, t_total, bwd_fp8, grad_dtype, x_dtype = ctx.meta
         dy = dy.contiguous()
         dx = dw = None
+        gt = None
         if ctx.needs_input_grad[0]:
-            qg, sg = kernels.quantize(dy, bwd_fp8, GX)
-            wt = torch.stack([transpose_payload(weight[g]) for g in range(groups)])
+            if ctx.needs_input_grad[1] and dy.shape[0]:
+                gt, sgt, qg, sg = quantize_transposed_segmented(dy, bwd_fp8, offsets_dev, padded_dev, groups, t_total, rowwise=True)
+            else:
+                qg, sg = kernels.quantize(dy, bwd_fp8, GX)
+            wt = transpose_payload(weight)
             st = weight_scale.transpose(1, 2).contiguous()
             dx = varlen_gemm(qg, wt, sg, st, offsets_dev, out_dtype=x_dtype)
         if ctx.needs_input_grad[1]:
-            gt, sgt = quantize_transposed_segmented(dy, bwd_fp8, offsets_dev, padded_dev, groups, t_total)
+            if gt is None:
+                gt, sgt = quantize_transposed_segmented(dy, bwd_fp8, offsets_dev, padded_dev, groups, t_total)
             dw = varlen_wgrad(gt, xt, sgt, sxt, padded_dev, groups, out_dtype=grad_dtype)
         return dx, dw, None, None, None, None, None
 
