@@ -149,6 +149,15 @@ int viola_adam_update(void* weight, int weight_dtype, const void* grad, int grad
                       int rounding, int64_t rounding_step, int64_t rounding_key, int64_t offset,
                       int adamw, int maximize, viola_stream_t stream);
 
+/* The same update for many tensors that share dtypes, hyper-parameters and step count, in one launch (the reference
+ * calls adam_update once per parameter, viola/optim/muon.py:122-128; vectors of a transformer are a few thousand
+ * elements each, so their launches dominate). table: device array of `tensors` rows of seven int64:
+ * {weight pointer, grad pointer, first pointer, second pointer, element count, rounding key, rounding offset};
+ * max_count: the largest element count. */
+int viola_adam_update_table(const int64_t* table, int64_t tensors, int64_t max_count, int weight_dtype, int grad_dtype,
+                            int state_dtype, float lr, float decay, float b1, float b2, float inv_c1, float inv_c2,
+                            float eps, int rounding, int64_t rounding_step, int adamw, int maximize, viola_stream_t stream);
+
 /* viola/optim/_kernels.py:318-322 `copy_scaled` (_copy_scaled_kernel :203-222). */
 int viola_copy_scaled(const void* update, int update_dtype, void* out, int out_dtype,
                       int64_t src, int64_t dst, int64_t count, float scale, viola_stream_t stream);

@@ -200,6 +200,36 @@ def test_stochastic_master_rounding(dtype):
     assert torch.equal(w2.cpu(), rw)
 
 
+@pytest.mark.parametrize("wdtype,rounding", [(torch.float32, "nearest"), (torch.bfloat16, "nearest"), (torch.bfloat16, "stochastic"),
+                                             (torch.float16, "stochastic")])
+def test_adam_table_equals_per_tensor_and_oracle(wdtype, rounding):
+    """One launch over a pointer table == one adam_update per tensor (viola/optim/muon.py:122-128), bit for bit,
+    ragged sizes from 1 element to beyond one grid stride, own rounding key per tensor."""
+    k = _k()
+    torch.manual_seed(31)
+    sizes = [1, 7, 256, 1152, 3 * 1152 + 5, 300001]
+    hyper = dict(lr=1e-3, weight_decay=.01, betas=(.9, .95), eps=1e-8)
+    weights = [(torch.randn(n) * .1).to(wdtype) for n in sizes]
+    grads = [torch.randn(n) * 1e-2 for n in sizes]
+    many = [(w.cuda(), g.cuda(), torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda"), 1000 + i, 3 * i)
+            for i, (w, g, n) in enumerate(zip(weights, grads, sizes))]
+    single = [(w.cuda(), g.cuda(), torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda"), 1000 + i, 3 * i)
+              for i, (w, g, n) in enumerate(zip(weights, grads, sizes))]
+    cache = {}
+    for step in (1, 2):
+        k.adam_update_many(many, step=step, rounding=rounding, cache=cache, **hyper)
+        for w, g, m, v, key, offset in single:
+            k.adam_update(w, g, m, v, step=step, rounding=rounding, key=key, offset=offset, **hyper)
+    assert len(cache["rows"]) == len(sizes)
+    for a, b in zip(many, single):
+        for x, y in zip(a[:4], b[:4]):
+            assert torch.equal(x, y)
+    rw, rm, rv = weights[4], torch.zeros(sizes[4]), torch.zeros(sizes[4])
+    for step in (1, 2):
+        rw, rm, rv = oo.adam_update(rw, grads[4], rm, rv, step=step, rounding=rounding, key=1004, offset=12, **hyper)
+    assert torch.equal(many[4][0].cpu(), rw) and torch.equal(many[4][2].cpu(), rm) and torch.equal(many[4][3].cpu(), rv)
+
+
 def test_copy_scaled():
     k = _k()
     matrix = torch.randn(17, 31).bfloat16().T

@@ -249,32 +249,56 @@ __global__ __launch_bounds__(256) void weight_quads_kernel(float* weight, const 
     }
 }
 
+struct AdamConstants {
+    float lr, decay, b1, b2, inv_c1, inv_c2, eps;
+    int adamw, maximize;
+};
+
+template <bool STOCHASTIC>
+__device__ __forceinline__ void adam_element(void* weight, int weight_dtype, const void* grad, int grad_dtype, void* first,
+                                             void* second, int state_dtype, int64_t j, const AdamConstants& c, uint64_t step,
+                                             uint64_t key, uint64_t offset) {
+    const float one_b1 = 1.0f - c.b1, one_b2 = 1.0f - c.b2;
+    const float keep = 1.0f - c.lr * c.decay;
+    float w = load_dtype(weight, j, weight_dtype);
+    float g = load_dtype(grad, j, grad_dtype);
+    if (c.maximize) g = -g;
+    if (!c.adamw) { const float t = c.decay * w; g = g + t; }
+    const float m0 = c.b1 * load_dtype(first, j, state_dtype);
+    const float m1 = one_b1 * g;
+    const float m = m0 + m1;
+    const float v0 = c.b2 * load_dtype(second, j, state_dtype);
+    const float v1 = (one_b2 * g) * g;
+    const float v = v0 + v1;
+    store_rounded<false>(first, j, state_dtype, m, 0, 0, 0);
+    store_rounded<false>(second, j, state_dtype, v, 0, 0, 0);
+    if (c.adamw) w = w * keep;
+    const float numerator = c.lr * (m * c.inv_c1);
+    const float denominator = sqrtf(v * c.inv_c2) + c.eps;
+    store_rounded<STOCHASTIC>(weight, j, weight_dtype, w - numerator / denominator, (uint64_t)j + offset, step, key);
+}
+
 template <bool STOCHASTIC>
 __global__ __launch_bounds__(256) void adam_kernel(void* weight, int weight_dtype, const void* __restrict__ grad,
                                                     int grad_dtype, void* first, void* second, int state_dtype, int64_t n,
-                                                    float lr, float decay, float b1, float b2, float inv_c1, float inv_c2,
-                                                    float eps, uint64_t step, uint64_t key, uint64_t offset, int adamw,
-                                                    int maximize) {
-    const float one_b1 = 1.0f - b1, one_b2 = 1.0f - b2;
-    const float keep = 1.0f - lr * decay;
-    for (int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < n; j += (int64_t)gridDim.x * blockDim.x) {
-        float w = load_dtype(weight, j, weight_dtype);
-        float g = load_dtype(grad, j, grad_dtype);
-        if (maximize) g = -g;
-        if (!adamw) { const float t = decay * w; g = g + t; }
-        const float m0 = b1 * load_dtype(first, j, state_dtype);
-        const float m1 = one_b1 * g;
-        const float m = m0 + m1;
-        const float v0 = b2 * load_dtype(second, j, state_dtype);
-        const float v1 = (one_b2 * g) * g;
-        const float v = v0 + v1;
-        store_rounded<false>(first, j, state_dtype, m, 0, 0, 0);
-        store_rounded<false>(second, j, state_dtype, v, 0, 0, 0);
-        if (adamw) w = w * keep;
-        const float numerator = lr * (m * inv_c1);
-        const float denominator = sqrtf(v * inv_c2) + eps;
-        store_rounded<STOCHASTIC>(weight, j, weight_dtype, w - numerator / denominator, (uint64_t)j + offset, step, key);
-    }
+                                                    AdamConstants c, uint64_t step, uint64_t key, uint64_t offset) {
+    for (int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < n; j += (int64_t)gridDim.x * blockDim.x)
+        adam_element<STOCHASTIC>(weight, weight_dtype, grad, grad_dtype, first, second, state_dtype, j, c, step, key, offset);
+}
+
+// Many small tensors in one launch: row t of `table` holds {weight, grad, first, second, count, key, offset} as
+// 64-bit words; blockIdx.y walks the tensors, blockIdx.x their elements.
+template <bool STOCHASTIC>
+__global__ __launch_bounds__(256) void adam_table_kernel(const int64_t* __restrict__ table, int weight_dtype, int grad_dtype,
+                                                          int state_dtype, AdamConstants c, uint64_t step) {
+    const int64_t* row = table + (int64_t)blockIdx.y * 7;
+    const int64_t n = row[4];
+    void* weight = reinterpret_cast<void*>(row[0]);
+    const void* grad = reinterpret_cast<const void*>(row[1]);
+    void* first = reinterpret_cast<void*>(row[2]);
+    void* second = reinterpret_cast<void*>(row[3]);
+    for (int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < n; j += (int64_t)gridDim.x * blockDim.x)
+        adam_element<STOCHASTIC>(weight, weight_dtype, grad, grad_dtype, first, second, state_dtype, j, c, step, (uint64_t)row[5], (uint64_t)row[6]);
 }
 
 __global__ __launch_bounds__(256) void copy_scaled_kernel(const void* __restrict__ update, int update_dtype, void* out,
@@ -402,10 +426,30 @@ extern "C" int viola_adam_update(void* weight, int weight_dtype, const void* gra
     VIOLA_CHECK_ARG(viola_is_float(weight_dtype) && viola_is_float(grad_dtype) && viola_is_float(state_dtype) && n >= 0);
     if (n == 0) return 0;
     VIOLA_CHECK_ARG(weight && grad && first && second);
+    const AdamConstants c{lr, decay, b1, b2, inv_c1, inv_c2, eps, adamw, maximize};
     if (rounding && weight_dtype != VIOLA_F32)
-        hipLaunchKernelGGL(adam_kernel<true>, dim3(grid_for(n)), dim3(256), 0, stream, weight, weight_dtype, grad, grad_dtype, first, second, state_dtype, n, lr, decay, b1, b2, inv_c1, inv_c2, eps, (uint64_t)rounding_step, (uint64_t)rounding_key, (uint64_t)offset, adamw, maximize);
+        hipLaunchKernelGGL(adam_kernel<true>, dim3(grid_for(n)), dim3(256), 0, stream, weight, weight_dtype, grad, grad_dtype, first, second, state_dtype, n, c, (uint64_t)rounding_step, (uint64_t)rounding_key, (uint64_t)offset);
     else
-        hipLaunchKernelGGL(adam_kernel<false>, dim3(grid_for(n)), dim3(256), 0, stream, weight, weight_dtype, grad, grad_dtype, first, second, state_dtype, n, lr, decay, b1, b2, inv_c1, inv_c2, eps, (uint64_t)rounding_step, (uint64_t)rounding_key, (uint64_t)offset, adamw, maximize);
+        hipLaunchKernelGGL(adam_kernel<false>, dim3(grid_for(n)), dim3(256), 0, stream, weight, weight_dtype, grad, grad_dtype, first, second, state_dtype, n, c, (uint64_t)rounding_step, (uint64_t)rounding_key, (uint64_t)offset);
+    return viola_launch_status();
+}
+
+extern "C" int viola_adam_update_table(const int64_t* table, int64_t tensors, int64_t max_count, int weight_dtype, int grad_dtype,
+                                       int state_dtype, float lr, float decay, float b1, float b2, float inv_c1, float inv_c2,
+                                       float eps, int rounding, int64_t rounding_step, int adamw, int maximize,
+                                       viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_float(weight_dtype) && viola_is_float(grad_dtype) && viola_is_float(state_dtype));
+    VIOLA_CHECK_ARG(tensors >= 0 && tensors <= 65535 && max_count >= 0);
+    if (tensors == 0 || max_count == 0) return 0;
+    VIOLA_CHECK_ARG(table);
+    const AdamConstants c{lr, decay, b1, b2, inv_c1, inv_c2, eps, adamw, maximize};
+    const int64_t blocks = (max_count + 255) / 256;
+    const dim3 grid((unsigned)(blocks > 1024 ? 1024 : blocks), (unsigned)tensors);
+    if (rounding && weight_dtype != VIOLA_F32)
+        hipLaunchKernelGGL(adam_table_kernel<true>, grid, dim3(256), 0, stream, table, weight_dtype, grad_dtype, state_dtype, c, (uint64_t)rounding_step);
+    else
+        hipLaunchKernelGGL(adam_table_kernel<false>, grid, dim3(256), 0, stream, table, weight_dtype, grad_dtype, state_dtype, c, (uint64_t)rounding_step);
     return viola_launch_status();
 }
 

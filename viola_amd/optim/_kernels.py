@@ -76,3 +76,29 @@ def adam_update(weight, grad, first, second, *, lr, weight_decay, betas, eps, st
               float(b1), float(b2), 1. / (1. - b1 ** step) if bias_correction else 1.,
               1. / (1. - b2 ** step) if bias_correction else 1., float(eps), _lib.ROUNDING[rounding],
               int(step - 1), int(key), int(offset), int(bool(adamw)), int(bool(maximize)))
+
+
+def adam_update_many(items, *, lr, weight_decay, betas, eps, step, rounding="nearest", adamw=True, maximize=False,
+                     bias_correction=True, cache=None):
+    """adam_update for a list of (weight, grad, first, second, key, offset) sharing dtypes and step, in one launch.
+    cache: a dict that keeps the device-side pointer table between calls (it is rebuilt when any pointer moves)."""
+    weight, grad, first, second, _, _ = items[0]
+    b1, b2 = betas
+    rows = []
+    for w, g, m, v, key, offset in items:
+        assert w.is_cuda and w.is_contiguous() and g.is_contiguous() and m.is_contiguous() and v.is_contiguous()
+        assert (w.dtype, g.dtype, m.dtype, v.dtype) == (weight.dtype, grad.dtype, first.dtype, first.dtype)
+        assert g.numel() == m.numel() == v.numel() == w.numel()
+        rows.append((w.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), w.numel(), int(key), int(offset)))
+    held = cache.get("rows") if cache is not None else None
+    if held == rows:
+        table = cache["table"]
+    else:
+        staging = torch.tensor(rows, dtype=torch.int64).pin_memory()
+        table = staging.to(weight.device, non_blocking=True)
+        if cache is not None:
+            cache.update(rows=rows, table=table, staging=staging)
+    _lib.call("viola_adam_update_table", _lib.ptr(table), len(rows), max(r[4] for r in rows), _lib.code(weight.dtype),
+              _lib.code(grad.dtype), _lib.code(first.dtype), float(lr), float(weight_decay), float(b1), float(b2),
+              1. / (1. - b1 ** step) if bias_correction else 1., 1. / (1. - b2 ** step) if bias_correction else 1.,
+              float(eps), _lib.ROUNDING[rounding], int(step - 1), int(bool(adamw)), int(bool(maximize)))

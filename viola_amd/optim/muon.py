@@ -9,7 +9,7 @@ import torch
 
 from .matrix import MatrixOptimizer
 from ..precision import _dtype, settings
-from ._kernels import adam_update, momentum_update, state_sizes, weight_update
+from ._kernels import adam_update, adam_update_many, momentum_update, state_sizes, weight_update
 from ._orthogonalize import METHODS
 
 _MODES = {"fast": (256, 3), "balanced": (256, 5), "stable": (128, 5)}
@@ -50,6 +50,7 @@ class FP8Muon(MatrixOptimizer):
             master_rounding_seed=policy["master_rounding_seed"])
         self.observer = None
         self._workspace = {}
+        self._adam_tables = {}
         super().__init__(params, defaults, shard_state=shard_state, skip_nonfinite=skip_nonfinite)
 
     def add_param_group(self, group):
@@ -115,11 +116,14 @@ class FP8Muon(MatrixOptimizer):
     def _step_all(self, work):
         if self.observer is not None:
             return super()._step_all(work)
-        buckets = {}
+        buckets, vectors = {}, {}
         for item in work:
             param, grad, state, group, index = item
             if not _use_muon(param, group):
-                self._step_local(*item)
+                state.setdefault("step", 0)
+                key = (param.device, param.dtype, grad.dtype, group["adam_state_dtype"], group["lr"], group["weight_decay"],
+                       tuple(group["betas"]), group["eps"], state["step"], group["master_rounding"])
+                vectors.setdefault(key, []).append(item)
                 continue
             shape = _shape(param, group)
             key = (shape, param.device, group["ns_method"], group["ns_steps"])
@@ -129,6 +133,32 @@ class FP8Muon(MatrixOptimizer):
                 self._step_bucket(buckets.pop(key))
         for bucket in buckets.values():
             self._step_bucket(bucket)
+        for key, bucket in vectors.items():
+            self._step_vectors(key, bucket)
+
+    # Vectors (biases, norms, modulation tables) are a few thousand elements each: those that share dtypes,
+    # hyper-parameters and step count take AdamW in one launch over a table of their pointers.
+    def _step_vectors(self, key, bucket):
+        if len(bucket) == 1 or any(not item[1].is_contiguous() or not item[0].is_contiguous() for item in bucket):
+            for item in bucket:
+                self._step_local(*item)
+            return
+        items = []
+        for param, grad, state, group, index in bucket:
+            assert param.is_cuda and not grad.is_sparse
+            assert param.dtype in (torch.float32, torch.bfloat16, torch.float16), \
+                "Bind FP8 modules with viola.optim.bind_optimizer before stepping."
+            if "exp_avg" not in state:
+                state["exp_avg"] = torch.zeros_like(param, dtype=group["adam_state_dtype"])
+                state["exp_avg_sq"] = torch.zeros_like(param, dtype=group["adam_state_dtype"])
+            master_key = (group["master_rounding_seed"] + index * 0x517CC1B727220A95) & _MASK63
+            items.append((param, grad, state["exp_avg"], state["exp_avg_sq"], master_key, 0))
+        param, grad, state, group, index = bucket[0]
+        adam_update_many(items, lr=group["lr"], weight_decay=group["weight_decay"], betas=group["betas"], eps=group["eps"],
+                         step=state["step"] + 1, rounding=group["master_rounding"],
+                         cache=self._adam_tables.setdefault(key[:4] + (len(bucket),), {}))
+        for _, _, state, _, _ in bucket:
+            state["step"] += 1
 
     def _step_bucket(self, bucket):
         param, _, _, group, _ = bucket[0]
