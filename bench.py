@@ -121,8 +121,8 @@ def cpu_baseline():
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=20)
-    parser.add_argument("--warmup", type=int, default=3)
+    parser.add_argument("--steps", type=int, default=200)
+    parser.add_argument("--warmup", type=int, default=50)
     parser.add_argument("--skip-cpu", action="store_true", help="leave out the CPU baseline leg")
     parser.add_argument("--skip-muon", action="store_true", help="leave out the FP8Muon / codec legs")
     parser.add_argument("--calibrate", action="store_true",

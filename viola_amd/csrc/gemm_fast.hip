@@ -199,24 +199,28 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
         goff_b[it] = (uint32_t)(b_global_row(r) * p.ldb + piece * 16);        // relative to bptr + k_begin (row span < 2 GiB)
         piece_k[it] = piece * 16;
     }
-    constexpr int B_LOADS = TN;                                              // 64 b rows per load instruction
     // scales: per block of 8 K groups the thread fetches groups 4 shalf .. 4 shalf + 3 of tile row srow
     const int srow = tid % BM, shalf = tid / BM;
     const uint32_t sa_off = (uint32_t)(a_global_row(srow) / p.ar * p.ldsa * 4 + ((k_begin >> 5) + shalf * 4) * 4);
     const uint32_t sb_off = (uint32_t)(b_global_row(srow) / p.br * p.ldsb * 4 + ((k_begin >> 5) + shalf * 4) * 4);
+    constexpr int B_LOADS = TN;                                              // 64 b rows per load instruction
     const int64_t k_len = k_end - k_begin;
     const int groups_total = (int)((k_len + 31) / 32);
     const int64_t chunks = (k_len + FBK - 1) / FBK;
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
-    auto issue = [&](int64_t c, int stage) {
+    // load instruction `which` (0, 1: a; 2, 3: b) of chunk c into ring stage `stage`
+    auto issue_one = [&](int64_t c, int stage, int which) {
         const int64_t k0 = c * FBK;                                          // relative to k_begin
         const uint32_t base = lds_base + (uint32_t)stage * F_STAGE + (uint32_t)wave * 1024;
+        const int it = which & 1;
+        const bool inside = k0 + piece_k[it] < k_len;
+        if (which < 2) load16_to_lds(res_a, base + it * 4096, inside ? goff_a[it] : OUTSIDE, (uint32_t)k0);
+        else load16_to_lds(res_b, base + F_TILE + it * 4096, inside ? goff_b[it] : OUTSIDE, (uint32_t)k0);
+    };
+    constexpr int CHUNK_LOADS = 2 + B_LOADS;
+    auto issue = [&](int64_t c, int stage) {
 #pragma unroll
-        for (int it = 0; it < 2; ++it) {
-            const bool inside = k0 + piece_k[it] < k_len;
-            load16_to_lds(res_a, base + it * 4096, inside ? goff_a[it] : OUTSIDE, (uint32_t)k0);
-            if (it < B_LOADS) load16_to_lds(res_b, base + F_TILE + it * 4096, inside ? goff_b[it] : OUTSIDE, (uint32_t)k0);
-        }
+        for (int i = 0; i < CHUNK_LOADS; ++i) issue_one(c, stage, i);
     };
     // scale block `block` (K groups 8 block .. 8 block + 7 of the k range) -> raw area, one 16-byte piece per thread
     // and operand; a piece wholly past the k range is not fetched
@@ -266,41 +270,49 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
     for (int r = 0; r < 16; ++r) acc[0][r] = acc[1][r] = acc[2][r] = acc[3][r] = 0.0f;
     auto as_long = [](uint32_t lo, uint32_t hi) -> long { return (long)(((uint64_t)hi << 32) | lo); };
 
-    auto compute = [&](int stage, int64_t c) {
+    // The MFMA operands and scales of one chunk, in registers. They are read from LDS one chunk ahead of their
+    // math (two register sets, the chunk loop is unrolled by two), so a wavefront goes from the barrier straight
+    // into its math and the LDS latency of the next chunk hides under it.
+    struct Operands {
+        uint4 a[FKG][TM], b[FKG][TN];
+        float sa[FKG][TM], sb[FKG][TN];
+    };
+    auto scale_block = [&](int64_t c) -> const float* {                      // a scales of chunk c: [kg][row]; b scales F_SBLOCK later
+        return reinterpret_cast<const float*>(lds + F_SCALE + ((c / F_SCHUNKS) & 1) * 2 * F_SBLOCK) + (c % F_SCHUNKS) * FKG * BM;
+    };
+    auto read_operands = [&](int stage, int64_t c, Operands& o) {
         const uint8_t* tile_a = lds + stage * F_STAGE;
         const uint8_t* tile_b = tile_a + F_TILE;
-        const float* scale_a = reinterpret_cast<const float*>(lds + F_SCALE + ((c / F_SCHUNKS) & 1) * 2 * F_SBLOCK) + (c % F_SCHUNKS) * FKG * BM;
+        const float* scale_a = scale_block(c);
         const float* scale_b = scale_a + F_SBLOCK / 4;
-        uint4 opa[FKG][TM], opb[FKG][TN];
-        float sa_l[FKG][TM], sb_u[FKG][TN];
-        float4 sb_q[FKG][TN][4];                                             // row-wise b scales of the lane's 16 columns
 #pragma unroll
         for (int kg = 0; kg < FKG; ++kg) {
 #pragma unroll
-            for (int j = 0; j < TM; ++j) opa[kg][j] = *reinterpret_cast<const uint4*>(tile_a + ((rd_a + j * 32 * FBK) ^ (kg * 32)));
+            for (int j = 0; j < TM; ++j) o.a[kg][j] = *reinterpret_cast<const uint4*>(tile_a + ((rd_a + j * 32 * FBK) ^ (kg * 32)));
 #pragma unroll
-            for (int i = 0; i < TN; ++i) opb[kg][i] = *reinterpret_cast<const uint4*>(tile_b + ((rd_b + (b_sub(i) - b_sub(0)) * FBK) ^ (kg * 32)));
+            for (int i = 0; i < TN; ++i) o.b[kg][i] = *reinterpret_cast<const uint4*>(tile_b + ((rd_b + (b_sub(i) - b_sub(0)) * FBK) ^ (kg * 32)));
 #pragma unroll
-            for (int j = 0; j < TM; ++j) sa_l[kg][j] = scale_a[kg * BM + a_sub(j) + l32];
-            if constexpr (!B_ROWSCALE) {
+            for (int j = 0; j < TM; ++j) o.sa[kg][j] = scale_a[kg * BM + a_sub(j) + l32];
 #pragma unroll
-                for (int i = 0; i < TN; ++i) sb_u[kg][i] = scale_b[kg * BM + b_sub(i)];
-            } else {
-#pragma unroll
-                for (int i = 0; i < TN; ++i)
-#pragma unroll
-                    for (int r4 = 0; r4 < 4; ++r4)
-                        sb_q[kg][i][r4] = *reinterpret_cast<const float4*>(&scale_b[kg * BM + b_sub(i) + r4 * 8 + lhi * 4]);
-            }
+            for (int i = 0; i < TN; ++i) o.sb[kg][i] = B_ROWSCALE ? 0.0f : scale_b[kg * BM + b_sub(i)];
         }
+    };
+
+    // Math of chunk c on the operands in `o`; `between(step)` runs after MFMA number `step` of the chunk (the
+    // caller's global loads and LDS reads for later chunks go there, spread over the chunk).
+    auto compute = [&](const Operands& o, int64_t c, auto&& between) {
+        // row-wise b scales of the lane's 16 columns for one pair of units (both share K group and b sub-tile): two
+        // slots, pair p loads slot p & 1 before its MFMAs and its fold reads it during pair p + 1
+        float4 sb_q[2][4];
+        const float* scale_b = scale_block(c) + F_SBLOCK / 4;
         // fold half `h` (registers 8h .. 8h+7) of accumulator `buf` into total[i][j]
-        auto fold_half = [&](int buf, int i, int j, int kg, int h, float scale) {
+        auto fold_half = [&](int buf, int i, int j, int slot, int h, float scale) {
 #pragma unroll
             for (int r = 8 * h; r < 8 * h + 8; ++r) {
                 if constexpr (!B_ROWSCALE) {
                     total[i][j][r] = fmaf(acc[buf][r], scale, total[i][j][r]);
                 } else {
-                    const float4 q = sb_q[kg][i][r / 4];
+                    const float4 q = sb_q[slot][r / 4];
                     const float sbv = r % 4 == 0 ? q.x : r % 4 == 1 ? q.y : r % 4 == 2 ? q.z : q.w;
                     total[i][j][r] = fmaf(acc[buf][r], scale * sbv, total[i][j][r]);
                 }
@@ -322,21 +334,27 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
                 const int unit = 2 * pair + h, prev = 2 * before + h;
                 kg[h] = unit / (TN * TM); ti[h] = unit / TM % TN; tj[h] = unit % TM;
                 pkg[h] = prev / (TN * TM); pi[h] = prev / TM % TN; pj[h] = prev % TM;
-                prev_scale[h] = B_ROWSCALE ? (pair > 0 ? sa_l[pkg[h]][pj[h]] : 0.0f) : pending_scale[h];
+                prev_scale[h] = B_ROWSCALE ? (pair > 0 ? o.sa[pkg[h]][pj[h]] : 0.0f) : pending_scale[h];
+            }
+            if constexpr (B_ROWSCALE) {
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4)
+                    sb_q[pair & 1][r4] = *reinterpret_cast<const float4*>(&scale_b[kg[0] * BM + b_sub(ti[0]) + r4 * 8 + lhi * 4]);
             }
 #pragma unroll
             for (int step = 0; step < 4; ++step) {
                 const int h = step & 1, ks = step >> 1;
-                const uint4 ob = opb[kg[h]][ti[h]], oa = opa[kg[h]][tj[h]];
+                const uint4 ob = o.b[kg[h]][ti[h]], oa = o.a[kg[h]][tj[h]];
                 if (ks == 0) acc[base + h] = mfma32<A_BF8, B_BF8>(as_long(ob.x, ob.y), as_long(oa.x, oa.y), zero);
                 else acc[base + h] = mfma32<A_BF8, B_BF8>(as_long(ob.z, ob.w), as_long(oa.z, oa.w), acc[base + h]);
-                if (fold_prev) fold_half(other + (step >> 1), pi[step >> 1], pj[step >> 1], pkg[step >> 1], step & 1, prev_scale[step >> 1]);
+                if (fold_prev) fold_half(other + (step >> 1), pi[step >> 1], pj[step >> 1], before & 1, step & 1, prev_scale[step >> 1]);
                 asm volatile("" : "+v"(total[pi[step >> 1]][pj[step >> 1]]));
                 __builtin_amdgcn_sched_barrier(0);
+                between(pair * 4 + step);
             }
             if constexpr (!B_ROWSCALE) {
 #pragma unroll
-                for (int h = 0; h < 2; ++h) pending_scale[h] = sa_l[kg[h]][tj[h]] * sb_u[kg[h]][ti[h]];
+                for (int h = 0; h < 2; ++h) pending_scale[h] = o.sa[kg[h]][tj[h]] * o.sb[kg[h]][ti[h]];
             }
         }
         if constexpr (!CARRY) {
@@ -345,33 +363,48 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
                 constexpr int last_pair = PAIRS - 1;
                 const int unit = 2 * last_pair + h;
                 const int lkg = unit / (TN * TM), li = unit / TM % TN, lj = unit % TM;
-                fold_half((last_pair & 1) * 2 + h, li, lj, lkg, 0, sa_l[lkg][lj]);
-                fold_half((last_pair & 1) * 2 + h, li, lj, lkg, 1, sa_l[lkg][lj]);
+                fold_half((last_pair & 1) * 2 + h, li, lj, last_pair & 1, 0, o.sa[lkg][lj]);
+                fold_half((last_pair & 1) * 2 + h, li, lj, last_pair & 1, 1, o.sa[lkg][lj]);
             }
         }
     };
 
-    // Per chunk: wait for its loads, one barrier, refill the stage read last, math. Every fourth chunk also fetches
-    // the next scale block (first chunk of a block) or rearranges it (last chunk of the block before).
+    // Ring of three stages, chunk c in stage c % 3. At the top of iteration c the wave waits for its own loads of
+    // chunk c+1 (issued two iterations ago) and for its LDS reads of chunk c; after the barrier chunk c+1 is in LDS
+    // for everybody and nobody reads chunk c's stage any more. Then: the loads of chunk c+3 into that stage (one
+    // instruction every few MFMAs, so the waves of a CU do not queue up at the memory pipe), the LDS reads of chunk
+    // c+1 into the other register set, the math of chunk c. Scale block b (K groups 8b ..) is fetched in iteration
+    // 4b-4, rearranged in 4b-2 and first read in 4b-1; it is issued before the chunk loads of its iteration, so the
+    // waits below cover it one iteration later.
+    constexpr int STEPS = FKG * TN * TM * 2, STRIDE = STEPS / CHUNK_LOADS;
+    int stage_now = 0, stage_next = 1;
+    auto chunk_step = [&](int64_t c, const Operands& now, Operands& next) {
+        if (c % F_SCHUNKS == 1) __builtin_amdgcn_s_waitcnt(0x0070 | (CHUNK_LOADS + 2));
+        else __builtin_amdgcn_s_waitcnt(0x0070 | CHUNK_LOADS);
+        __syncthreads();
+        if (c % F_SCHUNKS == 0) issue_scales(c / F_SCHUNKS + 1);
+        if (c % F_SCHUNKS == 2) arrange_scales(c / F_SCHUNKS + 1);
+        if (c + 1 < chunks) read_operands(stage_next, c + 1, next);
+        const int fill = stage_now;
+        compute(now, c, [&](int step) {
+            if (step % STRIDE == 0 && step / STRIDE < CHUNK_LOADS) issue_one(c + 3, fill, step / STRIDE);
+        });
+        stage_now = stage_next;
+        stage_next = stage_next == FSTAGES - 1 ? 0 : stage_next + 1;
+    };
     issue_scales(0);
     issue(0, 0);
     issue(1, 1);
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * (2 + B_LOADS)));               // scale block 0 is in LDS
+    issue(2, 2);
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * CHUNK_LOADS));                   // scale block 0 and chunk 0 are in LDS
     __syncthreads();
     arrange_scales(0);
-    int cur = 0, fill = 2;
-    for (int64_t c = 0; c < chunks; ++c) {
-        // all loads but the newest chunk's (and the scale pieces issued with it) have landed: chunk c is in LDS for
-        // this wave ...
-        if (c % F_SCHUNKS == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 + B_LOADS + 2));
-        else __builtin_amdgcn_s_waitcnt(0x0F70 | (2 + B_LOADS));
-        __syncthreads();                    // ... and for every wave; stage `fill` was last read in chunk c-1
-        issue(c + 2, fill);                 // past the end: zeros into a stage nobody reads
-        if (c % F_SCHUNKS == 0) issue_scales(c / F_SCHUNKS + 1);
-        if (c % F_SCHUNKS == F_SCHUNKS - 1) arrange_scales(c / F_SCHUNKS + 1);
-        compute(cur, c);
-        cur = cur == FSTAGES - 1 ? 0 : cur + 1;
-        fill = fill == FSTAGES - 1 ? 0 : fill + 1;
+    __syncthreads();
+    Operands set0, set1;
+    read_operands(0, 0, set0);
+    for (int64_t c = 0; c < chunks; c += 2) {
+        chunk_step(c, set0, set1);
+        if (c + 1 < chunks) chunk_step(c + 1, set1, set0);
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);     // drain the trailing loads before the LDS allocation is released
     if constexpr (CARRY) {
