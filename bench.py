@@ -3,7 +3,10 @@
 parameter set, the wire codec and quantizer bandwidths, a roofline object for the dominant kernel
 (the grouped-scale FP8 GEMM) and the CPU oracle timed on this host's cores.
 
-    python bench.py --gpus 1 --steps 20 --warmup 3
+    python bench.py --gpus 1 --steps 200 --warmup 50
+
+The defaults are long enough (tens of milliseconds of back-to-back launches) for the GPU to settle at its sustained
+clock: a 20-step run reads some 15 % slower than the steady state a training loop sees.
 
 A step is one `y = layer(x); y.backward(dy)` including every quantize / transpose launch, inputs
 resident in HBM. TFLOP/s = 6*M*K*N / t (the reference's definition, checks/benchmark_linear.py:165).
