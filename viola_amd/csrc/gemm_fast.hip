@@ -5,8 +5,9 @@
 // 2 x 2 sub-tiles of 32 x 32. Two blocks share a CU, so one block's prologue, barrier and output stores
 // run under the other block's math.
 //   * global -> LDS directly (buffer_load ... lds, no staging registers, lanes past the k range read
-//     zero), a ring of three stages: the loads of chunk c+2 fly during the math of chunk c, one barrier
-//     per chunk. Operand rows are 4 x 16 bytes, piece u = 2 * (K group) + half stored in slot
+//     zero), a ring of three stages, one barrier per chunk. During the math of chunk c a wave reads the
+//     MFMA operands of chunk c+1 from LDS into a second register set and issues the loads of chunk c+3,
+//     one instruction every few MFMAs, into the stage chunk c has vacated. Operand rows are 4 x 16 bytes, piece u = 2 * (K group) + half stored in slot
 //     u ^ ((row >> 2) & 3), which spreads the 16 rows of a ds_read_b128 group over all banks. A lane
 //     takes 16 consecutive bytes of a 32-byte K group (half = lane / 32): the first 8 feed the first
 //     MFMA of the group, the last 8 the second -- a and b use the same split, so every product meets its
