@@ -172,11 +172,13 @@ def main():
                     else:
                         ns_flops += 5 * 6 * m_ ** 3 if m_ == n_ else 8 * m_ * m_ * n_ + 28 * m_ ** 3
             ns_ms = b["viola_ns_gemm"]["avg_ms"] * b["viola_ns_gemm"]["launches_per_step"]
-            mom = b["viola_momentum_update"]
+            mom = b.get("viola_momentum_update_table") or b["viola_momentum_update"]
+            upd = b.get("viola_weight_update_table") or b["viola_weight_update"]
             extra[f"muon_{method}"] = dict(step_ms=step_ms, step_wall_ms=step_wall, muon_elements=elements,
                                            ns_gemm_ms=ns_ms, ns_tflops=ns_flops / (ns_ms * 1e-3) / 1e12,
                                            ns_frac_bf16_peak=ns_flops / (ns_ms * 1e-3) / 1e12 / PEAK["bf16_tflops"],
                                            momentum_gbs=8.03 * elements / (mom["avg_ms"] * mom["launches_per_step"] * 1e-3) / 1e9,
+                                           weight_update_gbs=10 * elements / (upd["avg_ms"] * upd["launches_per_step"] * 1e-3) / 1e9,
                                            launches_per_step=sum(v["launches_per_step"] for v in b.values()))
             del opt, params
             torch.cuda.empty_cache()

@@ -149,8 +149,23 @@ int viola_adam_update(void* weight, int weight_dtype, const void* grad, int grad
                       int rounding, int64_t rounding_step, int64_t rounding_key, int64_t offset,
                       int adamw, int maximize, viola_stream_t stream);
 
+/* viola_momentum_update (1-D tiles of 256 / 512 / 1024, whole tiles only) for many tensors with the same number of
+ * tiles, gradient dtype and hyper-parameters, in one launch (the reference launches once per matrix,
+ * viola/optim/muon.py:104-106). table: device array of `tensors` rows of eight int64: {grad, old_q, old_scale, new_q,
+ * new_scale, update, rounding key, 0}; the gradient must be aligned to four elements, the codes to 4
+ * bytes and the bf16 update to 8 bytes; old and new state may alias. */
+int viola_momentum_update_table(const int64_t* table, int64_t tensors, int64_t tiles, int grad_dtype, int tile_size,
+                                float beta, float inv_loss_scale, int nesterov, int rounding, int64_t rounding_step,
+                                viola_stream_t stream);
+
+/* viola_weight_update with nearest rounding for many fp32 tensors of `count` elements each (a multiple of 4), one
+ * launch (the reference: one launch per matrix, viola/optim/muon.py:131-132). table: rows of two int64:
+ * {weight (16-byte aligned), update (aligned to four elements of grad_dtype)}. */
+int viola_weight_update_table(const int64_t* table, int64_t tensors, int64_t count, int grad_dtype, float lr, float decay,
+                              float update_scale, viola_stream_t stream);
+
 /* The same update for many tensors that share dtypes, hyper-parameters and step count, in one launch (the reference
- * calls adam_update once per parameter, viola/optim/muon.py:122-128; vectors of a transformer are a few thousand
+ * calls adam_update once per parameter, viola/optim/muon.py:137-140; vectors of a transformer are a few thousand
  * elements each, so their launches dominate). table: device array of `tensors` rows of seven int64:
  * {weight pointer, grad pointer, first pointer, second pointer, element count, rounding key, rounding offset};
  * max_count: the largest element count. */

@@ -203,7 +203,7 @@ def test_stochastic_master_rounding(dtype):
 @pytest.mark.parametrize("wdtype,rounding", [(torch.float32, "nearest"), (torch.bfloat16, "nearest"), (torch.bfloat16, "stochastic"),
                                              (torch.float16, "stochastic")])
 def test_adam_table_equals_per_tensor_and_oracle(wdtype, rounding):
-    """One launch over a pointer table == one adam_update per tensor (viola/optim/muon.py:122-128), bit for bit,
+    """One launch over a pointer table == one adam_update per tensor (viola/optim/muon.py:137-140), bit for bit,
     ragged sizes from 1 element to beyond one grid stride, own rounding key per tensor."""
     k = _k()
     torch.manual_seed(31)
@@ -228,6 +228,41 @@ def test_adam_table_equals_per_tensor_and_oracle(wdtype, rounding):
     for step in (1, 2):
         rw, rm, rv = oo.adam_update(rw, grads[4], rm, rv, step=step, rounding=rounding, key=1004, offset=12, **hyper)
     assert torch.equal(many[4][0].cpu(), rw) and torch.equal(many[4][2].cpu(), rm) and torch.equal(many[4][3].cpu(), rv)
+
+
+@pytest.mark.parametrize("gdtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rounding", ["nearest", "stochastic"])
+@pytest.mark.parametrize("tile_size", [256, 1024])
+def test_momentum_and_weight_tables_equal_per_tensor(gdtype, rounding, tile_size):
+    """One launch over a pointer table == one momentum_update / weight_update per matrix (viola/optim/muon.py:104-106,
+    131-132), bit for bit: codes, scales, bf16 update and fp32 weights, over two steps (the second starts from state)."""
+    k = _k()
+    torch.manual_seed(41)
+    n, tensors = 12 * 1024, 5
+    grads = [(torch.randn(n, device="cuda") * 10. ** (i - 2)).to(gdtype) for i in range(tensors)]
+    grads[2][5] = float("inf")                                                  # a poisoned tile takes the division path
+    def state():
+        return [(torch.zeros(n, dtype=torch.uint8, device="cuda"), torch.ones(n // tile_size, device="cuda"),
+                 torch.empty(n, dtype=torch.bfloat16, device="cuda")) for _ in range(tensors)]
+    many, single = state(), state()
+    w_many = [torch.randn(n, device="cuda") for _ in range(tensors)]
+    w_single = [w.clone() for w in w_many]
+    caches = ({}, {})
+    for step in (0, 1):
+        assert k.momentum_update_many([(g, q, s, out, 77 + i) for i, (g, (q, s, out)) in enumerate(zip(grads, many))], beta=.95,
+                                      tile_size=tile_size, rounding=rounding, rounding_step=step, cache=caches[0])
+        assert k.weight_update_many([(w, out) for w, (_, _, out) in zip(w_many, many)], 1e-3, .01, update_scale=.7, cache=caches[1])
+        for i, (g, (q, s, out)) in enumerate(zip(grads, single)):
+            k.momentum_update(g, q, s, q, s, out, beta=.95, tile_size=tile_size, rounding=rounding, rounding_step=step, rounding_key=77 + i)
+            k.weight_update(w_single[i], out, 1e-3, .01, update_scale=.7)
+    for a, b in zip(many, single):
+        assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+        assert torch.equal(a[2].view(torch.int16), b[2].view(torch.int16))
+    for a, b in zip(w_many, w_single):
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+    # shapes the table kernels decline are reported, not mangled
+    assert not k.momentum_update_many([(grads[0][:300], many[0][0], many[0][1], many[0][2], 0)], beta=.95, tile_size=256)
+    assert not k.weight_update_many([(w_many[0][:6], many[0][2][:6])], 1e-3, .01)
 
 
 def test_copy_scaled():

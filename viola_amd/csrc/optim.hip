@@ -103,13 +103,10 @@ template <> __device__ __forceinline__ void load_quad<f16_t>(const f16_t* p, flo
 }
 
 template <typename TG, int EPL, bool STOCHASTIC>
-__global__ __launch_bounds__(256) void momentum_1d_quads(const TG* __restrict__ grad, const uint8_t* old_q,
-                                                          const float* old_scale, uint8_t* new_q, float* new_scale,
-                                                          uint16_t* __restrict__ update, int64_t blocks, float beta,
-                                                          float inv_loss_scale, int nesterov, uint64_t step, uint64_t key) {
+__device__ __forceinline__ void momentum_quads_tile(const TG* __restrict__ grad, const uint8_t* old_q, const float* old_scale,
+                                                    uint8_t* new_q, float* new_scale, uint16_t* __restrict__ update, int64_t b,
+                                                    float beta, float inv_loss_scale, int nesterov, uint64_t step, uint64_t key) {
     constexpr int TILE = EPL * WAVE, QUADS = EPL / 4;
-    const int64_t b = (int64_t)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
-    if (b >= blocks) return;
     const int lane = threadIdx.x % WAVE;
     const float scale_old = old_scale[b];
     const float one_minus = 1.0f - beta;
@@ -167,6 +164,30 @@ __global__ __launch_bounds__(256) void momentum_1d_quads(const TG* __restrict__ 
         }
         *reinterpret_cast<uint2*>(update + i) = make_uint2(f32_to_bf16x2_bits(u[0], u[1]), f32_to_bf16x2_bits(u[2], u[3]));
     }
+}
+
+template <typename TG, int EPL, bool STOCHASTIC>
+__global__ __launch_bounds__(256) void momentum_1d_quads(const TG* __restrict__ grad, const uint8_t* old_q,
+                                                          const float* old_scale, uint8_t* new_q, float* new_scale,
+                                                          uint16_t* __restrict__ update, int64_t blocks, float beta,
+                                                          float inv_loss_scale, int nesterov, uint64_t step, uint64_t key) {
+    const int64_t b = (int64_t)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (b >= blocks) return;
+    momentum_quads_tile<TG, EPL, STOCHASTIC>(grad, old_q, old_scale, new_q, new_scale, update, b, beta, inv_loss_scale, nesterov, step, key);
+}
+
+// Many tensors of `blocks` whole tiles each in one launch: row t of `table` holds {grad, old_q, old_scale, new_q,
+// new_scale, update, rounding key, 0} as 64-bit words; blockIdx.y walks the tensors.
+template <typename TG, int EPL, bool STOCHASTIC>
+__global__ __launch_bounds__(256) void momentum_table_quads(const int64_t* __restrict__ table, int64_t blocks, float beta,
+                                                             float inv_loss_scale, int nesterov, uint64_t step) {
+    const int64_t b = (int64_t)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (b >= blocks) return;
+    const int64_t* row = table + (int64_t)blockIdx.y * 8;
+    momentum_quads_tile<TG, EPL, STOCHASTIC>(reinterpret_cast<const TG*>(row[0]), reinterpret_cast<const uint8_t*>(row[1]),
+                                             reinterpret_cast<const float*>(row[2]), reinterpret_cast<uint8_t*>(row[3]),
+                                             reinterpret_cast<float*>(row[4]), reinterpret_cast<uint16_t*>(row[5]), b, beta,
+                                             inv_loss_scale, nesterov, step, (uint64_t)row[6]);
 }
 
 // ------------------------------------------------------------------ 2-D blocks: one wavefront per block
@@ -239,6 +260,24 @@ __global__ __launch_bounds__(256) void weight_quads_kernel(float* weight, const 
                                                             float decay, float update_scale) {
     const float keep = 1.0f - lr * decay;
     const float rate = lr * update_scale;
+    for (int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < quads; j += (int64_t)gridDim.x * blockDim.x) {
+        float4 w = reinterpret_cast<const float4*>(weight)[j];
+        float g[4];
+        load_quad<TG>(grad + 4 * j, g);
+        const float t0[4] = {w.x * keep, w.y * keep, w.z * keep, w.w * keep};
+        const float t1[4] = {rate * g[0], rate * g[1], rate * g[2], rate * g[3]};
+        reinterpret_cast<float4*>(weight)[j] = make_float4(t0[0] - t1[0], t0[1] - t1[1], t0[2] - t1[2], t0[3] - t1[3]);
+    }
+}
+
+// Many fp32 tensors of `quads` whole quads each: row t of `table` holds {weight, update}; blockIdx.y walks the tensors.
+template <typename TG>
+__global__ __launch_bounds__(256) void weight_table_quads_kernel(const int64_t* __restrict__ table, int64_t quads, float lr,
+                                                                  float decay, float update_scale) {
+    const float keep = 1.0f - lr * decay;
+    const float rate = lr * update_scale;
+    float* weight = reinterpret_cast<float*>(table[(int64_t)blockIdx.y * 2]);
+    const TG* grad = reinterpret_cast<const TG*>(table[(int64_t)blockIdx.y * 2 + 1]);
     for (int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < quads; j += (int64_t)gridDim.x * blockDim.x) {
         float4 w = reinterpret_cast<const float4*>(weight)[j];
         float g[4];
@@ -388,6 +427,44 @@ extern "C" int viola_momentum_update(const void* grad, int grad_dtype, const voi
     const dim3 grid((unsigned)((tiles + 3) / 4));
     if (rounding) hipLaunchKernelGGL((momentum_2d_kernel<true>), grid, dim3(256), 0, stream, grad, grad_dtype, oq, old_scale, nq, new_scale, up, planes, rows, cols, tr, tc, beta, inv_loss_scale, nesterov, step, key);
     else hipLaunchKernelGGL((momentum_2d_kernel<false>), grid, dim3(256), 0, stream, grad, grad_dtype, oq, old_scale, nq, new_scale, up, planes, rows, cols, tr, tc, beta, inv_loss_scale, nesterov, step, key);
+    return viola_launch_status();
+}
+
+extern "C" int viola_momentum_update_table(const int64_t* table, int64_t tensors, int64_t tiles, int grad_dtype, int tile_size,
+                                           float beta, float inv_loss_scale, int nesterov, int rounding, int64_t rounding_step,
+                                           viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_float(grad_dtype) && tensors >= 0 && tensors <= 65535 && tiles >= 0 && (tiles + 3) / 4 < (1ll << 31));
+    VIOLA_CHECK_ARG(tile_size == 256 || tile_size == 512 || tile_size == 1024);
+    VIOLA_CHECK_ARG(rounding == VIOLA_NEAREST || rounding == VIOLA_STOCHASTIC);
+    if (tensors == 0 || tiles == 0) return 0;
+    VIOLA_CHECK_ARG(table);
+    const dim3 grid((unsigned)((tiles + 3) / 4), (unsigned)tensors);
+#define VIOLA_MT(TG, EPL)                                                                                                   \
+    if (rounding) hipLaunchKernelGGL((momentum_table_quads<TG, EPL, true>), grid, dim3(256), 0, stream, table, tiles, beta, inv_loss_scale, nesterov, (uint64_t)rounding_step); \
+    else hipLaunchKernelGGL((momentum_table_quads<TG, EPL, false>), grid, dim3(256), 0, stream, table, tiles, beta, inv_loss_scale, nesterov, (uint64_t)rounding_step);
+#define VIOLA_MTT(EPL)                                                          \
+    if (grad_dtype == VIOLA_F32) { VIOLA_MT(float, EPL) }                        \
+    else if (grad_dtype == VIOLA_BF16) { VIOLA_MT(bf16_t, EPL) }                 \
+    else { VIOLA_MT(f16_t, EPL) }
+    if (tile_size == 256) { VIOLA_MTT(4) } else if (tile_size == 512) { VIOLA_MTT(8) } else { VIOLA_MTT(16) }
+#undef VIOLA_MTT
+#undef VIOLA_MT
+    return viola_launch_status();
+}
+
+extern "C" int viola_weight_update_table(const int64_t* table, int64_t tensors, int64_t count, int grad_dtype, float lr,
+                                         float decay, float update_scale, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_float(grad_dtype) && tensors >= 0 && tensors <= 65535 && count >= 0 && count % 4 == 0);
+    if (tensors == 0 || count == 0) return 0;
+    VIOLA_CHECK_ARG(table);
+    const int64_t quads = count / 4;
+    const int64_t blocks = (quads + 255) / 256;
+    const dim3 grid((unsigned)(blocks > 4096 ? 4096 : blocks), (unsigned)tensors);
+    if (grad_dtype == VIOLA_F32) hipLaunchKernelGGL(weight_table_quads_kernel<float>, grid, dim3(256), 0, stream, table, quads, lr, decay, update_scale);
+    else if (grad_dtype == VIOLA_BF16) hipLaunchKernelGGL(weight_table_quads_kernel<bf16_t>, grid, dim3(256), 0, stream, table, quads, lr, decay, update_scale);
+    else hipLaunchKernelGGL(weight_table_quads_kernel<f16_t>, grid, dim3(256), 0, stream, table, quads, lr, decay, update_scale);
     return viola_launch_status();
 }
 

@@ -78,6 +78,58 @@ def adam_update(weight, grad, first, second, *, lr, weight_decay, betas, eps, st
               int(step - 1), int(key), int(offset), int(bool(adamw)), int(bool(maximize)))
 
 
+def _device_table(rows, device, cache):
+    """int64 rows as a device tensor; `cache` (a dict) keeps it between calls and it is rebuilt when any entry changes."""
+    held = cache.get("rows") if cache is not None else None
+    if held == rows:
+        return cache["table"]
+    staging = torch.tensor(rows, dtype=torch.int64).pin_memory()
+    table = staging.to(device, non_blocking=True)
+    if cache is not None:
+        cache.update(rows=rows, table=table, staging=staging)
+    return table
+
+
+def momentum_update_many(items, *, beta, tile_size=256, nesterov=True, loss_scale=1.0, rounding="nearest", rounding_step=0,
+                         cache=None):
+    """momentum_update (granularity="tile", state advanced in place) for a list of (grad, q, scales, out, key) with
+    equal element counts (whole tiles), in one launch. Returns False, having done nothing, when the tensors do not fit
+    the kernel (ragged tiles, small tiles, odd alignment, mixed dtypes)."""
+    grad = items[0][0]
+    n = grad.numel()
+    if tile_size < 256 or n % tile_size or len(items) > 65535:
+        return False
+    rows = []
+    for g, q, s, out, key in items:
+        if (g.dtype != grad.dtype or g.numel() != n or not g.is_contiguous() or g.data_ptr() % (4 * g.element_size())
+                or q.data_ptr() % 4 or out.data_ptr() % 8 or out.dtype != torch.bfloat16):
+            return False
+        rows.append((g.data_ptr(), q.data_ptr(), s.data_ptr(), q.data_ptr(), s.data_ptr(), out.data_ptr(), int(key), 0))
+    table = _device_table(rows, grad.device, cache)
+    _lib.call("viola_momentum_update_table", _lib.ptr(table), len(rows), n // tile_size, _lib.code(grad.dtype), int(tile_size),
+              float(beta), 1.0 / float(loss_scale), int(bool(nesterov)), _lib.ROUNDING[rounding], int(rounding_step))
+    return True
+
+
+def weight_update_many(items, lr, weight_decay, *, update_scale=1.0, cache=None):
+    """weight_update with nearest rounding for a list of (fp32 weight, update) of equal element counts, one launch.
+    Returns False, having done nothing, when the tensors do not fit the kernel."""
+    weight, update = items[0]
+    n = weight.numel()
+    if n % 4 or len(items) > 65535:
+        return False
+    rows = []
+    for w, u in items:
+        if (w.dtype != torch.float32 or u.dtype != update.dtype or w.numel() != n or u.numel() != n or not w.is_contiguous()
+                or not u.is_contiguous() or w.data_ptr() % 16 or u.data_ptr() % (4 * u.element_size())):
+            return False
+        rows.append((w.data_ptr(), u.data_ptr()))
+    table = _device_table(rows, weight.device, cache)
+    _lib.call("viola_weight_update_table", _lib.ptr(table), len(rows), n, _lib.code(update.dtype), float(lr),
+              float(weight_decay), float(update_scale))
+    return True
+
+
 def adam_update_many(items, *, lr, weight_decay, betas, eps, step, rounding="nearest", adamw=True, maximize=False,
                      bias_correction=True, cache=None):
     """adam_update for a list of (weight, grad, first, second, key, offset) sharing dtypes and step, in one launch.
@@ -90,14 +142,7 @@ def adam_update_many(items, *, lr, weight_decay, betas, eps, step, rounding="nea
         assert (w.dtype, g.dtype, m.dtype, v.dtype) == (weight.dtype, grad.dtype, first.dtype, first.dtype)
         assert g.numel() == m.numel() == v.numel() == w.numel()
         rows.append((w.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), w.numel(), int(key), int(offset)))
-    held = cache.get("rows") if cache is not None else None
-    if held == rows:
-        table = cache["table"]
-    else:
-        staging = torch.tensor(rows, dtype=torch.int64).pin_memory()
-        table = staging.to(weight.device, non_blocking=True)
-        if cache is not None:
-            cache.update(rows=rows, table=table, staging=staging)
+    table = _device_table(rows, weight.device, cache)
     _lib.call("viola_adam_update_table", _lib.ptr(table), len(rows), max(r[4] for r in rows), _lib.code(weight.dtype),
               _lib.code(grad.dtype), _lib.code(first.dtype), float(lr), float(weight_decay), float(b1), float(b2),
               1. / (1. - b1 ** step) if bias_correction else 1., 1. / (1. - b2 ** step) if bias_correction else 1.,

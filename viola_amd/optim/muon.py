@@ -9,7 +9,7 @@ import torch
 
 from .matrix import MatrixOptimizer
 from ..precision import _dtype, settings
-from ._kernels import adam_update, adam_update_many, momentum_update, state_sizes, weight_update
+from ._kernels import adam_update, adam_update_many, momentum_update, momentum_update_many, weight_update_many, state_sizes, weight_update
 from ._orthogonalize import METHODS
 
 _MODES = {"fast": (256, 3), "balanced": (256, 5), "stable": (128, 5)}
@@ -51,6 +51,7 @@ class FP8Muon(MatrixOptimizer):
         self.observer = None
         self._workspace = {}
         self._adam_tables = {}
+        self._bucket_tables = {}
         super().__init__(params, defaults, shard_state=shard_state, skip_nonfinite=skip_nonfinite)
 
     def add_param_group(self, group):
@@ -167,22 +168,44 @@ class FP8Muon(MatrixOptimizer):
         work = self._workspace.get(param.device)
         if work is None or work.numel() < len(bucket) * count:
             work = self._workspace[param.device] = torch.empty(len(bucket) * count, device=param.device, dtype=torch.bfloat16)
-        keys = []
-        for slot, (param, grad, state, group, index) in enumerate(bucket):
+        tables = self._bucket_tables.setdefault((shape, param.device, len(bucket)), ({}, {}))
+        # one launch for the momentum of the whole bucket when its members share the recipe, else one per matrix
+        uniform = lambda *names: all(all(item[3][name] == group[name] for name in names) for item in bucket)
+        items = []
+        for slot, (param, grad, state, group_, index) in enumerate(bucket):
             assert param.is_cuda and not grad.is_sparse
             assert param.dtype in (torch.float32, torch.bfloat16, torch.float16), \
                 "Bind FP8 modules with viola.optim.bind_optimizer before stepping."
             state.setdefault("step", 0)
-            key = (group["rounding_seed"] + index * 0x9E3779B97F4A7C15) & _MASK63
-            self._momentum(param, grad, state, group, key, out=work[slot * count:(slot + 1) * count])
+            if "momentum_q" not in state:
+                payload, scales = state_sizes(shape, granularity=group_["granularity"], tile_size=group_["tile_size"],
+                                              block_shape=group_["block_shape"])
+                state["momentum_q"] = torch.zeros(payload, device=param.device, dtype=torch.uint8)
+                state["momentum_scale"] = torch.ones(scales, device=param.device, dtype=torch.float32)
+            key = (group_["rounding_seed"] + index * 0x9E3779B97F4A7C15) & _MASK63
+            items.append((grad, state["momentum_q"], state["momentum_scale"], work[slot * count:(slot + 1) * count], key))
+        step = bucket[0][2]["step"]
+        together = (group["granularity"] == "tile" and all(item[2]["step"] == step for item in bucket)
+                    and uniform("granularity", "tile_size", "momentum", "nesterov", "rounding")
+                    and momentum_update_many(items, beta=group["momentum"], tile_size=group["tile_size"],
+                                             nesterov=group["nesterov"], rounding=group["rounding"], rounding_step=step,
+                                             cache=tables[0]))
+        if not together:
+            for (param, grad, state, group_, index), item in zip(bucket, items):
+                self._momentum(param, grad, state, group_, item[4], out=item[3])
         stacked = work[:len(bucket) * count].view(len(bucket), -1, *shape[-2:])
         updates = METHODS[group["ns_method"]](stacked, steps=group["ns_steps"]).reshape(len(bucket), count)
         rows, cols = shape[-2:]
-        for slot, (param, grad, state, group, index) in enumerate(bucket):
-            master_key = (group["master_rounding_seed"] + index * 0x517CC1B727220A95) & _MASK63
-            scale = .2 * max(rows, cols) ** .5 if group["adjust_lr_fn"] == "match_rms_adamw" else max(1., rows / cols) ** .5
-            weight_update(param, updates[slot], group["lr"], group["weight_decay"], update_scale=scale,
-                          rounding=group["master_rounding"], step=state["step"], key=master_key)
+        scale_of = lambda g: .2 * max(rows, cols) ** .5 if g["adjust_lr_fn"] == "match_rms_adamw" else max(1., rows / cols) ** .5
+        together = (uniform("lr", "weight_decay", "adjust_lr_fn") and all(item[3]["master_rounding"] == "nearest" or
+                                                                          item[0].dtype == torch.float32 for item in bucket)
+                    and weight_update_many([(item[0], updates[slot]) for slot, item in enumerate(bucket)], group["lr"],
+                                           group["weight_decay"], update_scale=scale_of(group), cache=tables[1]))
+        for slot, (param, grad, state, group_, index) in enumerate(bucket):
+            if not together:
+                master_key = (group_["master_rounding_seed"] + index * 0x517CC1B727220A95) & _MASK63
+                weight_update(param, updates[slot], group_["lr"], group_["weight_decay"], update_scale=scale_of(group_),
+                              rounding=group_["master_rounding"], step=state["step"], key=master_key)
             state["step"] += 1
 
     def _step_local(self, param, grad, state, group, index):
