@@ -55,7 +55,7 @@ def test_software_codecs_all_codes():
 @pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("fp8", [E4, E5])
 @pytest.mark.parametrize("group,shape", [((1, 32), (65, 96)), ((1, 32), (256, 1024)), ((1, 64), (96, 136)), ((1, 128), (33, 256)),
-                                          ((32, 32), (96, 128)), ((32, 32), (70, 45)), ((32, 64), (64, 160)), ((64, 32), (130, 96)),
+                                          ((32, 32), (96, 128)), ((32, 32), (70, 45)), ((32, 32), (70, 132)), ((32, 32), (257, 1000)), ((32, 64), (64, 160)), ((64, 32), (130, 96)),
                                           ((1, 32), (7, 33)), ((1, 512), (9, 1024))])
 def test_quantize_rowwise_and_blocks(in_dtype, fp8, group, shape):
     g = _gpu()

@@ -5,6 +5,7 @@
 //   quantize_rowwise   gr == 1, not transposed: 8 elements per lane, amax over gc/8 lanes.
 //   quantize_tile      gc == 32, gr == 1: 128 x 64 tile through LDS, emits the row-wise layout,
 //                      the quantized transpose, or both from the one read.
+//   quantize_block32   gr == gc == 32, not transposed (weights and their masters): 32 x 128 strip per wavefront.
 //   quantize_generic   any (gr, gc), transposed or not, optional re-encode from codes+scales:
 //                      one wavefront per group, two passes over the group (second hits cache).
 //   dequantize, fp8 transpose, segmented transposed quantize for the variable-group path.
@@ -384,6 +385,71 @@ __global__ __launch_bounds__(256) void column_reduce_kernel(const float* __restr
     }
 }
 
+// ------------------------------------------------------------------ (32, 32) blocks, not transposed
+template <typename TIn> __device__ __forceinline__ void load4(const TIn* p, float (&v)[4]);
+template <> __device__ __forceinline__ void load4<float>(const float* p, float (&v)[4]) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+template <> __device__ __forceinline__ void load4<bf16_t>(const bf16_t* p, float (&v)[4]) {
+    const uint2 t = *reinterpret_cast<const uint2*>(p);
+    v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+    v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+}
+template <> __device__ __forceinline__ void load4<f16_t>(const f16_t* p, float (&v)[4]) {
+    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+    const h4 t = *reinterpret_cast<const h4*>(p);
+    v[0] = (float)t[0]; v[1] = (float)t[1]; v[2] = (float)t[2]; v[3] = (float)t[3];
+}
+
+// The weight recipe (a master matrix re-quantized after every optimizer step). A wavefront owns 32 rows x 128
+// columns = four blocks: load i of 16 takes rows 2i, 2i+1, a lane four consecutive columns, so every load and every
+// store instruction covers whole 512-byte (128-byte for the codes) row pieces; a block is the 8 lanes of a column
+// group in both half-waves, over the 16 loads. One read of x; cols must be a multiple of 4.
+template <typename TIn, typename TOut>
+__global__ __launch_bounds__(256) void quantize_block32(const TIn* __restrict__ x, uint8_t* __restrict__ q, float* __restrict__ scale,
+                                                         int64_t rows, int64_t cols, int64_t nc, float limit) {
+    const int64_t strips = (cols + 127) / 128;
+    const int64_t unit = (int64_t)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (unit >= (rows + 31) / 32 * strips) return;                      // whole wavefront leaves together
+    const int lane = threadIdx.x % WAVE;
+    const int64_t r0 = unit / strips * 32 + lane / 32, col = unit % strips * 128 + (lane % 32) * 4;
+    float v[16][4];
+    float amax = 0.0f, poison = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int64_t row = r0 + 2 * i;
+        if (row < rows && col < cols) load4<TIn>(x + row * cols + col, v[i]);
+        else v[i][0] = v[i][1] = v[i][2] = v[i][3] = 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            amax = fmaxf(amax, fabsf(v[i][e]));
+            poison = poison_of(poison, v[i][e]);
+        }
+    amax = group_max<8>(amax);
+    amax = fmaxf(amax, __shfl_xor(amax, 32, WAVE));
+    const bool any_bad = __builtin_amdgcn_ballot_w64(poison != poison) != 0;
+    const float s = group_scale(amax, limit);
+    if ((lane & 39) == 0 && col < cols) scale[(r0 / 32) * nc + col / 32] = s;
+    const SharedDivisor d(s, any_bad ? __uint_as_float(0x7fc00000u) : 0.0f);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int64_t row = r0 + 2 * i;
+        uint32_t word;
+        if (d.fast) {
+            word = fast_encode4<TOut>(d, limit, v[i][0], v[i][1], v[i][2], v[i][3]);
+        } else {
+            word = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) word |= (uint32_t)encode_clamped<TOut>(v[i][e], s, limit) << (8 * e);
+        }
+        if (row < rows && col < cols) *reinterpret_cast<uint32_t*>(q + row * cols + col) = word;
+    }
+}
+
 // ------------------------------------------------------------------ generic: one wavefront per group
 template <typename TIn, typename TOut, bool ENCODED>
 __global__ __launch_bounds__(256) void quantize_generic(const TIn* __restrict__ x, const float* __restrict__ source_scale,
@@ -629,6 +695,13 @@ static int launch_quantize(const void* x, int64_t rows, int64_t cols, void* q, f
         const dim3 grid((unsigned)((cols + TILE_C - 1) / TILE_C), (unsigned)((rows + TILE_R - 1) / TILE_R));
         if (vec) hipLaunchKernelGGL((quantize_tile<TIn, TOut, false, true, true>), grid, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit, nullptr);
         else hipLaunchKernelGGL((quantize_tile<TIn, TOut, false, true, false>), grid, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit, nullptr);
+        return viola_launch_status();
+    }
+    if (gr == 32 && gc == 32 && !transposed && cols % 4 == 0 && reinterpret_cast<uintptr_t>(x) % (4 * sizeof(TIn)) == 0 &&
+        reinterpret_cast<uintptr_t>(q) % 4 == 0) {
+        const int64_t units = (rows + 31) / 32 * ((cols + 127) / 128);
+        hipLaunchKernelGGL((quantize_block32<TIn, TOut>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, xp, qp, scale,
+                           rows, cols, (cols + 31) / 32, limit);
         return viola_launch_status();
     }
     const int64_t out_rows = transposed ? cols : rows, out_cols = transposed ? rows : cols;
