@@ -192,6 +192,32 @@ def main():
         extra["comm_codec"] = dict(bucket_elements=n, pack_ms=pack_ms, unpack_ms=unpack_ms,
                                    pack_gbs=5.016 * n / (pack_ms * 1e-3) / 1e9, unpack_gbs=5.016 * n / (unpack_ms * 1e-3) / 1e9)
 
+    if not args.skip_muon:
+        # the training loop closed: the same Linear under bind_optimizer (fp32 master, bf16 gradients), one
+        # forward + backward + FP8Muon step + write-back of the master as FP8 codes and (32, 32) scales
+        import viola_amd
+        from viola_amd.nn import _grouped_kernels as gk
+        viola_amd.set_master_weight_dtype("fp32")
+        viola_amd.set_gradient_dtype("bf16")
+        torch.manual_seed(1)
+        bound = viola_amd.nn.Linear(K, N, device="cuda", dtype=torch.bfloat16, scaling="grouped", forward_dtype="e4m3",
+                                    backward_dtype="e4m3", mode="memory", weight_dtype="fp8")
+        opt = viola_amd.optim.bind_optimizer(bound, viola_amd.optim.FP8Muon(bound.parameters(), lr=1e-3, weight_decay=.01))
+        xb = torch.randn(M, K, device="cuda").bfloat16().requires_grad_()
+
+        def train_step():
+            opt.zero_grad()
+            bound(xb).backward(dy)
+            opt.step()
+        train_ms, _ = timed(train_step, min(args.steps, 50), min(args.warmup, 10))
+        master = bound._master_ref().detach()
+        codes, scales = torch.empty_like(bound.weight), torch.empty_like(bound.weight_scale)
+        refresh_ms, _ = timed(lambda: gk.quantize(master, torch.float8_e4m3fn, (32, 32), out=codes, scale_out=scales), 100, 20)
+        extra["bound_training_step"] = dict(step_ms=train_ms, optimizer="FP8Muon standard, fp32 master, bf16 gradients",
+                                            refresh_quantize_ms=refresh_ms,
+                                            refresh_gbs=(4 + 1 + 4 / 1024) * K * N / (refresh_ms * 1e-3) / 1e9)
+        viola_amd.precision._settings.update(master_weight_dtype=torch.float32, gradient_dtype=None)
+
     if args.calibrate:
         from viola_amd.optim import _kernels as ok
         src = torch.ones(1 << 26, device="cuda")
