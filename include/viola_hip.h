@@ -69,6 +69,26 @@ int viola_group_dequantize(const void* q, int q_dtype, const float* scale, int64
  * out [batch, cols, rows] (the reference transposes one matrix per call; batch > 1 serves stacked expert weights). */
 int viola_fp8_transpose(const void* x, void* out, int64_t batch, int64_t rows, int64_t cols, viola_stream_t stream);
 
+/* ---------------------------------------------------------------- per-tensor scaling (`current` / `delayed`)
+ * viola/nn/_linear_kernels.py:231-242 `tensor_scale` = _amax_kernel :33-46 + _scale_kernel :49-71.
+ * viola_tensor_amax: maxima[i] = max |x| over part i of `parts` (NaN dropped); maxima is caller scratch of `parts`
+ * floats (the reference sizes it ceil(n / 2048)). viola_tensor_scale: amax = max(maxima);
+ * scale[0] = max(delayed && index != 0 ? max(history as it was) : amax, 1e-30) / limit; history[index % len] = amax. */
+int viola_tensor_amax(const void* x, int x_dtype, int64_t n, float* maxima, int64_t parts, viola_stream_t stream);
+int viola_tensor_scale(const float* maxima, int64_t parts, float* history, int history_len, int64_t index, int delayed,
+                       float limit, float* scale, viola_stream_t stream);
+
+/* viola/nn/_linear_kernels.py:245-250 `quantize` (_quantize_kernel :74-104): with the tensor's one scale,
+ * q[r, c] = fp8(isnan(x) ? x : clamp(x / scale[0], +-limit)) and / or qt[c, r] = the same code; q or qt may be NULL. */
+int viola_tensor_quantize(const void* x, int x_dtype, int64_t rows, int64_t cols, const float* scale, void* q, void* qt,
+                          int q_dtype, float limit, viola_stream_t stream);
+
+/* viola/nn/_linear_kernels.py:260-293 `gemm` (_gemm_kernel :124-163, _mixed_gemm_kernel :166-228):
+ * out[m, n] = (sum_k a[m, k] * b[n, k]) * sa[0] * sb[0] (+ bias[n]); a and b may mix e4m3 and e5m2. */
+int viola_tensor_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,
+                      int64_t m, int64_t n, int64_t k, const void* bias, int bias_dtype, void* out, int out_dtype,
+                      viola_stream_t stream);
+
 /* ---------------------------------------------------------------- grouped-scale FP8 GEMM
  * viola/nn/_grouped_kernels.py:310-328 `gemm` (gemm_kernel :195-293).
  * out[m, n] = sum over 32-wide K groups kg of (sum_{k in kg} a[m,k]*b[n,k]) * sa[m/ar, k/ak] * sb[n/br, k/bk]

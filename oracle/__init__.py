@@ -18,6 +18,9 @@ Pinning status (what fixes each function besides its own formula):
   momentum/weight/adam/comm codec : closed forms held by the reference's checks
   Newton-Schulz    : golden vectors written by tests/golden/make_ns_golden.py from the
                      reference's own optim/_orthogonalize.py + invariants   -> pinned
+  per-tensor scaling (oracle.tensor) : the reference's own CPU definitions (checks/linear.py:17-20,
+                     viola/nn/linear.py:298-312) + textbook matmul           -> pinned; an Inf inside the
+                     tensor (infinite scale, Inf / Inf)                       -> parity unpinned
   variable-group (MoE) linear : NOT in the reference; per-group loop of the Linear
                      restatement                                   -> parity unpinned
   NaN/Inf inside a quantize group: the reference's GPU and CPU branches disagree

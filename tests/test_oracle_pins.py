@@ -338,3 +338,49 @@ def test_linear_oracle_against_float_math():
         assert rel_l2(linear.gated_forward(g, u, name), out.detach()) < 1e-6
         dg, du = linear.gated_backward(d, g, u, name)
         assert rel_l2(dg, gg.grad) < 1e-5 and rel_l2(du, uu.grad) < 1e-6
+
+
+# ----------------------------------------------------------------------------- per-tensor scaling
+@pytest.mark.parametrize("dtype", [E4, E5])
+def test_tensor_oracle_matches_the_reference_cpu_definitions(dtype):
+    """checks/linear.py:17-20 `quantized` and viola/nn/linear.py:298-312 (CPU refresh_weight) written out here,
+    independently of oracle.tensor: same scale, same codes; delayed scaling reads the history as it was."""
+    from oracle import tensor
+    torch.manual_seed(51)
+    x = torch.randn(70, 45) * torch.logspace(-3, 2, 45)
+    limit = torch.finfo(dtype).max
+    expected_scale = x.float().abs().max().clamp_min(1e-30) / limit
+    scale, history = tensor.tensor_scale(x, torch.zeros(4), 0, limit=limit)
+    assert torch.equal(scale, expected_scale.reshape(1)) and history.tolist() == [x.abs().max().item(), 0, 0, 0]
+    expected = (x.float() / expected_scale).clamp(-limit, limit).to(dtype)
+    assert torch.equal(tensor.quantize(x, scale, dtype).view(torch.uint8), expected.view(torch.uint8))
+    assert torch.equal(tensor.quantize(x, scale, dtype, transpose=True).view(torch.uint8), expected.T.contiguous().view(torch.uint8))
+    assert tensor.quantize(x, scale, dtype).float().abs().max() == limit            # the largest element maps to the limit
+    # delayed: index 0 uses the tensor itself, later calls the history's maximum before the new amax is written
+    history = torch.zeros(3)
+    amaxes = [2.0, 8.0, 1.0, 0.5, 0.25, 0.125]
+    for index, a in enumerate(amaxes):
+        y = torch.full((5,), a)
+        y[2] = float("nan")                                                          # dropped by the reduction
+        before = history.clone()
+        scale, history = tensor.tensor_scale(y, history, index, delayed=True, limit=limit)
+        basis = a if index == 0 else before.max().item()
+        assert scale.item() == torch.tensor(basis) / limit and history[index % 3] == a
+    # all-zero tensor: the 1e-30 floor
+    assert tensor.tensor_scale(torch.zeros(9), torch.zeros(1), 0, limit=limit)[0].item() == (torch.tensor(1e-30) / limit).item()
+    # a reduced quantization limit clamps
+    q = tensor.quantize(x, scale=torch.tensor([x.abs().max().item() / 64]), dtype=dtype, limit=16.0)
+    assert q.float().abs().max() == 16.0
+
+
+def test_tensor_gemm_oracle_against_brute_force():
+    from oracle import tensor
+    torch.manual_seed(52)
+    a = torch.randn(5, 48).to(E5)
+    b = torch.randn(7, 48).to(E4)
+    sa, sb, bias = torch.tensor([.37]), torch.tensor([1.9]), torch.randn(7)
+    out = tensor.gemm(a, b, sa, sb, bias=bias)
+    for m in range(5):
+        for n in range(7):
+            acc = sum(float(a[m, k].float()) * float(b[n, k].float()) for k in range(48))
+            assert abs(out[m, n].item() - (acc * .37 * 1.9 + bias[n].item())) < 1e-4 * (1 + abs(acc))

@@ -358,6 +358,29 @@ extern "C" int viola_group_gemm(const void* a, int a_dtype, const void* b, int b
     return launch_out<MODE_PLAIN>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, vec, dim3((unsigned)gx, (unsigned)gy), stream);
 }
 
+extern "C" int viola_tensor_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,
+                                 int64_t m, int64_t n, int64_t k, const void* bias, int bias_dtype, void* out, int out_dtype,
+                                 viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_fp8(a_dtype) && viola_is_fp8(b_dtype) && viola_is_float(out_dtype));
+    VIOLA_CHECK_ARG(m >= 0 && n >= 0 && k >= 0 && k < (1ll << 30) && (!bias || viola_is_float(bias_dtype)));
+    if (m == 0 || n == 0) return 0;
+    VIOLA_CHECK_ARG(out && sa && sb && (k == 0 || (a && b)));
+    const int64_t gy = (m + BM - 1) / BM, gx = (n + BN - 1) / BN;
+    VIOLA_CHECK_ARG(gy <= 65535);
+    GemmArgs p = {};
+    p.a = static_cast<const uint8_t*>(a); p.b = static_cast<const uint8_t*>(b); p.sa = sa; p.sb = sb;
+    p.bias = bias; p.out = out; p.m = m; p.n = n; p.k = k; p.lda = k; p.ldb = k; p.ldo = n;
+    // one scale group per operand: every (row, k) lands on scale index 0
+    p.ldsa = 0; p.ldsb = 0; p.ar = 1 << 30; p.br = 1 << 30; p.ak_shift = 30; p.bk_shift = 30;
+    const dim3 grid((unsigned)gx, (unsigned)gy);
+    const bool vec = k % 16 == 0 && k > 0 && aligned16(a) && aligned16(b);
+    if (vec && n * k < (1ll << 31) && (int64_t)BM * k < (1ll << 31))
+        return launch_tensor_gemm_fast(p, a_dtype, b_dtype, bias_dtype, out_dtype, grid, stream);
+    // odd alignment: the generic kernel, which multiplies each 32-wide K group's sum by sa * sb as it goes
+    return launch_out<MODE_PLAIN>(p, a_dtype, b_dtype, bias_dtype, out_dtype, false, false, grid, stream);
+}
+
 extern "C" int viola_gated_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,
                                 int64_t m, int64_t h, int64_t k, int ar, int ak, int br, int bk, const void* bias,
                                 int bias_dtype, void* aux, void* out, int out_dtype, int activation, int backward,

@@ -32,4 +32,8 @@ struct GemmArgs {
 int launch_group_gemm_fast(const GemmArgs& p, int mode, int a_dtype, int b_dtype, int bias_dtype, int out_dtype,
                            bool rowscale, dim3 grid, hipStream_t stream);
 
+// Per-tensor scales on the same fast kernel (one v_mfma_f32_32x32x64_f8f6f4 per sub-tile and 64 k). Defined in gemm_fast.hip.
+int launch_tensor_gemm_fast(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, dim3 grid,
+                            hipStream_t stream);
+
 }  // namespace viola

@@ -113,8 +113,12 @@ template <typename TO> __device__ __forceinline__ float rounded(float v) { retur
 
 // TN: 32-column sub-tiles per wave; TN = 1 halves the tile to 128 x 64 for problems with too few 128 x 128 tiles to
 // give every CU two blocks (plain mode only).
-template <int MODE, bool A_BF8, bool B_BF8, bool B_ROWSCALE, typename TO, int TN>
+// TENSOR: one scale per operand (p.sa[0], p.sb[0]) applied to the finished sums, out = (acc * sa) * sb + bias: no
+// per-group fold, so a chunk's 64 k go through one v_mfma_f32_32x32x64_f8f6f4 per sub-tile straight into the totals.
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+template <int MODE, bool A_BF8, bool B_BF8, bool B_ROWSCALE, typename TO, int TN, bool TENSOR = false>
 __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int bias_dtype) {
+    static_assert(!TENSOR || (MODE == MODE_PLAIN && !B_ROWSCALE), "per-tensor scaling: plain mode only");
     __shared__ __attribute__((aligned(1024))) uint8_t lds[F_LDS];
 
     // wave grid 2 (m) x 2 (n), 2 x 2 sub-tiles each. Plain / gated backward: sub-tile i of wave wn covers b rows
@@ -293,15 +297,33 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
 #pragma unroll
             for (int i = 0; i < TN; ++i) o.b[kg][i] = *reinterpret_cast<const uint4*>(tile_b + ((rd_b + (b_sub(i) - b_sub(0)) * FBK) ^ (kg * 32)));
 #pragma unroll
-            for (int j = 0; j < TM; ++j) o.sa[kg][j] = scale_a[kg * BM + a_sub(j) + l32];
+            for (int j = 0; j < TM; ++j) o.sa[kg][j] = TENSOR ? 0.0f : scale_a[kg * BM + a_sub(j) + l32];
 #pragma unroll
-            for (int i = 0; i < TN; ++i) o.sb[kg][i] = B_ROWSCALE ? 0.0f : scale_b[kg * BM + b_sub(i)];
+            for (int i = 0; i < TN; ++i) o.sb[kg][i] = B_ROWSCALE || TENSOR ? 0.0f : scale_b[kg * BM + b_sub(i)];
         }
     };
 
     // Math of chunk c on the operands in `o`; `between(step)` runs after MFMA number `step` of the chunk (the
     // caller's global loads and LDS reads for later chunks go there, spread over the chunk).
     auto compute = [&](const Operands& o, int64_t c, auto&& between) {
+        if constexpr (TENSOR) {
+            constexpr int UNITS = TN * TM, STEPS_PER = FKG * 2;
+#pragma unroll
+            for (int unit = 0; unit < UNITS; ++unit) {
+                const int i = unit / TM, j = unit % TM;
+                const i32x8 ob = {(int)o.b[0][i].x, (int)o.b[0][i].y, (int)o.b[0][i].z, (int)o.b[0][i].w,
+                                  (int)o.b[1][i].x, (int)o.b[1][i].y, (int)o.b[1][i].z, (int)o.b[1][i].w};
+                const i32x8 oa = {(int)o.a[0][j].x, (int)o.a[0][j].y, (int)o.a[0][j].z, (int)o.a[0][j].w,
+                                  (int)o.a[1][j].x, (int)o.a[1][j].y, (int)o.a[1][j].z, (int)o.a[1][j].w};
+                // both operands give a lane the same 32 of the chunk's 64 k (16 of each K group), so every product
+                // meets its partner whatever order the instruction walks them in
+                total[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ob, oa, total[i][j], B_BF8 ? 1 : 0, A_BF8 ? 1 : 0, 0, 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int step = unit * STEPS_PER; step < (unit + 1) * STEPS_PER; ++step) between(step);
+            }
+            return;
+        }
         // row-wise b scales of the lane's 16 columns for one pair of units (both share K group and b sub-tile): two
         // slots, pair p loads slot p & 1 before its MFMAs and its fold reads it during pair p + 1
         float4 sb_q[2][4];
@@ -380,11 +402,13 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
     constexpr int STEPS = FKG * TN * TM * 2, STRIDE = STEPS / CHUNK_LOADS;
     int stage_now = 0, stage_next = 1;
     auto chunk_step = [&](int64_t c, const Operands& now, Operands& next) {
-        if (c % F_SCHUNKS == 1) __builtin_amdgcn_s_waitcnt(0x0070 | (CHUNK_LOADS + 2));
+        if (!TENSOR && c % F_SCHUNKS == 1) __builtin_amdgcn_s_waitcnt(0x0070 | (CHUNK_LOADS + 2));
         else __builtin_amdgcn_s_waitcnt(0x0070 | CHUNK_LOADS);
         __syncthreads();
-        if (c % F_SCHUNKS == 0) issue_scales(c / F_SCHUNKS + 1);
-        if (c % F_SCHUNKS == 2) arrange_scales(c / F_SCHUNKS + 1);
+        if constexpr (!TENSOR) {
+            if (c % F_SCHUNKS == 0) issue_scales(c / F_SCHUNKS + 1);
+            if (c % F_SCHUNKS == 2) arrange_scales(c / F_SCHUNKS + 1);
+        }
         if (c + 1 < chunks) read_operands(stage_next, c + 1, next);
         const int fill = stage_now;
         compute(now, c, [&](int step) {
@@ -393,14 +417,16 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
         stage_now = stage_next;
         stage_next = stage_next == FSTAGES - 1 ? 0 : stage_next + 1;
     };
-    issue_scales(0);
+    if constexpr (!TENSOR) issue_scales(0);
     issue(0, 0);
     issue(1, 1);
     issue(2, 2);
     __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * CHUNK_LOADS));                   // scale block 0 and chunk 0 are in LDS
     __syncthreads();
-    arrange_scales(0);
-    __syncthreads();
+    if constexpr (!TENSOR) {
+        arrange_scales(0);
+        __syncthreads();
+    }
     Operands set0, set1;
     read_operands(0, 0, set0);
     for (int64_t c = 0; c < chunks; c += 2) {
@@ -408,7 +434,15 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
         if (c + 1 < chunks) chunk_step(c + 1, set1, set0);
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);     // drain the trailing loads before the LDS allocation is released
-    if constexpr (CARRY) {
+    if constexpr (TENSOR) {
+        const float sa = p.sa[0], sb = p.sb[0];
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+            for (int j = 0; j < TM; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) { const float t = total[i][j][r] * sa; total[i][j][r] = t * sb; }
+    } else if constexpr (CARRY) {
         constexpr int UNITS = FKG * TN * TM, last_pair = UNITS / 2 - 1;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
@@ -593,6 +627,39 @@ static int launch_mode(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dty
         default: return VIOLA_EINVAL;
     }
 #undef VIOLA_FAST
+    return viola_launch_status();
+}
+
+// Per-tensor scales (args.sa / args.sb point at one float each). grid: (n tiles of 128, m tiles of 128).
+template <typename TO, int TN>
+static void launch_tensor_formats(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, dim3 grid, hipStream_t stream) {
+    const bool a5 = a_dtype == VIOLA_E5M2, b5 = b_dtype == VIOLA_E5M2;
+    if (!a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE_PLAIN, false, false, false, TO, TN, true>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    else if (a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE_PLAIN, true, false, false, TO, TN, true>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    else if (!a5 && b5) hipLaunchKernelGGL((group_gemm_fast<MODE_PLAIN, false, true, false, TO, TN, true>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    else hipLaunchKernelGGL((group_gemm_fast<MODE_PLAIN, true, true, false, TO, TN, true>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+}
+
+int launch_tensor_gemm_fast(const GemmArgs& args, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, dim3 grid,
+                            hipStream_t stream) {
+    GemmArgs p = args;
+    const bool narrow = (int64_t)grid.x * grid.y < 512 && p.n > 64;
+    if (narrow) grid.x = (unsigned)((p.n + 63) / 64);
+    if ((int64_t)grid.x * grid.y < (1 << 30)) {
+        p.tiles_n = (int)grid.x;
+        p.tiles_m = (int)grid.y;
+        grid = dim3((grid.x * grid.y + 7) / 8 * 8, 1, 1);
+    }
+#define VIOLA_TENSOR(TO)                                                                          \
+    if (narrow) launch_tensor_formats<TO, 1>(p, a_dtype, b_dtype, bias_dtype, grid, stream);      \
+    else launch_tensor_formats<TO, 2>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
+    switch (out_dtype) {
+        case VIOLA_F32: VIOLA_TENSOR(float) break;
+        case VIOLA_BF16: VIOLA_TENSOR(bf16_t) break;
+        case VIOLA_F16: VIOLA_TENSOR(f16_t) break;
+        default: return VIOLA_EINVAL;
+    }
+#undef VIOLA_TENSOR
     return viola_launch_status();
 }
 

@@ -1,5 +1,5 @@
-"""Byte-matrix kernels shared with the grouped path (operator seam of
-viola/nn/_linear_kernels.py; only `transpose` :253-257 is on the grouped hot path)."""
+"""Per-tensor FP8 scaling operators (operator seam of viola/nn/_linear_kernels.py:231-293): `tensor_scale`,
+`quantize`, `transpose`, `gemm`. `transpose` also serves the grouped path."""
 
 import torch
 
@@ -13,4 +13,49 @@ def transpose(x, out=None):
     if out is None:
         out = torch.empty((*x.shape[:-2], x.shape[-1], x.shape[-2]), device=x.device, dtype=x.dtype)
     _lib.call("viola_fp8_transpose", _lib.ptr(x), _lib.ptr(out), x.shape[0] if x.dim() == 3 else 1, x.shape[-2], x.shape[-1])
+    return out
+
+
+def tensor_scale(x, *, history=None, index=0, delayed=False, fp8_dtype=torch.float8_e4m3fn, quantization_limit=None):
+    """scale [1] = max(amax(x) or, delayed after the first call, the history's maximum, 1e-30) / limit; the new amax
+    goes into history[index % len]. Scratch is one float per 64 Ki elements, never a full-sized temporary."""
+    assert x.is_cuda
+    x = x.contiguous()
+    parts = max(1, min(-(-x.numel() // 65536), 1024))
+    maxima = torch.empty(parts, device=x.device, dtype=torch.float32)
+    if history is None:
+        history = torch.zeros(1, device=x.device, dtype=torch.float32)
+    scale = torch.empty(1, device=x.device, dtype=torch.float32)
+    _lib.call("viola_tensor_amax", _lib.ptr(x), _lib.code(x.dtype), x.numel(), _lib.ptr(maxima), parts)
+    limit = torch.finfo(fp8_dtype).max if quantization_limit is None else quantization_limit
+    _lib.call("viola_tensor_scale", _lib.ptr(maxima), parts, _lib.ptr(history), history.numel(), int(index),
+              int(bool(delayed)), float(limit), _lib.ptr(scale))
+    return scale
+
+
+def quantize(x, scale, *, rowwise=True, transpose=False, fp8_dtype=torch.float8_e4m3fn, out=None, out_t=None,
+             quantization_limit=None):
+    """(q, qt): the codes of x / scale in x's layout and / or transposed, from one read; absent ones are (0, 0)-shaped."""
+    assert x.is_cuda and x.dim() == 2
+    x = x.contiguous()
+    q = out if out is not None else torch.empty(x.shape if rowwise else (0, 0), device=x.device, dtype=fp8_dtype)
+    qt = out_t if out_t is not None else torch.empty(x.shape[::-1] if transpose else (0, 0), device=x.device, dtype=fp8_dtype)
+    assert q.is_contiguous() and qt.is_contiguous() and q.dtype == qt.dtype
+    limit = torch.finfo(q.dtype).max if quantization_limit is None else quantization_limit
+    _lib.call("viola_tensor_quantize", _lib.ptr(x), _lib.code(x.dtype), x.shape[0], x.shape[1], _lib.ptr(scale),
+              _lib.ptr(q), _lib.ptr(qt), _lib.code(q.dtype), float(limit))
+    return q, qt
+
+
+def gemm(a, b, sa, sb, *, out_dtype, bias=None, autotune=False, accum_dtype="fp32", accum_block_size=0,
+         accum_reduce_dtype="fp32"):
+    """(a * sa) @ (b * sb).T + bias with the scaling in the epilogue; a [m, k] and b [n, k] are FP8 codes."""
+    if accum_dtype != "fp32" or accum_block_size or accum_reduce_dtype != "fp32":
+        raise NotImplementedError("viola_amd builds FP32 accumulation only")
+    assert a.is_cuda and a.is_contiguous() and b.is_contiguous() and a.shape[1] == b.shape[1]
+    out = torch.empty((a.shape[0], b.shape[0]), device=a.device, dtype=out_dtype)
+    has_bias = bias is not None and bias.numel() > 0
+    _lib.call("viola_tensor_gemm", _lib.ptr(a), _lib.code(a.dtype), _lib.ptr(b), _lib.code(b.dtype), _lib.ptr(sa), _lib.ptr(sb),
+              a.shape[0], b.shape[0], a.shape[1], _lib.ptr(bias) if has_bias else None, _lib.code(bias.dtype) if has_bias else 0,
+              _lib.ptr(out), _lib.code(out_dtype))
     return out
