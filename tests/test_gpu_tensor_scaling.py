@@ -121,3 +121,154 @@ def test_tensor_gemm_exact_on_small_integers():
         out = kk.gemm(a.to(E4).cuda(), b.to(E5).cuda(), torch.tensor([.5], device="cuda"), torch.tensor([4.], device="cuda"),
                       out_dtype=torch.float32)
         assert torch.equal(out.cpu(), (a @ b.T) * 2)
+
+
+# ----------------------------------------------------------------------------- Linear(scaling="current" | "delayed")
+@pytest.fixture
+def precision_policy():
+    import viola_amd
+    saved = dict(viola_amd.precision._settings)
+    yield viola_amd
+    viola_amd.precision._settings.clear()
+    viola_amd.precision._settings.update(saved)
+
+
+@pytest.mark.parametrize("fmt,backward,mode", [("e4m3", "e5m2", "memory"), ("e4m3", "e5m2", "fast"), ("e4m3", "e4m3", "memory"),
+                                               ("e5m2", "e5m2", "fast")])
+@pytest.mark.parametrize("shape,gradient", [((65, 128, 96), "bf16"), ((256, 512, 384), "fp32"), ((100, 72, 40), "bf16")])
+def test_linear_current_scaling_numerics(precision_policy, fmt, backward, mode, shape, gradient):
+    """checks/linear.py:23-39: y, dx, dw against the matmul of the per-tensor-quantized operands (< .003 for bf16
+    results, < 2e-5 for fp32), db exact; the stored codes and scale are the oracle's quantize of the initial weight."""
+    viola = precision_policy
+    viola.set_master_weight_dtype("fp32")
+    viola.set_gradient_dtype(gradient)
+    m, k, n = shape
+    torch.manual_seed(127)
+    layer = viola.nn.Linear(k, n, mode=mode, forward_dtype=fmt, backward_dtype=backward, device="cuda", dtype=torch.bfloat16)
+    assert layer.weight_quantizer.scaling == "current" and layer.weight_scale.shape == (1,)
+    fp8, bwd = layer.fp8_dtype, layer.backward_fp8_dtype
+    master = layer._initial_weight.detach().cpu()
+    sw, _ = ot.tensor_scale(master, torch.zeros(1), 0, limit=torch.finfo(fp8).max)
+    assert torch.equal(layer.weight_scale.cpu(), sw) and torch.equal(_codes(layer.weight), _codes(ot.quantize(master, sw, fp8)))
+    if mode == "fast":
+        assert torch.equal(_codes(layer.weight_transpose), _codes(ot.quantize(master, sw, fp8, transpose=True)))
+    else:
+        assert layer.weight_transpose.numel() == 0
+    x = torch.randn(m, k, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    dy = torch.randn(m, n, device="cuda", dtype=torch.bfloat16)
+    y = layer(x)
+    y.backward(dy)
+    grad_dtype = torch.bfloat16 if gradient == "bf16" else torch.float32
+    ry, rdx, rdw, rdb = ot.linear(x.detach().cpu(), layer.weight.detach().cpu(), sw, layer.bias.detach().cpu(), dy.cpu(), fp8=fp8,
+                                  bwd_fp8=bwd, out_dtype=torch.bfloat16, grad_dtype=grad_dtype)
+    assert rel_l2(y, ry) < 3e-3 and rel_l2(x.grad, rdx) < 3e-3
+    assert layer.weight.grad.dtype == grad_dtype and rel_l2(layer.weight.grad, rdw) < (3e-3 if gradient == "bf16" else 2e-5)
+    torch.testing.assert_close(layer.bias.grad.cpu(), rdb)
+    # and against the float model: FP8 noise only
+    w = layer.dequantize_weight().cpu()
+    assert rel_l2(y, x.detach().float().cpu() @ w.T + layer.bias.detach().float().cpu()) < .08
+    assert torch.equal(w, layer.weight.detach().float().cpu() * sw)
+
+
+@pytest.mark.parametrize("weight_dtype", ["bf16", "fp16"])
+def test_linear_current_scaling_float_storage(precision_policy, weight_dtype):
+    """BF16/FP16 storage quantizes the weight per call with its own scale; frozen weights and no-grad calls work."""
+    viola = precision_policy
+    viola.set_gradient_dtype("bf16")
+    torch.manual_seed(128)
+    layer = viola.nn.Linear(96, 80, weight_dtype=weight_dtype, backward_dtype="e4m3", device="cuda", dtype=torch.bfloat16,
+                            saved_input_dtype="bf16", cache_weight_transpose=True)
+    assert layer.weight_scale.shape == (0,)
+    x = torch.randn(3, 50, 96, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    dy = torch.randn(3, 50, 80, device="cuda", dtype=torch.bfloat16)
+    y = layer(x)
+    y.backward(dy)
+    w = layer.weight.detach().float().cpu()
+    sw, _ = ot.tensor_scale(w, torch.zeros(1), 0)
+    ry, rdx, rdw, rdb = ot.linear(x.detach().cpu().reshape(-1, 96), ot.quantize(w, sw, E4), sw, layer.bias.detach().cpu(),
+                                  dy.cpu().reshape(-1, 80), bwd_fp8=E4)
+    assert rel_l2(y.reshape(-1, 80), ry) < 3e-3 and rel_l2(x.grad.reshape(-1, 96), rdx) < 3e-3 and rel_l2(layer.weight.grad, rdw) < 3e-3
+    with torch.no_grad():
+        assert torch.equal(layer(x), y)
+    layer.weight.requires_grad_(False)
+    x.grad = None
+    layer(x).backward(dy)
+    assert rel_l2(x.grad.reshape(-1, 96), rdx) < 3e-3 and layer.weight.grad is not None
+
+
+def test_linear_delayed_scaling_history(precision_policy):
+    """scaling="delayed": call n > 0 of each quantizer scales with the maximum of its amax history (linear.py:20-26,
+    _scale_kernel :49-71), the backward does not advance the weight history, state_dict round-trips the counters."""
+    viola = precision_policy
+    viola.set_gradient_dtype("bf16")
+    torch.manual_seed(129)
+    layer = viola.nn.Linear(64, 48, scaling="delayed", history_len=3, device="cuda", dtype=torch.bfloat16)
+    assert layer.weight_quantizer.index == 1                                    # the construction-time refresh
+    history = torch.zeros(3)
+    for index, gain in enumerate((1., 4., .25, .125, .0625)):
+        x = (torch.randn(32, 64) * gain).bfloat16()
+        expected_scale, history = ot.tensor_scale(x, history, index, delayed=True)
+        y = layer(x.cuda().requires_grad_())
+        assert torch.equal(layer.input_quantizer.history.cpu(), history) and layer.input_quantizer.index == index + 1
+        qx = ot.quantize(x, expected_scale, E4)
+        ry = ot.gemm(qx, layer.weight.detach().cpu(), expected_scale, layer.weight_scale.cpu(), bias=layer.bias.detach().cpu(),
+                     out_dtype=torch.bfloat16)
+        assert rel_l2(y, ry) < 3e-3
+        y.backward(torch.randn_like(y))
+        assert layer.grad_quantizer.index == index + 1 and layer.weight_quantizer.index == 1
+    state = layer.state_dict()
+    other = viola.nn.Linear(64, 48, scaling="delayed", history_len=3, device="cuda", dtype=torch.bfloat16)
+    other.load_state_dict(state)
+    assert other.input_quantizer.index == 5 and torch.equal(other.input_quantizer.history, layer.input_quantizer.history)
+    x = torch.randn(8, 64, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        assert torch.equal(other(x), layer(x))
+
+
+@pytest.mark.parametrize("fmt,mode,scaling,gradient", [("e4m3", "memory", "current", "bf16"), ("e4m3", "fast", "delayed", "fp32"),
+                                                       ("e5m2", "fast", "current", "bf16")])
+def test_linear_update_and_resume(precision_policy, fmt, mode, scaling, gradient):
+    """checks/linear.py:50-97: AdamW under bind_optimizer, three micro-batches per step; after a step the stored codes
+    are exactly quantize(master, stored scale); a restored model + optimizer repeats the next step bit for bit."""
+    import copy
+    viola = precision_policy
+    viola.set_master_weight_dtype("fp32")
+    viola.set_gradient_dtype(gradient)
+    torch.manual_seed(130)
+    make = lambda: viola.nn.Linear(256, 192, mode=mode, forward_dtype=fmt, scaling=scaling, device="cuda", dtype=torch.bfloat16)
+    layer = make()
+    optimizer = viola.optim.bind_optimizer(layer, torch.optim.AdamW(layer.parameters(), lr=.002))
+    assert layer._initial_weight is None
+    batches = [torch.randn(64, 256, device="cuda", dtype=torch.bfloat16) for _ in range(3)]
+
+    def step(model, opt):
+        opt.zero_grad()
+        for batch in batches:
+            model(batch).float().square().mean().div(len(batches)).backward()
+        before = model.weight.detach().view(torch.uint8).clone()
+        opt.step()
+        assert not torch.equal(before, model.weight.view(torch.uint8))
+        master = model._master_ref().detach().cpu()
+        assert torch.equal(_codes(model.weight), _codes(ot.quantize(master, model.weight_scale.cpu(), model.fp8_dtype)))
+        assert model.weight.grad.dtype == {"fp32": torch.float32, "bf16": torch.bfloat16}[gradient]
+        if model.cache_weight_transpose:
+            assert torch.equal(model.weight.T.contiguous().view(torch.uint8), model.weight_transpose.view(torch.uint8))
+        else:
+            assert model.weight_transpose.numel() == 0
+
+    step(layer, optimizer)
+    state = copy.deepcopy({"model": layer.state_dict(), "optimizer": optimizer.state_dict()})
+    restored = make()
+    restored.load_state_dict(state["model"])
+    second = viola.optim.bind_optimizer(restored, torch.optim.AdamW(restored.parameters(), lr=.002))
+    second.load_state_dict(state["optimizer"])
+    step(layer, optimizer)
+    step(restored, second)
+    assert torch.equal(layer.weight.view(torch.uint8), restored.weight.view(torch.uint8))
+    assert torch.equal(layer.bias, restored.bias) and torch.equal(layer.weight_scale, restored.weight_scale)
+    for p, q in zip(optimizer.param_groups[0]["params"], second.param_groups[0]["params"]):
+        assert torch.equal(p, q)
+    optimizer.zero_grad(set_to_none=False)
+    assert layer.weight.grad.count_nonzero() == 0
+    optimizer.zero_grad()
+    assert layer.weight.grad is None

@@ -1,0 +1,76 @@
+"""Forward / dgrad / wgrad of Linear(scaling="current" | "delayed"): one FP32 scale per tensor, applied in the
+GEMM epilogue (the role of `_Linear`, viola/nn/linear.py:36-147). Each operand is read twice at most: once for its
+amax, once by the quantizer, which writes the row-wise and the transposed codes together when both are needed."""
+
+import torch
+
+from . import _linear_kernels as kernels
+
+_FLOAT = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}
+
+
+class TensorLinear(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, bias, layer, need_backward):
+        shape = x.shape
+        x2 = x.reshape(-1, layer.in_features).contiguous()
+        fp8 = layer.fp8_dtype
+        input_limit = layer._quantization_limit(max(x2.shape), fp8)
+        sx = layer.input_quantizer.scale(x2, fp8, input_limit)
+        needs_x, needs_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        save_fp8 = need_backward and needs_w and layer.saved_input_dtype == "fp8"
+        qx, qxt = kernels.quantize(x2, sx, transpose=save_fp8, fp8_dtype=fp8, quantization_limit=input_limit)
+        if layer.weight_dtype != "fp8":
+            weight_limit = layer._quantization_limit(max(weight.shape), fp8)
+            sw = layer.weight_quantizer.scale(weight, fp8, weight_limit)
+            qw, wt = kernels.quantize(weight, sw, fp8_dtype=fp8, quantization_limit=weight_limit,
+                                      transpose=need_backward and needs_x and layer.cache_weight_transpose)
+        else:
+            qw, sw, wt = weight, layer.weight_scale, layer.weight_transpose
+        y = kernels.gemm(qx, qw, sx, sw, out_dtype=x2.dtype, bias=bias)
+        if need_backward:
+            if save_fp8:
+                saved_x = qxt
+            elif needs_w:
+                saved_x = x2.to(_FLOAT[layer.saved_input_dtype])
+            else:
+                saved_x = x2.new_empty(0)
+            # the scales this very forward used, not the quantizers' mutable state
+            ctx.save_for_backward(saved_x, sx, weight, sw, wt)
+            ctx.layer, ctx.shape, ctx.x_dtype, ctx.save_fp8, ctx.input_limit = layer, shape, x2.dtype, save_fp8, input_limit
+            ctx.weight_grad_dtype = weight.grad_dtype or weight.dtype
+            ctx.bias_grad_dtype = (bias.grad_dtype or bias.dtype) if bias is not None else None
+        return y.reshape(*shape[:-1], y.shape[-1])
+
+    @staticmethod
+    def backward(ctx, dy):
+        saved_x, sx, weight, sw, cached_wt = ctx.saved_tensors
+        layer = ctx.layer
+        fp8, bwd = layer.fp8_dtype, layer.backward_fp8_dtype
+        dy = dy.reshape(-1, layer.out_features).contiguous()
+        needs_x, needs_w, needs_b = ctx.needs_input_grad[:3]
+        grad_limit = layer._quantization_limit(max(dy.shape), bwd)
+        sg = layer.grad_quantizer.scale(dy, bwd, grad_limit)
+        # one read of dy serves dgrad (row-wise codes) and wgrad (transposed codes) when both are wanted
+        qg, qgt = kernels.quantize(dy, sg, rowwise=needs_x, transpose=needs_w, fp8_dtype=bwd, quantization_limit=grad_limit)
+        dx = dw = db = None
+        if needs_x:
+            if cached_wt.numel():
+                wt = cached_wt
+            elif layer.weight_dtype != "fp8":
+                # this forward's scale again: the delayed history does not advance in backward
+                _, wt = kernels.quantize(weight, sw, rowwise=False, transpose=True, fp8_dtype=fp8,
+                                         quantization_limit=layer._quantization_limit(max(weight.shape), fp8))
+            else:
+                wt = kernels.transpose(weight)
+            dx = kernels.gemm(qg, wt, sg, sw, out_dtype=ctx.x_dtype).reshape(*ctx.shape[:-1], layer.in_features)
+            del wt, qg
+        if needs_w:
+            if ctx.save_fp8:
+                xt = saved_x
+            else:
+                _, xt = kernels.quantize(saved_x, sx, rowwise=False, transpose=True, fp8_dtype=fp8, quantization_limit=ctx.input_limit)
+            dw = kernels.gemm(qgt, xt, sg, sx, out_dtype=ctx.weight_grad_dtype)
+        if needs_b:
+            db = dy.sum(dim=0, dtype=ctx.bias_grad_dtype)
+        return dx, dw, db, None, None

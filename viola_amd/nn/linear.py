@@ -1,9 +1,10 @@
 """FP8 Linear with FP8 / BF16 / FP16 weight storage (module surface of viola/nn/linear.py:150-412).
 
 Built here: `scaling="grouped"` (FP32 scales per 2-D weight block and per 1-D activation /
-gradient tile), FP32 accumulation, e4m3 / e5m2 operand formats. The reference's other recipes
-(per-tensor `current`/`delayed` scaling, `mxfp8`, blocked FP16 accumulation, Hadamard rotation) are
-accepted by the constructor signature but raise NotImplementedError.
+gradient tile) and the per-tensor recipes `scaling="current"` / `"delayed"` (one FP32 scale per tensor,
+delayed = the maximum of an amax history), FP32 accumulation, e4m3 / e5m2 operand formats. The
+reference's other recipes (`mxfp8`, blocked FP16 accumulation, quantization limits derived from it,
+Hadamard rotation) are accepted by the constructor signature but raise NotImplementedError.
 """
 
 import math
@@ -12,6 +13,7 @@ import torch
 from torch import nn
 
 from . import _grouped_kernels as grouped
+from . import _linear_kernels as kernels
 from ..precision import settings
 
 _FORMATS = {"e4m3": torch.float8_e4m3fn, "e5m2": torch.float8_e5m2}
@@ -19,13 +21,19 @@ _STORAGE = {"bf16": torch.bfloat16, "fp16": torch.float16}
 
 
 class _Quantizer(nn.Module):
-    """Amax history holder. Only the per-tensor recipes advance it; it is kept so that state_dicts
-    carry the same keys (`*_quantizer.history` + extra state) as the reference's (linear.py:14-33)."""
+    """Amax history and call counter of one per-tensor-scaled operand (viola/nn/linear.py:14-33); the grouped
+    recipe never advances it, but its state_dict carries the same keys."""
 
     def __init__(self, scaling, history_len, device):
         super().__init__()
         self.scaling, self.index = scaling, 0
         self.register_buffer("history", torch.zeros(history_len, device=device, dtype=torch.float32))
+
+    def scale(self, x, fp8_dtype=torch.float8_e4m3fn, quantization_limit=None):
+        scale = kernels.tensor_scale(x, history=self.history, index=self.index, delayed=self.scaling == "delayed",
+                                     fp8_dtype=fp8_dtype, quantization_limit=quantization_limit)
+        self.index += 1
+        return scale
 
     def get_extra_state(self):
         return {"index": self.index, "scaling": self.scaling}
@@ -57,15 +65,15 @@ class Linear(nn.Module):
         assert scaling in ("current", "delayed", "grouped", "mxfp8") and history_len > 0
         assert accum_dtype in ("fp32", "fp16") and accum_reduce_dtype in ("fp32", "bf16")
         assert accum_block_size >= 0 and accum_block_size % 32 == 0 and rotation_size in (0, 64)
-        if scaling != "grouped":
-            raise NotImplementedError(f"viola_amd builds scaling='grouped' only (got {scaling!r})")
+        if scaling == "mxfp8":
+            raise NotImplementedError("viola_amd builds scaling='grouped', 'current' and 'delayed' (got 'mxfp8')")
         if accum_dtype != "fp32" or accum_block_size or accum_reduce_dtype != "fp32" or rotation_size:
             raise NotImplementedError("viola_amd builds FP32 accumulation without rotation only")
         self.in_features, self.out_features = in_features, out_features
         self.mode, self.weight_dtype, self.saved_input_dtype = mode, weight_dtype, saved_input_dtype
         self.forward_dtype, self.backward_dtype = forward_dtype, backward_dtype
         self.fp8_dtype, self.backward_fp8_dtype = _FORMATS[forward_dtype], _FORMATS[backward_dtype]
-        self._grouped_scaling, self._native_scaling = True, False
+        self._grouped_scaling, self._native_scaling = scaling == "grouped", False
         self.weight_group_shape = tuple(weight_group_shape)
         self.input_group_shape = tuple(input_group_shape)
         self.grad_group_shape = tuple(grad_group_shape)
@@ -91,7 +99,10 @@ class Linear(nn.Module):
         self.bias = nn.Parameter(torch.empty(out_features, device=device, dtype=dtype)) if bias else None
         if self.bias is not None:
             self.bias.grad_dtype = gradient_dtype
-        scale_shape = grouped.scale_shape(shape, self.weight_group_shape) if fp8_storage else (0, 0)
+        if self._grouped_scaling:
+            scale_shape = grouped.scale_shape(shape, self.weight_group_shape) if fp8_storage else (0, 0)
+        else:
+            scale_shape = (1,) if fp8_storage else (0,)
         self.register_buffer("weight_scale", torch.ones(scale_shape, device=device, dtype=torch.float32), persistent=fp8_storage)
         self.register_buffer("weight_transpose", torch.empty(0, 0, device=device, dtype=self.fp8_dtype), persistent=False)
         self.register_buffer("weight_transpose_scale", torch.empty(0, 0, device=device, dtype=torch.float32), persistent=False)
@@ -105,6 +116,13 @@ class Linear(nn.Module):
         """Clamp magnitude for a group; None means the format's own maximum (linear.py:244-253)."""
         if self.quantization_limit is not None:
             return min(self.quantization_limit, torch.finfo(dtype).max)
+        return None
+
+    def _quantization_limit(self, reduction, fp8_dtype):
+        """Clamp magnitude of a per-tensor-scaled operand; None means the format's own maximum (linear.py:232-242,
+        whose FP16-accumulation branch is not built)."""
+        if self.quantization_limit is not None:
+            return min(self.quantization_limit, torch.finfo(fp8_dtype).max)
         return None
 
     def _group_gemm(self, a, b, sa, sb, ga, gb, *, out_dtype, bias=None):
@@ -138,6 +156,16 @@ class Linear(nn.Module):
             self._pending_refresh = True
             return
         self._pending_refresh = False
+        if not self._grouped_scaling:
+            # one scale for the tensor; the transposed codes, when cached, come from the same read (linear.py:288-297)
+            limit = self._quantization_limit(max(self.in_features, self.out_features), self.fp8_dtype)
+            if self.cache_weight_transpose and self.weight_transpose.numel() == 0:
+                self.weight_transpose = torch.empty((self.in_features, self.out_features), device=master.device, dtype=self.fp8_dtype)
+            scale = self.weight_quantizer.scale(master, self.fp8_dtype, limit)
+            self.weight_scale.copy_(scale)
+            kernels.quantize(master, scale, transpose=self.cache_weight_transpose, fp8_dtype=self.fp8_dtype, out=self.weight,
+                             out_t=self.weight_transpose if self.cache_weight_transpose else None, quantization_limit=limit)
+            return
         limit = self._group_limit(self.weight_group_shape, self.fp8_dtype, weight=True)
         grouped.quantize(master, self.fp8_dtype, self.weight_group_shape, limit=limit,
                          out=self.weight, scale_out=self.weight_scale)
@@ -145,6 +173,9 @@ class Linear(nn.Module):
             self._build_transpose(limit)
 
     def _build_transpose(self, limit):
+        if not self._grouped_scaling:
+            self.weight_transpose = kernels.transpose(self.weight)
+            return
         self.weight_transpose, self.weight_transpose_scale = grouped.transpose(
             self.weight, self.weight_scale, self.weight_group_shape, limit=limit)
 
@@ -152,6 +183,8 @@ class Linear(nn.Module):
         if self.weight_dtype != "fp8":
             return self.weight.float()
         assert self.weight.is_cuda, "viola_amd kernels run on the GPU only"
+        if not self._grouped_scaling:
+            return self.weight.float() * self.weight_scale
         return grouped.dequantize(self.weight, self.weight_scale, self.weight_group_shape)
 
     @classmethod
@@ -179,8 +212,11 @@ class Linear(nn.Module):
             self.refresh_weight(self._master())
         need_backward = torch.is_grad_enabled() and (
             x.requires_grad or self.weight.requires_grad or (self.bias is not None and self.bias.requires_grad))
-        from ._grouped_linear import GroupedLinear
-        return GroupedLinear.apply(x, self.weight, self.bias, self, need_backward)
+        if self._grouped_scaling:
+            from ._grouped_linear import GroupedLinear
+            return GroupedLinear.apply(x, self.weight, self.bias, self, need_backward)
+        from ._tensor_linear import TensorLinear
+        return TensorLinear.apply(x, self.weight, self.bias, self, need_backward)
 
     # ------------------------------------------------------------------ module plumbing
     def _apply(self, fn, recurse=True):
@@ -225,7 +261,7 @@ class Linear(nn.Module):
     def rebuild_weight_cache(self):
         """Rebuild W^T from the loaded codes and scales without requantizing W."""
         if self.cache_weight_transpose and self.weight_dtype == "fp8" and self.weight.is_cuda:
-            self._build_transpose(self._group_limit(self.weight_group_shape, self.fp8_dtype, weight=True))
+            self._build_transpose(self._group_limit(self.weight_group_shape, self.fp8_dtype, weight=True) if self._grouped_scaling else None)
 
     def extra_repr(self):
         return (f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, "

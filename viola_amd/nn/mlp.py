@@ -66,6 +66,8 @@ class MLP(nn.Module):
         self.hidden_features = hidden_features
         self.out_features = in_features if out_features is None else out_features
         self.activation, self.autotune = activation, autotune
+        if linear_options.get("scaling", "current") != "grouped":
+            raise NotImplementedError("viola_amd builds the fused gated MLP for scaling='grouped' only")
         self.gate_up = Linear(in_features, 2 * hidden_features, autotune=autotune, **linear_options)
         self.down = Linear(hidden_features, self.out_features, autotune=autotune, **linear_options)
 
