@@ -78,6 +78,10 @@ int viola_tensor_amax(const void* x, int x_dtype, int64_t n, float* maxima, int6
 int viola_tensor_scale(const float* maxima, int64_t parts, float* history, int history_len, int64_t index, int delayed,
                        float limit, float* scale, viola_stream_t stream);
 
+/* Both launches of `tensor_scale` behind one call. */
+int viola_tensor_amax_scale(const void* x, int x_dtype, int64_t n, float* maxima, int64_t parts, float* history,
+                            int history_len, int64_t index, int delayed, float limit, float* scale, viola_stream_t stream);
+
 /* viola/nn/_linear_kernels.py:245-250 `quantize` (_quantize_kernel :74-104): with the tensor's one scale,
  * q[r, c] = fp8(isnan(x) ? x : clamp(x / scale[0], +-limit)) and / or qt[c, r] = the same code; q or qt may be NULL. */
 int viola_tensor_quantize(const void* x, int x_dtype, int64_t rows, int64_t cols, const float* scale, void* q, void* qt,

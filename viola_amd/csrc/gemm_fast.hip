@@ -281,6 +281,7 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
     struct Operands {
         uint4 a[FKG][TM], b[FKG][TN];
         float sa[FKG][TM], sb[FKG][TN];
+        i32x8 wide_a[TM], wide_b[TN];                                        // TENSOR: both K groups of a sub-tile row, one operand
     };
     auto scale_block = [&](int64_t c) -> const float* {                      // a scales of chunk c: [kg][row]; b scales F_SBLOCK later
         return reinterpret_cast<const float*>(lds + F_SCALE + ((c / F_SCHUNKS) & 1) * 2 * F_SBLOCK) + (c % F_SCHUNKS) * FKG * BM;
@@ -290,6 +291,21 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
         const uint8_t* tile_b = tile_a + F_TILE;
         const float* scale_a = scale_block(c);
         const float* scale_b = scale_a + F_SBLOCK / 4;
+        if constexpr (TENSOR) {
+#pragma unroll
+            for (int j = 0; j < TM; ++j) {
+                const i32x4 lo = *reinterpret_cast<const i32x4*>(tile_a + (rd_a + j * 32 * FBK));
+                const i32x4 hi = *reinterpret_cast<const i32x4*>(tile_a + ((rd_a + j * 32 * FBK) ^ 32));
+                o.wide_a[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+#pragma unroll
+            for (int i = 0; i < TN; ++i) {
+                const i32x4 lo = *reinterpret_cast<const i32x4*>(tile_b + (rd_b + (b_sub(i) - b_sub(0)) * FBK));
+                const i32x4 hi = *reinterpret_cast<const i32x4*>(tile_b + ((rd_b + (b_sub(i) - b_sub(0)) * FBK) ^ 32));
+                o.wide_b[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+            return;
+        }
 #pragma unroll
         for (int kg = 0; kg < FKG; ++kg) {
 #pragma unroll
@@ -307,20 +323,18 @@ __global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int b
     // caller's global loads and LDS reads for later chunks go there, spread over the chunk).
     auto compute = [&](const Operands& o, int64_t c, auto&& between) {
         if constexpr (TENSOR) {
-            constexpr int UNITS = TN * TM, STEPS_PER = FKG * 2;
+            constexpr int STEPS_PER = FKG * 2;
 #pragma unroll
-            for (int unit = 0; unit < UNITS; ++unit) {
-                const int i = unit / TM, j = unit % TM;
-                const i32x8 ob = {(int)o.b[0][i].x, (int)o.b[0][i].y, (int)o.b[0][i].z, (int)o.b[0][i].w,
-                                  (int)o.b[1][i].x, (int)o.b[1][i].y, (int)o.b[1][i].z, (int)o.b[1][i].w};
-                const i32x8 oa = {(int)o.a[0][j].x, (int)o.a[0][j].y, (int)o.a[0][j].z, (int)o.a[0][j].w,
-                                  (int)o.a[1][j].x, (int)o.a[1][j].y, (int)o.a[1][j].z, (int)o.a[1][j].w};
-                // both operands give a lane the same 32 of the chunk's 64 k (16 of each K group), so every product
-                // meets its partner whatever order the instruction walks them in
-                total[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ob, oa, total[i][j], B_BF8 ? 1 : 0, A_BF8 ? 1 : 0, 0, 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
+            for (int i = 0; i < TN; ++i) {
 #pragma unroll
-                for (int step = unit * STEPS_PER; step < (unit + 1) * STEPS_PER; ++step) between(step);
+                for (int j = 0; j < TM; ++j) {
+                    // both operands give a lane the same 32 of the chunk's 64 k (16 of each K group), so every product
+                    // meets its partner whatever order the instruction walks them in
+                    total[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(o.wide_b[i], o.wide_a[j], total[i][j], B_BF8 ? 1 : 0, A_BF8 ? 1 : 0, 0, 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int step = 0; step < STEPS_PER; ++step) between((i * TM + j) * STEPS_PER + step);
+                }
             }
             return;
         }

@@ -216,6 +216,13 @@ extern "C" int viola_tensor_scale(const float* maxima, int64_t parts, float* his
     return viola_launch_status();
 }
 
+extern "C" int viola_tensor_amax_scale(const void* x, int x_dtype, int64_t n, float* maxima, int64_t parts, float* history,
+                                       int history_len, int64_t index, int delayed, float limit, float* scale,
+                                       viola_stream_t stream) {
+    const int status = viola_tensor_amax(x, x_dtype, n, maxima, parts, stream);
+    return status ? status : viola_tensor_scale(maxima, parts, history, history_len, index, delayed, limit, scale, stream);
+}
+
 extern "C" int viola_tensor_quantize(const void* x, int x_dtype, int64_t rows, int64_t cols, const float* scale, void* q,
                                      void* qt, int q_dtype, float limit, viola_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);

@@ -26,10 +26,9 @@ def tensor_scale(x, *, history=None, index=0, delayed=False, fp8_dtype=torch.flo
     if history is None:
         history = torch.zeros(1, device=x.device, dtype=torch.float32)
     scale = torch.empty(1, device=x.device, dtype=torch.float32)
-    _lib.call("viola_tensor_amax", _lib.ptr(x), _lib.code(x.dtype), x.numel(), _lib.ptr(maxima), parts)
     limit = torch.finfo(fp8_dtype).max if quantization_limit is None else quantization_limit
-    _lib.call("viola_tensor_scale", _lib.ptr(maxima), parts, _lib.ptr(history), history.numel(), int(index),
-              int(bool(delayed)), float(limit), _lib.ptr(scale))
+    _lib.call("viola_tensor_amax_scale", _lib.ptr(x), _lib.code(x.dtype), x.numel(), _lib.ptr(maxima), parts, _lib.ptr(history),
+              history.numel(), int(index), int(bool(delayed)), float(limit), _lib.ptr(scale))
     return scale
 
 
