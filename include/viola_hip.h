@@ -78,6 +78,13 @@ int viola_tensor_amax(const void* x, int x_dtype, int64_t n, float* maxima, int6
 int viola_tensor_scale(const float* maxima, int64_t parts, float* history, int history_len, int64_t index, int delayed,
                        float limit, float* scale, viola_stream_t stream);
 
+/* viola_tensor_amax for a [rows, cols] matrix that also leaves fp32 column sums of each of `slices` row slices in
+ * column_partial [slices, cols] (finish with viola_column_reduce): the bias gradient dy.sum(0) of
+ * viola/nn/linear.py:143 from the amax pass over dy. maxima receives ceil(cols / piece / 256) * slices values,
+ * piece = 16 bytes of x; cols must be a multiple of the piece, x and column_partial 16-byte aligned. */
+int viola_tensor_amax_columns(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t slices, float* maxima,
+                              float* column_partial, viola_stream_t stream);
+
 /* Both launches of `tensor_scale` behind one call. */
 int viola_tensor_amax_scale(const void* x, int x_dtype, int64_t n, float* maxima, int64_t parts, float* history,
                             int history_len, int64_t index, int delayed, float limit, float* scale, viola_stream_t stream);

@@ -46,6 +46,32 @@ def test_tensor_scale_current_and_delayed(dtype, n):
         assert torch.equal(scale.cpu(), expected) and torch.equal(history.cpu(), reference)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(1, 8), (65, 96), (300, 200), (8192, 4096), (7, 2056), (33, 45)])
+def test_tensor_scale_with_column_sums(dtype, shape):
+    """The amax pass that also returns x.sum(0): same scale and history as the plain pass, sums equal to fp32 column
+    sums within summation-order error (the reference compares db with torch's default closeness, checks/linear.py:40)."""
+    k = _k()
+    torch.manual_seed(65)
+    x = (torch.randn(shape) * 2).to(dtype)
+    x[0, 0] = float("nan") if shape[0] > 1 else x[0, 0]
+    history = torch.zeros(2, device="cuda")
+    scale, total = k.tensor_scale_and_column_sum(x.cuda(), torch.float32, history=history, index=0, fp8_dtype=E5)
+    expected, after = ot.tensor_scale(x, torch.zeros(2), 0, limit=torch.finfo(E5).max)
+    assert torch.equal(scale.cpu(), expected) and torch.equal(history.cpu(), after)
+    reference = x.double().sum(0)
+    keep = ~reference.isnan()
+    assert torch.equal(total.cpu().isnan(), reference.isnan())
+    magnitude = x.double().abs().nan_to_num(0).sum(0)
+    assert ((total.cpu().double() - reference)[keep].abs() <= 1e-6 * magnitude[keep] + 1e-30).all()
+    low = k.tensor_scale_and_column_sum(x.cuda(), torch.bfloat16)[1]
+    assert low.dtype == torch.bfloat16
+    if shape[1] % (16 // x.element_size()) == 0:                               # one read: the fp32 sums, rounded once
+        assert torch.equal(low[keep.cuda()], total.bfloat16()[keep.cuda()])
+    else:                                                                       # two passes: torch's own sum(0, dtype)
+        assert torch.equal(low, x.cuda().sum(0, dtype=torch.bfloat16)) or shape[0] > 1 and bool(x[0, 0].isnan())
+
+
 @pytest.mark.parametrize("in_dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("fp8", [E4, E5])
 @pytest.mark.parametrize("shape", [(65, 96), (64, 64), (70, 45), (1, 33), (300, 200), (129, 1024), (8192, 1024)])

@@ -36,6 +36,7 @@ _SIGNATURES = {
     "viola_adam_update": [_p, _i, _p, _i, _p, _p, _i, _l, _f, _f, _f, _f, _f, _f, _f, _i, _l, _l, _l, _i, _i, _p],
     "viola_tensor_amax": [_p, _i, _l, _p, _l, _p],
     "viola_tensor_scale": [_p, _l, _p, _i, _l, _i, _f, _p, _p],
+    "viola_tensor_amax_columns": [_p, _i, _l, _l, _l, _p, _p, _p],
     "viola_tensor_amax_scale": [_p, _i, _l, _p, _l, _p, _i, _l, _i, _f, _p, _p],
     "viola_tensor_quantize": [_p, _i, _l, _l, _p, _p, _p, _i, _f, _p],
     "viola_tensor_gemm": [_p, _i, _p, _i, _p, _p, _l, _l, _l, _p, _i, _p, _i, _p],

@@ -60,6 +60,56 @@ __global__ __launch_bounds__(256) void tensor_amax_kernel(const TIn* __restrict_
     if (threadIdx.x == 0) maxima[blockIdx.x] = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
 }
 
+// The same maximum together with column sums of a [rows, cols] matrix from the one read (the bias gradient of a
+// Linear rides on the amax pass over dY): block (x, y) covers 256 column pieces of 16 bytes and row slice y,
+// maxima[y * gridDim.x + x] = its max |x|, column_partial[y][c] = its fp32 column sums. cols is a multiple of the
+// piece, x 16-byte aligned.
+template <typename TIn>
+__global__ __launch_bounds__(256) void tensor_amax_columns_kernel(const TIn* __restrict__ x, int64_t rows, int64_t cols,
+                                                                   int64_t slice_rows, float* __restrict__ maxima,
+                                                                   float* __restrict__ column_partial) {
+    constexpr int N = Vec16<TIn>::N;
+    const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * N;
+    const int64_t begin = (int64_t)blockIdx.y * slice_rows, end = begin + slice_rows < rows ? begin + slice_rows : rows;
+    float sum[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) sum[i] = 0.0f;
+    float m = 0.0f;
+    if (col < cols) {
+        auto take = [&](int64_t r) {
+            const uint4 raw = *reinterpret_cast<const uint4*>(x + r * cols + col);
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+            float v[N];
+            if constexpr (sizeof(TIn) == 4) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) v[i] = __uint_as_float(w[i]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    TIn lo, hi;
+                    __builtin_memcpy(&lo, reinterpret_cast<const uint16_t*>(&w[i]), 2);
+                    __builtin_memcpy(&hi, reinterpret_cast<const uint16_t*>(&w[i]) + 1, 2);
+                    v[2 * i] = to_f32(lo);
+                    v[2 * i + 1] = to_f32(hi);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < N; ++i) { sum[i] += v[i]; m = fmaxf(m, fabsf(v[i])); }
+        };
+        int64_t r = begin;
+        for (; r + 3 < end; r += 4) { take(r); take(r + 1); take(r + 2); take(r + 3); }
+        for (; r < end; ++r) take(r);
+        float* dst = column_partial + (int64_t)blockIdx.y * cols + col;
+#pragma unroll
+        for (int i = 0; i < N; i += 4) *reinterpret_cast<float4*>(dst + i) = make_float4(sum[i], sum[i + 1], sum[i + 2], sum[i + 3]);
+    }
+    __shared__ float part[4];
+    m = wave_max(m);
+    if (threadIdx.x % WAVE == 0) part[threadIdx.x / WAVE] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) maxima[(int64_t)blockIdx.y * gridDim.x + blockIdx.x] = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
+}
+
 // One block: amax = max(maxima); scale = max(delayed and index != 0 ? max(history before this call) : amax, 1e-30) / limit;
 // history[index % history_len] = amax.
 __global__ __launch_bounds__(256) void tensor_scale_kernel(const float* __restrict__ maxima, int64_t parts, float* history,
@@ -213,6 +263,20 @@ extern "C" int viola_tensor_scale(const float* maxima, int64_t parts, float* his
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     VIOLA_CHECK_ARG(maxima && parts > 0 && history && history_len > 0 && index >= 0 && limit > 0.0f && scale);
     hipLaunchKernelGGL(tensor_scale_kernel, dim3(1), dim3(256), 0, stream, maxima, parts, history, history_len, index, delayed, limit, scale);
+    return viola_launch_status();
+}
+
+extern "C" int viola_tensor_amax_columns(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t slices, float* maxima,
+                                         float* column_partial, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_float(x_dtype) && rows > 0 && cols > 0 && slices > 0 && slices <= 65535 && x && maxima && column_partial);
+    const int piece = 16 / viola_dtype_size(x_dtype);
+    VIOLA_CHECK_ARG(cols % piece == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(column_partial) % 16 == 0);
+    const int64_t slice_rows = (rows + slices - 1) / slices;
+    const dim3 grid((unsigned)((cols / piece + 255) / 256), (unsigned)slices);
+    if (x_dtype == VIOLA_F32) hipLaunchKernelGGL(tensor_amax_columns_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(x), rows, cols, slice_rows, maxima, column_partial);
+    else if (x_dtype == VIOLA_BF16) hipLaunchKernelGGL(tensor_amax_columns_kernel<bf16_t>, grid, dim3(256), 0, stream, static_cast<const bf16_t*>(x), rows, cols, slice_rows, maxima, column_partial);
+    else hipLaunchKernelGGL(tensor_amax_columns_kernel<f16_t>, grid, dim3(256), 0, stream, static_cast<const f16_t*>(x), rows, cols, slice_rows, maxima, column_partial);
     return viola_launch_status();
 }
 

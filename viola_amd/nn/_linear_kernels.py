@@ -16,6 +16,34 @@ def transpose(x, out=None):
     return out
 
 
+def tensor_scale_and_column_sum(x, sum_dtype, *, history=None, index=0, delayed=False, fp8_dtype=torch.float8_e4m3fn,
+                                quantization_limit=None):
+    """(tensor_scale(x), x.sum(0, dtype=sum_dtype)) of a matrix from one read of x; fp32 sums in a fixed order. Falls
+    back to two passes when the columns are not whole 16-byte pieces."""
+    assert x.is_cuda and x.dim() == 2
+    x = x.contiguous()
+    rows, cols = x.shape
+    piece = 16 // x.element_size()
+    if rows == 0 or cols % piece or x.data_ptr() % 16:
+        scale = tensor_scale(x, history=history, index=index, delayed=delayed, fp8_dtype=fp8_dtype, quantization_limit=quantization_limit)
+        return scale, x.sum(dim=0, dtype=sum_dtype)
+    blocks_x = -(-(cols // piece) // 256)
+    slices = max(1, min(-(-rows // 8), 512 // blocks_x, 65535))
+    parts = blocks_x * slices
+    maxima = torch.empty(parts, device=x.device, dtype=torch.float32)
+    partial = torch.empty((slices, cols), device=x.device, dtype=torch.float32)
+    if history is None:
+        history = torch.zeros(1, device=x.device, dtype=torch.float32)
+    scale = torch.empty(1, device=x.device, dtype=torch.float32)
+    total = torch.empty(cols, device=x.device, dtype=sum_dtype)
+    limit = torch.finfo(fp8_dtype).max if quantization_limit is None else quantization_limit
+    _lib.call("viola_tensor_amax_columns", _lib.ptr(x), _lib.code(x.dtype), rows, cols, slices, _lib.ptr(maxima), _lib.ptr(partial))
+    _lib.call("viola_tensor_scale", _lib.ptr(maxima), parts, _lib.ptr(history), history.numel(), int(index), int(bool(delayed)),
+              float(limit), _lib.ptr(scale))
+    _lib.call("viola_column_reduce", _lib.ptr(partial), slices, cols, _lib.ptr(total), _lib.code(sum_dtype))
+    return scale, total
+
+
 def tensor_scale(x, *, history=None, index=0, delayed=False, fp8_dtype=torch.float8_e4m3fn, quantization_limit=None):
     """scale [1] = max(amax(x) or, delayed after the first call, the history's maximum, 1e-30) / limit; the new amax
     goes into history[index % len]. Scratch is one float per 64 Ki elements, never a full-sized temporary."""

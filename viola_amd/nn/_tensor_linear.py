@@ -50,10 +50,14 @@ class TensorLinear(torch.autograd.Function):
         dy = dy.reshape(-1, layer.out_features).contiguous()
         needs_x, needs_w, needs_b = ctx.needs_input_grad[:3]
         grad_limit = layer._quantization_limit(max(dy.shape), bwd)
-        sg = layer.grad_quantizer.scale(dy, bwd, grad_limit)
+        dx = dw = db = None
+        if needs_b:
+            # the bias gradient rides on the amax pass over dy
+            sg, db = layer.grad_quantizer.scale_and_column_sum(dy, ctx.bias_grad_dtype, bwd, grad_limit)
+        else:
+            sg = layer.grad_quantizer.scale(dy, bwd, grad_limit)
         # one read of dy serves dgrad (row-wise codes) and wgrad (transposed codes) when both are wanted
         qg, qgt = kernels.quantize(dy, sg, rowwise=needs_x, transpose=needs_w, fp8_dtype=bwd, quantization_limit=grad_limit)
-        dx = dw = db = None
         if needs_x:
             if cached_wt.numel():
                 wt = cached_wt
@@ -71,6 +75,4 @@ class TensorLinear(torch.autograd.Function):
             else:
                 _, xt = kernels.quantize(saved_x, sx, rowwise=False, transpose=True, fp8_dtype=fp8, quantization_limit=ctx.input_limit)
             dw = kernels.gemm(qgt, xt, sg, sx, out_dtype=ctx.weight_grad_dtype)
-        if needs_b:
-            db = dy.sum(dim=0, dtype=ctx.bias_grad_dtype)
         return dx, dw, db, None, None

@@ -35,6 +35,14 @@ class _Quantizer(nn.Module):
         self.index += 1
         return scale
 
+    def scale_and_column_sum(self, x, sum_dtype, fp8_dtype=torch.float8_e4m3fn, quantization_limit=None):
+        """scale(x) and x.sum(0) from one read of the matrix x."""
+        result = kernels.tensor_scale_and_column_sum(x, sum_dtype, history=self.history, index=self.index,
+                                                     delayed=self.scaling == "delayed", fp8_dtype=fp8_dtype,
+                                                     quantization_limit=quantization_limit)
+        self.index += 1
+        return result
+
     def get_extra_state(self):
         return {"index": self.index, "scaling": self.scaling}
 
