@@ -218,6 +218,28 @@ def main():
                                             refresh_gbs=(4 + 1 + 4 / 1024) * K * N / (refresh_ms * 1e-3) / 1e9)
         viola_amd.precision._settings.update(master_weight_dtype=torch.float32, gradient_dtype=None)
 
+    if not args.skip_muon:
+        # the reference's default recipe on the same layer: one scale per tensor, epilogue scaling (the GEMM runs on
+        # the K = 64 f8f6f4 MFMA, the kernel the 5 PFLOP/s figure belongs to)
+        import viola_amd
+        viola_amd.set_gradient_dtype("bf16")
+        torch.manual_seed(2)
+        current = viola_amd.nn.Linear(K, N, device="cuda", dtype=torch.bfloat16, scaling="current", forward_dtype="e4m3",
+                                      backward_dtype="e5m2", mode="memory", weight_dtype="fp8")
+        viola_amd.precision._settings["gradient_dtype"] = None
+        xc = torch.randn(M, K, device="cuda").bfloat16().requires_grad_()
+
+        def current_step():
+            xc.grad = current.weight.grad = current.bias.grad = None
+            current(xc).backward(dy)
+        c_ms, _ = timed(current_step, args.steps, args.warmup)
+        cb = kernel_breakdown(current_step, min(args.steps, 50))
+        cg = cb["viola_tensor_gemm"]
+        extra["linear_current_scaling"] = dict(step_ms=c_ms, tflops=flops / (c_ms * 1e-3) / 1e12, gemm_avg_ms=cg["avg_ms"],
+                                               gemm_tflops=2 * M * K * N / (cg["avg_ms"] * 1e-3) / 1e12,
+                                               gemm_frac_fp8_peak=2 * M * K * N / (cg["avg_ms"] * 1e-3) / 1e12 / PEAK["fp8_tflops"],
+                                               launches_per_step=sum(v["launches_per_step"] for v in cb.values()))
+
     if args.calibrate:
         from viola_amd.optim import _kernels as ok
         src = torch.ones(1 << 26, device="cuda")
