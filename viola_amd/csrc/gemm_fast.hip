@@ -117,9 +117,10 @@ template <typename TO> __device__ __forceinline__ float rounded(float v) { retur
 // per-group fold, so a chunk's 64 k go through one v_mfma_f32_32x32x64_f8f6f4 per sub-tile straight into the totals.
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 template <int MODE, bool A_BF8, bool B_BF8, bool B_ROWSCALE, typename TO, int TN, bool TENSOR = false>
-__global__ __launch_bounds__(FTHREADS, 2) void group_gemm_fast(GemmArgs p, int bias_dtype) {
+__global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(GemmArgs p, int bias_dtype) {
     static_assert(!TENSOR || (MODE == MODE_PLAIN && !B_ROWSCALE), "per-tensor scaling: plain mode only");
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[F_LDS];
+    // without scale blocks the ring plus the epilogue's bias row is all the LDS a block needs: three blocks share a CU
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[TENSOR ? F_RAW + 1024 : F_LDS];
 
     // wave grid 2 (m) x 2 (n), 2 x 2 sub-tiles each. Plain / gated backward: sub-tile i of wave wn covers b rows
     // 64 wn + 32 i. Gated forward: the tile's b rows are 64 gate rows then the 64 up rows of the same n, and
