@@ -100,6 +100,16 @@ int viola_tensor_gemm(const void* a, int a_dtype, const void* b, int b_dtype, co
                       int64_t m, int64_t n, int64_t k, const void* bias, int bias_dtype, void* out, int out_dtype,
                       viola_stream_t stream);
 
+/* ---------------------------------------------------------------- MXFP8: E8M0 scales per 32 k
+ * viola/nn/_grouped_kernels.py:310-328 `gemm` with native=True (gemm_kernel :195-293 on the block-scaled MMA of
+ * :174-192): out[m, n] = sum_kg (sum_{k in kg} a[m, k] b[n, k]) * 2^(sa[m / ar, kg] - 127) * 2^(sb[n / br, kg] - 127)
+ * (+ bias[n]), the scaling done by v_mfma_scale_f32_32x32x64_f8f6f4. sa [ceil(m / ar), k / 32], sb [ceil(n / br), k / 32]
+ * bytes. Returns VIOLA_EUNSUPPORTED unless k % 128 == 0, a and b are 16-byte and the scales 4-byte aligned and
+ * br is 1 or a multiple of 32: the caller then converts the scales to FP32 and calls viola_group_gemm (same values). */
+int viola_mx_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const uint8_t* sa, const uint8_t* sb,
+                  int64_t m, int64_t n, int64_t k, int ar, int br, const void* bias, int bias_dtype, void* out,
+                  int out_dtype, viola_stream_t stream);
+
 /* ---------------------------------------------------------------- grouped-scale FP8 GEMM
  * viola/nn/_grouped_kernels.py:310-328 `gemm` (gemm_kernel :195-293).
  * out[m, n] = sum over 32-wide K groups kg of (sum_{k in kg} a[m,k]*b[n,k]) * sa[m/ar, k/ak] * sb[n/br, k/bk]

@@ -381,6 +381,29 @@ extern "C" int viola_tensor_gemm(const void* a, int a_dtype, const void* b, int 
     return launch_out<MODE_PLAIN>(p, a_dtype, b_dtype, bias_dtype, out_dtype, false, false, grid, stream);
 }
 
+extern "C" int viola_mx_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const uint8_t* sa, const uint8_t* sb,
+                             int64_t m, int64_t n, int64_t k, int ar, int br, const void* bias, int bias_dtype, void* out,
+                             int out_dtype, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_fp8(a_dtype) && viola_is_fp8(b_dtype) && viola_is_float(out_dtype));
+    VIOLA_CHECK_ARG(m >= 0 && n >= 0 && k >= 0 && ar > 0 && br > 0 && (!bias || viola_is_float(bias_dtype)));
+    if (m == 0 || n == 0) return 0;
+    VIOLA_CHECK_ARG(out && (k == 0 || (a && b && sa && sb)));
+    const int64_t gy = (m + BM - 1) / BM, gx = (n + BN - 1) / BN;
+    VIOLA_CHECK_ARG(gy <= 65535);
+    // the block-scaled MFMA path only: whole 128-k scale pieces, 16-byte aligned codes, 4-byte aligned scale rows
+    if (k == 0 || k % 128 != 0 || !aligned16(a) || !aligned16(b) || reinterpret_cast<uintptr_t>(sa) % 4 != 0 ||
+        reinterpret_cast<uintptr_t>(sb) % 4 != 0 || n * k >= (1ll << 31) || (int64_t)BM * k >= (1ll << 31) ||
+        (br != 1 && br % 32 != 0))
+        return VIOLA_EUNSUPPORTED;
+    GemmArgs p = {};
+    p.a = static_cast<const uint8_t*>(a); p.b = static_cast<const uint8_t*>(b);
+    p.sa = reinterpret_cast<const float*>(sa); p.sb = reinterpret_cast<const float*>(sb);
+    p.bias = bias; p.out = out; p.m = m; p.n = n; p.k = k; p.lda = k; p.ldb = k; p.ldo = n;
+    p.ldsa = k / 32; p.ldsb = k / 32; p.ar = ar; p.br = br; p.ak_shift = 5; p.bk_shift = 5;
+    return launch_mx_gemm_fast(p, a_dtype, b_dtype, bias_dtype, out_dtype, dim3((unsigned)gx, (unsigned)gy), stream);
+}
+
 extern "C" int viola_gated_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,
                                 int64_t m, int64_t h, int64_t k, int ar, int ak, int br, int bk, const void* bias,
                                 int bias_dtype, void* aux, void* out, int out_dtype, int activation, int backward,

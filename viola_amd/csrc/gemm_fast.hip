@@ -116,11 +116,21 @@ template <typename TO> __device__ __forceinline__ float rounded(float v) { retur
 // TENSOR: one scale per operand (p.sa[0], p.sb[0]) applied to the finished sums, out = (acc * sa) * sb + bias: no
 // per-group fold, so a chunk's 64 k go through one v_mfma_f32_32x32x64_f8f6f4 per sub-tile straight into the totals.
 typedef int i32x8 __attribute__((ext_vector_type(8)));
-template <int MODE, bool A_BF8, bool B_BF8, bool B_ROWSCALE, typename TO, int TN, bool TENSOR = false>
+// MX: E8M0 scales (one byte per 32 k; p.sa / p.sb point at bytes, ldsa / ldsb are bytes per scale row) applied by the
+// hardware inside v_mfma_scale_f32_32x32x64_f8f6f4. The instruction's first 32-k block is operand registers 0..3 of all
+// 64 lanes and takes its scale from lanes 0..31 (one byte per row), the second block is registers 4..7 with the scale
+// of lanes 32..63 (measured: a scale change confined to one K group only gives the right product in this arrangement).
+// That is the layout the per-tensor path already has (registers 0..3 = the lane's 16 bytes of K group 0, 4..7 = of K
+// group 1), so lane (row, half) hands over the scale byte of K group `half` of its row. Scales travel in blocks of 16
+// K groups (one 16-byte piece per tile row and operand), double-buffered behind the ring; k must be a multiple of 128.
+constexpr int MX_GROUPS = 16, MX_CHUNKS = MX_GROUPS / FKG, MX_BLOCK = 2 * BM * MX_GROUPS;   // bytes of one block, a then b
+template <int MODE, bool A_BF8, bool B_BF8, bool B_ROWSCALE, typename TO, int TN, bool TENSOR = false, bool MX = false>
 __global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(GemmArgs p, int bias_dtype) {
     static_assert(!TENSOR || (MODE == MODE_PLAIN && !B_ROWSCALE), "per-tensor scaling: plain mode only");
+    static_assert(!MX || (MODE == MODE_PLAIN && !TENSOR), "block-scaled MFMA: plain mode only");
+    constexpr bool NOFOLD = TENSOR || MX;                                   // the products of a chunk go straight into the totals
     // without scale blocks the ring plus the epilogue's bias row is all the LDS a block needs: three blocks share a CU
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[TENSOR ? F_RAW + 1024 : F_LDS];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[TENSOR ? F_RAW + 1024 : MX ? F_RAW + 2 * MX_BLOCK : F_LDS];
 
     // wave grid 2 (m) x 2 (n), 2 x 2 sub-tiles each. Plain / gated backward: sub-tile i of wave wn covers b rows
     // 64 wn + 32 i. Gated forward: the tile's b rows are 64 gate rows then the 64 up rows of the same n, and
@@ -236,6 +246,16 @@ __global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(Gemm
         load16_to_lds(res_sa, at, inside ? sa_off : OUTSIDE, (uint32_t)(block * F_SGROUPS * 4));
         load16_to_lds(res_sb, at + F_SBLOCK, inside ? sb_off : OUTSIDE, (uint32_t)(block * F_SGROUPS * 4));
     };
+    // MX: scale block `block` (K groups 16 block ..) -> buffer block & 1: waves 0, 1 fetch the a rows' pieces, waves 2, 3 the b rows'
+    const i32x4 res_mxa = raw_resource(p.sa, (p.m + p.ar - 1) / p.ar * p.ldsa);
+    const i32x4 res_mxb = raw_resource(sbptr, (b_rows_total + p.br - 1) / p.br * p.ldsb);
+    const uint32_t mx_off = tid < BM ? (uint32_t)(a_global_row(tid) / p.ar * p.ldsa + (k_begin >> 5))
+                                     : (uint32_t)(b_global_row(tid - BM) / p.br * p.ldsb + (k_begin >> 5));
+    auto issue_mx_scales = [&](int64_t block) {
+        const bool inside = block * MX_GROUPS < groups_total;
+        const uint32_t at = lds_base + F_RAW + (uint32_t)(block & 1) * MX_BLOCK + (uint32_t)wave * 1024;
+        load16_to_lds(wave < 2 ? res_mxa : res_mxb, at, inside ? mx_off : OUTSIDE, (uint32_t)(block * MX_GROUPS));
+    };
     // raw area -> [group][row] floats of scale buffer `block & 1`; groups past the k range become zero (their
     // products are zero too, and a neighbouring row's value must not meet them)
     auto arrange_scales = [&](int64_t block) {
@@ -282,7 +302,8 @@ __global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(Gemm
     struct Operands {
         uint4 a[FKG][TM], b[FKG][TN];
         float sa[FKG][TM], sb[FKG][TN];
-        i32x8 wide_a[TM], wide_b[TN];                                        // TENSOR: both K groups of a sub-tile row, one operand
+        i32x8 wide_a[TM], wide_b[TN];                                        // TENSOR / MX: 16 k of either K group of a sub-tile row
+        int mx_a[TM], mx_b[TN];                                              // MX: the row's scale byte of K group lhi
     };
     auto scale_block = [&](int64_t c) -> const float* {                      // a scales of chunk c: [kg][row]; b scales F_SBLOCK later
         return reinterpret_cast<const float*>(lds + F_SCALE + ((c / F_SCHUNKS) & 1) * 2 * F_SBLOCK) + (c % F_SCHUNKS) * FKG * BM;
@@ -292,18 +313,28 @@ __global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(Gemm
         const uint8_t* tile_b = tile_a + F_TILE;
         const float* scale_a = scale_block(c);
         const float* scale_b = scale_a + F_SBLOCK / 4;
-        if constexpr (TENSOR) {
+        if constexpr (NOFOLD) {
+            // the lane's 16 bytes of either K group (slots lhi and lhi + 2)
+            const int first_a = rd_a, first_b = rd_b;
+            constexpr int SECOND = 32;
 #pragma unroll
             for (int j = 0; j < TM; ++j) {
-                const i32x4 lo = *reinterpret_cast<const i32x4*>(tile_a + (rd_a + j * 32 * FBK));
-                const i32x4 hi = *reinterpret_cast<const i32x4*>(tile_a + ((rd_a + j * 32 * FBK) ^ 32));
+                const i32x4 lo = *reinterpret_cast<const i32x4*>(tile_a + (first_a + j * 32 * FBK));
+                const i32x4 hi = *reinterpret_cast<const i32x4*>(tile_a + ((first_a + j * 32 * FBK) ^ SECOND));
                 o.wide_a[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
             }
 #pragma unroll
             for (int i = 0; i < TN; ++i) {
-                const i32x4 lo = *reinterpret_cast<const i32x4*>(tile_b + (rd_b + (b_sub(i) - b_sub(0)) * FBK));
-                const i32x4 hi = *reinterpret_cast<const i32x4*>(tile_b + ((rd_b + (b_sub(i) - b_sub(0)) * FBK) ^ 32));
+                const i32x4 lo = *reinterpret_cast<const i32x4*>(tile_b + (first_b + (b_sub(i) - b_sub(0)) * FBK));
+                const i32x4 hi = *reinterpret_cast<const i32x4*>(tile_b + ((first_b + (b_sub(i) - b_sub(0)) * FBK) ^ SECOND));
                 o.wide_b[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+            if constexpr (MX) {
+                const uint8_t* block = lds + F_RAW + ((c / MX_CHUNKS) & 1) * MX_BLOCK + (c % MX_CHUNKS) * FKG + lhi;
+#pragma unroll
+                for (int j = 0; j < TM; ++j) o.mx_a[j] = block[(a_sub(j) + l32) * MX_GROUPS];
+#pragma unroll
+                for (int i = 0; i < TN; ++i) o.mx_b[i] = block[BM * MX_GROUPS + (b_sub(i) + l32) * MX_GROUPS];
             }
             return;
         }
@@ -314,16 +345,16 @@ __global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(Gemm
 #pragma unroll
             for (int i = 0; i < TN; ++i) o.b[kg][i] = *reinterpret_cast<const uint4*>(tile_b + ((rd_b + (b_sub(i) - b_sub(0)) * FBK) ^ (kg * 32)));
 #pragma unroll
-            for (int j = 0; j < TM; ++j) o.sa[kg][j] = TENSOR ? 0.0f : scale_a[kg * BM + a_sub(j) + l32];
+            for (int j = 0; j < TM; ++j) o.sa[kg][j] = scale_a[kg * BM + a_sub(j) + l32];
 #pragma unroll
-            for (int i = 0; i < TN; ++i) o.sb[kg][i] = B_ROWSCALE || TENSOR ? 0.0f : scale_b[kg * BM + b_sub(i)];
+            for (int i = 0; i < TN; ++i) o.sb[kg][i] = B_ROWSCALE ? 0.0f : scale_b[kg * BM + b_sub(i)];
         }
     };
 
     // Math of chunk c on the operands in `o`; `between(step)` runs after MFMA number `step` of the chunk (the
     // caller's global loads and LDS reads for later chunks go there, spread over the chunk).
     auto compute = [&](const Operands& o, int64_t c, auto&& between) {
-        if constexpr (TENSOR) {
+        if constexpr (NOFOLD) {
             constexpr int STEPS_PER = FKG * 2;
 #pragma unroll
             for (int i = 0; i < TN; ++i) {
@@ -331,7 +362,10 @@ __global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(Gemm
                 for (int j = 0; j < TM; ++j) {
                     // both operands give a lane the same 32 of the chunk's 64 k (16 of each K group), so every product
                     // meets its partner whatever order the instruction walks them in
-                    total[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(o.wide_b[i], o.wide_a[j], total[i][j], B_BF8 ? 1 : 0, A_BF8 ? 1 : 0, 0, 0, 0, 0);
+                    if constexpr (MX)
+                        total[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(o.wide_b[i], o.wide_a[j], total[i][j], B_BF8 ? 1 : 0, A_BF8 ? 1 : 0, 0, o.mx_b[i], 0, o.mx_a[j]);
+                    else
+                        total[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(o.wide_b[i], o.wide_a[j], total[i][j], B_BF8 ? 1 : 0, A_BF8 ? 1 : 0, 0, 0, 0, 0);
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int step = 0; step < STEPS_PER; ++step) between((i * TM + j) * STEPS_PER + step);
@@ -417,12 +451,16 @@ __global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(Gemm
     constexpr int STEPS = FKG * TN * TM * 2, STRIDE = STEPS / CHUNK_LOADS;
     int stage_now = 0, stage_next = 1;
     auto chunk_step = [&](int64_t c, const Operands& now, Operands& next) {
-        if (!TENSOR && c % F_SCHUNKS == 1) __builtin_amdgcn_s_waitcnt(0x0070 | (CHUNK_LOADS + 2));
+        if (!NOFOLD && c % F_SCHUNKS == 1) __builtin_amdgcn_s_waitcnt(0x0070 | (CHUNK_LOADS + 2));
+        else if (MX && c % MX_CHUNKS == 1) __builtin_amdgcn_s_waitcnt(0x0070 | (CHUNK_LOADS + 1));
         else __builtin_amdgcn_s_waitcnt(0x0070 | CHUNK_LOADS);
         __syncthreads();
-        if constexpr (!TENSOR) {
+        if constexpr (!NOFOLD) {
             if (c % F_SCHUNKS == 0) issue_scales(c / F_SCHUNKS + 1);
             if (c % F_SCHUNKS == 2) arrange_scales(c / F_SCHUNKS + 1);
+        }
+        if constexpr (MX) {
+            if (c % MX_CHUNKS == 0) issue_mx_scales(c / MX_CHUNKS + 1);
         }
         if (c + 1 < chunks) read_operands(stage_next, c + 1, next);
         const int fill = stage_now;
@@ -432,13 +470,14 @@ __global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(Gemm
         stage_now = stage_next;
         stage_next = stage_next == FSTAGES - 1 ? 0 : stage_next + 1;
     };
-    if constexpr (!TENSOR) issue_scales(0);
+    if constexpr (MX) issue_mx_scales(0);
+    else if constexpr (!TENSOR) issue_scales(0);
     issue(0, 0);
     issue(1, 1);
     issue(2, 2);
     __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * CHUNK_LOADS));                   // scale block 0 and chunk 0 are in LDS
     __syncthreads();
-    if constexpr (!TENSOR) {
+    if constexpr (!NOFOLD) {
         arrange_scales(0);
         __syncthreads();
     }
@@ -457,7 +496,7 @@ __global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(Gemm
             for (int j = 0; j < TM; ++j)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) { const float t = total[i][j][r] * sa; total[i][j][r] = t * sb; }
-    } else if constexpr (CARRY) {
+    } else if constexpr (CARRY && !MX) {
         constexpr int UNITS = FKG * TN * TM, last_pair = UNITS / 2 - 1;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
@@ -675,6 +714,39 @@ int launch_tensor_gemm_fast(const GemmArgs& args, int a_dtype, int b_dtype, int 
         default: return VIOLA_EINVAL;
     }
 #undef VIOLA_TENSOR
+    return viola_launch_status();
+}
+
+// E8M0 block scales (args.sa / args.sb point at bytes; ldsa / ldsb = bytes per scale row). grid: (n tiles of 128, m tiles of 128).
+template <typename TO, int TN>
+static void launch_mx_formats(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, dim3 grid, hipStream_t stream) {
+    const bool a5 = a_dtype == VIOLA_E5M2, b5 = b_dtype == VIOLA_E5M2;
+    if (!a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE_PLAIN, false, false, false, TO, TN, false, true>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    else if (a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE_PLAIN, true, false, false, TO, TN, false, true>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    else if (!a5 && b5) hipLaunchKernelGGL((group_gemm_fast<MODE_PLAIN, false, true, false, TO, TN, false, true>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    else hipLaunchKernelGGL((group_gemm_fast<MODE_PLAIN, true, true, false, TO, TN, false, true>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+}
+
+int launch_mx_gemm_fast(const GemmArgs& args, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, dim3 grid,
+                        hipStream_t stream) {
+    GemmArgs p = args;
+    const bool narrow = (int64_t)grid.x * grid.y < 512 && p.n > 64;
+    if (narrow) grid.x = (unsigned)((p.n + 63) / 64);
+    if ((int64_t)grid.x * grid.y < (1 << 30)) {
+        p.tiles_n = (int)grid.x;
+        p.tiles_m = (int)grid.y;
+        grid = dim3((grid.x * grid.y + 7) / 8 * 8, 1, 1);
+    }
+#define VIOLA_MX(TO)                                                                          \
+    if (narrow) launch_mx_formats<TO, 1>(p, a_dtype, b_dtype, bias_dtype, grid, stream);      \
+    else launch_mx_formats<TO, 2>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
+    switch (out_dtype) {
+        case VIOLA_F32: VIOLA_MX(float) break;
+        case VIOLA_BF16: VIOLA_MX(bf16_t) break;
+        case VIOLA_F16: VIOLA_MX(f16_t) break;
+        default: return VIOLA_EINVAL;
+    }
+#undef VIOLA_MX
     return viola_launch_status();
 }
 
