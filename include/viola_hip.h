@@ -28,6 +28,8 @@ typedef void* viola_stream_t; /* hipStream_t */
 enum { VIOLA_F32 = 0, VIOLA_BF16 = 1, VIOLA_F16 = 2, VIOLA_E4M3 = 3, VIOLA_E5M2 = 4 };
 enum { VIOLA_SILU = 0, VIOLA_GELU = 1, VIOLA_RELU = 2 };
 enum { VIOLA_NEAREST = 0, VIOLA_STOCHASTIC = 1 };
+/* group scales: FP32 values, or E8M0 bytes (power-of-two scale 2^(byte - 127), the `native` / mxfp8 recipe) */
+enum { VIOLA_SCALE_F32 = 0, VIOLA_SCALE_E8M0 = 1 };
 enum { VIOLA_EINVAL = -1, VIOLA_EUNSUPPORTED = -2 };
 
 int viola_abi_version(void);
@@ -41,18 +43,21 @@ const char* viola_error_string(int code);
  * the output q is [rows, cols] and scale is [ceil(rows/gr), ceil(cols/gc)]; with
  * transposed = 1 the output is the quantized transpose, q [cols, rows] and scale
  * [ceil(cols/gr), ceil(rows/gc)], groups laid along the new last dimension.
- * Per group: s = max(amax, 1e-30) / limit; q = fp8(isnan(v/s) ? NaN : clamp(v/s, +-limit)). */
+ * Per group: s = max(amax, 1e-30) / limit; q = fp8(isnan(v/s) ? NaN : clamp(v/s, +-limit)).
+ * scale_format VIOLA_SCALE_E8M0 (native = True, :81-85): s is rounded up to a power of two, scale and source_scale
+ * are bytes log2(s) + 127. */
 int viola_group_quantize(const void* x, int x_dtype, int64_t rows, int64_t cols,
-                         void* q, int q_dtype, float* scale, int gr, int gc, float limit, int transposed,
-                         const float* source_scale, int source_gr, int source_gc, viola_stream_t stream);
+                         void* q, int q_dtype, void* scale, int gr, int gc, float limit, int transposed,
+                         const void* source_scale, int source_gr, int source_gc, int scale_format,
+                         viola_stream_t stream);
 
 /* One read pass that emits both layouts of a row-major matrix with 1-D groups: the row-wise
  * codes/scales (q [rows, cols], scale [rows, ceil(cols/gc)]) and the quantized transpose
  * (qt [cols, rows], scale_t [cols, ceil(rows/gc)]). Same arithmetic per group as two calls of
  * viola_group_quantize (viola/nn/_grouped_linear.py:21,46-47 and :73,92 make those two calls). */
 int viola_group_quantize_dual(const void* x, int x_dtype, int64_t rows, int64_t cols,
-                              void* q, float* scale, void* qt, float* scale_t, int q_dtype, int gc,
-                              float limit, float* column_partial, viola_stream_t stream);
+                              void* q, void* scale, void* qt, void* scale_t, int q_dtype, int gc,
+                              float limit, float* column_partial, int scale_format, viola_stream_t stream);
 
 /* column_partial (nullable) of viola_group_quantize_dual receives [ceil(rows/32), cols] fp32 sums of x over
  * each 32-row group, taken from the same read; viola_column_reduce adds the parts in a fixed order:

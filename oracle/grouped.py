@@ -15,13 +15,29 @@ def scale_shape(shape, group):
     return tuple((n + g - 1) // g for n, g in zip(shape, group))
 
 
+def decode_scale(scale):
+    """E8M0 bytes (uint8, the `native` recipe) -> 2^(byte - 127) (viola/nn/_grouped_kernels.py:35,72); FP32 passes."""
+    return torch.exp2(scale.float() - 127.) if scale.dtype == torch.uint8 else scale.float()
+
+
+def pow2_ceil(scales):
+    """The smallest power of two that is not below each (positive, finite) scale: the mathematical value of the
+    reference's exp2(ceil(log2(s))) (viola/nn/_grouped_kernels.py:81-83 on the GPU, :143-146 on the CPU), found from
+    the binary exponent instead of a rounded fp32 logarithm. PARITY UNPINNED where the reference's own log2 rounds:
+    for s within a few ulp above a power of two with |log2 s| >= 4 its fp32 log2 comes out an integer and the
+    reference keeps the smaller power; nothing in the reference pins that case (its CPU and CUDA log2 differ too)."""
+    mantissa, exponent = torch.frexp(scales.float())                       # s = mantissa * 2^exponent, mantissa in [0.5, 1)
+    exponent = torch.where(mantissa == 0.5, exponent - 1, exponent)
+    return torch.ldexp(torch.ones_like(scales, dtype=torch.float32), exponent), (exponent + 127).to(torch.uint8)
+
+
 def dequantize(q, scale, group):
     """float(q) * scale[r // gr, c // gc]  (viola/nn/_grouped_kernels.py:37-40,49-50)."""
-    expanded = scale.float().repeat_interleave(group[0], 0).repeat_interleave(group[1], 1)
+    expanded = decode_scale(scale).repeat_interleave(group[0], 0).repeat_interleave(group[1], 1)
     return q.float() * expanded[:q.shape[0], :q.shape[1]]
 
 
-def quantize(x, dtype, group, *, limit=None, transposed=False, source_scale=None, source_group=(1, 32)):
+def quantize(x, dtype, group, *, limit=None, transposed=False, source_scale=None, source_group=(1, 32), native=False):
     """Group amax quantization (viola/nn/_grouped_kernels.py:127-158).
 
     Follows the CPU branch at :135-151 (pad -> reshape (nr, gr, nc, gc) -> amax ->
@@ -39,9 +55,12 @@ def quantize(x, dtype, group, *, limit=None, transposed=False, source_scale=None
     blocks = F.pad(value, (0, nc * gc - shape[1], 0, nr * gr - shape[0])).reshape(nr, gr, nc, gc)
     magnitude = torch.where(blocks.isnan(), torch.zeros_like(blocks), blocks.abs())
     scales = magnitude.amax((1, 3)).clamp_min(1e-30) / limit
+    stored = scales
+    if native:                                                             # E8M0: power-of-two scale, stored as its exponent byte
+        scales, stored = pow2_ceil(scales)
     codes = (blocks / scales[:, None, :, None]).clamp(-limit, limit)      # clamp keeps NaN
     q = codes.reshape(nr * gr, nc * gc)[:shape[0], :shape[1]].to(dtype)
-    return q.contiguous(), scales.contiguous()
+    return q.contiguous(), stored.contiguous()
 
 
 def transpose_group(group):
@@ -49,11 +68,11 @@ def transpose_group(group):
     return group[::-1] if group[0] >= 32 else group
 
 
-def transpose(q, scale, group, *, limit=None):
+def transpose(q, scale, group, *, limit=None, native=False):
     """Byte transpose + scale.T for 2-D blocks, otherwise re-encode (:166-171)."""
     if group[0] >= 32:
         return q.T.contiguous(), scale.T.contiguous()
-    return quantize(q, q.dtype, group, limit=limit, transposed=True, source_scale=scale, source_group=group)
+    return quantize(q, q.dtype, group, limit=limit, transposed=True, source_scale=scale, source_group=group, native=native)
 
 
 def gemm(a, b, sa, sb, group_a, group_b, *, out_dtype=torch.float32, bias=None, witness=False):

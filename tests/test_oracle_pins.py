@@ -384,3 +384,35 @@ def test_tensor_gemm_oracle_against_brute_force():
         for n in range(7):
             acc = sum(float(a[m, k].float()) * float(b[n, k].float()) for k in range(48))
             assert abs(out[m, n].item() - (acc * .37 * 1.9 + bias[n].item())) < 1e-4 * (1 + abs(acc))
+
+
+# ----------------------------------------------------------------------------- MXFP8 (E8M0 scales)
+@pytest.mark.parametrize("dtype", [E4, E5])
+@pytest.mark.parametrize("group,shape", [((1, 32), (9, 96)), ((32, 32), (70, 45)), ((1, 32), (33, 64))])
+def test_native_quantize_matches_the_reference_cpu_branch(dtype, group, shape):
+    """viola/nn/_grouped_kernels.py:135-151 with native=True, written out with its own log2 / ceil / exp2: bytes and
+    codes equal the oracle's (random data does not sit within an ulp of a power of two, where the two could differ)."""
+    torch.manual_seed(70)
+    x = torch.randn(shape) * torch.logspace(-6, 4, shape[1])
+    limit = torch.finfo(dtype).max
+    gr, gc = group
+    nr, nc = grouped.scale_shape(shape, group)
+    blocks = F.pad(x, (0, nc * gc - shape[1], 0, nr * gr - shape[0])).reshape(nr, gr, nc, gc)
+    scales = blocks.abs().amax((1, 3)).clamp_min(1e-30) / limit
+    exponent = scales.log2().ceil()
+    expected_bytes = (exponent + 127).to(torch.uint8)
+    expected = (blocks / exponent.exp2()[:, None, :, None]).clamp(-limit, limit).reshape(nr * gr, nc * gc)[:shape[0], :shape[1]].to(dtype)
+    q, s = grouped.quantize(x, dtype, group, native=True)
+    assert s.dtype == torch.uint8 and torch.equal(s, expected_bytes)
+    assert torch.equal(q.view(torch.uint8), expected.view(torch.uint8))
+    assert torch.equal(grouped.decode_scale(s), exponent.exp2())
+    # the scale is the smallest power of two >= amax / limit: nothing clamps, and half of it would
+    assert (q.float().abs() <= limit).all() and (grouped.decode_scale(s) >= scales).all() and (grouped.decode_scale(s) < 2 * scales).all()
+    # an amax that is exactly limit * 2^k keeps the scale 2^k
+    y = torch.zeros(32, 32)
+    y[3, 5] = limit * 2. ** -9
+    assert grouped.quantize(y, dtype, (32, 32), native=True)[1].item() == 127 - 9
+    y[3, 5] = torch.nextafter(torch.tensor(limit * 2. ** -9), torch.tensor(float("inf")))
+    assert grouped.quantize(y, dtype, (32, 32), native=True)[1].item() == 127 - 8
+    # dequantize and the re-encoding transpose read the bytes
+    assert torch.equal(grouped.dequantize(q, s, group), q.float() * grouped.decode_scale(s).repeat_interleave(gr, 0).repeat_interleave(gc, 1)[:shape[0], :shape[1]])

@@ -19,8 +19,8 @@ LIBRARY = Path(__file__).resolve().parent / "csrc" / "libviola_hip.so"
 
 _i, _l, _f, _p = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 _SIGNATURES = {
-    "viola_group_quantize": [_p, _i, _l, _l, _p, _i, _p, _i, _i, _f, _i, _p, _i, _i, _p],
-    "viola_group_quantize_dual": [_p, _i, _l, _l, _p, _p, _p, _p, _i, _i, _f, _p, _p],
+    "viola_group_quantize": [_p, _i, _l, _l, _p, _i, _p, _i, _i, _f, _i, _p, _i, _i, _i, _p],
+    "viola_group_quantize_dual": [_p, _i, _l, _l, _p, _p, _p, _p, _i, _i, _f, _p, _i, _p],
     "viola_column_reduce": [_p, _l, _l, _p, _i, _p],
     "viola_group_dequantize": [_p, _i, _p, _l, _l, _i, _i, _p, _p],
     "viola_fp8_transpose": [_p, _p, _l, _l, _l, _p],
@@ -91,8 +91,9 @@ def stream():
 timeline = None   # when a list, every call appends (name, start_event, end_event) recorded on the current stream
 
 
-def call(name, *args):
-    """Invoke one entry point on the current stream; non-zero status raises."""
+def call(name, *args, unsupported_ok=False):
+    """Invoke one entry point on the current stream; non-zero status raises (VIOLA_EUNSUPPORTED is returned instead
+    when the caller has another route)."""
     lib = library()
     if timeline is not None:
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -102,8 +103,11 @@ def call(name, *args):
         timeline.append((name, start, end))
     else:
         status = getattr(lib, name)(*args, stream())
+    if status == -2 and unsupported_ok:
+        return status
     if status:
         raise RuntimeError(f"{name} failed: {lib.viola_error_string(status).decode()} (status {status})")
+    return status
 
 
 def code(dtype):

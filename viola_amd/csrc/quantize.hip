@@ -20,7 +20,23 @@ __device__ __forceinline__ uint8_t encode_clamped(float v, float s, float limit)
     return from_f32<TOut>(c).bits;
 }
 
-__device__ __forceinline__ float group_scale(float amax, float limit) { return scale_of(amax, limit); }
+// amax / limit, or for E8M0 scales the smallest power of two that is not below it (the reference's
+// exp2(ceil(log2(s))), viola/nn/_grouped_kernels.py:81-83, evaluated exactly on the bits)
+__device__ __forceinline__ float group_scale(float amax, float limit, int e8m0 = 0) {
+    const float s = scale_of(amax, limit);
+    if (!e8m0) return s;
+    const uint32_t bits = __float_as_uint(s);
+    if ((bits & 0x7f800000u) == 0x7f800000u) return s;                          // Inf / NaN stay
+    return __uint_as_float((bits & 0x7f800000u) + ((bits & 0x007fffffu) ? 0x00800000u : 0u));
+}
+// a scale goes out as FP32 or as its biased exponent byte (log2(s) + 127, _grouped_kernels.py:85)
+__device__ __forceinline__ void put_scale(float* scale, int64_t index, float s, int e8m0) {
+    if (e8m0) reinterpret_cast<uint8_t*>(scale)[index] = (uint8_t)(__float_as_uint(s) >> 23);
+    else scale[index] = s;
+}
+__device__ __forceinline__ float get_scale(const float* scale, int64_t index, int e8m0) {
+    return e8m0 ? __uint_as_float((uint32_t)reinterpret_cast<const uint8_t*>(scale)[index] << 23) : scale[index];
+}
 
 // ------------------------------------------------------------------ 8-element chunk loads
 template <typename TIn> struct Chunk8;
@@ -69,7 +85,7 @@ __device__ __forceinline__ uint2 encode8(const float (&v)[8], float s, float lim
 template <typename TIn, typename TOut, int GC>
 __global__ __launch_bounds__(256) void quantize_rowwise(const TIn* __restrict__ x, uint8_t* __restrict__ q,
                                                          float* __restrict__ scale, int64_t rows, int64_t cols,
-                                                         int64_t nc, float limit) {
+                                                         int64_t nc, float limit, int e8m0) {
     constexpr int LANES = GC / 8;                         // lanes that share one group
     const int64_t chunks_per_row = nc * LANES;
     const int64_t chunk = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -87,11 +103,11 @@ __global__ __launch_bounds__(256) void quantize_rowwise(const TIn* __restrict__ 
     amax = group_max<LANES>(amax);
 #pragma unroll
     for (int offset = LANES / 2; offset > 0; offset >>= 1) poison += __shfl_xor(poison, offset, WAVE);
-    const float s = group_scale(amax, limit);
+    const float s = group_scale(amax, limit, e8m0);
     const SharedDivisor divisor(s, poison);
     if (valid) {
         *reinterpret_cast<uint2*>(q + row * cols + c0) = encode8<TOut>(v, s, limit, divisor);
-        if ((threadIdx.x & (LANES - 1)) == 0) scale[row * nc + c0 / GC] = s;
+        if ((threadIdx.x & (LANES - 1)) == 0) put_scale(scale, row * nc + c0 / GC, s, e8m0);
     }
 }
 
@@ -153,7 +169,7 @@ template <typename TIn, typename TOut, bool ROWWISE, bool TRANSPOSED, bool VEC>
 __global__ __launch_bounds__(256) void quantize_tile(const TIn* __restrict__ x, uint8_t* __restrict__ q,
                                                       float* __restrict__ scale, uint8_t* __restrict__ qt,
                                                       float* __restrict__ scale_t, int64_t rows, int64_t cols,
-                                                      float limit, float* __restrict__ column_partial) {
+                                                      float limit, float* __restrict__ column_partial, int e8m0) {
     __shared__ float tile[TILE_R * TILE_LD];
     const int64_t r0 = (int64_t)blockIdx.y * TILE_R, c0 = (int64_t)blockIdx.x * TILE_C;
     load_tile<TIn, VEC>(x, tile, r0, c0, rows, cols);
@@ -171,9 +187,9 @@ __global__ __launch_bounds__(256) void quantize_tile(const TIn* __restrict__ x, 
                 amax = fmaxf(amax, fabsf(v[i]));
                 poison = poison_of(poison, v[i]);
             }
-            const float s = group_scale(amax, limit);
+            const float s = group_scale(amax, limit, e8m0);
             const int64_t nc = (cols + 31) / 32;
-            scale[row * nc + col / 32] = s;
+            put_scale(scale, row * nc + col / 32, s, e8m0);
             const int count = (int)(cols - col < 32 ? cols - col : 32);
             uint8_t* dst = q + row * cols + col;
             store_group32<TOut>(v, s, poison, limit, dst, count, (reinterpret_cast<uintptr_t>(dst) & 15) == 0);
@@ -191,9 +207,9 @@ __global__ __launch_bounds__(256) void quantize_tile(const TIn* __restrict__ x, 
                 amax = fmaxf(amax, fabsf(v[i]));
                 poison = poison_of(poison, v[i]);
             }
-            const float s = group_scale(amax, limit);
+            const float s = group_scale(amax, limit, e8m0);
             const int64_t nr = (rows + 31) / 32;
-            scale_t[col * nr + row / 32] = s;
+            put_scale(scale_t, col * nr + row / 32, s, e8m0);
             if (column_partial) {
                 float sum = 0.0f;
 #pragma unroll
@@ -225,7 +241,7 @@ template <typename TIn, typename TOut, bool ROWWISE>
 __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x, uint8_t* __restrict__ q,
                                                         float* __restrict__ scale, uint8_t* __restrict__ qt,
                                                         float* __restrict__ scale_t, int64_t rows, int64_t cols,
-                                                        float limit, float* __restrict__ column_partial) {
+                                                        float limit, float* __restrict__ column_partial, int e8m0) {
     constexpr int LD = 64 + 32;
     typedef short s16x4 __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
@@ -270,7 +286,7 @@ __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x
             amax = group_max<4>(amax);
             poison += __shfl_xor(poison, 1, WAVE);
             poison += __shfl_xor(poison, 2, WAVE);
-            s_row[i] = group_scale(amax, limit);
+            s_row[i] = group_scale(amax, limit, e8m0);
             d_row[i] = SharedDivisor(s_row[i], poison);
             fast = fast && d_row[i].fast;
         }
@@ -291,7 +307,7 @@ __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x
             poison = poison_of(poison, vc[4 * t + e]);
         }
     }
-    const float s_col = group_scale(amax, limit);
+    const float s_col = group_scale(amax, limit, e8m0);
     const SharedDivisor d_col(s_col, poison);
     fast = fast && d_col.fast;
 
@@ -327,13 +343,13 @@ __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x
             const int64_t row = r0 + lr + 8 * i;
             if (row < rows && col8 < cols) {
                 *reinterpret_cast<uint2*>(q + row * cols + col8) = row_codes[i];
-                if (ch % 4 == 0) scale[row * nc + col8 / 32] = s_row[i];
+                if (ch % 4 == 0) put_scale(scale, row * nc + col8 / 32, s_row[i], e8m0);
             }
         }
     }
     if (col < cols) {
         const int64_t nr = (rows + 31) / 32;
-        scale_t[col * nr + r0 / 32] = s_col;
+        put_scale(scale_t, col * nr + r0 / 32, s_col, e8m0);
         if (column_partial) {
             float sum = 0.0f;
 #pragma unroll
@@ -408,7 +424,7 @@ template <> __device__ __forceinline__ void load4<f16_t>(const f16_t* p, float (
 // group in both half-waves, over the 16 loads. One read of x; cols must be a multiple of 4.
 template <typename TIn, typename TOut>
 __global__ __launch_bounds__(256) void quantize_block32(const TIn* __restrict__ x, uint8_t* __restrict__ q, float* __restrict__ scale,
-                                                         int64_t rows, int64_t cols, int64_t nc, float limit) {
+                                                         int64_t rows, int64_t cols, int64_t nc, float limit, int e8m0) {
     const int64_t strips = (cols + 127) / 128;
     const int64_t unit = (int64_t)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
     if (unit >= (rows + 31) / 32 * strips) return;                      // whole wavefront leaves together
@@ -432,8 +448,8 @@ __global__ __launch_bounds__(256) void quantize_block32(const TIn* __restrict__ 
     amax = group_max<8>(amax);
     amax = fmaxf(amax, __shfl_xor(amax, 32, WAVE));
     const bool any_bad = __builtin_amdgcn_ballot_w64(poison != poison) != 0;
-    const float s = group_scale(amax, limit);
-    if ((lane & 39) == 0 && col < cols) scale[(r0 / 32) * nc + col / 32] = s;
+    const float s = group_scale(amax, limit, e8m0);
+    if ((lane & 39) == 0 && col < cols) put_scale(scale, (r0 / 32) * nc + col / 32, s, e8m0);
     const SharedDivisor d(s, any_bad ? __uint_as_float(0x7fc00000u) : 0.0f);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
@@ -455,7 +471,7 @@ template <typename TIn, typename TOut, bool ENCODED>
 __global__ __launch_bounds__(256) void quantize_generic(const TIn* __restrict__ x, const float* __restrict__ source_scale,
                                                          uint8_t* __restrict__ q, float* __restrict__ scale,
                                                          int64_t rows, int64_t cols, int gr, int gc, int transposed,
-                                                         int source_gr, int source_gc, float limit) {
+                                                         int source_gr, int source_gc, float limit, int e8m0) {
     const int64_t out_rows = transposed ? cols : rows, out_cols = transposed ? rows : cols;
     const int64_t nr = (out_rows + gr - 1) / gr, nc = (out_cols + gc - 1) / gc;
     const int64_t group = (int64_t)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
@@ -470,7 +486,7 @@ __global__ __launch_bounds__(256) void quantize_generic(const TIn* __restrict__ 
         inside = r < out_rows && c < out_cols;
         if (!inside) return 0.0f;
         float v = to_f32(x[xr * cols + xc]);
-        if constexpr (ENCODED) v *= source_scale[xr / source_gr * sc + xc / source_gc];
+        if constexpr (ENCODED) v *= get_scale(source_scale, xr / source_gr * sc + xc / source_gc, e8m0);
         return v;
     };
     float amax = 0.0f;
@@ -479,8 +495,8 @@ __global__ __launch_bounds__(256) void quantize_generic(const TIn* __restrict__ 
         amax = fmaxf(amax, fabsf(value(j, inside)));
     }
     amax = wave_max(amax);
-    const float s = group_scale(amax, limit);
-    if (lane == 0) scale[group] = s;
+    const float s = group_scale(amax, limit, e8m0);
+    if (lane == 0) put_scale(scale, group, s, e8m0);
     for (int j = lane; j < size; j += WAVE) {
         bool inside;
         const float v = value(j, inside);
@@ -666,7 +682,7 @@ __global__ __launch_bounds__(256) void quantize_segmented16(const TIn* __restric
 // ------------------------------------------------------------------ host dispatch
 template <typename TIn, typename TOut>
 static int launch_quantize(const void* x, int64_t rows, int64_t cols, void* q, float* scale, int gr, int gc,
-                           float limit, int transposed, hipStream_t stream) {
+                           float limit, int transposed, int e8m0, hipStream_t stream) {
     const TIn* xp = static_cast<const TIn*>(x);
     uint8_t* qp = static_cast<uint8_t*>(q);
     const bool vec = cols % 8 == 0 && reinterpret_cast<uintptr_t>(x) % (8 * sizeof(TIn)) == 0;
@@ -675,7 +691,7 @@ static int launch_quantize(const void* x, int64_t rows, int64_t cols, void* q, f
         const int64_t chunks = rows * nc * (gc / 8);
         const dim3 grid((unsigned)((chunks + 255) / 256));
 #define VIOLA_ROWWISE(GC) \
-    case GC: hipLaunchKernelGGL((quantize_rowwise<TIn, TOut, GC>), grid, dim3(256), 0, stream, xp, qp, scale, rows, cols, nc, limit); break;
+    case GC: hipLaunchKernelGGL((quantize_rowwise<TIn, TOut, GC>), grid, dim3(256), 0, stream, xp, qp, scale, rows, cols, nc, limit, e8m0); break;
         switch (gc) {
             VIOLA_ROWWISE(32) VIOLA_ROWWISE(64) VIOLA_ROWWISE(128) VIOLA_ROWWISE(256) VIOLA_ROWWISE(512)
             default: return VIOLA_EINVAL;
@@ -687,55 +703,55 @@ static int launch_quantize(const void* x, int64_t rows, int64_t cols, void* q, f
         if (gr == 1 && gc == 32 && transposed && vec) {
             const int64_t tiles16 = ((cols + 63) / 64) * ((rows + 127) / 128);
             const dim3 grid16((unsigned)(tiles16 < 256 * 6 ? tiles16 : 256 * 6));
-            hipLaunchKernelGGL((quantize_dual16<TIn, TOut, false>), grid16, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit, nullptr);
+            hipLaunchKernelGGL((quantize_dual16<TIn, TOut, false>), grid16, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit, nullptr, e8m0);
             return viola_launch_status();
         }
     }
     if (gr == 1 && gc == 32 && transposed) {
         const dim3 grid((unsigned)((cols + TILE_C - 1) / TILE_C), (unsigned)((rows + TILE_R - 1) / TILE_R));
-        if (vec) hipLaunchKernelGGL((quantize_tile<TIn, TOut, false, true, true>), grid, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit, nullptr);
-        else hipLaunchKernelGGL((quantize_tile<TIn, TOut, false, true, false>), grid, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit, nullptr);
+        if (vec) hipLaunchKernelGGL((quantize_tile<TIn, TOut, false, true, true>), grid, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit, nullptr, e8m0);
+        else hipLaunchKernelGGL((quantize_tile<TIn, TOut, false, true, false>), grid, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit, nullptr, e8m0);
         return viola_launch_status();
     }
     if (gr == 32 && gc == 32 && !transposed && cols % 4 == 0 && reinterpret_cast<uintptr_t>(x) % (4 * sizeof(TIn)) == 0 &&
         reinterpret_cast<uintptr_t>(q) % 4 == 0) {
         const int64_t units = (rows + 31) / 32 * ((cols + 127) / 128);
         hipLaunchKernelGGL((quantize_block32<TIn, TOut>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, xp, qp, scale,
-                           rows, cols, (cols + 31) / 32, limit);
+                           rows, cols, (cols + 31) / 32, limit, e8m0);
         return viola_launch_status();
     }
     const int64_t out_rows = transposed ? cols : rows, out_cols = transposed ? rows : cols;
     const int64_t ngroups = ((out_rows + gr - 1) / gr) * ((out_cols + gc - 1) / gc);
     hipLaunchKernelGGL((quantize_generic<TIn, TOut, false>), dim3((unsigned)((ngroups + 3) / 4)), dim3(256), 0, stream,
-                       xp, nullptr, qp, scale, rows, cols, gr, gc, transposed, 1, 32, limit);
+                       xp, nullptr, qp, scale, rows, cols, gr, gc, transposed, 1, 32, limit, e8m0);
     return viola_launch_status();
 }
 
 template <typename TOut>
 static int dispatch_in(int x_dtype, const void* x, int64_t rows, int64_t cols, void* q, float* scale, int gr, int gc,
-                       float limit, int transposed, hipStream_t stream) {
+                       float limit, int transposed, int e8m0, hipStream_t stream) {
     switch (x_dtype) {
-        case VIOLA_F32: return launch_quantize<float, TOut>(x, rows, cols, q, scale, gr, gc, limit, transposed, stream);
-        case VIOLA_BF16: return launch_quantize<bf16_t, TOut>(x, rows, cols, q, scale, gr, gc, limit, transposed, stream);
-        case VIOLA_F16: return launch_quantize<f16_t, TOut>(x, rows, cols, q, scale, gr, gc, limit, transposed, stream);
+        case VIOLA_F32: return launch_quantize<float, TOut>(x, rows, cols, q, scale, gr, gc, limit, transposed, e8m0, stream);
+        case VIOLA_BF16: return launch_quantize<bf16_t, TOut>(x, rows, cols, q, scale, gr, gc, limit, transposed, e8m0, stream);
+        case VIOLA_F16: return launch_quantize<f16_t, TOut>(x, rows, cols, q, scale, gr, gc, limit, transposed, e8m0, stream);
         default: return VIOLA_EINVAL;
     }
 }
 
 template <typename TIn, typename TOut>
 static int launch_reencode(const void* x, const float* source_scale, int64_t rows, int64_t cols, void* q, float* scale,
-                           int gr, int gc, float limit, int transposed, int sgr, int sgc, hipStream_t stream) {
+                           int gr, int gc, float limit, int transposed, int sgr, int sgc, int e8m0, hipStream_t stream) {
     const int64_t out_rows = transposed ? cols : rows, out_cols = transposed ? rows : cols;
     const int64_t ngroups = ((out_rows + gr - 1) / gr) * ((out_cols + gc - 1) / gc);
     hipLaunchKernelGGL((quantize_generic<TIn, TOut, true>), dim3((unsigned)((ngroups + 3) / 4)), dim3(256), 0, stream,
                        static_cast<const TIn*>(x), source_scale, static_cast<uint8_t*>(q), scale, rows, cols, gr, gc,
-                       transposed, sgr, sgc, limit);
+                       transposed, sgr, sgc, limit, e8m0);
     return viola_launch_status();
 }
 
 template <typename TIn, typename TOut>
 static int launch_dual(const void* x, int64_t rows, int64_t cols, void* q, float* scale, void* qt, float* scale_t,
-                       float limit, float* column_partial, hipStream_t stream) {
+                       float limit, float* column_partial, int e8m0, hipStream_t stream) {
     const bool vec = cols % 8 == 0 && reinterpret_cast<uintptr_t>(x) % (8 * sizeof(TIn)) == 0;
     const dim3 grid((unsigned)((cols + TILE_C - 1) / TILE_C), (unsigned)((rows + TILE_R - 1) / TILE_R));
     const TIn* xp = static_cast<const TIn*>(x);
@@ -744,12 +760,12 @@ static int launch_dual(const void* x, int64_t rows, int64_t cols, void* q, float
             const int64_t tiles16 = ((cols + 63) / 64) * ((rows + 127) / 128);
             const dim3 grid16((unsigned)(tiles16 < 256 * 6 ? tiles16 : 256 * 6));
             hipLaunchKernelGGL((quantize_dual16<TIn, TOut, true>), grid16, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale,
-                               static_cast<uint8_t*>(qt), scale_t, rows, cols, limit, column_partial);
+                               static_cast<uint8_t*>(qt), scale_t, rows, cols, limit, column_partial, e8m0);
             return viola_launch_status();
         }
     }
-    if (vec) hipLaunchKernelGGL((quantize_tile<TIn, TOut, true, true, true>), grid, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale, static_cast<uint8_t*>(qt), scale_t, rows, cols, limit, column_partial);
-    else hipLaunchKernelGGL((quantize_tile<TIn, TOut, true, true, false>), grid, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale, static_cast<uint8_t*>(qt), scale_t, rows, cols, limit, column_partial);
+    if (vec) hipLaunchKernelGGL((quantize_tile<TIn, TOut, true, true, true>), grid, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale, static_cast<uint8_t*>(qt), scale_t, rows, cols, limit, column_partial, e8m0);
+    else hipLaunchKernelGGL((quantize_tile<TIn, TOut, true, true, false>), grid, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale, static_cast<uint8_t*>(qt), scale_t, rows, cols, limit, column_partial, e8m0);
     return viola_launch_status();
 }
 
@@ -780,15 +796,20 @@ static bool pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
 using namespace viola;
 
 extern "C" int viola_group_quantize(const void* x, int x_dtype, int64_t rows, int64_t cols, void* q, int q_dtype,
-                                    float* scale, int gr, int gc, float limit, int transposed,
-                                    const float* source_scale, int source_gr, int source_gc, viola_stream_t stream_) {
+                                    void* scale_, int gr, int gc, float limit, int transposed,
+                                    const void* source_scale_, int source_gr, int source_gc, int scale_format,
+                                    viola_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
+    float* scale = static_cast<float*>(scale_);
+    const float* source_scale = static_cast<const float*>(source_scale_);
+    VIOLA_CHECK_ARG(scale_format == VIOLA_SCALE_F32 || scale_format == VIOLA_SCALE_E8M0);
+    const int e8m0 = scale_format == VIOLA_SCALE_E8M0;
     VIOLA_CHECK_ARG(viola_is_fp8(q_dtype) && rows >= 0 && cols >= 0 && pow2(gr) && pow2(gc) && limit > 0.0f);
     if (rows == 0 || cols == 0) return 0;
     VIOLA_CHECK_ARG(x && q && scale);
     if (source_scale) {
         VIOLA_CHECK_ARG(viola_is_fp8(x_dtype) && source_gr > 0 && source_gc > 0);
-#define VIOLA_RE(TI, TO) return launch_reencode<TI, TO>(x, source_scale, rows, cols, q, scale, gr, gc, limit, transposed, source_gr, source_gc, stream)
+#define VIOLA_RE(TI, TO) return launch_reencode<TI, TO>(x, source_scale, rows, cols, q, scale, gr, gc, limit, transposed, source_gr, source_gc, e8m0, stream)
         if (x_dtype == VIOLA_E4M3 && q_dtype == VIOLA_E4M3) VIOLA_RE(e4m3_t, e4m3_t);
         if (x_dtype == VIOLA_E4M3 && q_dtype == VIOLA_E5M2) VIOLA_RE(e4m3_t, e5m2_t);
         if (x_dtype == VIOLA_E5M2 && q_dtype == VIOLA_E4M3) VIOLA_RE(e5m2_t, e4m3_t);
@@ -796,19 +817,23 @@ extern "C" int viola_group_quantize(const void* x, int x_dtype, int64_t rows, in
 #undef VIOLA_RE
     }
     VIOLA_CHECK_ARG(viola_is_float(x_dtype));
-    if (q_dtype == VIOLA_E4M3) return dispatch_in<e4m3_t>(x_dtype, x, rows, cols, q, scale, gr, gc, limit, transposed, stream);
-    return dispatch_in<e5m2_t>(x_dtype, x, rows, cols, q, scale, gr, gc, limit, transposed, stream);
+    if (q_dtype == VIOLA_E4M3) return dispatch_in<e4m3_t>(x_dtype, x, rows, cols, q, scale, gr, gc, limit, transposed, e8m0, stream);
+    return dispatch_in<e5m2_t>(x_dtype, x, rows, cols, q, scale, gr, gc, limit, transposed, e8m0, stream);
 }
 
-extern "C" int viola_group_quantize_dual(const void* x, int x_dtype, int64_t rows, int64_t cols, void* q, float* scale,
-                                         void* qt, float* scale_t, int q_dtype, int gc, float limit,
-                                         float* column_partial, viola_stream_t stream_) {
+extern "C" int viola_group_quantize_dual(const void* x, int x_dtype, int64_t rows, int64_t cols, void* q, void* scale_,
+                                         void* qt, void* scale_t_, int q_dtype, int gc, float limit,
+                                         float* column_partial, int scale_format, viola_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
+    float* scale = static_cast<float*>(scale_);
+    float* scale_t = static_cast<float*>(scale_t_);
+    VIOLA_CHECK_ARG(scale_format == VIOLA_SCALE_F32 || scale_format == VIOLA_SCALE_E8M0);
+    const int e8m0 = scale_format == VIOLA_SCALE_E8M0;
     VIOLA_CHECK_ARG(viola_is_fp8(q_dtype) && viola_is_float(x_dtype) && rows >= 0 && cols >= 0 && limit > 0.0f);
     if (gc != 32) return VIOLA_EUNSUPPORTED;
     if (rows == 0 || cols == 0) return 0;
     VIOLA_CHECK_ARG(x && q && scale && qt && scale_t);
-#define VIOLA_DUAL(TI, TO) return launch_dual<TI, TO>(x, rows, cols, q, scale, qt, scale_t, limit, column_partial, stream)
+#define VIOLA_DUAL(TI, TO) return launch_dual<TI, TO>(x, rows, cols, q, scale, qt, scale_t, limit, column_partial, e8m0, stream)
     if (q_dtype == VIOLA_E4M3) {
         if (x_dtype == VIOLA_F32) VIOLA_DUAL(float, e4m3_t);
         if (x_dtype == VIOLA_BF16) VIOLA_DUAL(bf16_t, e4m3_t);

@@ -2,7 +2,8 @@
 viola/nn/_grouped_kernels.py: scale_shape :16, dequantize :44, quantize :127,
 transpose_group :161, transpose :166, gemm :310), each one call into libviola_hip.
 
-FP32 scales only; the reference's `native=True` (E8M0 / MXFP8) variant is not built.
+`native=True` is the MXFP8 recipe: scales are E8M0 bytes (uint8, value 2^(byte - 127)) of 32-wide K groups, and the
+GEMM scales inside the block-scaled MFMA.
 """
 
 import torch
@@ -15,15 +16,20 @@ def scale_shape(shape, group):
     return tuple(-(-n // g) for n, g in zip(shape, group))
 
 
-def _no_native(native):
-    if native:
-        raise NotImplementedError("MXFP8 (E8M0 scales) is not built in viola_amd; use FP32 group scales")
+def _scale_dtype(native):
+    return torch.uint8 if native else torch.float32
+
+
+def decode_scale(scale):
+    """E8M0 bytes -> the FP32 scales they stand for (exact); FP32 scales pass through."""
+    return torch.exp2(scale.float() - 127.) if scale.dtype == torch.uint8 else scale
 
 
 def dequantize(q, scale, group):
     """fp32 [rows, cols] = float(q) * scale[r // gr, c // gc]."""
     assert q.is_cuda, "viola_amd kernels run on the GPU only"
     q = q.contiguous()
+    scale = decode_scale(scale)
     out = torch.empty(q.shape, device=q.device, dtype=torch.float32)
     _lib.call("viola_group_dequantize", _lib.ptr(q), _lib.code(q.dtype), _lib.ptr(scale.contiguous()),
               q.shape[0], q.shape[1], group[0], group[1], _lib.ptr(out))
@@ -32,28 +38,28 @@ def dequantize(q, scale, group):
 
 def quantize(x, dtype, group, *, native=False, limit=None, transposed=False,
              source_scale=None, source_group=(1, 32), out=None, scale_out=None):
-    """Group amax quantization of a 2-D tensor; returns (codes, fp32 scales).
+    """Group amax quantization of a 2-D tensor; returns (codes, fp32 scales), or (codes, E8M0 bytes) with native=True.
 
     transposed=True yields the quantized transpose (codes [cols, rows]) with the groups laid
     along the new last dimension, read straight from the floating input. source_scale re-encodes
     existing codes. out/scale_out let the caller own the outputs (nothing is allocated then).
     """
-    _no_native(native)
     assert x.is_cuda and x.dim() == 2, "viola_amd kernels run on the GPU only"
     x = x.contiguous()
     shape = tuple(x.shape[::-1]) if transposed else tuple(x.shape)
     limit = torch.finfo(dtype).max if limit is None else limit
     q = out if out is not None else torch.empty(shape, device=x.device, dtype=dtype)
-    s = scale_out if scale_out is not None else torch.empty(scale_shape(shape, group), device=x.device, dtype=torch.float32)
+    s = scale_out if scale_out is not None else torch.empty(scale_shape(shape, group), device=x.device, dtype=_scale_dtype(native))
     assert q.is_contiguous() and s.is_contiguous() and tuple(q.shape) == shape and tuple(s.shape) == scale_shape(shape, group)
+    assert s.dtype == _scale_dtype(native) and (source_scale is None or source_scale.dtype == s.dtype)
     source = source_scale.contiguous() if source_scale is not None else None
     _lib.call("viola_group_quantize", _lib.ptr(x), _lib.code(x.dtype), x.shape[0], x.shape[1],
               _lib.ptr(q), _lib.code(q.dtype), _lib.ptr(s), group[0], group[1], float(limit), int(transposed),
-              _lib.ptr(source), source_group[0], source_group[1])
+              _lib.ptr(source), source_group[0], source_group[1], int(bool(native)))
     return q, s
 
 
-def quantize_dual(x, dtype, group, *, limit=None, column_sum_dtype=None):
+def quantize_dual(x, dtype, group, *, limit=None, column_sum_dtype=None, native=False):
     """Row-wise codes/scales and the quantized transpose of x from ONE read of x.
 
     Same values as quantize(x, ...) and quantize(x, ..., transposed=True); 1-D groups of 32 only.
@@ -65,13 +71,13 @@ def quantize_dual(x, dtype, group, *, limit=None, column_sum_dtype=None):
     rows, cols = x.shape
     limit = torch.finfo(dtype).max if limit is None else limit
     q = torch.empty((rows, cols), device=x.device, dtype=dtype)
-    s = torch.empty(scale_shape((rows, cols), group), device=x.device, dtype=torch.float32)
+    s = torch.empty(scale_shape((rows, cols), group), device=x.device, dtype=_scale_dtype(native))
     qt = torch.empty((cols, rows), device=x.device, dtype=dtype)
-    st = torch.empty(scale_shape((cols, rows), group), device=x.device, dtype=torch.float32)
+    st = torch.empty(scale_shape((cols, rows), group), device=x.device, dtype=_scale_dtype(native))
     parts = -(-rows // 32)
     partial = torch.empty((parts, cols), device=x.device, dtype=torch.float32) if column_sum_dtype is not None else None
     _lib.call("viola_group_quantize_dual", _lib.ptr(x), _lib.code(x.dtype), rows, cols, _lib.ptr(q), _lib.ptr(s),
-              _lib.ptr(qt), _lib.ptr(st), _lib.code(dtype), group[1], float(limit), _lib.ptr(partial))
+              _lib.ptr(qt), _lib.ptr(st), _lib.code(dtype), group[1], float(limit), _lib.ptr(partial), int(bool(native)))
     if column_sum_dtype is None:
         return q, s, qt, st
     total = torch.empty(cols, device=x.device, dtype=column_sum_dtype)
@@ -85,16 +91,14 @@ def transpose_group(group):
 
 
 def transpose(q, scale, group, *, native=False, limit=None):
-    _no_native(native)
     if group[0] >= 32:
         return transpose_payload(q), scale.T.contiguous()
-    return quantize(q, q.dtype, group, limit=limit, transposed=True, source_scale=scale, source_group=group)
+    return quantize(q, q.dtype, group, native=native, limit=limit, transposed=True, source_scale=scale, source_group=group)
 
 
 def gemm(a, b, sa, sb, group_a, group_b, *, out_dtype, native=False, bias=None, autotune=False,
          accum_dtype="fp32", accum_block_size=0, accum_reduce_dtype="fp32"):
     """out[m, n] = sum over 32-wide K groups of (a_codes . b_codes^T) * sa * sb (+ bias); a [m, k], b [n, k]."""
-    _no_native(native)
     if accum_dtype != "fp32" or accum_block_size or accum_reduce_dtype != "fp32":
         raise NotImplementedError("viola_amd accumulates in FP32 only (blocked FP16 accumulation is not built)")
     assert a.is_cuda and b.is_cuda and a.shape[1] == b.shape[1]
@@ -104,6 +108,16 @@ def gemm(a, b, sa, sb, group_a, group_b, *, out_dtype, native=False, bias=None, 
     assert tuple(sa.shape) == scale_shape((m, k), group_a) and tuple(sb.shape) == scale_shape((n, k), group_b)
     out = torch.empty((m, n), device=a.device, dtype=out_dtype)
     bias_c = bias.contiguous() if bias is not None else None
+    if native:
+        assert sa.dtype == torch.uint8 and sb.dtype == torch.uint8 and group_a[1] == 32 and group_b[1] == 32
+        status = _lib.call("viola_mx_gemm", _lib.ptr(a), _lib.code(a.dtype), _lib.ptr(b), _lib.code(b.dtype), _lib.ptr(sa),
+                           _lib.ptr(sb), m, n, k, group_a[0], group_b[0], _lib.ptr(bias_c),
+                           _lib.code(bias_c.dtype) if bias_c is not None else 0, _lib.ptr(out), _lib.code(out_dtype),
+                           unsupported_ok=True)
+        if status == 0:
+            return out
+        # shapes the block-scaled MFMA kernel declines: the same products with the scales spelled out in FP32
+        sa, sb = decode_scale(sa), decode_scale(sb)
     _lib.call("viola_group_gemm", _lib.ptr(a), _lib.code(a.dtype), _lib.ptr(b), _lib.code(b.dtype), _lib.ptr(sa), _lib.ptr(sb),
               m, n, k, group_a[0], group_a[1], group_b[0], group_b[1],
               _lib.ptr(bias_c), _lib.code(bias_c.dtype) if bias_c is not None else 0, _lib.ptr(out), _lib.code(out_dtype))
