@@ -12,23 +12,24 @@ import torch.nn.functional as F
 from . import grouped
 
 
-def _deq(x, dtype, group, limit=None, transposed=False):
-    q, s = grouped.quantize(x, dtype, group, limit=limit, transposed=transposed)
+def _deq(x, dtype, group, limit=None, transposed=False, native=False):
+    q, s = grouped.quantize(x, dtype, group, limit=limit, transposed=transposed, native=native)
     return grouped.dequantize(q, s, group)
 
 
 def linear(x, w_real, bias, dy, *, fp8=torch.float8_e4m3fn, bwd_fp8=torch.float8_e4m3fn,
-           gx=(1, 32), gw=(32, 32), gg=(1, 32), out_dtype=torch.bfloat16, grad_dtype=torch.bfloat16):
-    """Expected y, dx, dw, db of Linear(scaling='grouped') (check_grouped_linear.py:64-75).
+           gx=(1, 32), gw=(32, 32), gg=(1, 32), out_dtype=torch.bfloat16, grad_dtype=torch.bfloat16, native=False):
+    """Expected y, dx, dw, db of Linear(scaling='grouped') (check_grouped_linear.py:64-75); native=True is the same
+    recipe with E8M0 scales (scaling='mxfp8').
 
     w_real is the dequantized weight in its original coordinates ([out, in] fp32).
     """
     x2, dy2 = x.reshape(-1, x.shape[-1]), dy.reshape(-1, dy.shape[-1])
-    ref_x = _deq(x2, fp8, gx)
-    ref_g = _deq(dy2, bwd_fp8, gg)
-    wt = w_real.T if gw[0] >= 32 else _deq(w_real, fp8, gw, transposed=True)
-    xt = _deq(x2, fp8, gx, transposed=True)
-    gt = _deq(dy2, bwd_fp8, gg, transposed=True)
+    ref_x = _deq(x2, fp8, gx, native=native)
+    ref_g = _deq(dy2, bwd_fp8, gg, native=native)
+    wt = w_real.T if gw[0] >= 32 else _deq(w_real, fp8, gw, transposed=True, native=native)
+    xt = _deq(x2, fp8, gx, transposed=True, native=native)
+    gt = _deq(dy2, bwd_fp8, gg, transposed=True, native=native)
     y = ref_x @ w_real.T
     if bias is not None:
         y = y + bias.float()

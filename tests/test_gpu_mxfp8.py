@@ -109,3 +109,81 @@ def test_mx_gemm_exact_on_integers():
     da = a * og.decode_scale(sa).repeat_interleave(32, 1)
     db = b * og.decode_scale(sb).repeat_interleave(32, 0).repeat_interleave(32, 1)
     assert torch.equal(out.cpu(), (da.double() @ db.double().T).float())
+
+
+# ----------------------------------------------------------------------------- Linear(scaling="mxfp8")
+@pytest.fixture
+def precision_policy():
+    import viola_amd
+    saved = dict(viola_amd.precision._settings)
+    yield viola_amd
+    viola_amd.precision._settings.clear()
+    viola_amd.precision._settings.update(saved)
+
+
+@pytest.mark.parametrize("mode,storage,backward", [("memory", "fp8", "e4m3"), ("fast", "fp8", "e5m2"), ("memory", "bf16", "e4m3")])
+@pytest.mark.parametrize("shape", [(65, 128, 96), (256, 512, 384), (3 * 40, 160, 72)])
+def test_linear_mxfp8(precision_policy, mode, storage, backward, shape):
+    """checks/check_grouped_linear.py:50-107 with native scales: uint8 scale buffers, codes and bytes of the stored
+    weight equal the oracle's, y / dx / dw within .003 of the dequantized-operand matmuls, db exact, state_dict reload
+    reproduces the forward bit for bit."""
+    from oracle import linear as ol
+    viola = precision_policy
+    viola.set_gradient_dtype("bf16")
+    m, k, n = shape
+    torch.manual_seed(90)
+    layer = viola.nn.Linear(k, n, device="cuda", dtype=torch.bfloat16, scaling="mxfp8", mode=mode, weight_dtype=storage,
+                            backward_dtype=backward)
+    bwd = E4 if backward == "e4m3" else E5
+    if storage == "fp8":
+        assert layer.weight_scale.dtype == torch.uint8 and layer.weight_scale.shape == og.scale_shape((n, k), (32, 32))
+        master = layer._initial_weight.detach().cpu()
+        rq, rs = og.quantize(master, E4, (32, 32), native=True)
+        assert torch.equal(layer.weight.detach().view(torch.uint8).cpu(), rq.view(torch.uint8)) and torch.equal(layer.weight_scale.cpu(), rs)
+        if mode == "fast":
+            assert layer.weight_transpose_scale.dtype == torch.uint8 and torch.equal(layer.weight_transpose_scale.cpu(), rs.T)
+        w_real = og.dequantize(rq, rs, (32, 32))
+    else:
+        q, s = og.quantize(layer.weight.detach().float().cpu(), E4, (32, 32), native=True)
+        w_real = og.dequantize(q, s, (32, 32))
+    assert torch.equal(layer.dequantize_weight().cpu(), w_real if storage == "fp8" else layer.weight.detach().float().cpu())
+    x = (torch.randn(m, k) * torch.exp2(torch.randint(-5, 6, (m, 1)).float())).bfloat16().cuda().requires_grad_()
+    dy = torch.randn(m, n, device="cuda", dtype=torch.bfloat16)
+    y = layer(x)
+    y.backward(dy)
+    expected = ol.linear(x.detach().cpu(), w_real, layer.bias.detach().cpu(), dy.cpu(), fp8=E4, bwd_fp8=bwd, native=True)
+    assert rel_l2(y, expected["y"]) < 3e-3 and rel_l2(x.grad, expected["dx"]) < 3e-3 and rel_l2(layer.weight.grad, expected["dw"]) < 3e-3
+    assert rel_l2(layer.bias.grad, expected["db"]) < 4e-3
+    if storage == "fp8":
+        other = viola.nn.Linear(k, n, device="cuda", dtype=torch.bfloat16, scaling="mxfp8", mode=mode, weight_dtype=storage,
+                                backward_dtype=backward)
+        other.load_state_dict(layer.state_dict())
+        with torch.no_grad():
+            assert torch.equal(other(x), y)
+
+
+def test_linear_mxfp8_under_bind_optimizer(precision_policy):
+    """A bound AdamW step re-quantizes the master into codes and E8M0 bytes that equal the oracle's."""
+    viola = precision_policy
+    viola.set_master_weight_dtype("fp32")
+    viola.set_gradient_dtype("bf16")
+    torch.manual_seed(91)
+    layer = viola.nn.Linear(256, 192, device="cuda", dtype=torch.bfloat16, scaling="mxfp8", mode="fast")
+    opt = viola.optim.bind_optimizer(layer, torch.optim.AdamW(layer.parameters(), lr=.01))
+    x = torch.randn(64, 256, device="cuda", dtype=torch.bfloat16)
+    for _ in range(2):
+        opt.zero_grad()
+        layer(x).float().square().mean().backward()
+        before = layer.weight.detach().view(torch.uint8).clone()
+        opt.step()
+        assert not torch.equal(before, layer.weight.view(torch.uint8))
+        rq, rs = og.quantize(layer._master_ref().detach().cpu(), E4, (32, 32), native=True)
+        assert torch.equal(layer.weight.detach().view(torch.uint8).cpu(), rq.view(torch.uint8)) and torch.equal(layer.weight_scale.cpu(), rs)
+        assert torch.equal(layer.weight_transpose.view(torch.uint8), layer.weight.T.contiguous().view(torch.uint8))
+        assert torch.equal(layer.weight_transpose_scale, layer.weight_scale.T)
+
+
+def test_mlp_mxfp8_is_declined():
+    import viola_amd
+    with pytest.raises(NotImplementedError):
+        viola_amd.nn.MLP(64, 96, device="cuda", scaling="mxfp8")

@@ -29,18 +29,19 @@ def forward_core(x, weight, bias, layer, need_backward, needs, *, gated=None):
     x_dtype = x.dtype
     x2 = x.reshape(-1, layer.in_features).contiguous()
     gx, gw = layer.input_group_shape, layer.weight_group_shape
+    native = layer._native_scaling
     limit = layer._group_limit(gx, layer.fp8_dtype)
     save_fp8 = need_backward and needs[1] and layer.saved_input_dtype == "fp8"
     xt = sxt = None
     if save_fp8 and _one_d32(gx):
-        qx, sx, xt, sxt = kernels.quantize_dual(x2, layer.fp8_dtype, gx, limit=limit)
+        qx, sx, xt, sxt = kernels.quantize_dual(x2, layer.fp8_dtype, gx, limit=limit, native=native)
     else:
-        qx, sx = kernels.quantize(x2, layer.fp8_dtype, gx, limit=limit)
+        qx, sx = kernels.quantize(x2, layer.fp8_dtype, gx, limit=limit, native=native)
         if save_fp8:
-            xt, sxt = kernels.quantize(x2, layer.fp8_dtype, gx, limit=limit, transposed=True)
+            xt, sxt = kernels.quantize(x2, layer.fp8_dtype, gx, limit=limit, transposed=True, native=native)
     weight_limit = layer._group_limit(gw, layer.fp8_dtype, weight=True)
     if layer.weight_dtype != "fp8":
-        qw, sw = kernels.quantize(weight, layer.fp8_dtype, gw, limit=weight_limit)
+        qw, sw = kernels.quantize(weight, layer.fp8_dtype, gw, limit=weight_limit, native=native)
     else:
         qw, sw = weight, layer.weight_scale
     aux = None
@@ -53,7 +54,7 @@ def forward_core(x, weight, bias, layer, need_backward, needs, *, gated=None):
     if need_backward:
         wt, st = layer.weight_transpose, layer.weight_transpose_scale
         if layer.weight_dtype != "fp8" and needs[0] and layer.cache_weight_transpose:
-            wt, st = kernels.quantize(weight, layer.fp8_dtype, kernels.transpose_group(gw), limit=weight_limit, transposed=True)
+            wt, st = kernels.quantize(weight, layer.fp8_dtype, kernels.transpose_group(gw), limit=weight_limit, transposed=True, native=native)
         if save_fp8:
             saved_x, saved_scale = xt, sxt
         elif needs[1]:
@@ -75,6 +76,7 @@ def backward_core(record, tensors, dy, needs, *, gated=None, aux=None):
     dy = dy.reshape(-1, layer.out_features).contiguous()
     gg, gx, gw = layer.grad_group_shape, layer.input_group_shape, layer.weight_group_shape
     fp8, bwd = layer.fp8_dtype, layer.backward_fp8_dtype
+    native = layer._native_scaling
     limit = layer._group_limit(gg, bwd)
     weight_limit = layer._group_limit(gw, fp8, weight=True)
     qg = sg = gt = sgt = None
@@ -82,19 +84,19 @@ def backward_core(record, tensors, dy, needs, *, gated=None, aux=None):
     if needs[0] and needs[1] and _one_d32(gg):
         if needs[2] and dy.shape[0] > 0:
             # the bias gradient rides on the quantizer's read of dy
-            qg, sg, gt, sgt, db = kernels.quantize_dual(dy, bwd, gg, limit=limit, column_sum_dtype=record.bias_grad_dtype)
+            qg, sg, gt, sgt, db = kernels.quantize_dual(dy, bwd, gg, limit=limit, column_sum_dtype=record.bias_grad_dtype, native=native)
         else:
-            qg, sg, gt, sgt = kernels.quantize_dual(dy, bwd, gg, limit=limit)
+            qg, sg, gt, sgt = kernels.quantize_dual(dy, bwd, gg, limit=limit, native=native)
     for op in ((1, 0) if gated else (0, 1)):
         if op == 0 and needs[0]:
             if qg is None:
-                qg, sg = kernels.quantize(dy, bwd, gg, limit=limit)
+                qg, sg = kernels.quantize(dy, bwd, gg, limit=limit, native=native)
             if cached_wt.numel():
                 wt, st = cached_wt, cached_st
             elif layer.weight_dtype != "fp8":
-                wt, st = kernels.quantize(w, fp8, kernels.transpose_group(gw), limit=weight_limit, transposed=True)
+                wt, st = kernels.quantize(w, fp8, kernels.transpose_group(gw), limit=weight_limit, transposed=True, native=native)
             else:
-                wt, st = kernels.transpose(w, sw, gw, limit=weight_limit)
+                wt, st = kernels.transpose(w, sw, gw, native=native, limit=weight_limit)
             gwt = kernels.transpose_group(gw)
             if gated:
                 dx, _, _ = _mlp_kernels.gemm(qg, wt, sg, st, layer=layer, out_dtype=record.x_dtype, backward=True,
@@ -105,11 +107,11 @@ def backward_core(record, tensors, dy, needs, *, gated=None, aux=None):
             qg = sg = wt = st = None
         if op == 1 and needs[1]:
             if gt is None:
-                gt, sgt = kernels.quantize(dy, bwd, gg, limit=limit, transposed=True)
+                gt, sgt = kernels.quantize(dy, bwd, gg, limit=limit, transposed=True, native=native)
             if record.save_fp8:
                 xt, sxt = saved_x, saved_scale
             else:
-                xt, sxt = kernels.quantize(saved_x, fp8, gx, limit=record.input_limit, transposed=True)
+                xt, sxt = kernels.quantize(saved_x, fp8, gx, limit=record.input_limit, transposed=True, native=native)
             dw = layer._group_gemm(gt, xt, sgt, sxt, gg, gx, out_dtype=record.weight_grad_dtype)
             gt = sgt = xt = sxt = None
     if needs[2] and db is None:

@@ -1,9 +1,10 @@
 """FP8 Linear with FP8 / BF16 / FP16 weight storage (module surface of viola/nn/linear.py:150-412).
 
 Built here: `scaling="grouped"` (FP32 scales per 2-D weight block and per 1-D activation /
-gradient tile) and the per-tensor recipes `scaling="current"` / `"delayed"` (one FP32 scale per tensor,
+gradient tile), `scaling="mxfp8"` (the same groups with E8M0 power-of-two scales, GEMMs on the block-scaled
+MFMA) and the per-tensor recipes `scaling="current"` / `"delayed"` (one FP32 scale per tensor,
 delayed = the maximum of an amax history), FP32 accumulation, e4m3 / e5m2 operand formats. The
-reference's other recipes (`mxfp8`, blocked FP16 accumulation, quantization limits derived from it,
+reference's other recipes (blocked FP16 accumulation, quantization limits derived from it,
 Hadamard rotation) are accepted by the constructor signature but raise NotImplementedError.
 """
 
@@ -73,15 +74,14 @@ class Linear(nn.Module):
         assert scaling in ("current", "delayed", "grouped", "mxfp8") and history_len > 0
         assert accum_dtype in ("fp32", "fp16") and accum_reduce_dtype in ("fp32", "bf16")
         assert accum_block_size >= 0 and accum_block_size % 32 == 0 and rotation_size in (0, 64)
-        if scaling == "mxfp8":
-            raise NotImplementedError("viola_amd builds scaling='grouped', 'current' and 'delayed' (got 'mxfp8')")
+
         if accum_dtype != "fp32" or accum_block_size or accum_reduce_dtype != "fp32" or rotation_size:
             raise NotImplementedError("viola_amd builds FP32 accumulation without rotation only")
         self.in_features, self.out_features = in_features, out_features
         self.mode, self.weight_dtype, self.saved_input_dtype = mode, weight_dtype, saved_input_dtype
         self.forward_dtype, self.backward_dtype = forward_dtype, backward_dtype
         self.fp8_dtype, self.backward_fp8_dtype = _FORMATS[forward_dtype], _FORMATS[backward_dtype]
-        self._grouped_scaling, self._native_scaling = scaling == "grouped", False
+        self._grouped_scaling, self._native_scaling = scaling in ("grouped", "mxfp8"), scaling == "mxfp8"
         self.weight_group_shape = tuple(weight_group_shape)
         self.input_group_shape = tuple(input_group_shape)
         self.grad_group_shape = tuple(grad_group_shape)
@@ -111,9 +111,12 @@ class Linear(nn.Module):
             scale_shape = grouped.scale_shape(shape, self.weight_group_shape) if fp8_storage else (0, 0)
         else:
             scale_shape = (1,) if fp8_storage else (0,)
-        self.register_buffer("weight_scale", torch.ones(scale_shape, device=device, dtype=torch.float32), persistent=fp8_storage)
+        # FP32 scales start at 1, E8M0 bytes at 127 = 2^0 (linear.py:221-226)
+        scale_dtype = torch.uint8 if self._native_scaling else torch.float32
+        self.register_buffer("weight_scale", torch.full(scale_shape, 127 if self._native_scaling else 1, device=device, dtype=scale_dtype),
+                             persistent=fp8_storage)
         self.register_buffer("weight_transpose", torch.empty(0, 0, device=device, dtype=self.fp8_dtype), persistent=False)
-        self.register_buffer("weight_transpose_scale", torch.empty(0, 0, device=device, dtype=torch.float32), persistent=False)
+        self.register_buffer("weight_transpose_scale", torch.empty(0, 0, device=device, dtype=scale_dtype), persistent=False)
         self.weight_quantizer = _Quantizer(scaling, history_len, device)
         self.input_quantizer = _Quantizer(scaling, history_len, device)
         self.grad_quantizer = _Quantizer(scaling, history_len, device)
@@ -134,7 +137,7 @@ class Linear(nn.Module):
         return None
 
     def _group_gemm(self, a, b, sa, sb, ga, gb, *, out_dtype, bias=None):
-        return grouped.gemm(a, b, sa, sb, ga, gb, out_dtype=out_dtype, bias=bias)
+        return grouped.gemm(a, b, sa, sb, ga, gb, out_dtype=out_dtype, bias=bias, native=self._native_scaling)
 
     # ------------------------------------------------------------------ weights
     def _master(self):
@@ -175,7 +178,7 @@ class Linear(nn.Module):
                              out_t=self.weight_transpose if self.cache_weight_transpose else None, quantization_limit=limit)
             return
         limit = self._group_limit(self.weight_group_shape, self.fp8_dtype, weight=True)
-        grouped.quantize(master, self.fp8_dtype, self.weight_group_shape, limit=limit,
+        grouped.quantize(master, self.fp8_dtype, self.weight_group_shape, limit=limit, native=self._native_scaling,
                          out=self.weight, scale_out=self.weight_scale)
         if self.cache_weight_transpose:
             self._build_transpose(limit)
@@ -185,7 +188,7 @@ class Linear(nn.Module):
             self.weight_transpose = kernels.transpose(self.weight)
             return
         self.weight_transpose, self.weight_transpose_scale = grouped.transpose(
-            self.weight, self.weight_scale, self.weight_group_shape, limit=limit)
+            self.weight, self.weight_scale, self.weight_group_shape, native=self._native_scaling, limit=limit)
 
     def dequantize_weight(self):
         if self.weight_dtype != "fp8":
