@@ -235,6 +235,22 @@ def main():
         c_ms, _ = timed(current_step, args.steps, args.warmup)
         cb = kernel_breakdown(current_step, min(args.steps, 50))
         cg = cb["viola_tensor_gemm"]
+        # and the grouped recipe with E8M0 scales: same groups as the headline, the scaling done by the block-scaled MFMA
+        viola_amd.set_gradient_dtype("bf16")
+        mx = viola_amd.nn.Linear(K, N, device="cuda", dtype=torch.bfloat16, scaling="mxfp8", forward_dtype="e4m3",
+                                 backward_dtype="e4m3", mode="memory", weight_dtype="fp8")
+        viola_amd.precision._settings["gradient_dtype"] = None
+
+        def mx_step():
+            xc.grad = mx.weight.grad = mx.bias.grad = None
+            mx(xc).backward(dy)
+        m_ms, _ = timed(mx_step, args.steps, args.warmup)
+        mb = kernel_breakdown(mx_step, min(args.steps, 50))
+        mg = mb["viola_mx_gemm"]
+        extra["linear_mxfp8"] = dict(step_ms=m_ms, tflops=flops / (m_ms * 1e-3) / 1e12, gemm_avg_ms=mg["avg_ms"],
+                                     gemm_tflops=2 * M * K * N / (mg["avg_ms"] * 1e-3) / 1e12,
+                                     gemm_frac_fp8_peak=2 * M * K * N / (mg["avg_ms"] * 1e-3) / 1e12 / PEAK["fp8_tflops"],
+                                     launches_per_step=sum(v["launches_per_step"] for v in mb.values()))
         extra["linear_current_scaling"] = dict(step_ms=c_ms, tflops=flops / (c_ms * 1e-3) / 1e12, gemm_avg_ms=cg["avg_ms"],
                                                gemm_tflops=2 * M * K * N / (cg["avg_ms"] * 1e-3) / 1e12,
                                                gemm_frac_fp8_peak=2 * M * K * N / (cg["avg_ms"] * 1e-3) / 1e12 / PEAK["fp8_tflops"],
