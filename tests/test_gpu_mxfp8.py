@@ -183,7 +183,33 @@ def test_linear_mxfp8_under_bind_optimizer(precision_policy):
         assert torch.equal(layer.weight_transpose_scale, layer.weight_scale.T)
 
 
-def test_mlp_mxfp8_is_declined():
-    import viola_amd
-    with pytest.raises(NotImplementedError):
-        viola_amd.nn.MLP(64, 96, device="cuda", scaling="mxfp8")
+@pytest.mark.parametrize("scaling,activation", [("mxfp8", "silu"), ("current", "gelu"), ("delayed", "relu")])
+def test_mlp_other_recipes_are_the_unfused_composition(precision_policy, scaling, activation):
+    """checks/mlp.py:12-52 for the recipes without a fused epilogue: y, dx and every parameter gradient equal (to the
+    reference's .025) the model written out with its own two Linears and a float gated activation."""
+    import torch.nn.functional as F
+    viola = precision_policy
+    viola.set_gradient_dtype("bf16")
+    torch.manual_seed(131)
+    model = viola.nn.MLP(128, 160, 96, device="cuda", dtype=torch.bfloat16, scaling=scaling, activation=activation,
+                         backward_dtype="e4m3")
+    x = torch.randn(2, 33, 128, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    dy = torch.randn(2, 33, 96, device="cuda", dtype=torch.bfloat16)
+    y = model(x)
+    y.backward(dy)
+    got = [y.detach().clone(), x.grad.clone()] + [p.grad.clone() for p in model.parameters()]
+    x.grad = None
+    for p in model.parameters():
+        p.grad = None
+    for layer in (model.gate_up, model.down):                                  # delayed scaling: replay the same history slots
+        for quantizer in (layer.input_quantizer, layer.grad_quantizer):
+            quantizer.index = 0
+            quantizer.history.zero_()
+    act = {"silu": F.silu, "relu": F.relu, "gelu": lambda t: F.gelu(t, approximate="tanh")}[activation]
+    z = model.gate_up(x)
+    g, u = z[..., :160], z[..., 160:]
+    reference = model.down((act(g.float()) * u.float()).to(z.dtype))
+    reference.backward(dy)
+    want = [reference.detach(), x.grad] + [p.grad for p in model.parameters()]
+    for a, b in zip(got, want):
+        assert rel_l2(a, b) < .025

@@ -1,5 +1,6 @@
-"""Gated MLP: down(act(gate(x)) * up(x)) with the gating fused into the FP8 GEMMs
-(module surface of viola/nn/mlp.py:76-113; autograd wiring :22-73)."""
+"""Gated MLP: down(act(gate(x)) * up(x)) with the gating fused into the FP8 GEMMs for scaling="grouped"
+(module surface of viola/nn/mlp.py:76-113; autograd wiring :22-73); the per-tensor and MXFP8 recipes run the two
+Linears with the elementwise gated kernel between them."""
 
 import torch
 from torch import nn
@@ -66,8 +67,6 @@ class MLP(nn.Module):
         self.hidden_features = hidden_features
         self.out_features = in_features if out_features is None else out_features
         self.activation, self.autotune = activation, autotune
-        if linear_options.get("scaling", "current") != "grouped":
-            raise NotImplementedError("viola_amd builds the fused gated MLP for scaling='grouped' only")
         self.gate_up = Linear(in_features, 2 * hidden_features, autotune=autotune, **linear_options)
         self.down = Linear(hidden_features, self.out_features, autotune=autotune, **linear_options)
 
@@ -75,6 +74,12 @@ class MLP(nn.Module):
         assert x.is_cuda, "viola.nn.MLP executes on CUDA."
         if torch.is_autocast_enabled("cuda"):
             x = x.to(torch.get_autocast_dtype("cuda"))
+        if not (self.gate_up._grouped_scaling and not self.gate_up._native_scaling):
+            # per-tensor and MXFP8 recipes: the same arithmetic, un-fused (z = gate_up(x) rounded to the activation
+            # dtype, act(g) * u in fp32, rounded once: the expression the fused epilogue is checked against,
+            # checks/mlp.py:12-16); only the FP32-group-scale GEMM has the gated epilogues
+            from ._gated_kernels import GatedActivation
+            return self.down(GatedActivation.apply(self.gate_up(x), self.activation))
         need_backward = torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters()))
         need_up = need_backward and (x.requires_grad or any(p.requires_grad for p in self.gate_up.parameters()))
         shape = x.shape
