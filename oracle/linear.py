@@ -18,18 +18,21 @@ def _deq(x, dtype, group, limit=None, transposed=False, native=False):
 
 
 def linear(x, w_real, bias, dy, *, fp8=torch.float8_e4m3fn, bwd_fp8=torch.float8_e4m3fn,
-           gx=(1, 32), gw=(32, 32), gg=(1, 32), out_dtype=torch.bfloat16, grad_dtype=torch.bfloat16, native=False):
+           gx=(1, 32), gw=(32, 32), gg=(1, 32), out_dtype=torch.bfloat16, grad_dtype=torch.bfloat16, native=False,
+           limits=(None, None, None)):
     """Expected y, dx, dw, db of Linear(scaling='grouped') (check_grouped_linear.py:64-75); native=True is the same
     recipe with E8M0 scales (scaling='mxfp8').
 
-    w_real is the dequantized weight in its original coordinates ([out, in] fp32).
+    w_real is the dequantized weight in its original coordinates ([out, in] fp32); limits = the clamp
+    magnitudes of (input, weight, gradient) groups, None = the format's maximum (layer._group_limit there).
     """
     x2, dy2 = x.reshape(-1, x.shape[-1]), dy.reshape(-1, dy.shape[-1])
-    ref_x = _deq(x2, fp8, gx, native=native)
-    ref_g = _deq(dy2, bwd_fp8, gg, native=native)
-    wt = w_real.T if gw[0] >= 32 else _deq(w_real, fp8, gw, transposed=True, native=native)
-    xt = _deq(x2, fp8, gx, transposed=True, native=native)
-    gt = _deq(dy2, bwd_fp8, gg, transposed=True, native=native)
+    lx, lw, lg = limits
+    ref_x = _deq(x2, fp8, gx, lx, native=native)
+    ref_g = _deq(dy2, bwd_fp8, gg, lg, native=native)
+    wt = w_real.T if gw[0] >= 32 else _deq(w_real, fp8, gw, lw, transposed=True, native=native)
+    xt = _deq(x2, fp8, gx, lx, transposed=True, native=native)
+    gt = _deq(dy2, bwd_fp8, gg, lg, transposed=True, native=native)
     y = ref_x @ w_real.T
     if bias is not None:
         y = y + bias.float()

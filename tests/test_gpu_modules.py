@@ -83,7 +83,9 @@ def test_linear_host_construction_then_move_and_no_grad_paths():
     with pytest.raises(AssertionError):
         layer(x.cpu())
     with pytest.raises(NotImplementedError):
-        viola_amd.nn.Linear(64, 32, scaling="grouped", accum_dtype="fp16")       # blocked FP16 accumulation is not built
+        viola_amd.nn.Linear(64, 64, scaling="current", rotation_size=64)         # the Hadamard rotation recipe is not built
+    with pytest.raises(AssertionError):
+        viola_amd.nn.Linear(64, 32, scaling="mxfp8", accum_dtype="fp16")         # linear.py:187-188
     layer.weight.requires_grad_(False)
     layer.bias.requires_grad_(False)
     xg = x.clone().requires_grad_()

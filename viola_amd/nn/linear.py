@@ -3,9 +3,15 @@
 Built here: `scaling="grouped"` (FP32 scales per 2-D weight block and per 1-D activation /
 gradient tile), `scaling="mxfp8"` (the same groups with E8M0 power-of-two scales, GEMMs on the block-scaled
 MFMA) and the per-tensor recipes `scaling="current"` / `"delayed"` (one FP32 scale per tensor,
-delayed = the maximum of an amax history), FP32 accumulation, e4m3 / e5m2 operand formats. The
-reference's other recipes (blocked FP16 accumulation, quantization limits derived from it,
-Hadamard rotation) are accepted by the constructor signature but raise NotImplementedError.
+delayed = the maximum of an amax history), e4m3 / e5m2 operand formats.
+
+Accumulation: the FP8 MFMA of gfx950 accumulates in FP32 and has no narrower accumulator, so
+`accum_dtype="fp16"`, `accum_block_size` and `accum_reduce_dtype="bf16"` (a speed / register knob of
+the reference's tensor-core kernels) change no GEMM here. What they change in the reference's DATA is
+kept: the quantization limits derived from them (linear.py:232-253), so codes and scales are the
+ones the reference stores, and the products are summed in FP32, inside the tolerance the reference
+checks its FP16 sums against (checks/check_grouped_linear.py:41,73). Hadamard rotation
+(`rotation_size=64`) raises NotImplementedError.
 """
 
 import math
@@ -55,6 +61,12 @@ def _pow2(v):
     return v > 0 and v & (v - 1) == 0
 
 
+def _half_sum_limit(reduction):
+    """Largest power of two L with reduction * L * L <= 32768: `reduction` products of two codes of
+    magnitude <= L then sum to at most half of FP16's range (linear.py:237-241, :250-253)."""
+    return 2.0 ** math.floor(math.log2(math.sqrt(32768.0 / reduction)))
+
+
 class Linear(nn.Module):
     """y = x W^T + b computed with FP8 GEMMs on the GPU; inputs/outputs are ordinary BF16/FP16/FP32.
 
@@ -75,8 +87,10 @@ class Linear(nn.Module):
         assert accum_dtype in ("fp32", "fp16") and accum_reduce_dtype in ("fp32", "bf16")
         assert accum_block_size >= 0 and accum_block_size % 32 == 0 and rotation_size in (0, 64)
 
-        if accum_dtype != "fp32" or accum_block_size or accum_reduce_dtype != "fp32" or rotation_size:
-            raise NotImplementedError("viola_amd builds FP32 accumulation without rotation only")
+        if rotation_size:
+            raise NotImplementedError("viola_amd does not build the Hadamard rotation recipe")
+        if scaling == "mxfp8":
+            assert accum_dtype == "fp32" and accum_block_size == 0 and accum_reduce_dtype == "fp32", "MXFP8 MMA uses FP32 accumulation."
         self.in_features, self.out_features = in_features, out_features
         self.mode, self.weight_dtype, self.saved_input_dtype = mode, weight_dtype, saved_input_dtype
         self.forward_dtype, self.backward_dtype = forward_dtype, backward_dtype
@@ -127,14 +141,21 @@ class Linear(nn.Module):
         """Clamp magnitude for a group; None means the format's own maximum (linear.py:244-253)."""
         if self.quantization_limit is not None:
             return min(self.quantization_limit, torch.finfo(dtype).max)
-        return None
+        if self.accum_dtype == "fp32":
+            return None
+        # a weight block is reduced along either of its sides (forward and dgrad)
+        reduction = max(shape) if weight else shape[1]
+        if self.accum_block_size:
+            reduction = math.gcd(reduction, self.accum_block_size)
+        return min(_half_sum_limit(reduction), torch.finfo(dtype).max)
 
     def _quantization_limit(self, reduction, fp8_dtype):
-        """Clamp magnitude of a per-tensor-scaled operand; None means the format's own maximum (linear.py:232-242,
-        whose FP16-accumulation branch is not built)."""
+        """Clamp magnitude of a per-tensor-scaled operand; None means the format's own maximum (linear.py:232-242)."""
         if self.quantization_limit is not None:
             return min(self.quantization_limit, torch.finfo(fp8_dtype).max)
-        return None
+        if self.accum_dtype == "fp32":
+            return None
+        return min(_half_sum_limit(self.accum_block_size or reduction), torch.finfo(fp8_dtype).max)
 
     def _group_gemm(self, a, b, sa, sb, ga, gb, *, out_dtype, bias=None):
         return grouped.gemm(a, b, sa, sb, ga, gb, out_dtype=out_dtype, bias=bias, native=self._native_scaling)
