@@ -99,6 +99,20 @@ int viola_tensor_amax_scale(const void* x, int x_dtype, int64_t n, float* maxima
 int viola_tensor_quantize(const void* x, int x_dtype, int64_t rows, int64_t cols, const float* scale, void* q, void* qt,
                           int q_dtype, float limit, viola_stream_t stream);
 
+/* ---------------------------------------------------------------- Hadamard-64 rotation (`rotation_size=64`)
+ * H64 = H4 (x) H4 (x) H4, H4 = (ones(4, 4) - 2 flip(eye(4))) / 2, applied to each run of 64 consecutive columns of a
+ * [rows, cols] matrix in FP32, in the operation order of viola/nn/_rotation_kernels.py:11-25 (_regular64); a last
+ * group that reaches past `cols` is completed with zeros.
+ * viola_rotation_amax (_rotation_amax :28-47, first half of `tensor_scale` :100-108): maxima[i] = max |rotated x| over
+ * tile i of 64 x 64; parts must be ceil(rows / 64) * ceil(cols / 64); finish with viola_tensor_scale.
+ * viola_rotation_quantize (_rotation_quantize :50-80, `quantize` :111-117): viola_tensor_quantize of the rotated values.
+ * viola_rotation_inverse (_rotation_inplace :83-97, `inverse_` :120-123): x <- rotated x in place, rounded to x's type. */
+int viola_rotation_amax(const void* x, int x_dtype, int64_t rows, int64_t cols, float* maxima, int64_t parts,
+                        viola_stream_t stream);
+int viola_rotation_quantize(const void* x, int x_dtype, int64_t rows, int64_t cols, const float* scale, void* q, void* qt,
+                            int q_dtype, float limit, viola_stream_t stream);
+int viola_rotation_inverse(void* x, int x_dtype, int64_t rows, int64_t cols, viola_stream_t stream);
+
 /* viola/nn/_linear_kernels.py:260-293 `gemm` (_gemm_kernel :124-163, _mixed_gemm_kernel :166-228):
  * out[m, n] = (sum_k a[m, k] * b[n, k]) * sa[0] * sb[0] (+ bias[n]); a and b may mix e4m3 and e5m2. */
 int viola_tensor_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,

@@ -21,6 +21,8 @@ Pinning status (what fixes each function besides its own formula):
   per-tensor scaling (oracle.tensor) : the reference's own CPU definitions (checks/linear.py:17-20,
                      viola/nn/linear.py:298-312) + textbook matmul           -> pinned; an Inf inside the
                      tensor (infinite scale, Inf / Inf)                       -> parity unpinned
+  Hadamard-64 rotation (oracle.rotation) : the matrix the reference defines it by (rotate_cpu,
+                     _rotation_kernels.py:126-130): exact on integers, one-hot rows, involution  -> pinned
   variable-group (MoE) linear : NOT in the reference; per-group loop of the Linear
                      restatement                                   -> parity unpinned
   NaN/Inf inside a quantize group: the reference's GPU and CPU branches disagree

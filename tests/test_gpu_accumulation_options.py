@@ -69,11 +69,11 @@ def test_kernel_with_the_half_sum_limit():
     assert torch.equal(qb.cpu().view(torch.uint8), rb.view(torch.uint8)) and torch.equal(sb.cpu(), rsb)
     assert ra.float().abs().max() == 8.0 and rb.float().abs().max() == 8.0
     bias = torch.randn(n)
-    actual = g.gemm(qa, qb, sa, sb, (1, 32), (32, 32), out_dtype=torch.float32, bias=bias.cuda())
+    actual = g.gemm(qa, qb, sa, sb, (1, 32), (32, 32), out_dtype=torch.float32, bias=bias.cuda(), accum_dtype="fp16")
     expected = og.dequantize(ra, rsa, (1, 32)) @ og.dequantize(rb, rsb, (32, 32)).T + bias
     assert torch.isfinite(actual).all()
     assert rel_l2(actual, expected) < 2e-5                                    # the FP32 bound (:41); the FP16 one is .01
-    again = g.gemm(qa, qb, sa, sb, (1, 32), (32, 32), out_dtype=torch.float32, bias=bias.cuda())
+    again = g.gemm(qa, qb, sa, sb, (1, 32), (32, 32), out_dtype=torch.float32, bias=bias.cuda(), accum_dtype="fp16")
     assert torch.equal(again, actual)
 
 

@@ -82,8 +82,10 @@ def test_linear_host_construction_then_move_and_no_grad_paths():
     assert y.shape == (3, 5, 32) and y.dtype == torch.float32
     with pytest.raises(AssertionError):
         layer(x.cpu())
-    with pytest.raises(NotImplementedError):
-        viola_amd.nn.Linear(64, 64, scaling="current", rotation_size=64)         # the Hadamard rotation recipe is not built
+    with pytest.raises(AssertionError):
+        viola_amd.nn.Linear(64, 64, scaling="grouped", rotation_size=64)         # linear.py:183
+    with pytest.raises(AssertionError):
+        viola_amd.nn.Linear(96, 64, scaling="current", rotation_size=64)         # linear.py:200
     with pytest.raises(AssertionError):
         viola_amd.nn.Linear(64, 32, scaling="mxfp8", accum_dtype="fp16")         # linear.py:187-188
     layer.weight.requires_grad_(False)

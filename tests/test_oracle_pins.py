@@ -416,3 +416,33 @@ def test_native_quantize_matches_the_reference_cpu_branch(dtype, group, shape):
     assert grouped.quantize(y, dtype, (32, 32), native=True)[1].item() == 127 - 8
     # dequantize and the re-encoding transpose read the bytes
     assert torch.equal(grouped.dequantize(q, s, group), q.float() * grouped.decode_scale(s).repeat_interleave(gr, 0).repeat_interleave(gc, 1)[:shape[0], :shape[1]])
+
+
+# ----------------------------------------------------------------------------- Hadamard-64 rotation
+def test_rotation_is_the_kronecker_hadamard_matrix():
+    """The staged butterflies of oracle.rotation.rotate against the matrix the reference defines the rotation by
+    (rotate_cpu, viola/nn/_rotation_kernels.py:126-130): equal bit for bit on small integers (every sum exact), to
+    rounding otherwise; H64 is symmetric, orthogonal and has entries +-1/8; rotating twice gives the input back; a
+    group cut off by the matrix edge is completed with zeros. A wrong stride, digit or sign fails the first check."""
+    from oracle import rotation
+    h = rotation.hadamard64()
+    assert torch.equal(h, h.T) and torch.equal(h.abs(), torch.full((64, 64), 0.125))
+    assert torch.equal(h @ h, torch.eye(64))
+    torch.manual_seed(9)
+    k = torch.randint(-50, 51, (7, 192)).float()
+    assert torch.equal(rotation.rotate(k), (k.reshape(-1, 64) @ h).reshape(k.shape))
+    assert torch.equal(rotation.rotate(rotation.rotate(k)), k)
+    # one-hot rows pick out the rows of H64: every output position and sign is checked
+    assert torch.equal(rotation.rotate(torch.eye(64)), h)
+    x = torch.randn(5, 128)
+    exact = (x.double().reshape(-1, 64) @ h.double()).reshape(x.shape)
+    assert (rotation.rotate(x).double() - exact).abs().max() < 1e-6
+    z = torch.randn(3, 100)
+    padded = torch.zeros(3, 128)
+    padded[:, :100] = z
+    assert torch.equal(rotation.rotate(z), rotation.rotate(padded)[:, :100])
+    # the norm of every group is preserved (orthogonality), which is why one scale serves the rotated tensor
+    assert torch.allclose(rotation.rotate(x).reshape(-1, 64).norm(dim=1), x.reshape(-1, 64).norm(dim=1), rtol=1e-5)
+    n = x.clone()
+    n[2, 5] = float("nan")
+    assert rotation.amax(n) == rotation.rotate(x)[torch.arange(5) != 2].abs().max().maximum(rotation.rotate(x)[2, 64:].abs().max())

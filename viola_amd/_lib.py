@@ -39,6 +39,9 @@ _SIGNATURES = {
     "viola_tensor_amax_columns": [_p, _i, _l, _l, _l, _p, _p, _p],
     "viola_tensor_amax_scale": [_p, _i, _l, _p, _l, _p, _i, _l, _i, _f, _p, _p],
     "viola_tensor_quantize": [_p, _i, _l, _l, _p, _p, _p, _i, _f, _p],
+    "viola_rotation_amax": [_p, _i, _l, _l, _p, _l, _p],
+    "viola_rotation_quantize": [_p, _i, _l, _l, _p, _p, _p, _i, _f, _p],
+    "viola_rotation_inverse": [_p, _i, _l, _l, _p],
     "viola_tensor_gemm": [_p, _i, _p, _i, _p, _p, _l, _l, _l, _p, _i, _p, _i, _p],
     "viola_mx_gemm": [_p, _i, _p, _i, _p, _p, _l, _l, _l, _i, _i, _p, _i, _p, _i, _p],
     "viola_momentum_update_table": [_p, _l, _l, _i, _i, _f, _f, _i, _i, _l, _p],

@@ -170,10 +170,103 @@ __device__ __forceinline__ void load16(const TIn* row, int64_t c0, int64_t cols,
     }
 }
 
+// ------------------------------------------------------------------ Hadamard-64 rotation of channel groups
+// H64 = H4 (x) H4 (x) H4 with H4 = (ones(4, 4) - 2 flip(eye(4))) / 2, symmetric and its own inverse, applied to 64
+// consecutive columns. Three stages with strides 1, 4 and 16, each in the reference's operation order
+// (_rotation_kernels.py:11-25): out[j] = ((v[b] + v[b + s]) + (v[b + 2s] + v[b + 3s])) * 0.5 - v[b + (3 - digit) s],
+// b = j with base-4 digit `digit` of weight s cleared. A quad of lanes holds the 64 values, 16 consecutive ones each:
+// strides 1 and 4 stay inside a lane, stride 16 pairs the same register of the four lanes (DPP quad permutes; float
+// addition commutes, so every lane forms (v0 + v1) + (v2 + v3) bit for bit).
+__device__ __forceinline__ float quad_perm(float v, int control) {
+    if (control == 0xB1) return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xf, 0xf, true));   // lanes 1 0 3 2
+    if (control == 0x4E) return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xf, 0xf, true));   // lanes 2 3 0 1
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x1B, 0xf, 0xf, true));                        // lanes 3 2 1 0
+}
+
+__device__ __forceinline__ void rotate64(float (&v)[16]) {
+    float t[16];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {                                           // stride 1
+        const float half = ((v[4 * g] + v[4 * g + 1]) + (v[4 * g + 2] + v[4 * g + 3])) * 0.5f;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) t[4 * g + d] = half - v[4 * g + 3 - d];
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {                                           // stride 4
+        const float half = ((t[r] + t[r + 4]) + (t[r + 8] + t[r + 12])) * 0.5f;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) v[r + 4 * d] = half - t[r + 4 * (3 - d)];
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {                                          // stride 16: digit = lane % 4
+        const float pair = v[i] + quad_perm(v[i], 0xB1);
+        const float half = (pair + quad_perm(pair, 0x4E)) * 0.5f;
+        t[i] = half - quad_perm(v[i], 0x1B);
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) v[i] = t[i];
+}
+
+// maxima[block] = max |rotated x| over a 64 x 64 tile (columns past the end count as zeros inside their group, as in
+// _rotation_kernels.py:28-47; fmaxf drops NaN like the reference's reduction).
+template <typename TIn>
+__global__ __launch_bounds__(256) void rotation_amax_kernel(const TIn* __restrict__ x, int64_t rows, int64_t cols, int vector_in,
+                                                             float* __restrict__ maxima) {
+    const int tid = threadIdx.x;
+    const int64_t row = (int64_t)blockIdx.y * 64 + tid / 4, col = (int64_t)blockIdx.x * 64 + (tid % 4) * 16;
+    float v[16];
+    load16<TIn>(x + row * cols, col, cols, row < rows, vector_in != 0, v);
+    rotate64(v);
+    float m = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) m = fmaxf(m, fabsf(v[i]));
+    __shared__ float part[4];
+    m = wave_max(m);
+    if (tid % WAVE == 0) part[tid / WAVE] = m;
+    __syncthreads();
+    if (tid == 0) maxima[(int64_t)blockIdx.y * gridDim.x + blockIdx.x] = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
+}
+
+// x <- rotated x, rounded to the tensor's own type (_rotation_kernels.py:83-97): every block owns whole groups.
+template <typename T>
+__global__ __launch_bounds__(256) void rotation_inplace_kernel(T* __restrict__ x, int64_t rows, int64_t cols, int vector_in) {
+    const int tid = threadIdx.x;
+    const int64_t row = (int64_t)blockIdx.y * 64 + tid / 4, col = (int64_t)blockIdx.x * 64 + (tid % 4) * 16;
+    float v[16];
+    load16<T>(x + row * cols, col, cols, row < rows, vector_in != 0, v);
+    rotate64(v);
+    if (row >= rows) return;
+    T* dst = x + row * cols + col;
+    if (vector_in && col + 16 <= cols) {
+        if constexpr (sizeof(T) == 4) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) *reinterpret_cast<float4*>(dst + 4 * i) = make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                uint32_t w[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const T lo = from_f32<T>(v[8 * i + 2 * j]), hi = from_f32<T>(v[8 * i + 2 * j + 1]);
+                    uint16_t a, b;
+                    __builtin_memcpy(&a, &lo, 2);
+                    __builtin_memcpy(&b, &hi, 2);
+                    w[j] = (uint32_t)a | ((uint32_t)b << 16);
+                }
+                *reinterpret_cast<uint4*>(dst + 8 * i) = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+        }
+    } else {
+        for (int i = 0; i < 16; ++i)
+            if (col + i < cols) dst[i] = from_f32<T>(v[i]);
+    }
+}
+
 // 64 x 64 tile per 256-thread block: thread t quantizes 16 consecutive elements of tile row t / 4, stores them
 // row-wise (16 bytes) and, for the transposed layout, parks them in LDS, from where thread t collects 16 consecutive
 // rows of tile column t / 4. q = fp8(isnan(v) ? v : clamp(v / scale, +-limit)) with the one scale of the tensor.
-template <typename TIn, typename TOut>
+// ROTATE: the values are Hadamard-rotated in their 64-column groups first (_rotation_kernels.py:50-80).
+template <typename TIn, typename TOut, bool ROTATE>
 __global__ __launch_bounds__(256) void tensor_quantize_kernel(const TIn* __restrict__ x, const float* __restrict__ scale,
                                                                uint8_t* __restrict__ q, uint8_t* __restrict__ qt, int64_t rows,
                                                                int64_t cols, float limit, int vector_in, int vector_q,
@@ -186,6 +279,7 @@ __global__ __launch_bounds__(256) void tensor_quantize_kernel(const TIn* __restr
     const float s = scale[0];
     float v[16];
     load16<TIn>(x + row * cols, col, cols, row < rows, vector_in != 0, v);
+    if constexpr (ROTATE) rotate64(v);
     float poison = 0.0f;
 #pragma unroll
     for (int i = 0; i < 16; ++i) poison = poison_of(poison, v[i]);
@@ -232,14 +326,14 @@ __global__ __launch_bounds__(256) void tensor_quantize_kernel(const TIn* __restr
     }
 }
 
-template <typename TIn, typename TOut>
+template <typename TIn, typename TOut, bool ROTATE>
 static int launch_tensor_quantize(const void* x, const float* scale, void* q, void* qt, int64_t rows, int64_t cols, float limit,
                                   hipStream_t stream) {
     const int vector_in = reinterpret_cast<uintptr_t>(x) % 16 == 0 && (cols * sizeof(TIn)) % 16 == 0;
     const int vector_q = q && reinterpret_cast<uintptr_t>(q) % 16 == 0 && cols % 16 == 0;
     const int vector_qt = qt && reinterpret_cast<uintptr_t>(qt) % 16 == 0 && rows % 16 == 0;
     const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64));
-    hipLaunchKernelGGL((tensor_quantize_kernel<TIn, TOut>), grid, dim3(256), 0, stream, static_cast<const TIn*>(x), scale,
+    hipLaunchKernelGGL((tensor_quantize_kernel<TIn, TOut, ROTATE>), grid, dim3(256), 0, stream, static_cast<const TIn*>(x), scale,
                        static_cast<uint8_t*>(q), static_cast<uint8_t*>(qt), rows, cols, limit, vector_in, vector_q, vector_qt);
     return viola_launch_status();
 }
@@ -287,13 +381,13 @@ extern "C" int viola_tensor_amax_scale(const void* x, int x_dtype, int64_t n, fl
     return status ? status : viola_tensor_scale(maxima, parts, history, history_len, index, delayed, limit, scale, stream);
 }
 
-extern "C" int viola_tensor_quantize(const void* x, int x_dtype, int64_t rows, int64_t cols, const float* scale, void* q,
-                                     void* qt, int q_dtype, float limit, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+template <bool ROTATE>
+static int tensor_quantize_entry(const void* x, int x_dtype, int64_t rows, int64_t cols, const float* scale, void* q,
+                                 void* qt, int q_dtype, float limit, hipStream_t stream) {
     VIOLA_CHECK_ARG(viola_is_float(x_dtype) && viola_is_fp8(q_dtype) && rows >= 0 && cols >= 0 && limit > 0.0f);
     if (rows == 0 || cols == 0 || (!q && !qt)) return 0;
     VIOLA_CHECK_ARG(x && scale && (rows + 63) / 64 <= 65535);
-#define VIOLA_TQ(TI, TO) return launch_tensor_quantize<TI, TO>(x, scale, q, qt, rows, cols, limit, stream)
+#define VIOLA_TQ(TI, TO) return launch_tensor_quantize<TI, TO, ROTATE>(x, scale, q, qt, rows, cols, limit, stream)
     if (q_dtype == VIOLA_E4M3) {
         if (x_dtype == VIOLA_F32) VIOLA_TQ(float, e4m3_t);
         if (x_dtype == VIOLA_BF16) VIOLA_TQ(bf16_t, e4m3_t);
@@ -303,4 +397,40 @@ extern "C" int viola_tensor_quantize(const void* x, int x_dtype, int64_t rows, i
     if (x_dtype == VIOLA_BF16) VIOLA_TQ(bf16_t, e5m2_t);
     VIOLA_TQ(f16_t, e5m2_t);
 #undef VIOLA_TQ
+}
+
+extern "C" int viola_tensor_quantize(const void* x, int x_dtype, int64_t rows, int64_t cols, const float* scale, void* q,
+                                     void* qt, int q_dtype, float limit, viola_stream_t stream) {
+    return tensor_quantize_entry<false>(x, x_dtype, rows, cols, scale, q, qt, q_dtype, limit, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int viola_rotation_quantize(const void* x, int x_dtype, int64_t rows, int64_t cols, const float* scale, void* q,
+                                       void* qt, int q_dtype, float limit, viola_stream_t stream) {
+    return tensor_quantize_entry<true>(x, x_dtype, rows, cols, scale, q, qt, q_dtype, limit, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int viola_rotation_amax(const void* x, int x_dtype, int64_t rows, int64_t cols, float* maxima, int64_t parts,
+                                   viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_float(x_dtype) && rows > 0 && cols > 0 && x && maxima && (rows + 63) / 64 <= 65535);
+    const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64));
+    VIOLA_CHECK_ARG(parts == (int64_t)grid.x * grid.y);
+    const int vector_in = reinterpret_cast<uintptr_t>(x) % 16 == 0 && (cols * viola_dtype_size(x_dtype)) % 16 == 0;
+    if (x_dtype == VIOLA_F32) hipLaunchKernelGGL(rotation_amax_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(x), rows, cols, vector_in, maxima);
+    else if (x_dtype == VIOLA_BF16) hipLaunchKernelGGL(rotation_amax_kernel<bf16_t>, grid, dim3(256), 0, stream, static_cast<const bf16_t*>(x), rows, cols, vector_in, maxima);
+    else hipLaunchKernelGGL(rotation_amax_kernel<f16_t>, grid, dim3(256), 0, stream, static_cast<const f16_t*>(x), rows, cols, vector_in, maxima);
+    return viola_launch_status();
+}
+
+extern "C" int viola_rotation_inverse(void* x, int x_dtype, int64_t rows, int64_t cols, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_float(x_dtype) && rows >= 0 && cols >= 0);
+    if (rows == 0 || cols == 0) return 0;
+    VIOLA_CHECK_ARG(x && (rows + 63) / 64 <= 65535);
+    const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64));
+    const int vector_in = reinterpret_cast<uintptr_t>(x) % 16 == 0 && (cols * viola_dtype_size(x_dtype)) % 16 == 0;
+    if (x_dtype == VIOLA_F32) hipLaunchKernelGGL(rotation_inplace_kernel<float>, grid, dim3(256), 0, stream, static_cast<float*>(x), rows, cols, vector_in);
+    else if (x_dtype == VIOLA_BF16) hipLaunchKernelGGL(rotation_inplace_kernel<bf16_t>, grid, dim3(256), 0, stream, static_cast<bf16_t*>(x), rows, cols, vector_in);
+    else hipLaunchKernelGGL(rotation_inplace_kernel<f16_t>, grid, dim3(256), 0, stream, static_cast<f16_t*>(x), rows, cols, vector_in);
+    return viola_launch_status();
 }

@@ -77,8 +77,8 @@ def quantize(x, scale, *, rowwise=True, transpose=False, fp8_dtype=torch.float8_
 def gemm(a, b, sa, sb, *, out_dtype, bias=None, autotune=False, accum_dtype="fp32", accum_block_size=0,
          accum_reduce_dtype="fp32"):
     """(a * sa) @ (b * sb).T + bias with the scaling in the epilogue; a [m, k] and b [n, k] are FP8 codes."""
-    if accum_dtype != "fp32" or accum_block_size or accum_reduce_dtype != "fp32":
-        raise NotImplementedError("viola_amd builds FP32 accumulation only")
+    # the accumulation arguments select no other kernel: the FP8 MFMA sums in FP32
+    assert accum_dtype in ("fp32", "fp16") and accum_reduce_dtype in ("fp32", "bf16") and accum_block_size % 32 == 0
     assert a.is_cuda and a.is_contiguous() and b.is_contiguous() and a.shape[1] == b.shape[1]
     out = torch.empty((a.shape[0], b.shape[0]), device=a.device, dtype=out_dtype)
     has_bias = bias is not None and bias.numel() > 0

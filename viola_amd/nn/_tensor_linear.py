@@ -1,10 +1,15 @@
 """Forward / dgrad / wgrad of Linear(scaling="current" | "delayed"): one FP32 scale per tensor, applied in the
 GEMM epilogue (the role of `_Linear`, viola/nn/linear.py:36-147). Each operand is read twice at most: once for its
-amax, once by the quantizer, which writes the row-wise and the transposed codes together when both are needed."""
+amax, once by the quantizer, which writes the row-wise and the transposed codes together when both are needed.
+
+With `rotation_size=64`, X and W are Hadamard-rotated along in_features inside their amax and quantize kernels
+((X H)(W H)^T = X W^T), dY is not, and the two gradients that come out in rotated coordinates, dX = dY (W H) and
+dW = dY^T (X H), are rotated back in place (linear.py:42-52, :113-115, :142-143)."""
 
 import torch
 
 from . import _linear_kernels as kernels
+from . import _rotation_kernels as rotation
 
 _FLOAT = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}
 
@@ -16,15 +21,16 @@ class TensorLinear(torch.autograd.Function):
         x2 = x.reshape(-1, layer.in_features).contiguous()
         fp8 = layer.fp8_dtype
         input_limit = layer._quantization_limit(max(x2.shape), fp8)
-        sx = layer.input_quantizer.scale(x2, fp8, input_limit)
+        sx = layer.input_quantizer.scale(x2, fp8, input_limit, layer.rotation_size)
+        quantize = rotation.quantize if layer.rotation_size else kernels.quantize
         needs_x, needs_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         save_fp8 = need_backward and needs_w and layer.saved_input_dtype == "fp8"
-        qx, qxt = kernels.quantize(x2, sx, transpose=save_fp8, fp8_dtype=fp8, quantization_limit=input_limit)
+        qx, qxt = quantize(x2, sx, transpose=save_fp8, fp8_dtype=fp8, quantization_limit=input_limit)
         if layer.weight_dtype != "fp8":
             weight_limit = layer._quantization_limit(max(weight.shape), fp8)
-            sw = layer.weight_quantizer.scale(weight, fp8, weight_limit)
-            qw, wt = kernels.quantize(weight, sw, fp8_dtype=fp8, quantization_limit=weight_limit,
-                                      transpose=need_backward and needs_x and layer.cache_weight_transpose)
+            sw = layer.weight_quantizer.scale(weight, fp8, weight_limit, layer.rotation_size)
+            qw, wt = quantize(weight, sw, fp8_dtype=fp8, quantization_limit=weight_limit,
+                              transpose=need_backward and needs_x and layer.cache_weight_transpose)
         else:
             qw, sw, wt = weight, layer.weight_scale, layer.weight_transpose
         y = kernels.gemm(qx, qw, sx, sw, out_dtype=x2.dtype, bias=bias)
@@ -51,6 +57,7 @@ class TensorLinear(torch.autograd.Function):
         needs_x, needs_w, needs_b = ctx.needs_input_grad[:3]
         grad_limit = layer._quantization_limit(max(dy.shape), bwd)
         dx = dw = db = None
+        quantize = rotation.quantize if layer.rotation_size else kernels.quantize
         if needs_b:
             # the bias gradient rides on the amax pass over dy
             sg, db = layer.grad_quantizer.scale_and_column_sum(dy, ctx.bias_grad_dtype, bwd, grad_limit)
@@ -63,16 +70,21 @@ class TensorLinear(torch.autograd.Function):
                 wt = cached_wt
             elif layer.weight_dtype != "fp8":
                 # this forward's scale again: the delayed history does not advance in backward
-                _, wt = kernels.quantize(weight, sw, rowwise=False, transpose=True, fp8_dtype=fp8,
-                                         quantization_limit=layer._quantization_limit(max(weight.shape), fp8))
+                _, wt = quantize(weight, sw, rowwise=False, transpose=True, fp8_dtype=fp8,
+                                 quantization_limit=layer._quantization_limit(max(weight.shape), fp8))
             else:
                 wt = kernels.transpose(weight)
-            dx = kernels.gemm(qg, wt, sg, sw, out_dtype=ctx.x_dtype).reshape(*ctx.shape[:-1], layer.in_features)
+            dx = kernels.gemm(qg, wt, sg, sw, out_dtype=ctx.x_dtype)
+            if layer.rotation_size:
+                rotation.inverse_(dx)
+            dx = dx.reshape(*ctx.shape[:-1], layer.in_features)
             del wt, qg
         if needs_w:
             if ctx.save_fp8:
                 xt = saved_x
             else:
-                _, xt = kernels.quantize(saved_x, sx, rowwise=False, transpose=True, fp8_dtype=fp8, quantization_limit=ctx.input_limit)
+                _, xt = quantize(saved_x, sx, rowwise=False, transpose=True, fp8_dtype=fp8, quantization_limit=ctx.input_limit)
             dw = kernels.gemm(qgt, xt, sg, sx, out_dtype=ctx.weight_grad_dtype)
+            if layer.rotation_size:
+                rotation.inverse_(dw)
         return dx, dw, db, None, None

@@ -10,8 +10,8 @@ Accumulation: the FP8 MFMA of gfx950 accumulates in FP32 and has no narrower acc
 the reference's tensor-core kernels) change no GEMM here. What they change in the reference's DATA is
 kept: the quantization limits derived from them (linear.py:232-253), so codes and scales are the
 ones the reference stores, and the products are summed in FP32, inside the tolerance the reference
-checks its FP16 sums against (checks/check_grouped_linear.py:41,73). Hadamard rotation
-(`rotation_size=64`) raises NotImplementedError.
+checks its FP16 sums against (checks/check_grouped_linear.py:41,73). `rotation_size=64` (per-tensor recipes only)
+stores and multiplies Hadamard-rotated X and W.
 """
 
 import math
@@ -21,6 +21,7 @@ from torch import nn
 
 from . import _grouped_kernels as grouped
 from . import _linear_kernels as kernels
+from . import _rotation_kernels as rotation
 from ..precision import settings
 
 _FORMATS = {"e4m3": torch.float8_e4m3fn, "e5m2": torch.float8_e5m2}
@@ -36,9 +37,10 @@ class _Quantizer(nn.Module):
         self.scaling, self.index = scaling, 0
         self.register_buffer("history", torch.zeros(history_len, device=device, dtype=torch.float32))
 
-    def scale(self, x, fp8_dtype=torch.float8_e4m3fn, quantization_limit=None):
-        scale = kernels.tensor_scale(x, history=self.history, index=self.index, delayed=self.scaling == "delayed",
-                                     fp8_dtype=fp8_dtype, quantization_limit=quantization_limit)
+    def scale(self, x, fp8_dtype=torch.float8_e4m3fn, quantization_limit=None, rotation_size=0):
+        implementation = rotation if rotation_size else kernels
+        scale = implementation.tensor_scale(x, history=self.history, index=self.index, delayed=self.scaling == "delayed",
+                                            fp8_dtype=fp8_dtype, quantization_limit=quantization_limit)
         self.index += 1
         return scale
 
@@ -87,8 +89,9 @@ class Linear(nn.Module):
         assert accum_dtype in ("fp32", "fp16") and accum_reduce_dtype in ("fp32", "bf16")
         assert accum_block_size >= 0 and accum_block_size % 32 == 0 and rotation_size in (0, 64)
 
-        if rotation_size:
-            raise NotImplementedError("viola_amd does not build the Hadamard rotation recipe")
+        assert not rotation_size or in_features % rotation_size == 0
+        if scaling in ("grouped", "mxfp8"):
+            assert rotation_size == 0, "Grouped scaling does not combine with rotation_size."
         if scaling == "mxfp8":
             assert accum_dtype == "fp32" and accum_block_size == 0 and accum_reduce_dtype == "fp32", "MXFP8 MMA uses FP32 accumulation."
         self.in_features, self.out_features = in_features, out_features
@@ -193,10 +196,11 @@ class Linear(nn.Module):
             limit = self._quantization_limit(max(self.in_features, self.out_features), self.fp8_dtype)
             if self.cache_weight_transpose and self.weight_transpose.numel() == 0:
                 self.weight_transpose = torch.empty((self.in_features, self.out_features), device=master.device, dtype=self.fp8_dtype)
-            scale = self.weight_quantizer.scale(master, self.fp8_dtype, limit)
+            scale = self.weight_quantizer.scale(master, self.fp8_dtype, limit, self.rotation_size)
             self.weight_scale.copy_(scale)
-            kernels.quantize(master, scale, transpose=self.cache_weight_transpose, fp8_dtype=self.fp8_dtype, out=self.weight,
-                             out_t=self.weight_transpose if self.cache_weight_transpose else None, quantization_limit=limit)
+            quantize = rotation.quantize if self.rotation_size else kernels.quantize
+            quantize(master, scale, transpose=self.cache_weight_transpose, fp8_dtype=self.fp8_dtype, out=self.weight,
+                     out_t=self.weight_transpose if self.cache_weight_transpose else None, quantization_limit=limit)
             return
         limit = self._group_limit(self.weight_group_shape, self.fp8_dtype, weight=True)
         grouped.quantize(master, self.fp8_dtype, self.weight_group_shape, limit=limit, native=self._native_scaling,
@@ -216,7 +220,8 @@ class Linear(nn.Module):
             return self.weight.float()
         assert self.weight.is_cuda, "viola_amd kernels run on the GPU only"
         if not self._grouped_scaling:
-            return self.weight.float() * self.weight_scale
+            weight = self.weight.float() * self.weight_scale
+            return rotation.inverse_(weight) if self.rotation_size else weight   # back to the original coordinates
         return grouped.dequantize(self.weight, self.weight_scale, self.weight_group_shape)
 
     @classmethod
@@ -300,5 +305,7 @@ class Linear(nn.Module):
                 f"mode={self.mode!r}, weight_dtype={self.weight_dtype!r}, forward_dtype={self.forward_dtype!r}, "
                 f"backward_dtype={self.backward_dtype!r}, cache_weight_transpose={self.cache_weight_transpose}, "
                 f"saved_input_dtype={self.saved_input_dtype!r}, scaling={self.weight_quantizer.scaling!r}, "
+                f"accum_dtype={self.accum_dtype!r}, accum_block_size={self.accum_block_size}, "
+                f"accum_reduce_dtype={self.accum_reduce_dtype!r}, rotation_size={self.rotation_size}, "
                 f"weight_group_shape={self.weight_group_shape}, input_group_shape={self.input_group_shape}, "
                 f"grad_group_shape={self.grad_group_shape}")
