@@ -147,6 +147,17 @@ int viola_gated_gemm(const void* a, int a_dtype, const void* b, int b_dtype, con
                      const void* bias, int bias_dtype, void* aux, void* out, int out_dtype,
                      int activation, int backward, viola_stream_t stream);
 
+/* The same two gated projections under the other recipes of viola/nn/_mlp_kernels.py:16-231 (`grouped` false:
+ * value *= sa[0] * sb[0], :157-166; native E8M0 scales, :120-127). viola_tensor_gated_gemm: one FP32 scale per
+ * operand. viola_mx_gated_gemm: E8M0 bytes per 32 k as in viola_mx_gemm (ar, br = rows per scale row); returns
+ * VIOLA_EUNSUPPORTED where viola_mx_gemm does, and in forward when h is not a multiple of br. */
+int viola_tensor_gated_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,
+                            int64_t m, int64_t h, int64_t k, const void* bias, int bias_dtype, void* aux, void* out,
+                            int out_dtype, int activation, int backward, viola_stream_t stream);
+int viola_mx_gated_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const uint8_t* sa, const uint8_t* sb,
+                        int64_t m, int64_t h, int64_t k, int ar, int br, const void* bias, int bias_dtype, void* aux,
+                        void* out, int out_dtype, int activation, int backward, viola_stream_t stream);
+
 /* Variable-group (MoE-expert style) GEMM: `groups` independent problems that share n and k and
  * differ in their row range. Group g owns rows [offsets[g], offsets[g+1]) of a and out
  * (offsets: groups+1 int64 on the device, ascending) and operand b + g*b_group_stride (elements),

@@ -94,6 +94,62 @@ def test_gated_gemm_forward_backward(activation, m, h, k, dtype):
     assert dz.shape == (m, 2 * h) and rel_l2(dz, torch.cat([dg, du], 1).to(dtype)) < 6e-3
 
 
+class _TensorLayer:
+    _grouped_scaling, _native_scaling = False, False
+
+
+class _NativeLayer(_Layer):
+    _native_scaling = True
+
+
+@pytest.mark.parametrize("recipe", ["tensor", "mxfp8"])
+@pytest.mark.parametrize("activation,formats", [("silu", (E4, E4)), ("gelu", (E5, E4)), ("relu", (E4, E5))])
+@pytest.mark.parametrize("m,h,k,k2", [(66, 160, 128, 256), (130, 64, 96, 96), (64, 40, 64, 128), (300, 256, 384, 128)])
+def test_gated_gemm_other_recipes(recipe, activation, formats, m, h, k, k2):
+    """viola_tensor_gated_gemm / viola_mx_gated_gemm (viola/nn/_mlp_kernels.py:157-194 with `grouped` false or native
+    scales): aux = the plain GEMM's [g, u], out = act(g) * u, and the backward pair, for aligned shapes (the fused
+    kernels) and others (generic kernel, or plain GEMM + elementwise kernels)."""
+    from viola_amd.nn import _mlp_kernels as mk
+    from oracle import tensor as ot
+    dtype = torch.bfloat16
+    native = recipe == "mxfp8"
+    torch.manual_seed(7)
+    a = (torch.randn(m, k) * torch.exp2(torch.randint(-3, 4, (m, 1)).float())).bfloat16()
+    w = (torch.randn(2 * h, k) * torch.exp2(torch.randint(-3, 4, (2 * h, 1)).float())).bfloat16()
+    dy = (torch.randn(m, k2) * torch.exp2(torch.randint(-3, 4, (m, 1)).float())).bfloat16()
+    w2 = (torch.randn(h, k2) * torch.exp2(torch.randint(-3, 4, (h, 1)).float())).bfloat16()
+    bias = torch.randn(2 * h).to(dtype)
+    if native:
+        gw = (32, 32) if h % 32 == 0 else (1, 32)
+        layer = _NativeLayer()
+        layer.weight_group_shape = gw
+        (qa, sa), (qb, sb) = og.quantize(a, formats[0], (1, 32), native=True), og.quantize(w, formats[1], gw, native=True)
+        (qg, sg), (qw, sw) = og.quantize(dy, formats[0], (1, 32), native=True), og.quantize(w2, formats[1], (32, 32), native=True)
+        z = og.gemm(qa, qb, og.decode_scale(sa), og.decode_scale(sb), (1, 32), gw, bias=bias.float()).to(dtype)
+        d = og.gemm(qg, qw, og.decode_scale(sg), og.decode_scale(sw), (1, 32), (32, 32)).to(dtype)
+        extra = dict(group_a=(1, 32), group_b=(32, 32))
+    else:
+        layer = _TensorLayer()
+        zero = torch.zeros(1)
+        sa, sb = ot.tensor_scale(a, zero, 0, limit=torch.finfo(formats[0]).max)[0], ot.tensor_scale(w, zero, 0, limit=torch.finfo(formats[1]).max)[0]
+        sg, sw = ot.tensor_scale(dy, zero, 0, limit=torch.finfo(formats[0]).max)[0], ot.tensor_scale(w2, zero, 0, limit=torch.finfo(formats[1]).max)[0]
+        qa, qb, qg, qw = ot.quantize(a, sa, formats[0]), ot.quantize(w, sb, formats[1]), ot.quantize(dy, sg, formats[0]), ot.quantize(w2, sw, formats[1])
+        z = ot.gemm(qa, qb, sa, sb, bias=bias, out_dtype=dtype)
+        d = ot.gemm(qg, qw, sg, sw, out_dtype=dtype)
+        extra = {}
+    out, aux, _ = mk.gemm(qa.cuda(), qb.cuda(), sa.cuda(), sb.cuda(), layer=layer, out_dtype=dtype, bias=bias.cuda(),
+                          activation=activation, save=True)
+    assert aux.shape == (m, 2 * h) and rel_l2(aux, z) < 4e-3
+    assert rel_l2(out, ol.gated_forward(aux.cpu()[:, :h], aux.cpu()[:, h:], activation).to(dtype)) < 4e-3
+    nosave, aux2, _ = mk.gemm(qa.cuda(), qb.cuda(), sa.cuda(), sb.cuda(), layer=layer, out_dtype=dtype, bias=bias.cuda(),
+                              activation=activation, save=False)
+    assert aux2.numel() == 0 and torch.equal(nosave, out)
+    dz, _, _ = mk.gemm(qg.cuda(), qw.cuda(), sg.cuda(), sw.cuda(), layer=layer, out_dtype=dtype, backward=True,
+                       activation=activation, aux=aux, **extra)
+    dg, du = ol.gated_backward(d, aux.cpu()[:, :h], aux.cpu()[:, h:], activation)
+    assert dz.shape == (m, 2 * h) and rel_l2(dz, torch.cat([dg, du], 1).to(dtype)) < 6e-3
+
+
 @pytest.mark.parametrize("activation", ["silu", "gelu", "relu"])
 def test_gated_elementwise(activation):
     from viola_amd.nn._gated_kernels import GatedActivation

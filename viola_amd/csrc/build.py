@@ -17,7 +17,7 @@ ARCH = "gfx950"
 # scale with an explicit fmaf.
 COMMON = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17", "-ffp-contract=off", "-fno-fast-math",
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
-SOURCES = ["quantize.hip", "gemm.hip", "gemm_fast.hip", "ns.hip", "ns_fast.hip", "optim.hip", "misc.hip", "tensor.hip"]
+SOURCES = ["quantize.hip", "gemm.hip", "gemm_fast.hip", "gemm_fast_tensor.hip", "gemm_fast_mx.hip", "ns.hip", "ns_fast.hip", "optim.hip", "misc.hip", "tensor.hip"]
 
 
 def hipcc():
@@ -51,7 +51,7 @@ def build(verbose=True, incremental=False):
             print(message, file=sys.stderr)
         return obj
 
-    with ThreadPoolExecutor(max_workers=min(6, len(SOURCES))) as pool:
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
         objects = list(pool.map(compile_one, SOURCES))
     link = [compiler, f"--offload-arch={ARCH}", "-shared", "-fPIC", *map(str, objects), "-o", str(LIBRARY)]
     result = subprocess.run(link, capture_output=True, text=True)

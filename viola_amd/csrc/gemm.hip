@@ -376,7 +376,7 @@ extern "C" int viola_tensor_gemm(const void* a, int a_dtype, const void* b, int 
     const dim3 grid((unsigned)gx, (unsigned)gy);
     const bool vec = k % 16 == 0 && k > 0 && aligned16(a) && aligned16(b);
     if (vec && n * k < (1ll << 31) && (int64_t)BM * k < (1ll << 31))
-        return launch_tensor_gemm_fast(p, a_dtype, b_dtype, bias_dtype, out_dtype, grid, stream);
+        return launch_tensor_gemm_fast(p, MODE_PLAIN, a_dtype, b_dtype, bias_dtype, out_dtype, grid, stream);
     // odd alignment: the generic kernel, which multiplies each 32-wide K group's sum by sa * sb as it goes
     return launch_out<MODE_PLAIN>(p, a_dtype, b_dtype, bias_dtype, out_dtype, false, false, grid, stream);
 }
@@ -401,7 +401,63 @@ extern "C" int viola_mx_gemm(const void* a, int a_dtype, const void* b, int b_dt
     p.sa = reinterpret_cast<const float*>(sa); p.sb = reinterpret_cast<const float*>(sb);
     p.bias = bias; p.out = out; p.m = m; p.n = n; p.k = k; p.lda = k; p.ldb = k; p.ldo = n;
     p.ldsa = k / 32; p.ldsb = k / 32; p.ar = ar; p.br = br; p.ak_shift = 5; p.bk_shift = 5;
-    return launch_mx_gemm_fast(p, a_dtype, b_dtype, bias_dtype, out_dtype, dim3((unsigned)gx, (unsigned)gy), stream);
+    return launch_mx_gemm_fast(p, MODE_PLAIN, a_dtype, b_dtype, bias_dtype, out_dtype, dim3((unsigned)gx, (unsigned)gy), stream);
+}
+
+// The gated projections of an MLP under the per-tensor recipes: viola_gated_gemm's epilogues behind
+// (acc * sa[0]) * sb[0].
+extern "C" int viola_tensor_gated_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,
+                                       int64_t m, int64_t h, int64_t k, const void* bias, int bias_dtype, void* aux, void* out,
+                                       int out_dtype, int activation, int backward, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_fp8(a_dtype) && viola_is_fp8(b_dtype) && viola_is_float(out_dtype));
+    VIOLA_CHECK_ARG(m >= 0 && h >= 0 && k >= 0 && k < (1ll << 30));
+    VIOLA_CHECK_ARG(activation >= VIOLA_SILU && activation <= VIOLA_RELU && (!bias || viola_is_float(bias_dtype)));
+    if (m == 0 || h == 0) return 0;
+    VIOLA_CHECK_ARG(out && sa && sb && (k == 0 || (a && b)) && (!backward || aux));
+    GemmArgs p = {};
+    p.a = static_cast<const uint8_t*>(a); p.b = static_cast<const uint8_t*>(b); p.sa = sa; p.sb = sb;
+    p.bias = backward ? nullptr : bias; p.out = out; p.aux = aux; p.m = m; p.n = h; p.k = k; p.lda = k; p.ldb = k;
+    p.ldo = backward ? 2 * h : h; p.activation = activation;
+    p.ldsa = 0; p.ldsb = 0; p.ar = 1 << 30; p.br = 1 << 30; p.ak_shift = 30; p.bk_shift = 30;
+    const int64_t gy = (m + BM - 1) / BM;
+    VIOLA_CHECK_ARG(gy <= 65535);
+    const int mode = backward ? MODE_GATED_BWD : MODE_GATED_FWD;
+    const int64_t width = backward ? BN : BN / 2;
+    const dim3 grid((unsigned)((h + width - 1) / width), (unsigned)gy);
+    const bool vec = k % 16 == 0 && k > 0 && aligned16(a) && aligned16(b);
+    if (vec && 2 * h * k < (1ll << 31) && (int64_t)BM * k < (1ll << 31))
+        return launch_tensor_gemm_fast(p, mode, a_dtype, b_dtype, bias_dtype, out_dtype, grid, stream);
+    if (backward) return launch_out<MODE_GATED_BWD>(p, a_dtype, b_dtype, bias_dtype, out_dtype, false, false, grid, stream);
+    return launch_out<MODE_GATED_FWD>(p, a_dtype, b_dtype, bias_dtype, out_dtype, false, false, grid, stream);
+}
+
+// The same under E8M0 block scales; VIOLA_EUNSUPPORTED where viola_mx_gemm returns it, and when the up rows of b do
+// not start on a scale-row boundary (h not a multiple of br).
+extern "C" int viola_mx_gated_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const uint8_t* sa, const uint8_t* sb,
+                                   int64_t m, int64_t h, int64_t k, int ar, int br, const void* bias, int bias_dtype, void* aux,
+                                   void* out, int out_dtype, int activation, int backward, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_fp8(a_dtype) && viola_is_fp8(b_dtype) && viola_is_float(out_dtype));
+    VIOLA_CHECK_ARG(m >= 0 && h >= 0 && k >= 0 && ar > 0 && br > 0);
+    VIOLA_CHECK_ARG(activation >= VIOLA_SILU && activation <= VIOLA_RELU && (!bias || viola_is_float(bias_dtype)));
+    if (m == 0 || h == 0) return 0;
+    VIOLA_CHECK_ARG(out && (k == 0 || (a && b && sa && sb)) && (!backward || aux));
+    const int64_t gy = (m + BM - 1) / BM;
+    VIOLA_CHECK_ARG(gy <= 65535);
+    if (k == 0 || k % 128 != 0 || !aligned16(a) || !aligned16(b) || reinterpret_cast<uintptr_t>(sa) % 4 != 0 ||
+        reinterpret_cast<uintptr_t>(sb) % 4 != 0 || 2 * h * k >= (1ll << 31) || (int64_t)BM * k >= (1ll << 31) ||
+        (br != 1 && br % 32 != 0) || (!backward && h % br != 0))
+        return VIOLA_EUNSUPPORTED;
+    GemmArgs p = {};
+    p.a = static_cast<const uint8_t*>(a); p.b = static_cast<const uint8_t*>(b);
+    p.sa = reinterpret_cast<const float*>(sa); p.sb = reinterpret_cast<const float*>(sb);
+    p.bias = backward ? nullptr : bias; p.out = out; p.aux = aux; p.m = m; p.n = h; p.k = k; p.lda = k; p.ldb = k;
+    p.ldo = backward ? 2 * h : h; p.activation = activation;
+    p.ldsa = k / 32; p.ldsb = k / 32; p.ar = ar; p.br = br; p.ak_shift = 5; p.bk_shift = 5;
+    const int64_t width = backward ? BN : BN / 2;
+    return launch_mx_gemm_fast(p, backward ? MODE_GATED_BWD : MODE_GATED_FWD, a_dtype, b_dtype, bias_dtype, out_dtype,
+                               dim3((unsigned)((h + width - 1) / width), (unsigned)gy), stream);
 }
 
 extern "C" int viola_gated_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,

@@ -32,12 +32,13 @@ struct GemmArgs {
 int launch_group_gemm_fast(const GemmArgs& p, int mode, int a_dtype, int b_dtype, int bias_dtype, int out_dtype,
                            bool rowscale, dim3 grid, hipStream_t stream);
 
-// Per-tensor scales on the same fast kernel (one v_mfma_f32_32x32x64_f8f6f4 per sub-tile and 64 k). Defined in gemm_fast.hip.
-int launch_tensor_gemm_fast(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, dim3 grid,
+// Per-tensor scales on the same fast kernel (one v_mfma_f32_32x32x64_f8f6f4 per sub-tile and 64 k); mode = MODE_PLAIN or a
+// gated mode (grid.x then counts the gated tile width). Defined in gemm_fast.hip.
+int launch_tensor_gemm_fast(const GemmArgs& p, int mode, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, dim3 grid,
                             hipStream_t stream);
 
 // E8M0 block scales applied by v_mfma_scale_f32_32x32x64_f8f6f4 (k a multiple of 128). Defined in gemm_fast.hip.
-int launch_mx_gemm_fast(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, dim3 grid,
+int launch_mx_gemm_fast(const GemmArgs& p, int mode, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, dim3 grid,
                         hipStream_t stream);
 
 }  // namespace viola

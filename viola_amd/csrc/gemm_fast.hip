@@ -1,664 +1,9 @@
-// Fast path of the grouped-scale FP8 GEMM for gfx950 (see gemm.hip for the contract and the operand
-// orientation). Requires 16-byte aligned operand rows and k ranges that are multiples of 16.
-//
-// Block: 256 threads = 2 x 2 wavefronts, tile 128 (m) x 128 (b rows), 64 k per LDS stage; a wavefront owns
-// 2 x 2 sub-tiles of 32 x 32. Two blocks share a CU, so one block's prologue, barrier and output stores
-// run under the other block's math.
-//   * global -> LDS directly (buffer_load ... lds, no staging registers, lanes past the k range read
-//     zero), a ring of three stages, one barrier per chunk. During the math of chunk c a wave reads the
-//     MFMA operands of chunk c+1 from LDS into a second register set and issues the loads of chunk c+3,
-//     one instruction every few MFMAs, into the stage chunk c has vacated. Operand rows are 4 x 16 bytes, piece u = 2 * (K group) + half stored in slot
-//     u ^ ((row >> 2) & 3), which spreads the 16 rows of a ds_read_b128 group over all banks. A lane
-//     takes 16 consecutive bytes of a 32-byte K group (half = lane / 32): the first 8 feed the first
-//     MFMA of the group, the last 8 the second -- a and b use the same split, so every product meets its
-//     partner. The scales come in blocks of 8 K groups (32 bytes per row, so a scale row's cache
-//     line is touched once per 256 k) and are rearranged in LDS to [group][row].
-//   * math per (K group, sub-tile): 2 x v_mfma_f32_32x32x16 into one of two 16-register accumulators,
-//     then total += acc * (sa * sb), one FMA per output element, issued between the MFMAs of the next
-//     sub-tile so the matrix pipe and the VALU run together inside a wavefront as well as across the
-//     two wavefronts of a SIMD. The last fold of a chunk rides into the next chunk (uniform b scales;
-//     with row-wise b scales, which live in registers per chunk, that fold stays in its own chunk).
-//   * epilogue stores runs of four consecutive n as one 8- or 16-byte store.
-#include "gemm_args.hpp"
+// Grouped FP32-scale instances of the fast FP8 GEMM kernel (plain, gated forward, gated backward; uniform or
+// row-wise b scales).
+#include "gemm_fast_kernel.hpp"
 
 namespace viola {
 
-typedef int i32x4 __attribute__((ext_vector_type(4)));
-
-constexpr int FBK = 64, FKG = FBK / 32;                           // k bytes and K groups per LDS stage
-constexpr int FTHREADS = 256, FSTAGES = 3;
-constexpr int F_TILE = BM * FBK;                                  // bytes of one operand tile
-constexpr int F_STAGE = 2 * F_TILE;
-// Scales travel in blocks of 8 K groups (4 chunks): 32 bytes per row and operand, fetched as two 16-byte pieces
-// ("raw", piece = 4 groups of one row) and then rearranged in LDS to [group][row] floats, double-buffered.
-constexpr int F_SGROUPS = 8, F_SCHUNKS = F_SGROUPS / FKG;
-constexpr int F_SBLOCK = F_SGROUPS * BM * 4;                      // bytes of one operand's scale block
-constexpr int F_RAW = FSTAGES * F_STAGE;                          // raw a block, raw b block
-constexpr int F_SCALE = F_RAW + 2 * F_SBLOCK;                     // [buffer][operand][group][row]
-constexpr int F_LDS = F_SCALE + 4 * F_SBLOCK;
-
-// 64 lanes x 16 (or 4) bytes from a raw buffer straight into LDS at lds_addr + 16 (4) * lane. The compiler
-// is not told that these touch LDS (it would drain every outstanding load before each LDS read); the kernel
-// orders them against its LDS reads with s_waitcnt vmcnt + barrier itself.
-__device__ __forceinline__ void load16_to_lds(i32x4 rsrc, uint32_t lds_addr, uint32_t voffset, uint32_t soffset) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                 :: "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
-}
-__device__ __forceinline__ i32x4 raw_resource(const void* base, int64_t bytes = 0x7fffffff) {
-    const uint64_t address = reinterpret_cast<uint64_t>(base);
-    i32x4 r = {__builtin_amdgcn_readfirstlane((int)(uint32_t)address), __builtin_amdgcn_readfirstlane((int)(uint32_t)(address >> 32)),
-               __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000};
-    return r;
-}
-
-template <bool A_BF8, bool B_BF8>
-__device__ __forceinline__ f32x16 mfma32(long x, long y, f32x16 c) {
-    // x: 8 codes of the b matrix (MFMA srcA), y: 8 codes of the a matrix (MFMA srcB)
-    if constexpr (!B_BF8 && !A_BF8) return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(x, y, c, 0, 0, 0);
-    else if constexpr (!B_BF8 && A_BF8) return __builtin_amdgcn_mfma_f32_32x32x16_fp8_bf8(x, y, c, 0, 0, 0);
-    else if constexpr (B_BF8 && !A_BF8) return __builtin_amdgcn_mfma_f32_32x32x16_bf8_fp8(x, y, c, 0, 0, 0);
-    else return __builtin_amdgcn_mfma_f32_32x32x16_bf8_bf8(x, y, c, 0, 0, 0);
-}
-
-__device__ __forceinline__ float load_bias(const void* p, int64_t i, int dtype) {
-    if (dtype == VIOLA_F32) return static_cast<const float*>(p)[i];
-    if (dtype == VIOLA_BF16) return bf16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
-    return (float)static_cast<const _Float16*>(p)[i];
-}
-
-__device__ __forceinline__ void gate_math(int activation, float g, float& act, float& derivative) {
-    if (activation == VIOLA_SILU) {
-        const float s = 1.0f / (1.0f + expf(-g));
-        act = g * s;
-        derivative = s * (1.0f + g * (1.0f - s));
-    } else if (activation == VIOLA_GELU) {
-        const float t = tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g));
-        act = 0.5f * g * (1.0f + t);
-        derivative = 0.5f * (1.0f + t) + 0.5f * g * (1.0f - t * t) * 0.7978845608028654f * (1.0f + 0.134145f * g * g);
-    } else {
-        act = fmaxf(g, 0.0f);
-        derivative = g > 0.0f ? 1.0f : 0.0f;
-    }
-}
-
-// Four consecutive outputs of one row.
-template <typename TO> struct Quad;
-template <> struct Quad<float> {
-    static __device__ __forceinline__ void store(float* p, const float (&v)[4]) { *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]); }
-    static __device__ __forceinline__ void load(const float* p, float (&v)[4]) { const float4 t = *reinterpret_cast<const float4*>(p); v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w; }
-};
-template <> struct Quad<bf16_t> {
-    static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[4]) {
-        *reinterpret_cast<uint2*>(p) = make_uint2(f32_to_bf16x2_bits(v[0], v[1]), f32_to_bf16x2_bits(v[2], v[3]));
-    }
-    static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[4]) {
-        const uint2 t = *reinterpret_cast<const uint2*>(p);
-        v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
-        v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
-    }
-};
-template <> struct Quad<f16_t> {
-    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
-    static __device__ __forceinline__ void store(f16_t* p, const float (&v)[4]) {
-        h4 t = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
-        *reinterpret_cast<h4*>(p) = t;
-    }
-    static __device__ __forceinline__ void load(const f16_t* p, float (&v)[4]) {
-        const h4 t = *reinterpret_cast<const h4*>(p);
-        v[0] = (float)t[0]; v[1] = (float)t[1]; v[2] = (float)t[2]; v[3] = (float)t[3];
-    }
-};
-
-template <typename TO> __device__ __forceinline__ float rounded(float v) { return to_f32(from_f32<TO>(v)); }
-
-// TN: 32-column sub-tiles per wave; TN = 1 halves the tile to 128 x 64 for problems with too few 128 x 128 tiles to
-// give every CU two blocks (plain mode only).
-// TENSOR: one scale per operand (p.sa[0], p.sb[0]) applied to the finished sums, out = (acc * sa) * sb + bias: no
-// per-group fold, so a chunk's 64 k go through one v_mfma_f32_32x32x64_f8f6f4 per sub-tile straight into the totals.
-typedef int i32x8 __attribute__((ext_vector_type(8)));
-// MX: E8M0 scales (one byte per 32 k; p.sa / p.sb point at bytes, ldsa / ldsb are bytes per scale row) applied by the
-// hardware inside v_mfma_scale_f32_32x32x64_f8f6f4. The instruction's first 32-k block is operand registers 0..3 of all
-// 64 lanes and takes its scale from lanes 0..31 (one byte per row), the second block is registers 4..7 with the scale
-// of lanes 32..63 (measured: a scale change confined to one K group only gives the right product in this arrangement).
-// That is the layout the per-tensor path already has (registers 0..3 = the lane's 16 bytes of K group 0, 4..7 = of K
-// group 1), so lane (row, half) hands over the scale byte of K group `half` of its row. Scales travel in blocks of 16
-// K groups (one 16-byte piece per tile row and operand), double-buffered behind the ring; k must be a multiple of 128.
-constexpr int MX_GROUPS = 16, MX_CHUNKS = MX_GROUPS / FKG, MX_BLOCK = 2 * BM * MX_GROUPS;   // bytes of one block, a then b
-template <int MODE, bool A_BF8, bool B_BF8, bool B_ROWSCALE, typename TO, int TN, bool TENSOR = false, bool MX = false>
-__global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(GemmArgs p, int bias_dtype) {
-    static_assert(!TENSOR || (MODE == MODE_PLAIN && !B_ROWSCALE), "per-tensor scaling: plain mode only");
-    static_assert(!MX || (MODE == MODE_PLAIN && !TENSOR), "block-scaled MFMA: plain mode only");
-    constexpr bool NOFOLD = TENSOR || MX;                                   // the products of a chunk go straight into the totals
-    // without scale blocks the ring plus the epilogue's bias row is all the LDS a block needs: three blocks share a CU
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[TENSOR ? F_RAW + 1024 : MX ? F_RAW + 2 * MX_BLOCK : F_LDS];
-
-    // wave grid 2 (m) x 2 (n), 2 x 2 sub-tiles each. Plain / gated backward: sub-tile i of wave wn covers b rows
-    // 64 wn + 32 i. Gated forward: the tile's b rows are 64 gate rows then the 64 up rows of the same n, and
-    // i = 0 / 1 is the gate / up sub-tile of columns 32 wn .. 32 wn + 31, so one lane holds g and u of the same n.
-    constexpr bool GATED = MODE == MODE_GATED_FWD;
-    constexpr int TM = 2;
-    constexpr int PANEL = GATED ? BN / 2 : 64 * TN;
-    static_assert(!GATED || TN == 2, "gated forward pairs a gate and an up sub-tile");
-    const int tid = threadIdx.x, lane = tid % WAVE;
-    const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
-    const int wm = wave / 2, wn = wave % 2;
-    const int l32 = lane % 32, lhi = lane / 32;
-
-    // ---- which problem / tile (uniform per block)
-    // Workgroups are dealt round-robin to the 8 XCDs (block i -> XCD i % 8), each with its own L2. Give every XCD a
-    // contiguous range of output tiles, walked in groups of 8 m tiles x all n tiles (n slowest inside a group), so the
-    // blocks resident on one XCD at a time share a few rows of a and b.
-    int tile_m = blockIdx.y, tile_n = blockIdx.x;
-    if (p.tiles_m) {
-        const int per_xcd = gridDim.x / 8;
-        const int t = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-        if (t >= p.tiles_m * p.tiles_n) return;
-        const int group = 8 * p.tiles_n;
-        const int first_m = t / group * 8;
-        const int rows = p.tiles_m - first_m < 8 ? p.tiles_m - first_m : 8;
-        tile_m = first_m + t % group % rows;
-        tile_n = t % group / rows;
-    }
-    int64_t m_begin = (int64_t)tile_m * BM, m_end = p.m;
-    int64_t k_begin = 0, k_end = p.k;
-    const uint8_t* bptr = p.b;
-    const float* sbptr = p.sb;
-    uint8_t* outptr = static_cast<uint8_t*>(p.out);
-    if (p.offsets) {
-        int64_t tile = tile_m;
-        int g = 0;
-        bool found = false;
-        for (; g < p.groups; ++g) {
-            const int64_t lo = p.offsets[g], hi = p.offsets[g + 1];
-            const int64_t tiles = (hi - lo + BM - 1) / BM;
-            if (tile < tiles) { m_begin = lo + tile * BM; m_end = hi; found = true; break; }
-            tile -= tiles;
-        }
-        if (!found) return;
-        bptr += (int64_t)g * p.b_group_stride;
-        sbptr += (int64_t)g * p.sb_group_stride;
-    }
-    if (p.koffsets) {
-        const int g = blockIdx.z;
-        k_begin = p.koffsets[g];
-        k_end = p.koffsets[g + 1];
-        outptr += (int64_t)g * p.out_group_stride * (int64_t)sizeof(TO);
-    }
-    if (m_begin >= m_end) return;
-    const int64_t n_begin = (int64_t)tile_n * PANEL;
-    const int64_t b_rows_total = GATED ? 2 * p.n : p.n;
-    auto b_global_row = [&](int r) -> int64_t {                               // tile-local b row -> row of b
-        int64_t bn;
-        if constexpr (GATED) bn = (int64_t)(r / PANEL) * p.n + n_begin + r % PANEL;
-        else bn = n_begin + r;
-        return bn < b_rows_total ? bn : b_rows_total - 1;
-    };
-    auto a_global_row = [&](int r) -> int64_t {                               // rows past the end repeat the last row
-        const int64_t am = m_begin + r;
-        return am < m_end ? am : m_end - 1;
-    };
-
-    // ---- load plan. Instruction `it` of this wave fills 16-byte LDS units [it * 256 + wave * 64, +64) of an operand
-    // tile: unit U = 4 * row + slot holds piece (slot ^ ((row >> 2) & 3)) of the row's 64 k bytes.
-    const i32x4 res_a = raw_resource(p.a + m_begin * p.lda + k_begin);
-    const i32x4 res_b = raw_resource(bptr + k_begin);
-    // scale buffers carry their true size: a 16-byte piece may reach past the last row, and must then read zero
-    const i32x4 res_sa = raw_resource(p.sa, (p.m + p.ar - 1) / p.ar * p.ldsa * 4);
-    const i32x4 res_sb = raw_resource(sbptr, (b_rows_total + p.br - 1) / p.br * p.ldsb * 4);
-    constexpr uint32_t OUTSIDE = 0x80000000u;
-    uint32_t goff_a[2], goff_b[2];
-    int piece_k[2];
-#pragma unroll
-    for (int it = 0; it < 2; ++it) {
-        const int unit = it * 256 + tid, r = unit >> 2, piece = (unit & 3) ^ ((r >> 2) & 3);
-        goff_a[it] = (uint32_t)((a_global_row(r) - m_begin) * p.lda + piece * 16);
-        goff_b[it] = (uint32_t)(b_global_row(r) * p.ldb + piece * 16);        // relative to bptr + k_begin (row span < 2 GiB)
-        piece_k[it] = piece * 16;
-    }
-    // scales: per block of 8 K groups the thread fetches groups 4 shalf .. 4 shalf + 3 of tile row srow
-    const int srow = tid % BM, shalf = tid / BM;
-    const uint32_t sa_off = (uint32_t)(a_global_row(srow) / p.ar * p.ldsa * 4 + ((k_begin >> 5) + shalf * 4) * 4);
-    const uint32_t sb_off = (uint32_t)(b_global_row(srow) / p.br * p.ldsb * 4 + ((k_begin >> 5) + shalf * 4) * 4);
-    constexpr int B_LOADS = TN;                                              // 64 b rows per load instruction
-    const int64_t k_len = k_end - k_begin;
-    const int groups_total = (int)((k_len + 31) / 32);
-    const int64_t chunks = (k_len + FBK - 1) / FBK;
-    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
-    // load instruction `which` (0, 1: a; 2, 3: b) of chunk c into ring stage `stage`
-    auto issue_one = [&](int64_t c, int stage, int which) {
-        const int64_t k0 = c * FBK;                                          // relative to k_begin
-        const uint32_t base = lds_base + (uint32_t)stage * F_STAGE + (uint32_t)wave * 1024;
-        const int it = which & 1;
-        const bool inside = k0 + piece_k[it] < k_len;
-        if (which < 2) load16_to_lds(res_a, base + it * 4096, inside ? goff_a[it] : OUTSIDE, (uint32_t)k0);
-        else load16_to_lds(res_b, base + F_TILE + it * 4096, inside ? goff_b[it] : OUTSIDE, (uint32_t)k0);
-    };
-    constexpr int CHUNK_LOADS = 2 + B_LOADS;
-    auto issue = [&](int64_t c, int stage) {
-#pragma unroll
-        for (int i = 0; i < CHUNK_LOADS; ++i) issue_one(c, stage, i);
-    };
-    // scale block `block` (K groups 8 block .. 8 block + 7 of the k range) -> raw area, one 16-byte piece per thread
-    // and operand; a piece wholly past the k range is not fetched
-    auto issue_scales = [&](int64_t block) {
-        const bool inside = block * F_SGROUPS + shalf * 4 < groups_total;
-        const uint32_t at = lds_base + F_RAW + (uint32_t)wave * 1024;
-        load16_to_lds(res_sa, at, inside ? sa_off : OUTSIDE, (uint32_t)(block * F_SGROUPS * 4));
-        load16_to_lds(res_sb, at + F_SBLOCK, inside ? sb_off : OUTSIDE, (uint32_t)(block * F_SGROUPS * 4));
-    };
-    // MX: scale block `block` (K groups 16 block ..) -> buffer block & 1: waves 0, 1 fetch the a rows' pieces, waves 2, 3 the b rows'
-    const i32x4 res_mxa = raw_resource(p.sa, (p.m + p.ar - 1) / p.ar * p.ldsa);
-    const i32x4 res_mxb = raw_resource(sbptr, (b_rows_total + p.br - 1) / p.br * p.ldsb);
-    const uint32_t mx_off = tid < BM ? (uint32_t)(a_global_row(tid) / p.ar * p.ldsa + (k_begin >> 5))
-                                     : (uint32_t)(b_global_row(tid - BM) / p.br * p.ldsb + (k_begin >> 5));
-    auto issue_mx_scales = [&](int64_t block) {
-        const bool inside = block * MX_GROUPS < groups_total;
-        const uint32_t at = lds_base + F_RAW + (uint32_t)(block & 1) * MX_BLOCK + (uint32_t)wave * 1024;
-        load16_to_lds(wave < 2 ? res_mxa : res_mxb, at, inside ? mx_off : OUTSIDE, (uint32_t)(block * MX_GROUPS));
-    };
-    // raw area -> [group][row] floats of scale buffer `block & 1`; groups past the k range become zero (their
-    // products are zero too, and a neighbouring row's value must not meet them)
-    auto arrange_scales = [&](int64_t block) {
-        const float4 va = *reinterpret_cast<const float4*>(lds + F_RAW + tid * 16);
-        const float4 vb = *reinterpret_cast<const float4*>(lds + F_RAW + F_SBLOCK + tid * 16);
-        float* ta = reinterpret_cast<float*>(lds + F_SCALE + (block & 1) * 2 * F_SBLOCK);
-        float* tb = ta + F_SBLOCK / 4;
-        const int left = groups_total - (int)(block * F_SGROUPS + shalf * 4);
-        const float a4[4] = {va.x, va.y, va.z, va.w}, b4[4] = {vb.x, vb.y, vb.z, vb.w};
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            ta[(shalf * 4 + q) * BM + srow] = q < left ? a4[q] : 0.0f;
-            tb[(shalf * 4 + q) * BM + srow] = q < left ? b4[q] : 0.0f;
-        }
-    };
-
-    // ---- MFMA operand reads: 16 bytes = this lane's half (lhi) of K group kg for row l32 of a sub-tile
-    auto a_sub = [&](int j) -> int { return (wm * TM + j) * 32; };
-    auto b_sub = [&](int i) -> int { return GATED ? i * PANEL + wn * 32 : (wn * TN + i) * 32; };
-    const int sw = (l32 >> 2) & 3;
-    const int rd_a = (a_sub(0) + l32) * FBK + ((lhi ^ sw) * 16);             // K group 1: ^ 32
-    const int rd_b = (b_sub(0) + l32) * FBK + ((lhi ^ sw) * 16);
-
-    f32x16 total[TN][TM];                                                    // [b sub-tile i][a sub-tile j]
-#pragma unroll
-    for (int i = 0; i < TN; ++i)
-#pragma unroll
-        for (int j = 0; j < TM; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) total[i][j][r] = 0.0f;
-
-    // Four 16-register accumulators: two receive the MFMAs of the current pair of (K group, sub-tile) units while the
-    // two of the pair before are folded into the totals (across chunk boundaries when CARRY).
-    constexpr bool CARRY = !B_ROWSCALE;
-    f32x16 acc[4];
-    float pending_scale[2] = {0.0f, 0.0f};                                   // sa * sb of the pending pair (uniform b scales)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[0][r] = acc[1][r] = acc[2][r] = acc[3][r] = 0.0f;
-    auto as_long = [](uint32_t lo, uint32_t hi) -> long { return (long)(((uint64_t)hi << 32) | lo); };
-
-    // The MFMA operands and scales of one chunk, in registers. They are read from LDS one chunk ahead of their
-    // math (two register sets, the chunk loop is unrolled by two), so a wavefront goes from the barrier straight
-    // into its math and the LDS latency of the next chunk hides under it.
-    struct Operands {
-        uint4 a[FKG][TM], b[FKG][TN];
-        float sa[FKG][TM], sb[FKG][TN];
-        i32x8 wide_a[TM], wide_b[TN];                                        // TENSOR / MX: 16 k of either K group of a sub-tile row
-        int mx_a[TM], mx_b[TN];                                              // MX: the row's scale byte of K group lhi
-    };
-    auto scale_block = [&](int64_t c) -> const float* {                      // a scales of chunk c: [kg][row]; b scales F_SBLOCK later
-        return reinterpret_cast<const float*>(lds + F_SCALE + ((c / F_SCHUNKS) & 1) * 2 * F_SBLOCK) + (c % F_SCHUNKS) * FKG * BM;
-    };
-    auto read_operands = [&](int stage, int64_t c, Operands& o) {
-        const uint8_t* tile_a = lds + stage * F_STAGE;
-        const uint8_t* tile_b = tile_a + F_TILE;
-        const float* scale_a = scale_block(c);
-        const float* scale_b = scale_a + F_SBLOCK / 4;
-        if constexpr (NOFOLD) {
-            // the lane's 16 bytes of either K group (slots lhi and lhi + 2)
-            const int first_a = rd_a, first_b = rd_b;
-            constexpr int SECOND = 32;
-#pragma unroll
-            for (int j = 0; j < TM; ++j) {
-                const i32x4 lo = *reinterpret_cast<const i32x4*>(tile_a + (first_a + j * 32 * FBK));
-                const i32x4 hi = *reinterpret_cast<const i32x4*>(tile_a + ((first_a + j * 32 * FBK) ^ SECOND));
-                o.wide_a[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            }
-#pragma unroll
-            for (int i = 0; i < TN; ++i) {
-                const i32x4 lo = *reinterpret_cast<const i32x4*>(tile_b + (first_b + (b_sub(i) - b_sub(0)) * FBK));
-                const i32x4 hi = *reinterpret_cast<const i32x4*>(tile_b + ((first_b + (b_sub(i) - b_sub(0)) * FBK) ^ SECOND));
-                o.wide_b[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            }
-            if constexpr (MX) {
-                const uint8_t* block = lds + F_RAW + ((c / MX_CHUNKS) & 1) * MX_BLOCK + (c % MX_CHUNKS) * FKG + lhi;
-#pragma unroll
-                for (int j = 0; j < TM; ++j) o.mx_a[j] = block[(a_sub(j) + l32) * MX_GROUPS];
-#pragma unroll
-                for (int i = 0; i < TN; ++i) o.mx_b[i] = block[BM * MX_GROUPS + (b_sub(i) + l32) * MX_GROUPS];
-            }
-            return;
-        }
-#pragma unroll
-        for (int kg = 0; kg < FKG; ++kg) {
-#pragma unroll
-            for (int j = 0; j < TM; ++j) o.a[kg][j] = *reinterpret_cast<const uint4*>(tile_a + ((rd_a + j * 32 * FBK) ^ (kg * 32)));
-#pragma unroll
-            for (int i = 0; i < TN; ++i) o.b[kg][i] = *reinterpret_cast<const uint4*>(tile_b + ((rd_b + (b_sub(i) - b_sub(0)) * FBK) ^ (kg * 32)));
-#pragma unroll
-            for (int j = 0; j < TM; ++j) o.sa[kg][j] = scale_a[kg * BM + a_sub(j) + l32];
-#pragma unroll
-            for (int i = 0; i < TN; ++i) o.sb[kg][i] = B_ROWSCALE ? 0.0f : scale_b[kg * BM + b_sub(i)];
-        }
-    };
-
-    // Math of chunk c on the operands in `o`; `between(step)` runs after MFMA number `step` of the chunk (the
-    // caller's global loads and LDS reads for later chunks go there, spread over the chunk).
-    auto compute = [&](const Operands& o, int64_t c, auto&& between) {
-        if constexpr (NOFOLD) {
-            constexpr int STEPS_PER = FKG * 2;
-#pragma unroll
-            for (int i = 0; i < TN; ++i) {
-#pragma unroll
-                for (int j = 0; j < TM; ++j) {
-                    // both operands give a lane the same 32 of the chunk's 64 k (16 of each K group), so every product
-                    // meets its partner whatever order the instruction walks them in
-                    if constexpr (MX)
-                        total[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(o.wide_b[i], o.wide_a[j], total[i][j], B_BF8 ? 1 : 0, A_BF8 ? 1 : 0, 0, o.mx_b[i], 0, o.mx_a[j]);
-                    else
-                        total[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(o.wide_b[i], o.wide_a[j], total[i][j], B_BF8 ? 1 : 0, A_BF8 ? 1 : 0, 0, 0, 0, 0);
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int step = 0; step < STEPS_PER; ++step) between((i * TM + j) * STEPS_PER + step);
-                }
-            }
-            return;
-        }
-        // row-wise b scales of the lane's 16 columns for one pair of units (both share K group and b sub-tile): two
-        // slots, pair p loads slot p & 1 before its MFMAs and its fold reads it during pair p + 1
-        float4 sb_q[2][4];
-        const float* scale_b = scale_block(c) + F_SBLOCK / 4;
-        // fold half `h` (registers 8h .. 8h+7) of accumulator `buf` into total[i][j]
-        auto fold_half = [&](int buf, int i, int j, int slot, int h, float scale) {
-#pragma unroll
-            for (int r = 8 * h; r < 8 * h + 8; ++r) {
-                if constexpr (!B_ROWSCALE) {
-                    total[i][j][r] = fmaf(acc[buf][r], scale, total[i][j][r]);
-                } else {
-                    const float4 q = sb_q[slot][r / 4];
-                    const float sbv = r % 4 == 0 ? q.x : r % 4 == 1 ? q.y : r % 4 == 2 ? q.z : q.w;
-                    total[i][j][r] = fmaf(acc[buf][r], scale * sbv, total[i][j][r]);
-                }
-            }
-        };
-        const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        // Units go in pairs: the four MFMAs of a pair alternate between its two accumulators, so an MFMA never waits
-        // for the one issued just before it, and a quarter of the previous pair's fold follows each of them.
-        constexpr int UNITS = FKG * TN * TM, PAIRS = UNITS / 2;
-#pragma unroll
-        for (int pair = 0; pair < PAIRS; ++pair) {
-            const int base = (pair & 1) * 2, other = base ^ 2;
-            const int before = (pair + PAIRS - 1) % PAIRS;                   // the pair folded now (last of the chunk before for pair 0)
-            const bool fold_prev = pair > 0 || CARRY;
-            int kg[2], ti[2], tj[2], pkg[2], pi[2], pj[2];
-            float prev_scale[2];
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const int unit = 2 * pair + h, prev = 2 * before + h;
-                kg[h] = unit / (TN * TM); ti[h] = unit / TM % TN; tj[h] = unit % TM;
-                pkg[h] = prev / (TN * TM); pi[h] = prev / TM % TN; pj[h] = prev % TM;
-                prev_scale[h] = B_ROWSCALE ? (pair > 0 ? o.sa[pkg[h]][pj[h]] : 0.0f) : pending_scale[h];
-            }
-            if constexpr (B_ROWSCALE) {
-#pragma unroll
-                for (int r4 = 0; r4 < 4; ++r4)
-                    sb_q[pair & 1][r4] = *reinterpret_cast<const float4*>(&scale_b[kg[0] * BM + b_sub(ti[0]) + r4 * 8 + lhi * 4]);
-            }
-#pragma unroll
-            for (int step = 0; step < 4; ++step) {
-                const int h = step & 1, ks = step >> 1;
-                const uint4 ob = o.b[kg[h]][ti[h]], oa = o.a[kg[h]][tj[h]];
-                if (ks == 0) acc[base + h] = mfma32<A_BF8, B_BF8>(as_long(ob.x, ob.y), as_long(oa.x, oa.y), zero);
-                else acc[base + h] = mfma32<A_BF8, B_BF8>(as_long(ob.z, ob.w), as_long(oa.z, oa.w), acc[base + h]);
-                if (fold_prev) fold_half(other + (step >> 1), pi[step >> 1], pj[step >> 1], before & 1, step & 1, prev_scale[step >> 1]);
-                asm volatile("" : "+v"(total[pi[step >> 1]][pj[step >> 1]]));
-                __builtin_amdgcn_sched_barrier(0);
-                between(pair * 4 + step);
-            }
-            if constexpr (!B_ROWSCALE) {
-#pragma unroll
-                for (int h = 0; h < 2; ++h) pending_scale[h] = o.sa[kg[h]][tj[h]] * o.sb[kg[h]][ti[h]];
-            }
-        }
-        if constexpr (!CARRY) {
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                constexpr int last_pair = PAIRS - 1;
-                const int unit = 2 * last_pair + h;
-                const int lkg = unit / (TN * TM), li = unit / TM % TN, lj = unit % TM;
-                fold_half((last_pair & 1) * 2 + h, li, lj, last_pair & 1, 0, o.sa[lkg][lj]);
-                fold_half((last_pair & 1) * 2 + h, li, lj, last_pair & 1, 1, o.sa[lkg][lj]);
-            }
-        }
-    };
-
-    // Ring of three stages, chunk c in stage c % 3. At the top of iteration c the wave waits for its own loads of
-    // chunk c+1 (issued two iterations ago) and for its LDS reads of chunk c; after the barrier chunk c+1 is in LDS
-    // for everybody and nobody reads chunk c's stage any more. Then: the loads of chunk c+3 into that stage (one
-    // instruction every few MFMAs, so the waves of a CU do not queue up at the memory pipe), the LDS reads of chunk
-    // c+1 into the other register set, the math of chunk c. Scale block b (K groups 8b ..) is fetched in iteration
-    // 4b-4, rearranged in 4b-2 and first read in 4b-1; it is issued before the chunk loads of its iteration, so the
-    // waits below cover it one iteration later.
-    constexpr int STEPS = FKG * TN * TM * 2, STRIDE = STEPS / CHUNK_LOADS;
-    int stage_now = 0, stage_next = 1;
-    auto chunk_step = [&](int64_t c, const Operands& now, Operands& next) {
-        if (!NOFOLD && c % F_SCHUNKS == 1) __builtin_amdgcn_s_waitcnt(0x0070 | (CHUNK_LOADS + 2));
-        else if (MX && c % MX_CHUNKS == 1) __builtin_amdgcn_s_waitcnt(0x0070 | (CHUNK_LOADS + 1));
-        else __builtin_amdgcn_s_waitcnt(0x0070 | CHUNK_LOADS);
-        __syncthreads();
-        if constexpr (!NOFOLD) {
-            if (c % F_SCHUNKS == 0) issue_scales(c / F_SCHUNKS + 1);
-            if (c % F_SCHUNKS == 2) arrange_scales(c / F_SCHUNKS + 1);
-        }
-        if constexpr (MX) {
-            if (c % MX_CHUNKS == 0) issue_mx_scales(c / MX_CHUNKS + 1);
-        }
-        if (c + 1 < chunks) read_operands(stage_next, c + 1, next);
-        const int fill = stage_now;
-        compute(now, c, [&](int step) {
-            if (step % STRIDE == 0 && step / STRIDE < CHUNK_LOADS) issue_one(c + 3, fill, step / STRIDE);
-        });
-        stage_now = stage_next;
-        stage_next = stage_next == FSTAGES - 1 ? 0 : stage_next + 1;
-    };
-    if constexpr (MX) issue_mx_scales(0);
-    else if constexpr (!TENSOR) issue_scales(0);
-    issue(0, 0);
-    issue(1, 1);
-    issue(2, 2);
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * CHUNK_LOADS));                   // scale block 0 and chunk 0 are in LDS
-    __syncthreads();
-    if constexpr (!NOFOLD) {
-        arrange_scales(0);
-        __syncthreads();
-    }
-    Operands set0, set1;
-    read_operands(0, 0, set0);
-    for (int64_t c = 0; c < chunks; c += 2) {
-        chunk_step(c, set0, set1);
-        if (c + 1 < chunks) chunk_step(c + 1, set1, set0);
-    }
-    __builtin_amdgcn_s_waitcnt(0x0F70);     // drain the trailing loads before the LDS allocation is released
-    if constexpr (TENSOR) {
-        const float sa = p.sa[0], sb = p.sb[0];
-#pragma unroll
-        for (int i = 0; i < TN; ++i)
-#pragma unroll
-            for (int j = 0; j < TM; ++j)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) { const float t = total[i][j][r] * sa; total[i][j][r] = t * sb; }
-    } else if constexpr (CARRY && !MX) {
-        constexpr int UNITS = FKG * TN * TM, last_pair = UNITS / 2 - 1;
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int unit = 2 * last_pair + h, li = unit / TM % TN, lj = unit % TM;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) total[li][lj][r] = fmaf(acc[(last_pair & 1) * 2 + h][r], pending_scale[h], total[li][lj][r]);
-        }
-    }
-
-    // ---- epilogue: for sub-tiles (i, j) the lane holds row m = 32*j + l32 and, per register quad r4, columns
-    // n = 8*r4 + 4*lhi + 0..3
-    TO* out = reinterpret_cast<TO*>(outptr);
-    const bool vec_out = p.ldo % 4 == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
-    const bool vec_aux = p.n % 4 == 0 && (reinterpret_cast<uintptr_t>(p.aux) & 15) == 0;
-    if constexpr (MODE == MODE_PLAIN) {
-        // Row-major output: as stores, "one row per lane, four columns" would touch 32 cache lines per instruction. When
-        // rows of out are 16-byte aligned, each wavefront parks its finished values, 32 rows at a time, in LDS (the
-        // stage ring is free now) and stores them as 16-byte pieces along the rows instead.
-        constexpr int PER = 16 / (int)sizeof(TO);                            // values per piece
-        constexpr int WCOLS = 32 * TN, PLD = WCOLS + PER, PIECES = WCOLS / PER;
-        static_assert(4 * 32 * PLD * (int)sizeof(TO) <= F_RAW, "parking area fits in the stage ring");
-        if ((p.ldo * sizeof(TO)) % 16 == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
-            __syncthreads();                                                 // every wave has left the ring
-            TO* park = reinterpret_cast<TO*>(lds) + wave * 32 * PLD;
-            const int64_t ncol0 = n_begin + wn * WCOLS;
-            // the tile's bias as fp32 in the (now idle) raw scale area: one global load per column, not per element
-            float4 bias_q[TN][4];
-            if (p.bias) {
-                float* bias_lds = reinterpret_cast<float*>(lds + F_RAW);
-                if (tid < 64 * TN) bias_lds[tid] = n_begin + tid < p.n ? load_bias(p.bias, n_begin + tid, bias_dtype) : 0.0f;
-                __syncthreads();
-#pragma unroll
-                for (int i = 0; i < TN; ++i)
-#pragma unroll
-                    for (int r4 = 0; r4 < 4; ++r4) bias_q[i][r4] = *reinterpret_cast<const float4*>(&bias_lds[wn * WCOLS + i * 32 + r4 * 8 + lhi * 4]);
-            } else {
-#pragma unroll
-                for (int i = 0; i < TN; ++i)
-#pragma unroll
-                    for (int r4 = 0; r4 < 4; ++r4) bias_q[i][r4] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-            }
-#pragma unroll
-            for (int j = 0; j < TM; ++j) {
-#pragma unroll
-                for (int i = 0; i < TN; ++i)
-#pragma unroll
-                    for (int r4 = 0; r4 < 4; ++r4) {
-                        float v[4];
-                        const float bq[4] = {bias_q[i][r4].x, bias_q[i][r4].y, bias_q[i][r4].z, bias_q[i][r4].w};
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = total[i][j][r4 * 4 + e] + bq[e];
-                        Quad<TO>::store(&park[l32 * PLD + i * 32 + r4 * 8 + lhi * 4], v);
-                    }
-#pragma unroll
-                for (int it = 0; it < 32 * PIECES / WAVE; ++it) {
-                    const int id = it * WAVE + lane, pr = id / PIECES, pc = id % PIECES;
-                    const int64_t mrow = m_begin + a_sub(j) + pr, ncol = ncol0 + pc * PER;
-                    const uint4 piece = *reinterpret_cast<const uint4*>(&park[pr * PLD + pc * PER]);
-                    if (mrow >= m_end || ncol >= p.n) continue;
-                    if (ncol + PER <= p.n) {
-                        *reinterpret_cast<uint4*>(out + mrow * p.ldo + ncol) = piece;
-                    } else {
-                        const TO* values = reinterpret_cast<const TO*>(&piece);
-                        for (int e = 0; e < PER; ++e)
-                            if (ncol + e < p.n) out[mrow * p.ldo + ncol + e] = values[e];
-                    }
-                }
-            }
-            return;
-        }
-    }
-#pragma unroll
-    for (int j = 0; j < TM; ++j) {
-        const int64_t mrow = m_begin + a_sub(j) + l32;
-        if (mrow >= m_end) continue;
-#pragma unroll
-        for (int i = 0; i < (GATED ? 1 : TN); ++i)
-#pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-            const int64_t ncol = n_begin + (GATED ? wn * 32 : b_sub(i)) + r4 * 8 + lhi * 4;
-            if (ncol >= p.n) continue;
-            const bool full = ncol + 3 < p.n;
-            if constexpr (GATED) {
-                TO* aux = static_cast<TO*>(p.aux);
-                float gq[4], uq[4], h[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float gv = total[0][j][r4 * 4 + e], uv = total[1][j][r4 * 4 + e];
-                    if (p.bias && ncol + e < p.n) {
-                        gv += load_bias(p.bias, ncol + e, bias_dtype);
-                        uv += load_bias(p.bias, p.n + ncol + e, bias_dtype);
-                    }
-                    gq[e] = rounded<TO>(gv);
-                    uq[e] = rounded<TO>(uv);
-                    float act, derivative;
-                    gate_math(p.activation, gq[e], act, derivative);
-                    h[e] = act * uq[e];
-                }
-                if (full && vec_out) Quad<TO>::store(out + mrow * p.ldo + ncol, h);
-                else for (int e = 0; e < 4; ++e) if (ncol + e < p.n) out[mrow * p.ldo + ncol + e] = from_f32<TO>(h[e]);
-                if (aux) {
-                    if (full && vec_aux) {
-                        Quad<TO>::store(aux + mrow * 2 * p.n + ncol, gq);
-                        Quad<TO>::store(aux + mrow * 2 * p.n + p.n + ncol, uq);
-                    } else {
-                        for (int e = 0; e < 4; ++e)
-                            if (ncol + e < p.n) {
-                                aux[mrow * 2 * p.n + ncol + e] = from_f32<TO>(gq[e]);
-                                aux[mrow * 2 * p.n + p.n + ncol + e] = from_f32<TO>(uq[e]);
-                            }
-                    }
-                }
-            } else {
-                float v[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = total[i][j][r4 * 4 + e];
-                if constexpr (MODE == MODE_PLAIN) {
-                    if (p.bias) {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (ncol + e < p.n) v[e] += load_bias(p.bias, ncol + e, bias_dtype);
-                    }
-                    if (full && vec_out) Quad<TO>::store(out + mrow * p.ldo + ncol, v);
-                    else for (int e = 0; e < 4; ++e) if (ncol + e < p.n) out[mrow * p.ldo + ncol + e] = from_f32<TO>(v[e]);
-                } else {
-                    const TO* aux = static_cast<const TO*>(p.aux);
-                    float g[4] = {0, 0, 0, 0}, u[4] = {0, 0, 0, 0}, dg[4], du[4];
-                    if (full && vec_aux) {
-                        Quad<TO>::load(aux + mrow * 2 * p.n + ncol, g);
-                        Quad<TO>::load(aux + mrow * 2 * p.n + p.n + ncol, u);
-                    } else {
-                        for (int e = 0; e < 4; ++e)
-                            if (ncol + e < p.n) {
-                                g[e] = to_f32(aux[mrow * 2 * p.n + ncol + e]);
-                                u[e] = to_f32(aux[mrow * 2 * p.n + p.n + ncol + e]);
-                            }
-                    }
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const float d = rounded<TO>(v[e]);
-                        float act, derivative;
-                        gate_math(p.activation, g[e], act, derivative);
-                        dg[e] = d * u[e] * derivative;
-                        du[e] = d * act;
-                    }
-                    if (full && vec_out && vec_aux) {
-                        Quad<TO>::store(out + mrow * p.ldo + ncol, dg);
-                        Quad<TO>::store(out + mrow * p.ldo + p.n + ncol, du);
-                    } else {
-                        for (int e = 0; e < 4; ++e)
-                            if (ncol + e < p.n) {
-                                out[mrow * p.ldo + ncol + e] = from_f32<TO>(dg[e]);
-                                out[mrow * p.ldo + p.n + ncol + e] = from_f32<TO>(du[e]);
-                            }
-                    }
-                }
-            }
-        }
-    }
-}
-
-#ifndef VIOLA_GEMM_PROBE   // a probe build instantiates single kernels itself
 template <int MODE, bool B_ROWSCALE, typename TO, int TN>
 static void launch_formats(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, dim3 grid, hipStream_t stream) {
     const bool a5 = a_dtype == VIOLA_E5M2, b5 = b_dtype == VIOLA_E5M2;
@@ -684,72 +29,6 @@ static int launch_mode(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dty
     return viola_launch_status();
 }
 
-// Per-tensor scales (args.sa / args.sb point at one float each). grid: (n tiles of 128, m tiles of 128).
-template <typename TO, int TN>
-static void launch_tensor_formats(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, dim3 grid, hipStream_t stream) {
-    const bool a5 = a_dtype == VIOLA_E5M2, b5 = b_dtype == VIOLA_E5M2;
-    if (!a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE_PLAIN, false, false, false, TO, TN, true>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else if (a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE_PLAIN, true, false, false, TO, TN, true>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else if (!a5 && b5) hipLaunchKernelGGL((group_gemm_fast<MODE_PLAIN, false, true, false, TO, TN, true>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else hipLaunchKernelGGL((group_gemm_fast<MODE_PLAIN, true, true, false, TO, TN, true>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-}
-
-int launch_tensor_gemm_fast(const GemmArgs& args, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, dim3 grid,
-                            hipStream_t stream) {
-    GemmArgs p = args;
-    const bool narrow = (int64_t)grid.x * grid.y < 512 && p.n > 64;
-    if (narrow) grid.x = (unsigned)((p.n + 63) / 64);
-    if ((int64_t)grid.x * grid.y < (1 << 30)) {
-        p.tiles_n = (int)grid.x;
-        p.tiles_m = (int)grid.y;
-        grid = dim3((grid.x * grid.y + 7) / 8 * 8, 1, 1);
-    }
-#define VIOLA_TENSOR(TO)                                                                          \
-    if (narrow) launch_tensor_formats<TO, 1>(p, a_dtype, b_dtype, bias_dtype, grid, stream);      \
-    else launch_tensor_formats<TO, 2>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
-    switch (out_dtype) {
-        case VIOLA_F32: VIOLA_TENSOR(float) break;
-        case VIOLA_BF16: VIOLA_TENSOR(bf16_t) break;
-        case VIOLA_F16: VIOLA_TENSOR(f16_t) break;
-        default: return VIOLA_EINVAL;
-    }
-#undef VIOLA_TENSOR
-    return viola_launch_status();
-}
-
-// E8M0 block scales (args.sa / args.sb point at bytes; ldsa / ldsb = bytes per scale row). grid: (n tiles of 128, m tiles of 128).
-template <typename TO, int TN>
-static void launch_mx_formats(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, dim3 grid, hipStream_t stream) {
-    const bool a5 = a_dtype == VIOLA_E5M2, b5 = b_dtype == VIOLA_E5M2;
-    if (!a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE_PLAIN, false, false, false, TO, TN, false, true>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else if (a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE_PLAIN, true, false, false, TO, TN, false, true>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else if (!a5 && b5) hipLaunchKernelGGL((group_gemm_fast<MODE_PLAIN, false, true, false, TO, TN, false, true>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else hipLaunchKernelGGL((group_gemm_fast<MODE_PLAIN, true, true, false, TO, TN, false, true>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-}
-
-int launch_mx_gemm_fast(const GemmArgs& args, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, dim3 grid,
-                        hipStream_t stream) {
-    GemmArgs p = args;
-    const bool narrow = (int64_t)grid.x * grid.y < 512 && p.n > 64;
-    if (narrow) grid.x = (unsigned)((p.n + 63) / 64);
-    if ((int64_t)grid.x * grid.y < (1 << 30)) {
-        p.tiles_n = (int)grid.x;
-        p.tiles_m = (int)grid.y;
-        grid = dim3((grid.x * grid.y + 7) / 8 * 8, 1, 1);
-    }
-#define VIOLA_MX(TO)                                                                          \
-    if (narrow) launch_mx_formats<TO, 1>(p, a_dtype, b_dtype, bias_dtype, grid, stream);      \
-    else launch_mx_formats<TO, 2>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
-    switch (out_dtype) {
-        case VIOLA_F32: VIOLA_MX(float) break;
-        case VIOLA_BF16: VIOLA_MX(bf16_t) break;
-        case VIOLA_F16: VIOLA_MX(f16_t) break;
-        default: return VIOLA_EINVAL;
-    }
-#undef VIOLA_MX
-    return viola_launch_status();
-}
-
 int launch_group_gemm_fast(const GemmArgs& args, int mode, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, bool rowscale,
                            dim3 grid, hipStream_t stream) {
     GemmArgs p = args;
@@ -766,6 +45,5 @@ int launch_group_gemm_fast(const GemmArgs& args, int mode, int a_dtype, int b_dt
     if (mode == MODE_GATED_FWD) return launch_mode<MODE_GATED_FWD, 2>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
     return launch_mode<MODE_GATED_BWD, 2>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
 }
-#endif
 
 }  // namespace viola

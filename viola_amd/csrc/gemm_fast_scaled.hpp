@@ -1,0 +1,45 @@
+// Launchers of the fast FP8 GEMM kernel for the recipes whose scales need no per-group fold: per-tensor scales and
+// E8M0 block scales. Included by the one file that instantiates each.
+#pragma once
+#include "gemm_fast_kernel.hpp"
+
+namespace viola {
+
+// Per-tensor scales (TENSOR: args.sa / args.sb point at one float each) or E8M0 block scales (MX: they point at
+// bytes; ldsa / ldsb = bytes per scale row). grid: (n tiles, m tiles of 128); n tiles are 128 wide, 64 for gated forward.
+template <int MODE, typename TO, int TN, bool TENSOR, bool MX>
+static void launch_scaled_formats(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, dim3 grid, hipStream_t stream) {
+    const bool a5 = a_dtype == VIOLA_E5M2, b5 = b_dtype == VIOLA_E5M2;
+    if (!a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE, false, false, false, TO, TN, TENSOR, MX>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    else if (a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE, true, false, false, TO, TN, TENSOR, MX>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    else if (!a5 && b5) hipLaunchKernelGGL((group_gemm_fast<MODE, false, true, false, TO, TN, TENSOR, MX>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    else hipLaunchKernelGGL((group_gemm_fast<MODE, true, true, false, TO, TN, TENSOR, MX>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+}
+
+template <bool TENSOR, bool MX>
+static int launch_scaled_gemm_fast(const GemmArgs& args, int mode, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, dim3 grid,
+                                   hipStream_t stream) {
+    GemmArgs p = args;
+    const bool narrow = mode == MODE_PLAIN && (int64_t)grid.x * grid.y < 512 && p.n > 64;
+    if (narrow) grid.x = (unsigned)((p.n + 63) / 64);
+    if ((int64_t)grid.x * grid.y < (1 << 30)) {
+        p.tiles_n = (int)grid.x;
+        p.tiles_m = (int)grid.y;
+        grid = dim3((grid.x * grid.y + 7) / 8 * 8, 1, 1);
+    }
+#define VIOLA_SCALED(TO)                                                                                                        \
+    if (narrow) launch_scaled_formats<MODE_PLAIN, TO, 1, TENSOR, MX>(p, a_dtype, b_dtype, bias_dtype, grid, stream);             \
+    else if (mode == MODE_PLAIN) launch_scaled_formats<MODE_PLAIN, TO, 2, TENSOR, MX>(p, a_dtype, b_dtype, bias_dtype, grid, stream); \
+    else if (mode == MODE_GATED_FWD) launch_scaled_formats<MODE_GATED_FWD, TO, 2, TENSOR, MX>(p, a_dtype, b_dtype, bias_dtype, grid, stream); \
+    else launch_scaled_formats<MODE_GATED_BWD, TO, 2, TENSOR, MX>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
+    switch (out_dtype) {
+        case VIOLA_F32: VIOLA_SCALED(float) break;
+        case VIOLA_BF16: VIOLA_SCALED(bf16_t) break;
+        case VIOLA_F16: VIOLA_SCALED(f16_t) break;
+        default: return VIOLA_EINVAL;
+    }
+#undef VIOLA_SCALED
+    return viola_launch_status();
+}
+
+}  // namespace viola

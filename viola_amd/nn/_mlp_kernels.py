@@ -1,9 +1,11 @@
 """FP8 GEMMs with the gated-activation forward/backward epilogues fused (operator seam of
-viola/nn/_mlp_kernels.py `gemm` :243-277), FP32 group scales."""
+viola/nn/_mlp_kernels.py `gemm` :243-277) for every scaling recipe: FP32 group scales, E8M0 block scales on the
+block-scaled MFMA, and one FP32 scale per tensor."""
 
 import torch
 
 from .. import _lib
+from . import _gated_kernels, _grouped_kernels
 
 
 def gemm(a, b, sa, sb, *, layer, out_dtype, activation, backward=False, aux=None, bias=None, save=True,
@@ -11,24 +13,44 @@ def gemm(a, b, sa, sb, *, layer, out_dtype, activation, backward=False, aux=None
     """forward: out = act(a.Wg^T) * (a.Wu^T), aux = [g, u] if save; backward: out = [d*u*act'(g), d*act(g)].
 
     Returns (out, aux, (out_scale, out_t, out_t_scale)); the last triple is the reference's
-    in-kernel MXFP8 re-encode of H, which only its E8M0 path produces: always empty here.
+    in-kernel MXFP8 re-encode of H (_mlp_kernels.py:195-230), which is not built: always empty here, and the
+    caller quantizes H with the ordinary quantizer (the same codes and scales).
     """
-    if encode_output or save_output_transpose or layer._native_scaling:
+    if encode_output or save_output_transpose:
         raise NotImplementedError("in-kernel MXFP8 re-encode of H is not built in viola_amd")
-    assert layer._grouped_scaling and a.is_cuda
+    assert a.is_cuda
     a, b, sa, sb = a.contiguous(), b.contiguous(), sa.contiguous(), sb.contiguous()
     m, k = a.shape
     h = b.shape[0] if backward else b.shape[0] // 2
-    ga = tuple(group_a or layer.input_group_shape)
-    gb = tuple(group_b or layer.weight_group_shape)
     out = torch.empty((m, 2 * h if backward else h), device=a.device, dtype=out_dtype)
     if aux is None:
         aux = torch.empty((m, 2 * h) if save else (0, 0), device=a.device, dtype=out_dtype)
     else:
         assert aux.dtype == out_dtype and aux.is_contiguous() and tuple(aux.shape) == (m, 2 * h)
     bias_c = bias.contiguous() if bias is not None else None
-    _lib.call("viola_gated_gemm", _lib.ptr(a), _lib.code(a.dtype), _lib.ptr(b), _lib.code(b.dtype), _lib.ptr(sa), _lib.ptr(sb),
-              m, h, k, ga[0], ga[1], gb[0], gb[1], _lib.ptr(bias_c), _lib.code(bias_c.dtype) if bias_c is not None else 0,
-              _lib.ptr(aux), _lib.ptr(out), _lib.code(out_dtype), _lib.ACTIVATION[activation], int(backward))
+    bias_code = _lib.code(bias_c.dtype) if bias_c is not None else 0
     empty = torch.empty((0, 0), device=a.device, dtype=torch.uint8)
-    return out, aux, (empty, out.new_empty((0, 0), dtype=a.dtype), empty)
+    extra = (empty, out.new_empty((0, 0), dtype=a.dtype), empty)
+    operands = (_lib.ptr(a), _lib.code(a.dtype), _lib.ptr(b), _lib.code(b.dtype), _lib.ptr(sa), _lib.ptr(sb), m, h, k)
+    tail = (_lib.ptr(bias_c), bias_code, _lib.ptr(aux), _lib.ptr(out), _lib.code(out_dtype), _lib.ACTIVATION[activation], int(backward))
+    if not layer._grouped_scaling:
+        _lib.call("viola_tensor_gated_gemm", *operands, *tail)
+        return out, aux, extra
+    ga = tuple(group_a or layer.input_group_shape)
+    gb = tuple(group_b or layer.weight_group_shape)
+    if not layer._native_scaling:
+        _lib.call("viola_gated_gemm", *operands, ga[0], ga[1], gb[0], gb[1], *tail)
+        return out, aux, extra
+    status = -2
+    if ga[1] == 32 and gb[1] == 32:
+        status = _lib.call("viola_mx_gated_gemm", *operands, ga[0], gb[0], *tail, unsupported_ok=True)
+    if status != 0:
+        # shapes the block-scaled MFMA path does not take: the same values from the plain GEMM and the elementwise kernels
+        if backward:
+            d = _grouped_kernels.gemm(a, b, sa, sb, ga, gb, out_dtype=out_dtype, native=True)
+            out = _gated_kernels.gated_backward(aux, d, activation)
+        else:
+            z = _grouped_kernels.gemm(a, b, sa, sb, ga, gb, out_dtype=out_dtype, native=True, bias=bias)
+            z, out = _gated_kernels.gated_forward(z, activation)
+            aux = z if save else aux
+    return out, aux, extra

@@ -1,12 +1,21 @@
-"""Gated MLP: down(act(gate(x)) * up(x)) with the gating fused into the FP8 GEMMs for scaling="grouped"
-(module surface of viola/nn/mlp.py:76-113; autograd wiring :22-73); the per-tensor and MXFP8 recipes run the two
-Linears with the elementwise gated kernel between them."""
+"""Gated MLP: down(act(gate(x)) * up(x)) with the gating fused into the FP8 GEMMs' epilogues under every scaling
+recipe (module surface of viola/nn/mlp.py:76-113; autograd wiring :22-73)."""
 
 import torch
 from torch import nn
 
 from .linear import Linear
-from ._grouped_linear import backward_core, forward_core
+from . import _grouped_linear, _tensor_linear
+
+
+def forward_core(x, weight, bias, layer, *args, **kwargs):
+    cores = _grouped_linear if layer._grouped_scaling else _tensor_linear
+    return cores.forward_core(x, weight, bias, layer, *args, **kwargs)
+
+
+def backward_core(record, *args, **kwargs):
+    cores = _grouped_linear if record.layer._grouped_scaling else _tensor_linear
+    return cores.backward_core(record, *args, **kwargs)
 
 
 class _GateUp(torch.autograd.Function):
@@ -74,12 +83,6 @@ class MLP(nn.Module):
         assert x.is_cuda, "viola.nn.MLP executes on CUDA."
         if torch.is_autocast_enabled("cuda"):
             x = x.to(torch.get_autocast_dtype("cuda"))
-        if not (self.gate_up._grouped_scaling and not self.gate_up._native_scaling):
-            # per-tensor and MXFP8 recipes: the same arithmetic, un-fused (z = gate_up(x) rounded to the activation
-            # dtype, act(g) * u in fp32, rounded once: the expression the fused epilogue is checked against,
-            # checks/mlp.py:12-16); only the FP32-group-scale GEMM has the gated epilogues
-            from ._gated_kernels import GatedActivation
-            return self.down(GatedActivation.apply(self.gate_up(x), self.activation))
         need_backward = torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters()))
         need_up = need_backward and (x.requires_grad or any(p.requires_grad for p in self.gate_up.parameters()))
         shape = x.shape
