@@ -164,6 +164,34 @@ def test_gated_elementwise(activation):
     assert rel_l2(z.grad, torch.cat([dg, du], -1).bfloat16()) < 4e-3
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("activation", ["silu", "gelu", "relu"])
+def test_gated_elementwise_pieces_equal_the_scalar_kernel(dtype, activation):
+    """Rows of 16-byte pieces take the vectorised kernels, anything else the element-wise ones: the same values bit
+    for bit (hidden 160 against the same data at hidden 160 behind a one-element pointer offset), and against the
+    oracle at an odd hidden size."""
+    from viola_amd.nn import _gated_kernels as gk
+    torch.manual_seed(11)
+    rows, hidden = 77, 160
+    z = (torch.randn(rows, 2 * hidden) * 3).to(dtype).cuda()
+    dy = torch.randn(rows, hidden).to(dtype).cuda()
+    _, out = gk.gated_forward(z, activation)
+    dz = gk.gated_backward(z, dy, activation)
+    shifted_z = torch.empty(z.numel() + 1, device="cuda", dtype=dtype)[1:].view_as(z).copy_(z)      # 2- or 4-byte aligned only
+    shifted_dy = torch.empty(dy.numel() + 1, device="cuda", dtype=dtype)[1:].view_as(dy).copy_(dy)
+    assert shifted_z.data_ptr() % 16 != 0 and shifted_z.is_contiguous()
+    _, out_scalar = gk.gated_forward(shifted_z, activation)
+    dz_scalar = gk.gated_backward(shifted_z, shifted_dy, activation)
+    assert torch.equal(out, out_scalar) and torch.equal(dz, dz_scalar)
+    g, u = z.cpu()[:, :hidden], z.cpu()[:, hidden:]
+    assert rel_l2(out, ol.gated_forward(g, u, activation).to(dtype)) < 4e-3
+    dg, du = ol.gated_backward(dy.cpu(), g, u, activation)
+    assert rel_l2(dz, torch.cat([dg, du], -1).to(dtype)) < 4e-3
+    odd = (torch.randn(9, 2 * 37) * 3).to(dtype).cuda()
+    _, out_odd = gk.gated_forward(odd, activation)
+    assert rel_l2(out_odd, ol.gated_forward(odd.cpu()[:, :37], odd.cpu()[:, 37:], activation).to(dtype)) < 4e-3
+
+
 @pytest.mark.parametrize("counts", [[130, 0, 3, 64, 1, 200], [5], [0, 0, 7]])
 def test_varlen_group_gemm_and_wgrad(counts):
     from viola_amd.nn import _varlen as v

@@ -190,6 +190,109 @@ __global__ __launch_bounds__(256) void gated_backward_kernel(const void* __restr
     }
 }
 
+// The same two maps for rows whose halves start on 16-byte boundaries: one 16-byte piece of g, u (and dy) per thread,
+// element type and activation fixed at compile time. Every element goes through the expressions above.
+template <typename T> struct Piece {
+    static constexpr int N = 16 / (int)sizeof(T);
+    static __device__ __forceinline__ void load(const T* p, float (&v)[N]) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(p);
+        T t[N];
+        __builtin_memcpy(t, &raw, 16);
+#pragma unroll
+        for (int i = 0; i < N; ++i) v[i] = to_f32(t[i]);
+    }
+    static __device__ __forceinline__ void store(T* p, const float (&v)[N]) {
+        T t[N];
+#pragma unroll
+        for (int i = 0; i < N; ++i) t[i] = from_f32<T>(v[i]);
+        uint4 raw;
+        __builtin_memcpy(&raw, t, 16);
+        *reinterpret_cast<uint4*>(p) = raw;
+    }
+};
+
+template <typename T, int ACT>
+__global__ __launch_bounds__(256) void gated_forward_pieces(const T* __restrict__ z, T* __restrict__ out, int64_t pieces, int64_t per_row) {
+    constexpr int N = Piece<T>::N;
+    const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (id >= pieces) return;
+    const int64_t r = id / per_row, c = id % per_row * N, h = per_row * N;
+    float g[N], u[N], o[N];
+    Piece<T>::load(z + r * 2 * h + c, g);
+    Piece<T>::load(z + r * 2 * h + h + c, u);
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        float a;
+        if constexpr (ACT == VIOLA_SILU) a = g[i] / (1.0f + expf(-g[i]));
+        else if constexpr (ACT == VIOLA_GELU) a = 0.5f * g[i] * (1.0f + tanhf(0.7978845608028654f * (g[i] + 0.044715f * g[i] * g[i] * g[i])));
+        else a = fmaxf(g[i], 0.0f);
+        o[i] = a * u[i];
+    }
+    Piece<T>::store(out + r * h + c, o);
+}
+
+template <typename T, int ACT>
+__global__ __launch_bounds__(256) void gated_backward_pieces(const T* __restrict__ z, const T* __restrict__ dy, T* __restrict__ dz,
+                                                              int64_t pieces, int64_t per_row) {
+    constexpr int N = Piece<T>::N;
+    const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (id >= pieces) return;
+    const int64_t r = id / per_row, c = id % per_row * N, h = per_row * N;
+    float g[N], u[N], d[N], dg[N], du[N];
+    Piece<T>::load(z + r * 2 * h + c, g);
+    Piece<T>::load(z + r * 2 * h + h + c, u);
+    Piece<T>::load(dy + r * h + c, d);
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        float a, derivative;
+        if constexpr (ACT == VIOLA_SILU) {
+            const float s = 1.0f / (1.0f + expf(-g[i]));
+            a = g[i] * s;
+            derivative = s * (1.0f + g[i] * (1.0f - s));
+        } else if constexpr (ACT == VIOLA_GELU) {
+            const float t = tanhf(0.7978845608028654f * (g[i] + 0.044715f * g[i] * g[i] * g[i]));
+            a = 0.5f * g[i] * (1.0f + t);
+            derivative = 0.5f * (1.0f + t) + 0.5f * g[i] * (1.0f - t * t) * 0.7978845608028654f * (1.0f + 0.134145f * g[i] * g[i]);
+        } else {
+            a = fmaxf(g[i], 0.0f);
+            derivative = g[i] > 0.0f ? 1.0f : 0.0f;
+        }
+        dg[i] = d[i] * u[i] * derivative;
+        du[i] = d[i] * a;
+    }
+    Piece<T>::store(dz + r * 2 * h + c, dg);
+    Piece<T>::store(dz + r * 2 * h + h + c, du);
+}
+
+template <typename T>
+static bool launch_gated_pieces(const void* z, const void* dy, void* out, int64_t rows, int64_t h, int activation, bool backward,
+                                hipStream_t stream) {
+    constexpr int N = Piece<T>::N;
+    const auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    if (h % N != 0 || !aligned(z) || !aligned(out) || (backward && !aligned(dy))) return false;
+    const int64_t per_row = h / N, pieces = rows * per_row, blocks = (pieces + 255) / 256;
+    if (blocks > 0x7fffffff) return false;
+    const dim3 grid((unsigned)blocks);
+    const T* zp = static_cast<const T*>(z);
+    const T* dp = static_cast<const T*>(dy);
+    T* op = static_cast<T*>(out);
+#define VIOLA_GATED(ACT)                                                                                                   \
+    if (backward) hipLaunchKernelGGL((gated_backward_pieces<T, ACT>), grid, dim3(256), 0, stream, zp, dp, op, pieces, per_row); \
+    else hipLaunchKernelGGL((gated_forward_pieces<T, ACT>), grid, dim3(256), 0, stream, zp, op, pieces, per_row);
+    if (activation == VIOLA_SILU) { VIOLA_GATED(VIOLA_SILU) }
+    else if (activation == VIOLA_GELU) { VIOLA_GATED(VIOLA_GELU) }
+    else { VIOLA_GATED(VIOLA_RELU) }
+#undef VIOLA_GATED
+    return true;
+}
+
+static bool launch_gated_pieces(const void* z, const void* dy, void* out, int64_t rows, int64_t h, int dtype, int activation,
+                                bool backward, hipStream_t stream) {
+    if (dtype == VIOLA_F32) return launch_gated_pieces<float>(z, dy, out, rows, h, activation, backward, stream);
+    if (dtype == VIOLA_BF16) return launch_gated_pieces<bf16_t>(z, dy, out, rows, h, activation, backward, stream);
+    return launch_gated_pieces<f16_t>(z, dy, out, rows, h, activation, backward, stream);
+}
+
 // ------------------------------------------------------------------ self checks
 // Hardware v_cvt_pk_{fp8,bf8}_f32 / v_cvt_f32_{fp8,bf8} against the software codecs.
 __global__ __launch_bounds__(256) void selftest_fp8_kernel(unsigned long long* counts) {
@@ -290,6 +393,7 @@ extern "C" int viola_gated_forward(const void* z, void* out, int64_t rows, int64
     VIOLA_CHECK_ARG(viola_is_float(dtype) && rows >= 0 && h >= 0 && activation >= VIOLA_SILU && activation <= VIOLA_RELU);
     if (rows == 0 || h == 0) return 0;
     VIOLA_CHECK_ARG(z && out);
+    if (launch_gated_pieces(z, nullptr, out, rows, h, dtype, activation, false, stream)) return viola_launch_status();
     hipLaunchKernelGGL(gated_forward_kernel, dim3(grid_for(rows * h)), dim3(256), 0, stream, z, out, rows, h, dtype, activation);
     return viola_launch_status();
 }
@@ -300,6 +404,7 @@ extern "C" int viola_gated_backward(const void* z, const void* dy, void* dz, int
     VIOLA_CHECK_ARG(viola_is_float(dtype) && rows >= 0 && h >= 0 && activation >= VIOLA_SILU && activation <= VIOLA_RELU);
     if (rows == 0 || h == 0) return 0;
     VIOLA_CHECK_ARG(z && dy && dz);
+    if (launch_gated_pieces(z, dy, dz, rows, h, dtype, activation, true, stream)) return viola_launch_status();
     hipLaunchKernelGGL(gated_backward_kernel, dim3(grid_for(rows * h)), dim3(256), 0, stream, z, dy, dz, rows, h, dtype, activation);
     return viola_launch_status();
 }
