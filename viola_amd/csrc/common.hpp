@@ -187,10 +187,20 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// The value of the lane whose index differs in bit 0 (OFFSET 1) or bit 1 (OFFSET 2): a DPP quad permute, which stays
+// in the vector ALU (a shuffle goes through the LDS crossbar and its wait).
+template <int OFFSET> __device__ __forceinline__ float quad_xor(float v) {
+    static_assert(OFFSET == 1 || OFFSET == 2, "inside a quad of lanes");
+    if constexpr (OFFSET == 1) return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xf, 0xf, true));   // lanes 1 0 3 2
+    else return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xf, 0xf, true));                        // lanes 2 3 0 1
+}
+
 // max over aligned sub-groups of WIDTH lanes (WIDTH a power of two <= 64)
 template <int WIDTH> __device__ __forceinline__ float group_max(float v) {
 #pragma unroll
-    for (int offset = WIDTH / 2; offset > 0; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, WAVE));
+    for (int offset = WIDTH / 2; offset > 2; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, WAVE));
+    if constexpr (WIDTH >= 4) v = fmaxf(v, quad_xor<2>(v));
+    if constexpr (WIDTH >= 2) v = fmaxf(v, quad_xor<1>(v));
     return v;
 }
 

@@ -247,7 +247,7 @@ __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x
     typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     __shared__ __attribute__((aligned(16))) uint16_t park[4][32 * LD];
-    const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+    const int lane = threadIdx.x % WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);   // uniform: so is the buffer descriptor
     uint16_t* mine = park[wave];
     const int lr = lane / 8, ch = lane % 8;
     const int64_t nc = (cols + 31) / 32;
@@ -284,8 +284,8 @@ __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x
                 poison = poison_of(poison, vr[i][e]);
             }
             amax = group_max<4>(amax);
-            poison += __shfl_xor(poison, 1, WAVE);
-            poison += __shfl_xor(poison, 2, WAVE);
+            poison += quad_xor<1>(poison);
+            poison += quad_xor<2>(poison);
             s_row[i] = group_scale(amax, limit, e8m0);
             d_row[i] = SharedDivisor(s_row[i], poison);
             fast = fast && d_row[i].fast;
@@ -608,7 +608,7 @@ __global__ __launch_bounds__(256) void quantize_segmented16(const TIn* __restric
     typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     __shared__ __attribute__((aligned(16))) uint16_t park[4][32 * LD];
-    const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+    const int lane = threadIdx.x % WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);   // uniform: so is the buffer descriptor
     uint16_t* mine = park[wave];
     const int lr = lane / 8, ch = lane % 8;
     const int64_t nc = (cols + 31) / 32;
@@ -644,8 +644,8 @@ __global__ __launch_bounds__(256) void quantize_segmented16(const TIn* __restric
                 poison = poison_of(poison, v[e]);
             }
             amax = group_max<4>(amax);
-            poison += __shfl_xor(poison, 1, WAVE);
-            poison += __shfl_xor(poison, 2, WAVE);
+            poison += quad_xor<1>(poison);
+            poison += quad_xor<2>(poison);
             const float s = group_scale(amax, limit);
             const SharedDivisor divisor(s, poison);
             const uint2 codes = encode8<TOut>(v, s, limit, divisor);
