@@ -128,6 +128,7 @@ def main():
     parser.add_argument("--warmup", type=int, default=50)
     parser.add_argument("--skip-cpu", action="store_true", help="leave out the CPU baseline leg")
     parser.add_argument("--skip-muon", action="store_true", help="leave out the FP8Muon / codec legs")
+    parser.add_argument("--skip-mlp", action="store_true", help="leave out the gated MLP leg")
     parser.add_argument("--calibrate", action="store_true",
                         help="also launch copy_scaled_kernel once over 64 Mi floats (256 MiB read, 256 MiB written): "
                              "the known-size kernel that FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -255,6 +256,33 @@ def main():
                                                gemm_tflops=2 * M * K * N / (cg["avg_ms"] * 1e-3) / 1e12,
                                                gemm_frac_fp8_peak=2 * M * K * N / (cg["avg_ms"] * 1e-3) / 1e12 / PEAK["fp8_tflops"],
                                                launches_per_step=sum(v["launches_per_step"] for v in cb.values()))
+
+    if not args.skip_mlp:
+        # the gated MLP of the reference's MLP benchmark shape (16384 tokens, 4096 -> 11008 -> 4096, SwiGLU), forward +
+        # backward, under the three recipes: gating fused into the gate/up GEMM's and the down dgrad GEMM's epilogues
+        import viola_amd
+        Mm, Dm, Hm = 16384, 4096, 11008
+        mlp_flops = 3 * (2 * Mm * Dm * 2 * Hm + 2 * Mm * Hm * Dm)
+        xm = torch.randn(Mm, Dm, device="cuda").bfloat16().requires_grad_()
+        dym = torch.randn(Mm, Dm, device="cuda").bfloat16()
+        extra["mlp_step"] = {"shape": [Mm, Dm, Hm], "flops": mlp_flops}
+        for scaling in ("grouped", "current", "mxfp8"):
+            viola_amd.set_gradient_dtype("bf16")
+            torch.manual_seed(4)
+            mlp = viola_amd.nn.MLP(Dm, Hm, activation="silu", weight_dtype="fp8", scaling=scaling, mode="memory", backward_dtype="e4m3",
+                                   device="cuda", dtype=torch.bfloat16)
+            viola_amd.precision._settings["gradient_dtype"] = None
+
+            def mlp_step():
+                xm.grad = None
+                for parameter in mlp.parameters():
+                    parameter.grad = None
+                mlp(xm).backward(dym)
+            mlp_ms, _ = timed(mlp_step, min(args.steps, 20), min(args.warmup, 5))
+            gated = {k: v for k, v in kernel_breakdown(mlp_step, 3).items() if "gated" in k}
+            extra["mlp_step"][scaling] = dict(step_ms=mlp_ms, tflops=mlp_flops / (mlp_ms * 1e-3) / 1e12, gated_gemm=gated)
+            del mlp
+        del xm, dym
 
     if args.calibrate:
         from viola_amd.optim import _kernels as ok
