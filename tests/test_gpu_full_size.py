@@ -87,6 +87,73 @@ def test_gated_mlp_gemms_at_16384x4096x11008():
     assert torch.equal(plain, aux)
 
 
+@pytest.mark.parametrize("recipe", ["tensor", "mxfp8"])
+def test_gated_mlp_gemms_other_recipes_at_16384x4096x11008(recipe):
+    """The gated epilogues under per-tensor and E8M0 scales at the full MLP shape: the fused forward's [g, u] is the
+    plain GEMM's output bit for bit, h is the elementwise kernel's to rounding, and the fused backward equals the plain
+    dgrad GEMM followed by the elementwise backward kernel bit for bit (same expressions, same rounding points)."""
+    import types
+    from viola_amd.nn import _gated_kernels as gk, _grouped_kernels as g, _linear_kernels as lk, _mlp_kernels as mk
+    m, d, h = 16384, 4096, 11008
+    torch.manual_seed(6)
+    x = (torch.randn(m, d, device="cuda") * torch.exp2(torch.randint(-3, 4, (m, 1), device="cuda").float())).bfloat16()
+    w = torch.empty(2 * h, d, device="cuda").uniform_(-1 / 64, 1 / 64)
+    dy = torch.randn(m, d, device="cuda").bfloat16()
+    w2 = torch.empty(h, d, device="cuda").uniform_(-1 / 64, 1 / 64)          # the down projection's W^T: [hidden, out]
+    if recipe == "mxfp8":
+        layer = types.SimpleNamespace(_native_scaling=True, _grouped_scaling=True, input_group_shape=(1, 32), weight_group_shape=(32, 32))
+        (qx, sx), (qw, sw) = g.quantize(x, E4, (1, 32), native=True), g.quantize(w, E4, (32, 32), native=True)
+        (qg, sg), (qw2, sw2) = g.quantize(dy, E4, (1, 32), native=True), g.quantize(w2, E4, (32, 32), native=True)
+        plain = lambda a, b, sa, sb: g.gemm(a, b, sa, sb, (1, 32), (32, 32), out_dtype=torch.bfloat16, native=True)
+        extra = dict(group_a=(1, 32), group_b=(32, 32))
+    else:
+        layer = types.SimpleNamespace(_native_scaling=False, _grouped_scaling=False)
+        sx, sw, sg, sw2 = (lk.tensor_scale(t) for t in (x, w, dy, w2))
+        qx, qw, qg, qw2 = (lk.quantize(t, s)[0] for t, s in ((x, sx), (w, sw), (dy, sg), (w2, sw2)))
+        plain = lambda a, b, sa, sb: lk.gemm(a, b, sa, sb, out_dtype=torch.bfloat16)
+        extra = {}
+    del w, w2
+    out, aux, _ = mk.gemm(qx, qw, sx, sw, layer=layer, out_dtype=torch.bfloat16, activation="silu", save=True)
+    assert out.shape == (m, h) and aux.shape == (m, 2 * h)
+    assert torch.equal(aux, plain(qx, qw, sx, sw))
+    assert rel_l2(out, gk.gated_forward(aux, "silu")[1]) < 3e-3
+    rows = torch.arange(0, m, 61, device="cuda")
+    assert rel_l2(out[rows], (torch.nn.functional.silu(aux[rows, :h].float()) * aux[rows, h:].float()).bfloat16()) < 3e-3
+    dz, _, _ = mk.gemm(qg, qw2, sg, sw2, layer=layer, out_dtype=torch.bfloat16, activation="silu", backward=True, aux=aux, **extra)
+    assert torch.equal(dz, gk.gated_backward(aux, plain(qg, qw2, sg, sw2), "silu"))
+
+
+@pytest.mark.parametrize("scaling,backward", [("current", "e5m2"), ("mxfp8", "e4m3")])
+def test_linear_module_other_recipes_at_8192x1024x4096(scaling, backward):
+    """The headline layer under the per-tensor and the MXFP8 recipe against fp32 GPU matmuls of the dequantized operands."""
+    import viola_amd
+    from viola_amd.nn import _grouped_kernels as g, _linear_kernels as lk
+    viola_amd.set_gradient_dtype("bf16")
+    try:
+        torch.manual_seed(3)
+        layer = viola_amd.nn.Linear(1024, 4096, device="cuda", dtype=torch.bfloat16, scaling=scaling, forward_dtype="e4m3",
+                                    backward_dtype=backward, mode="memory", weight_dtype="fp8")
+    finally:
+        viola_amd.precision._settings["gradient_dtype"] = None
+    bwd = torch.float8_e5m2 if backward == "e5m2" else E4
+    x = torch.randn(8192, 1024, device="cuda").bfloat16().requires_grad_()
+    dy = (torch.randn(8192, 4096, device="cuda") * 1e-2).bfloat16()
+    y = layer(x)
+    y.backward(dy)
+    w = layer.dequantize_weight()
+    if scaling == "mxfp8":
+        deq = lambda t, fmt, transposed=False: g.dequantize(*g.quantize(t, fmt, (1, 32), native=True, transposed=transposed), (1, 32))
+        xq, gq, xt, gt = deq(x.detach(), E4), deq(dy, bwd), deq(x.detach(), E4, True), deq(dy, bwd, True)
+    else:
+        fake = lambda t, fmt: lk.quantize(t, lk.tensor_scale(t, fp8_dtype=fmt), fp8_dtype=fmt)[0].float() * lk.tensor_scale(t, fp8_dtype=fmt)
+        xq, gq = fake(x.detach(), E4), fake(dy, bwd)
+        xt, gt = xq.T, gq.T
+    assert rel_l2(y, (xq @ w.T + layer.bias.float()).bfloat16()) < 3e-3
+    assert rel_l2(x.grad, (gq @ w).bfloat16()) < 3e-3
+    assert rel_l2(layer.weight.grad, (gt @ xt.T).bfloat16()) < 3e-3
+    assert rel_l2(layer.bias.grad, dy.float().sum(0).bfloat16()) < 3e-3
+
+
 def test_variable_groups_at_16x32768x4096x1024():
     from viola_amd.nn import _varlen as v, _grouped_kernels as g
     groups, k, n, total = 16, 4096, 1024, 32768
