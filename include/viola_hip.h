@@ -158,6 +158,16 @@ int viola_mx_gated_gemm(const void* a, int a_dtype, const void* b, int b_dtype, 
                         int64_t m, int64_t h, int64_t k, int ar, int br, const void* bias, int bias_dtype, void* aux,
                         void* out, int out_dtype, int activation, int backward, viola_stream_t stream);
 
+/* viola/nn/_mlp_kernels.py:195-230 (`encode_output`, `save_output_transpose`): the gate/up projection of an MXFP8 MLP
+ * whose h = act(g) * u, rounded to aux_dtype, leaves the kernel as FP8 codes with E8M0 scales per 32 values: along its
+ * rows (enc [m, h], enc_scale [m, h / 32]) for the down projection's forward GEMM and, when enc_t is not NULL, along
+ * its columns (enc_t [h, m], enc_t_scale [h, m / 32]) for its wgrad. aux [m, 2h] (NULL allowed) receives [g, u].
+ * VIOLA_EUNSUPPORTED where viola_mx_gated_gemm returns it, and when m or h is not a multiple of 32. */
+int viola_mx_gated_gemm_encode(const void* a, int a_dtype, const void* b, int b_dtype, const uint8_t* sa, const uint8_t* sb,
+                               int64_t m, int64_t h, int64_t k, int ar, int br, const void* bias, int bias_dtype, void* aux,
+                               int aux_dtype, void* enc, uint8_t* enc_scale, void* enc_t, uint8_t* enc_t_scale, int enc_dtype,
+                               float limit, int activation, viola_stream_t stream);
+
 /* Variable-group (MoE-expert style) GEMM: `groups` independent problems that share n and k and
  * differ in their row range. Group g owns rows [offsets[g], offsets[g+1]) of a and out
  * (offsets: groups+1 int64 on the device, ascending) and operand b + g*b_group_stride (elements),

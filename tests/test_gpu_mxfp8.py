@@ -229,3 +229,75 @@ def test_mlp_recipes_match_their_unfused_composition(precision_policy, options, 
         assert a.dtype == b.dtype and rel_l2(a, b) < .025
     # same GEMM sums, same rounding points: the fused epilogue gives the composition's y to bf16 / fp16 rounding
     assert rel_l2(got[0], want[0]) < 2e-3
+
+
+@pytest.mark.parametrize("fmt", [E4, E5])
+@pytest.mark.parametrize("m,h,k,transpose,dtype", [(128, 64, 128, True, torch.bfloat16), (96, 160, 256, True, torch.bfloat16),
+                                                   (320, 256, 128, False, torch.float16), (64, 96, 384, True, torch.float32),
+                                                   (66, 64, 128, True, torch.bfloat16), (64, 64, 96, True, torch.bfloat16)])
+def test_gate_up_gemm_hands_h_over_as_mxfp8_codes(fmt, m, h, k, transpose, dtype):
+    """viola/nn/_mlp_kernels.py:195-230 (encode_output, save_output_transpose): the codes and E8M0 bytes of h in both
+    layouts equal the oracle's quantization of the h the plain fused kernel writes, bit for bit; [g, u] is unchanged.
+    The last two shapes (m not a multiple of 32, k not of 128) take the quantizer after the GEMM instead."""
+    import types
+    from viola_amd.nn import _mlp_kernels as mk
+    torch.manual_seed(23)
+    spread = 1 if dtype == torch.float16 else 3                               # keep g * u inside fp16's range
+    a = (torch.randn(m, k) * torch.exp2(torch.randint(-spread, spread + 1, (m, 1)).float())).bfloat16()
+    w = (torch.randn(2 * h, k) / 8 * torch.exp2(torch.randint(-spread, spread + 1, (2 * h, 1)).float())).bfloat16()
+    (qa, sa), (qb, sb) = og.quantize(a, E4, (1, 32), native=True), og.quantize(w, E4, (32, 32), native=True)
+    bias = torch.randn(2 * h).to(dtype)
+    layer = types.SimpleNamespace(_native_scaling=True, _grouped_scaling=True, input_group_shape=(1, 32), weight_group_shape=(32, 32),
+                                  fp8_dtype=fmt, _group_limit=lambda *args, **kwargs: None)
+    args = (qa.cuda(), qb.cuda(), sa.cuda(), sb.cuda())
+    plain, aux, _ = mk.gemm(*args, layer=layer, out_dtype=dtype, bias=bias.cuda(), activation="silu", save=True)
+    codes, aux2, (scale, codes_t, scale_t) = mk.gemm(*args, layer=layer, out_dtype=dtype, bias=bias.cuda(), activation="silu",
+                                                     save=True, encode_output=True, save_output_transpose=transpose)
+    assert torch.equal(aux2, aux)
+    want_q, want_s = og.quantize(plain.cpu(), fmt, (1, 32), native=True)
+    assert codes.dtype == fmt and scale.dtype == torch.uint8
+    assert torch.equal(scale.cpu(), want_s) and torch.equal(codes.cpu().view(torch.uint8), want_q.view(torch.uint8))
+    if transpose:
+        want_qt, want_st = og.quantize(plain.cpu(), fmt, (1, 32), native=True, transposed=True)
+        assert torch.equal(scale_t.cpu(), want_st) and torch.equal(codes_t.cpu().view(torch.uint8), want_qt.view(torch.uint8))
+    else:
+        assert codes_t.numel() == 0 and scale_t.numel() == 0
+    nosave = mk.gemm(*args, layer=layer, out_dtype=dtype, bias=bias.cuda(), activation="silu", save=False, encode_output=True)
+    assert nosave[1].numel() == 0 and torch.equal(nosave[0].view(torch.uint8), codes.view(torch.uint8))
+
+
+@pytest.mark.parametrize("dims,tokens", [((128, 256, 128), 128), ((256, 384, 256), 96), ((128, 160, 96), 64)])
+@pytest.mark.parametrize("options", [dict(weight_dtype="fp8", mode="fast", activation="gelu"), dict(weight_dtype="bf16"),
+                                     dict(weight_dtype="bf16", bias=False, saved_input_dtype="bf16")],
+                         ids=lambda o: "-".join(str(v) for v in o.values()))
+def test_mxfp8_mlp_with_encoded_h_matches_its_unfused_composition(precision_policy, options, dims, tokens):
+    """The MXFP8 MLP at token counts that are multiples of 32, where h travels from the gate/up GEMM to the down
+    projection as codes (mlp.py:103-107), against the two Linears with a float activation between them."""
+    import torch.nn.functional as F
+    viola = precision_policy
+    viola.set_gradient_dtype("bf16")
+    torch.manual_seed(131)
+    activation = options.get("activation", "silu")
+    d_in, hidden, d_out = dims
+    model = viola.nn.MLP(d_in, hidden, d_out, device="cuda", dtype=torch.bfloat16, scaling="mxfp8", **options)
+    x = torch.randn(tokens, d_in, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    dy = torch.randn(tokens, d_out, device="cuda", dtype=torch.bfloat16)
+    y = model(x)
+    y.backward(dy)
+    got = [y.detach().clone(), x.grad.clone()] + [p.grad.clone() for p in model.parameters()]
+    x.grad = None
+    for p in model.parameters():
+        p.grad = None
+    act = {"silu": F.silu, "relu": F.relu, "gelu": lambda t: F.gelu(t, approximate="tanh")}[activation]
+    z = model.gate_up(x)
+    g, u = z[..., :hidden], z[..., hidden:]
+    reference = model.down((act(g.float()) * u.float()).to(z.dtype))
+    reference.backward(dy)
+    want = [reference.detach(), x.grad] + [p.grad for p in model.parameters()]
+    for a, b in zip(got, want):
+        assert a.dtype == b.dtype and rel_l2(a, b) < .025
+    assert rel_l2(got[0], want[0]) < 2e-3
+    # frozen down weight: no transposed codes are produced, the forward still runs on codes
+    model.down.weight.requires_grad_(False)
+    with torch.no_grad():
+        assert torch.equal(model(x), y)

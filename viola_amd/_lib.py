@@ -46,6 +46,7 @@ _SIGNATURES = {
     "viola_mx_gemm": [_p, _i, _p, _i, _p, _p, _l, _l, _l, _i, _i, _p, _i, _p, _i, _p],
     "viola_tensor_gated_gemm": [_p, _i, _p, _i, _p, _p, _l, _l, _l, _p, _i, _p, _p, _i, _i, _i, _p],
     "viola_mx_gated_gemm": [_p, _i, _p, _i, _p, _p, _l, _l, _l, _i, _i, _p, _i, _p, _p, _i, _i, _i, _p],
+    "viola_mx_gated_gemm_encode": [_p, _i, _p, _i, _p, _p, _l, _l, _l, _i, _i, _p, _i, _p, _i, _p, _p, _p, _p, _i, _f, _i, _p],
     "viola_momentum_update_table": [_p, _l, _l, _i, _i, _f, _f, _i, _i, _l, _p],
     "viola_weight_update_table": [_p, _l, _l, _i, _f, _f, _f, _p],
     "viola_adam_update_table": [_p, _l, _l, _i, _i, _i, _f, _f, _f, _f, _f, _f, _f, _i, _l, _i, _i, _p],

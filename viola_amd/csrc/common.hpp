@@ -180,6 +180,32 @@ __device__ __forceinline__ uint32_t fast_encode4(const SharedDivisor& d, float l
                          __builtin_amdgcn_fmed3f(d.quotient(c), -limit, limit), __builtin_amdgcn_fmed3f(d.quotient(e), -limit, limit));
 }
 
+// ------------------------------------------------------------------ group scales and the clamped encoder
+template <typename TOut>
+__device__ __forceinline__ uint8_t encode_clamped(float v, float s, float limit) {
+    const float t = v / s;
+    const float c = t != t ? t : fminf(fmaxf(t, -limit), limit);
+    return from_f32<TOut>(c).bits;
+}
+
+// amax / limit, or for E8M0 scales the smallest power of two that is not below it (the reference's
+// exp2(ceil(log2(s))), viola/nn/_grouped_kernels.py:81-83, evaluated exactly on the bits)
+__device__ __forceinline__ float group_scale(float amax, float limit, int e8m0 = 0) {
+    const float s = scale_of(amax, limit);
+    if (!e8m0) return s;
+    const uint32_t bits = __float_as_uint(s);
+    if ((bits & 0x7f800000u) == 0x7f800000u) return s;                          // Inf / NaN stay
+    return __uint_as_float((bits & 0x7f800000u) + ((bits & 0x007fffffu) ? 0x00800000u : 0u));
+}
+// a scale goes out as FP32 or as its biased exponent byte (log2(s) + 127, _grouped_kernels.py:85)
+__device__ __forceinline__ void put_scale(float* scale, int64_t index, float s, int e8m0) {
+    if (e8m0) reinterpret_cast<uint8_t*>(scale)[index] = (uint8_t)(__float_as_uint(s) >> 23);
+    else scale[index] = s;
+}
+__device__ __forceinline__ float get_scale(const float* scale, int64_t index, int e8m0) {
+    return e8m0 ? __uint_as_float((uint32_t)reinterpret_cast<const uint8_t*>(scale)[index] << 23) : scale[index];
+}
+
 // ------------------------------------------------------------------ wavefront reductions
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll

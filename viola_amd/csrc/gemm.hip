@@ -488,6 +488,37 @@ extern "C" int viola_gated_gemm(const void* a, int a_dtype, const void* b, int b
                                       dim3((unsigned)((h + BN / 2 - 1) / (BN / 2)), (unsigned)gy), stream);
 }
 
+// viola_mx_gated_gemm forward whose h leaves the kernel as FP8 codes with E8M0 scales in both layouts.
+extern "C" int viola_mx_gated_gemm_encode(const void* a, int a_dtype, const void* b, int b_dtype, const uint8_t* sa, const uint8_t* sb,
+                                          int64_t m, int64_t h, int64_t k, int ar, int br, const void* bias, int bias_dtype,
+                                          void* aux, int aux_dtype, void* enc, uint8_t* enc_scale, void* enc_t,
+                                          uint8_t* enc_t_scale, int enc_dtype, float limit, int activation,
+                                          viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_fp8(a_dtype) && viola_is_fp8(b_dtype) && viola_is_float(aux_dtype) && viola_is_fp8(enc_dtype));
+    VIOLA_CHECK_ARG(m >= 0 && h >= 0 && k >= 0 && ar > 0 && br > 0 && limit > 0.0f);
+    VIOLA_CHECK_ARG(activation >= VIOLA_SILU && activation <= VIOLA_RELU && (!bias || viola_is_float(bias_dtype)));
+    if (m == 0 || h == 0) return 0;
+    VIOLA_CHECK_ARG(enc && enc_scale && (!enc_t || enc_t_scale) && (k == 0 || (a && b && sa && sb)));
+    const int64_t gy = (m + BM - 1) / BM;
+    VIOLA_CHECK_ARG(gy <= 65535);
+    if (k == 0 || k % 128 != 0 || !aligned16(a) || !aligned16(b) || reinterpret_cast<uintptr_t>(sa) % 4 != 0 ||
+        reinterpret_cast<uintptr_t>(sb) % 4 != 0 || 2 * h * k >= (1ll << 31) || (int64_t)BM * k >= (1ll << 31) ||
+        (br != 1 && br % 32 != 0) || h % br != 0 || h % 32 != 0 || m % 32 != 0 || !aligned16(aux) || !aligned16(enc) ||
+        !aligned16(enc_t))
+        return VIOLA_EUNSUPPORTED;
+    GemmArgs p = {};
+    p.a = static_cast<const uint8_t*>(a); p.b = static_cast<const uint8_t*>(b);
+    p.sa = reinterpret_cast<const float*>(sa); p.sb = reinterpret_cast<const float*>(sb);
+    p.bias = bias; p.out = nullptr; p.aux = aux; p.m = m; p.n = h; p.k = k; p.lda = k; p.ldb = k; p.ldo = h;
+    p.activation = activation;
+    p.ldsa = k / 32; p.ldsb = k / 32; p.ar = ar; p.br = br; p.ak_shift = 5; p.bk_shift = 5;
+    p.enc = static_cast<uint8_t*>(enc); p.enc_scale = enc_scale; p.enc_t = static_cast<uint8_t*>(enc_t); p.enc_t_scale = enc_t_scale;
+    p.enc_limit = limit; p.enc_bf8 = enc_dtype == VIOLA_E5M2;
+    return launch_mx_gemm_fast(p, MODE_GATED_FWD, a_dtype, b_dtype, bias_dtype, aux_dtype,
+                               dim3((unsigned)((h + BN / 2 - 1) / (BN / 2)), (unsigned)gy), stream);
+}
+
 extern "C" int viola_varlen_group_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa,
                                        const float* sb, const int64_t* offsets, int groups, int64_t m_total, int64_t n,
                                        int64_t k, int ar, int ak, int br, int bk, int64_t b_group_stride,

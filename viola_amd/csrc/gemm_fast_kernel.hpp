@@ -642,7 +642,79 @@ __global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(Gemm
                     }
                     const int64_t row0 = m_begin + a_sub(j);
                     put(park_a, h);
-                    flush(park_a, out, p.ldo, row0, col0);
+                    bool encoded = false;
+                    if constexpr (MX) {
+                        if (p.enc) {
+                            // The rounded h goes out as FP8 codes with E8M0 scales instead (viola/nn/_mlp_kernels.py:195-230).
+                            // The wave's 32 columns are one group of a row: lanes l32 and l32 + 32 hold its two halves.
+                            encoded = true;
+                            const float limit = p.enc_limit;
+                            auto encode_words = [&](const float (&v)[16], float s, float poison, uint32_t (&w)[4]) {
+                                const SharedDivisor dv(s, poison);
+                                if (__builtin_amdgcn_ballot_w64(!dv.fast) == 0) {
+#pragma unroll
+                                    for (int q = 0; q < 4; ++q)
+                                        w[q] = p.enc_bf8 ? fast_encode4<e5m2_t>(dv, limit, v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3])
+                                                         : fast_encode4<e4m3_t>(dv, limit, v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]);
+                                } else {
+#pragma unroll
+                                    for (int q = 0; q < 4; ++q) {
+                                        w[q] = 0;
+#pragma unroll
+                                        for (int e = 0; e < 4; ++e)
+                                            w[q] |= (uint32_t)(p.enc_bf8 ? encode_clamped<e5m2_t>(v[4 * q + e], s, limit)
+                                                                         : encode_clamped<e4m3_t>(v[4 * q + e], s, limit)) << (8 * e);
+                                    }
+                                }
+                            };
+                            float hq[16];                                    // what the parked tile holds: h rounded to TO
+                            float amax = 0.0f, poison = 0.0f;
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) {
+                                hq[r] = rounded<TO>(h[r]);
+                                amax = fmaxf(amax, fabsf(hq[r]));
+                                poison = poison_of(poison, hq[r]);
+                            }
+                            amax = fmaxf(amax, __shfl_xor(amax, 32, WAVE));
+                            poison += __shfl_xor(poison, 32, WAVE);
+                            const float s_row = group_scale(amax, limit, 1);
+                            uint32_t w[4];
+                            encode_words(hq, s_row, poison, w);
+                            // codes -> a byte tile [row][48] in the second area, then one 16-byte piece per lane to enc
+                            uint8_t* bytes = reinterpret_cast<uint8_t*>(park_b);
+                            constexpr int QLD = 48;
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) *reinterpret_cast<uint32_t*>(&bytes[l32 * QLD + q * 8 + lhi * 4]) = w[q];
+                            const int64_t grow = row0 + lane / 2;
+                            const uint4 piece = *reinterpret_cast<const uint4*>(&bytes[(lane / 2) * QLD + (lane % 2) * 16]);
+                            if (grow < m_end && col0 < p.n) *reinterpret_cast<uint4*>(p.enc + grow * p.n + col0 + (lane % 2) * 16) = piece;
+                            if (lhi == 0 && row0 + l32 < m_end && col0 < p.n)
+                                p.enc_scale[(row0 + l32) * (p.n / 32) + col0 / 32] = (uint8_t)(__float_as_uint(s_row) >> 23);
+                            if (p.enc_t) {
+                                // a column's 32 rows are one group of the transposed layout: lane (column l32, half lhi)
+                                // collects rows 16 lhi .. 16 lhi + 15 of the parked h
+                                float c[16];
+                                float cmax = 0.0f, cpoison = 0.0f;
+#pragma unroll
+                                for (int r = 0; r < 16; ++r) {
+                                    c[r] = to_f32(park_a[(lhi * 16 + r) * PLD + l32]);
+                                    cmax = fmaxf(cmax, fabsf(c[r]));
+                                    cpoison = poison_of(cpoison, c[r]);
+                                }
+                                cmax = fmaxf(cmax, __shfl_xor(cmax, 32, WAVE));
+                                cpoison += __shfl_xor(cpoison, 32, WAVE);
+                                const float s_col = group_scale(cmax, limit, 1);
+                                uint32_t t[4];
+                                encode_words(c, s_col, cpoison, t);
+                                const int64_t gcol = col0 + l32;
+                                if (gcol < p.n && row0 < m_end) {
+                                    *reinterpret_cast<uint4*>(p.enc_t + gcol * p.m + row0 + lhi * 16) = make_uint4(t[0], t[1], t[2], t[3]);
+                                    if (lhi == 0) p.enc_t_scale[gcol * (p.m / 32) + row0 / 32] = (uint8_t)(__float_as_uint(s_col) >> 23);
+                                }
+                            }
+                        }
+                    }
+                    if (!encoded) flush(park_a, out, p.ldo, row0, col0);
                     if (aux) {
                         put(park_b, g);
                         flush(park_b, aux, 2 * p.n, row0, col0);

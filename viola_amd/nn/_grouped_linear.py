@@ -22,18 +22,27 @@ def _one_d32(group):
     return tuple(group) == (1, 32)
 
 
-def forward_core(x, weight, bias, layer, need_backward, needs, *, gated=None):
+def forward_core(x, weight, bias, layer, need_backward, needs, *, gated=None, encode=(False, False), encoded=None,
+                 input_dtype=None):
     """Returns (y, aux, record). `needs` = (needs dX, needs dW, needs db); aux is the gated
-    projection's [g, u] (None otherwise); record carries what backward_core needs."""
+    projection's [g, u] (None otherwise); record carries what backward_core needs.
+
+    encode = (codes, transposed codes too): the gated projection hands h over as MXFP8 codes, and y becomes the tuple
+    (codes, scale, codes_t, scale_t) (_grouped_linear.py:28-32). encoded = (scale, codes_t, scale_t) marks x as such
+    codes, of an activation of dtype input_dtype (_grouped_linear.py:11-18, 44-46)."""
     shape = x.shape
-    x_dtype = x.dtype
+    x_dtype = x.dtype if encoded is None else input_dtype
     x2 = x.reshape(-1, layer.in_features).contiguous()
     gx, gw = layer.input_group_shape, layer.weight_group_shape
     native = layer._native_scaling
     limit = layer._group_limit(gx, layer.fp8_dtype)
     save_fp8 = need_backward and needs[1] and layer.saved_input_dtype == "fp8"
     xt = sxt = None
-    if save_fp8 and _one_d32(gx):
+    if encoded is not None:
+        qx, sx = x2, encoded[0]
+        if save_fp8:
+            xt, sxt = encoded[1:]
+    elif save_fp8 and _one_d32(gx):
         qx, sx, xt, sxt = kernels.quantize_dual(x2, layer.fp8_dtype, gx, limit=limit, native=native)
     else:
         qx, sx = kernels.quantize(x2, layer.fp8_dtype, gx, limit=limit, native=native)
@@ -45,9 +54,11 @@ def forward_core(x, weight, bias, layer, need_backward, needs, *, gated=None):
     else:
         qw, sw = weight, layer.weight_scale
     aux = None
+    extra = None
     if gated:
-        y, aux, _ = _mlp_kernels.gemm(qx, qw, sx, sw, layer=layer, out_dtype=x_dtype, bias=bias,
-                                      activation=gated, save=need_backward)
+        y, aux, extra = _mlp_kernels.gemm(qx, qw, sx, sw, layer=layer, out_dtype=x_dtype, bias=bias,
+                                          activation=gated, save=need_backward, encode_output=encode[0],
+                                          save_output_transpose=encode[1])
     else:
         y = layer._group_gemm(qx, qw, sx, sw, gx, gw, out_dtype=x_dtype, bias=bias)
     record = None
@@ -65,6 +76,8 @@ def forward_core(x, weight, bias, layer, need_backward, needs, *, gated=None):
                                  x_dtype=x_dtype, save_fp8=save_fp8, input_limit=limit,
                                  weight_grad_dtype=weight.grad_dtype or weight.dtype,
                                  bias_grad_dtype=(bias.grad_dtype or bias.dtype) if bias is not None else None)
+    if encode[0]:
+        return (y, *extra), aux, record
     return y.reshape(*shape[:-1], y.shape[-1]), aux, record
 
 

@@ -12,13 +12,16 @@ def gemm(a, b, sa, sb, *, layer, out_dtype, activation, backward=False, aux=None
          group_a=None, group_b=None, encode_output=False, save_output_transpose=False):
     """forward: out = act(a.Wg^T) * (a.Wu^T), aux = [g, u] if save; backward: out = [d*u*act'(g), d*act(g)].
 
-    Returns (out, aux, (out_scale, out_t, out_t_scale)); the last triple is the reference's
-    in-kernel MXFP8 re-encode of H (_mlp_kernels.py:195-230), which is not built: always empty here, and the
-    caller quantizes H with the ordinary quantizer (the same codes and scales).
+    Returns (out, aux, (out_scale, out_t, out_t_scale)). With encode_output (MXFP8 forward only,
+    _mlp_kernels.py:195-230) out holds the FP8 codes of h with E8M0 scales per 32 columns in out_scale, and with
+    save_output_transpose out_t / out_t_scale hold the quantized transpose: written by the GEMM's epilogue where
+    the block-scaled MFMA path takes the shape, by the dual-layout quantizer from a BF16 h otherwise (the same
+    codes and scales either way). Without encode_output the triple is empty.
     """
-    if encode_output or save_output_transpose:
-        raise NotImplementedError("in-kernel MXFP8 re-encode of H is not built in viola_amd")
-    assert a.is_cuda
+    assert a.is_cuda and not (save_output_transpose and not encode_output)
+    if encode_output:
+        return _encoded_forward(a, b, sa, sb, layer=layer, out_dtype=out_dtype, activation=activation, bias=bias, save=save,
+                                group_a=group_a, group_b=group_b, transpose=save_output_transpose)
     a, b, sa, sb = a.contiguous(), b.contiguous(), sa.contiguous(), sb.contiguous()
     m, k = a.shape
     h = b.shape[0] if backward else b.shape[0] // 2
@@ -54,3 +57,37 @@ def gemm(a, b, sa, sb, *, layer, out_dtype, activation, backward=False, aux=None
             z, out = _gated_kernels.gated_forward(z, activation)
             aux = z if save else aux
     return out, aux, extra
+
+
+def _encoded_forward(a, b, sa, sb, *, layer, out_dtype, activation, bias, save, group_a, group_b, transpose):
+    assert layer._native_scaling, "only the MXFP8 recipe re-encodes H in the GEMM"
+    a, b, sa, sb = a.contiguous(), b.contiguous(), sa.contiguous(), sb.contiguous()
+    m, k = a.shape
+    h = b.shape[0] // 2
+    ga = tuple(group_a or layer.input_group_shape)
+    gb = tuple(group_b or layer.weight_group_shape)
+    fp8 = layer.fp8_dtype
+    limit = layer._group_limit(layer.input_group_shape, fp8) or torch.finfo(fp8).max
+    if ga[1] == 32 and gb[1] == 32 and m % 32 == 0 and h % 32 == 0:
+        aux = torch.empty((m, 2 * h) if save else (0, 0), device=a.device, dtype=out_dtype)
+        codes = torch.empty((m, h), device=a.device, dtype=fp8)
+        scale = torch.empty((m, h // 32), device=a.device, dtype=torch.uint8)
+        codes_t = torch.empty((h, m) if transpose else (0, 0), device=a.device, dtype=fp8)
+        scale_t = torch.empty((h, m // 32) if transpose else (0, 0), device=a.device, dtype=torch.uint8)
+        bias_c = bias.contiguous() if bias is not None else None
+        status = _lib.call("viola_mx_gated_gemm_encode", _lib.ptr(a), _lib.code(a.dtype), _lib.ptr(b), _lib.code(b.dtype),
+                           _lib.ptr(sa), _lib.ptr(sb), m, h, k, ga[0], gb[0], _lib.ptr(bias_c),
+                           _lib.code(bias_c.dtype) if bias_c is not None else 0, _lib.ptr(aux) if save else None,
+                           _lib.code(out_dtype), _lib.ptr(codes), _lib.ptr(scale), _lib.ptr(codes_t) if transpose else None,
+                           _lib.ptr(scale_t) if transpose else None, _lib.code(fp8), float(limit), _lib.ACTIVATION[activation],
+                           unsupported_ok=True)
+        if status == 0:
+            return codes, aux, (scale, codes_t, scale_t)
+    hidden, aux, _ = gemm(a, b, sa, sb, layer=layer, out_dtype=out_dtype, activation=activation, bias=bias, save=save,
+                          group_a=group_a, group_b=group_b)
+    if transpose:
+        codes, scale, codes_t, scale_t = _grouped_kernels.quantize_dual(hidden, fp8, (1, 32), limit=limit, native=True)
+    else:
+        codes, scale = _grouped_kernels.quantize(hidden, fp8, (1, 32), limit=limit, native=True)
+        codes_t, scale_t = hidden.new_empty((0, 0), dtype=fp8), scale.new_empty((0, 0))
+    return codes, aux, (scale, codes_t, scale_t)
