@@ -74,6 +74,12 @@ int viola_group_dequantize(const void* q, int q_dtype, const float* scale, int64
  * out [batch, cols, rows] (the reference transposes one matrix per call; batch > 1 serves stacked expert weights). */
 int viola_fp8_transpose(const void* x, void* out, int64_t batch, int64_t rows, int64_t cols, viola_stream_t stream);
 
+/* viola/nn/_grouped_kernels.py:161-164 `transpose` of a 2-D-block-scaled code matrix (gr >= 32): the payload transposes
+ * exactly and the scale grid [ceil(rows / gr), ceil(cols / gc)] (FP32 or E8M0 bytes, scale_format) is transposed with
+ * it: out [cols, rows], scale_out [ceil(cols / gc), ceil(rows / gr)], one launch. */
+int viola_block_transpose(const void* x, void* out, int64_t rows, int64_t cols, const void* scale, void* scale_out,
+                          int gr, int gc, int scale_format, viola_stream_t stream);
+
 /* ---------------------------------------------------------------- per-tensor scaling (`current` / `delayed`)
  * viola/nn/_linear_kernels.py:231-242 `tensor_scale` = _amax_kernel :33-46 + _scale_kernel :49-71.
  * viola_tensor_amax: maxima[i] = max |x| over part i of `parts` (NaN dropped); maxima is caller scratch of `parts`

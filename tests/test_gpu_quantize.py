@@ -198,3 +198,19 @@ def test_full_size_properties():
     # idempotence: quantizing the dequantized tensor reproduces codes and scales
     q3, s3 = g.quantize(g.dequantize(q, s, (1, 32)), E4, (1, 32))
     assert torch.equal(q3.view(torch.uint8), q.view(torch.uint8)) and torch.equal(s3, s)
+
+
+@pytest.mark.parametrize("native", [False, True])
+@pytest.mark.parametrize("shape,group", [((96, 128), (32, 32)), ((4096, 1024), (32, 32)), ((65, 100), (32, 64)), ((130, 33), (64, 32)),
+                                         ((7, 5), (32, 32))])
+def test_block_transpose_moves_codes_and_scale_grid_in_one_launch(shape, group, native):
+    """viola/nn/_grouped_kernels.py:161-164: a 2-D-block-scaled matrix transposes exactly, payload and scale grid."""
+    from viola_amd.nn import _grouped_kernels as g
+    torch.manual_seed(19)
+    x = torch.randn(shape) * torch.logspace(-3, 3, shape[1])
+    q, s = og.quantize(x, E4, group, native=native)
+    qt, st = g.transpose(q.cuda(), s.cuda(), group, native=native)
+    want_q, want_s = og.transpose(q, s, group, native=native)
+    assert qt.shape == (shape[1], shape[0]) and st.dtype == s.dtype
+    assert torch.equal(qt.cpu().view(torch.uint8), want_q.view(torch.uint8)) and torch.equal(st.cpu(), want_s)
+    assert torch.equal(st.cpu(), s.T) and torch.equal(qt.cpu().view(torch.uint8), q.view(torch.uint8).T)

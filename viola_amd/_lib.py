@@ -24,6 +24,7 @@ _SIGNATURES = {
     "viola_column_reduce": [_p, _l, _l, _p, _i, _p],
     "viola_group_dequantize": [_p, _i, _p, _l, _l, _i, _i, _p, _p],
     "viola_fp8_transpose": [_p, _p, _l, _l, _l, _p],
+    "viola_block_transpose": [_p, _p, _l, _l, _p, _p, _i, _i, _i, _p],
     "viola_group_gemm": [_p, _i, _p, _i, _p, _p, _l, _l, _l, _i, _i, _i, _i, _p, _i, _p, _i, _p],
     "viola_gated_gemm": [_p, _i, _p, _i, _p, _p, _l, _l, _l, _i, _i, _i, _i, _p, _i, _p, _p, _i, _i, _i, _p],
     "viola_varlen_group_gemm": [_p, _i, _p, _i, _p, _p, _p, _i, _l, _l, _l, _i, _i, _i, _i, _l, _l, _p, _i, _p],

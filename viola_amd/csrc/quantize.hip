@@ -496,10 +496,23 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const TQ* __restrict__ 
 // WORDS: rows and cols multiples of 4 and both pointers 4-byte aligned. A thread then owns a 4 x 4 byte block: four
 // 4-byte loads (16 lanes cover 64 contiguous bytes of a row), a 4 x 4 transpose with byte permutes, the four words
 // handed over through LDS so that the stores are again 64 contiguous bytes per 16 lanes.
+// With a scale grid (one entry of scale_bytes bytes per block of codes, [srows, scols]), the grid is transposed in the
+// same launch: the blocks share out its entries, thread 0 .. moving one each.
 template <bool WORDS>
 __global__ __launch_bounds__(256) void transpose_bytes(const uint8_t* __restrict__ x, uint8_t* __restrict__ out,
-                                                        int64_t rows, int64_t cols) {
+                                                        int64_t rows, int64_t cols, const uint8_t* __restrict__ scale = nullptr,
+                                                        uint8_t* __restrict__ scale_out = nullptr, int64_t srows = 0,
+                                                        int64_t scols = 0, int scale_bytes = 0) {
     const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+    if (scale) {
+        const int64_t entries = srows * scols, blocks = (int64_t)gridDim.x * gridDim.y;
+        const int64_t per = (entries + blocks - 1) / blocks, first = ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * per;
+        for (int64_t e = first + threadIdx.x; e < first + per && e < entries; e += blockDim.x) {
+            const int64_t sr = e / scols, sc = e % scols;
+            if (scale_bytes == 4) reinterpret_cast<float*>(scale_out)[sc * srows + sr] = reinterpret_cast<const float*>(scale)[e];
+            else scale_out[sc * srows + sr] = scale[e];
+        }
+    }
     x += (int64_t)blockIdx.z * rows * cols;
     out += (int64_t)blockIdx.z * rows * cols;
     if constexpr (WORDS) {
@@ -869,6 +882,22 @@ extern "C" int viola_group_dequantize(const void* q, int q_dtype, const float* s
     return viola_launch_status();
 }
 
+extern "C" int viola_block_transpose(const void* x, void* out, int64_t rows, int64_t cols, const void* scale, void* scale_out,
+                                     int gr, int gc, int scale_format, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(rows >= 0 && cols >= 0 && gr > 0 && gc > 0 && (scale_format == VIOLA_SCALE_F32 || scale_format == VIOLA_SCALE_E8M0));
+    if (rows == 0 || cols == 0) return 0;
+    VIOLA_CHECK_ARG(x && out && scale && scale_out && (rows + 63) / 64 <= 65535);
+    const int scale_bytes = scale_format == VIOLA_SCALE_F32 ? 4 : 1;
+    VIOLA_CHECK_ARG(reinterpret_cast<uintptr_t>(scale) % scale_bytes == 0 && reinterpret_cast<uintptr_t>(scale_out) % scale_bytes == 0);
+    const int64_t srows = (rows + gr - 1) / gr, scols = (cols + gc - 1) / gc;
+    const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64), 1);
+    const bool words = rows % 4 == 0 && cols % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 4 == 0;
+    if (words) hipLaunchKernelGGL(transpose_bytes<true>, grid, dim3(256), 0, stream, static_cast<const uint8_t*>(x), static_cast<uint8_t*>(out), rows, cols, static_cast<const uint8_t*>(scale), static_cast<uint8_t*>(scale_out), srows, scols, scale_bytes);
+    else hipLaunchKernelGGL(transpose_bytes<false>, grid, dim3(256), 0, stream, static_cast<const uint8_t*>(x), static_cast<uint8_t*>(out), rows, cols, static_cast<const uint8_t*>(scale), static_cast<uint8_t*>(scale_out), srows, scols, scale_bytes);
+    return viola_launch_status();
+}
+
 extern "C" int viola_fp8_transpose(const void* x, void* out, int64_t batch, int64_t rows, int64_t cols, viola_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     VIOLA_CHECK_ARG(batch >= 0 && rows >= 0 && cols >= 0);
@@ -876,7 +905,7 @@ extern "C" int viola_fp8_transpose(const void* x, void* out, int64_t batch, int6
     VIOLA_CHECK_ARG(x && out && (rows + 63) / 64 <= 65535 && batch <= 65535);
     const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64), (unsigned)batch);
     const bool words = rows % 4 == 0 && cols % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 4 == 0;
-    if (words) hipLaunchKernelGGL(transpose_bytes<true>, grid, dim3(256), 0, stream, static_cast<const uint8_t*>(x), static_cast<uint8_t*>(out), rows, cols);
-    else hipLaunchKernelGGL(transpose_bytes<false>, grid, dim3(256), 0, stream, static_cast<const uint8_t*>(x), static_cast<uint8_t*>(out), rows, cols);
+    if (words) hipLaunchKernelGGL(transpose_bytes<true>, grid, dim3(256), 0, stream, static_cast<const uint8_t*>(x), static_cast<uint8_t*>(out), rows, cols, nullptr, nullptr, 0, 0, 0);
+    else hipLaunchKernelGGL(transpose_bytes<false>, grid, dim3(256), 0, stream, static_cast<const uint8_t*>(x), static_cast<uint8_t*>(out), rows, cols, nullptr, nullptr, 0, 0, 0);
     return viola_launch_status();
 }

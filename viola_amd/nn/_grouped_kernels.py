@@ -92,7 +92,15 @@ def transpose_group(group):
 
 def transpose(q, scale, group, *, native=False, limit=None):
     if group[0] >= 32:
-        return transpose_payload(q), scale.T.contiguous()
+        # a 2-D block transposes exactly: codes and scale grid move in one launch
+        assert q.is_cuda and q.dim() == 2 and scale.dim() == 2
+        q, scale = q.contiguous(), scale.contiguous()
+        out = torch.empty((q.shape[1], q.shape[0]), device=q.device, dtype=q.dtype)
+        scale_out = torch.empty((scale.shape[1], scale.shape[0]), device=q.device, dtype=scale.dtype)
+        if q.numel():
+            _lib.call("viola_block_transpose", _lib.ptr(q), _lib.ptr(out), q.shape[0], q.shape[1], _lib.ptr(scale), _lib.ptr(scale_out),
+                      group[0], group[1], int(scale.dtype == torch.uint8))
+        return out, scale_out
     return quantize(q, q.dtype, group, native=native, limit=limit, transposed=True, source_scale=scale, source_group=group)
 
 
