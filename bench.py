@@ -163,6 +163,10 @@ def main():
         for method in ("standard", "gram"):
             opt, params, elements = muon_case(method)
             step_ms, step_wall = timed(opt.step, 5, 3)
+            # the step runs its shape buckets on several streams; for per-launch durations that do not overlap each
+            # other the instrumented pass (and one timing next to it) keeps them on one
+            lanes, opt._LANES = opt._LANES, 1
+            serial_ms, _ = timed(opt.step, 3, 1)
             b = kernel_breakdown(opt.step, 2)
             ns_flops = 0.0
             for p in params:
@@ -175,7 +179,8 @@ def main():
             ns_ms = b["viola_ns_gemm"]["avg_ms"] * b["viola_ns_gemm"]["launches_per_step"]
             mom = b.get("viola_momentum_update_table") or b["viola_momentum_update"]
             upd = b.get("viola_weight_update_table") or b["viola_weight_update"]
-            extra[f"muon_{method}"] = dict(step_ms=step_ms, step_wall_ms=step_wall, muon_elements=elements,
+            extra[f"muon_{method}"] = dict(step_ms=step_ms, step_wall_ms=step_wall, streams=lanes, step_one_stream_ms=serial_ms,
+                                           muon_elements=elements,
                                            ns_gemm_ms=ns_ms, ns_tflops=ns_flops / (ns_ms * 1e-3) / 1e12,
                                            ns_frac_bf16_peak=ns_flops / (ns_ms * 1e-3) / 1e12 / PEAK["bf16_tflops"],
                                            momentum_gbs=8.03 * elements / (mom["avg_ms"] * mom["launches_per_step"] * 1e-3) / 1e9,

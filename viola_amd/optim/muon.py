@@ -50,6 +50,7 @@ class FP8Muon(MatrixOptimizer):
             master_rounding_seed=policy["master_rounding_seed"])
         self.observer = None
         self._workspace = {}
+        self._streams = {}
         self._adam_tables = {}
         self._bucket_tables = {}
         super().__init__(params, defaults, shard_state=shard_state, skip_nonfinite=skip_nonfinite)
@@ -117,7 +118,7 @@ class FP8Muon(MatrixOptimizer):
     def _step_all(self, work):
         if self.observer is not None:
             return super()._step_all(work)
-        buckets, vectors = {}, {}
+        buckets, vectors, ready = {}, {}, []
         for item in work:
             param, grad, state, group, index = item
             if not _use_muon(param, group):
@@ -131,11 +132,42 @@ class FP8Muon(MatrixOptimizer):
             bucket = buckets.setdefault(key, [])
             bucket.append(item)
             if (len(bucket) + 1) * param.numel() > self._BATCH_ELEMENTS:
-                self._step_bucket(buckets.pop(key))
-        for bucket in buckets.values():
-            self._step_bucket(bucket)
+                ready.append(buckets.pop(key))
+        ready.extend(buckets.values())
+        self._step_buckets(ready)
         for key, bucket in vectors.items():
             self._step_vectors(key, bucket)
+
+    # The chains of different buckets are independent, and a single chain leaves the GPU partly idle at every launch
+    # boundary (a Newton-Schulz GEMM of 28 matrices is ~590 tiles for 512 tile slots: its second round is nearly
+    # empty). Buckets therefore go to up to _LANES streams of default priority, each with its own workspace, so the
+    # blocks of one chain fill the tails of the others; the caller's stream waits for all of them at the end.
+    _LANES = 4
+
+    def _step_buckets(self, ready):
+        devices = {bucket[0][0].device for bucket in ready}
+        if len(ready) < 2 or self._LANES < 2 or len(devices) != 1 or not ready[0][0][0].is_cuda:
+            for bucket in ready:
+                self._step_bucket(bucket)
+            return
+        device = ready[0][0][0].device
+        lanes = self._streams.setdefault(device, [])
+        while len(lanes) < min(self._LANES, len(ready)):
+            lanes.append(torch.cuda.Stream(device=device))
+        main = torch.cuda.current_stream(device)
+        start = torch.cuda.Event()
+        start.record(main)
+        # largest chains first, one lane after the other: the long ones start together and the short ones pack behind
+        order = sorted(range(len(ready)), key=lambda i: -len(ready[i]) * ready[i][0][0].numel())
+        for slot, i in enumerate(order):
+            lane = slot % len(lanes)
+            lanes[lane].wait_event(start)
+            with torch.cuda.stream(lanes[lane]):
+                self._step_bucket(ready[i], lane=lane)
+        for stream in lanes:
+            done = torch.cuda.Event()
+            done.record(stream)
+            main.wait_event(done)
 
     # Vectors (biases, norms, modulation tables) are a few thousand elements each: those that share dtypes,
     # hyper-parameters and step count take AdamW in one launch over a table of their pointers.
@@ -161,13 +193,13 @@ class FP8Muon(MatrixOptimizer):
         for _, _, state, _, _ in bucket:
             state["step"] += 1
 
-    def _step_bucket(self, bucket):
+    def _step_bucket(self, bucket, lane=0):
         param, _, _, group, _ = bucket[0]
         shape = _shape(param, group)
         count = param.numel()
-        work = self._workspace.get(param.device)
+        work = self._workspace.get((param.device, lane))
         if work is None or work.numel() < len(bucket) * count:
-            work = self._workspace[param.device] = torch.empty(len(bucket) * count, device=param.device, dtype=torch.bfloat16)
+            work = self._workspace[(param.device, lane)] = torch.empty(len(bucket) * count, device=param.device, dtype=torch.bfloat16)
         tables = self._bucket_tables.setdefault((shape, param.device, len(bucket)), ({}, {}))
         # one launch for the momentum of the whole bucket when its members share the recipe, else one per matrix
         uniform = lambda *names: all(all(item[3][name] == group[name] for name in names) for item in bucket)
