@@ -129,6 +129,8 @@ def main():
     parser.add_argument("--skip-cpu", action="store_true", help="leave out the CPU baseline leg")
     parser.add_argument("--skip-muon", action="store_true", help="leave out the FP8Muon / codec legs")
     parser.add_argument("--skip-mlp", action="store_true", help="leave out the gated MLP leg")
+    parser.add_argument("--muon-streams", type=int, default=0, help="streams FP8Muon.step spreads its shape buckets over "
+                        "(0: the optimizer's default; 1 keeps a kernel trace free of overlapping launches)")
     parser.add_argument("--calibrate", action="store_true",
                         help="also launch copy_scaled_kernel once over 64 Mi floats (256 MiB read, 256 MiB written): "
                              "the known-size kernel that FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -162,6 +164,8 @@ def main():
     if not args.skip_muon:
         for method in ("standard", "gram"):
             opt, params, elements = muon_case(method)
+            if args.muon_streams:
+                opt._LANES = args.muon_streams
             step_ms, step_wall = timed(opt.step, 5, 3)
             # the step runs its shape buckets on several streams; for per-launch durations that do not overlap each
             # other the instrumented pass (and one timing next to it) keeps them on one
