@@ -288,3 +288,35 @@ def test_full_size_momentum_properties():
     q2, s2 = torch.zeros_like(q), torch.ones_like(s)
     k.momentum_update(g, q2, s2, q2, s2, u, beta=.95, tile_size=256, nesterov=False)
     assert torch.equal(q, q2) and torch.equal(s, s2)
+
+
+@pytest.mark.parametrize("method", ["standard", "gram"])
+def test_fp8muon_buckets_on_several_streams_equal_one_stream(method):
+    """FP8Muon.step spreads independent shape buckets over streams; a shape that is split into several buckets (batch
+    limit) gives those their own pointer tables. Parameters and states after three steps are bit-equal to the
+    single-stream, unsplit optimizer."""
+    import viola_amd
+    shapes = [(256, 128)] * 6 + [(128, 384)] * 3 + [(192, 192)] * 2 + [(64,)] * 4
+    def build(lanes, limit):
+        torch.manual_seed(5)
+        params = [torch.nn.Parameter(torch.randn(*shape, device="cuda") * .05) for shape in shapes]
+        opt = viola_amd.optim.FP8Muon(params, lr=2e-3, weight_decay=.01, tile_size=64, ns_method=method, rounding="stochastic",
+                                      rounding_seed=9)
+        opt._LANES, opt._BATCH_ELEMENTS = lanes, limit
+        return params, opt
+    many, opt_many = build(4, 2 * 256 * 128 + 1)                              # (256, 128) goes in three buckets of two
+    one, opt_one = build(1, 1 << 28)
+    for step in range(3):
+        torch.manual_seed(100 + step)
+        grads = [torch.randn(*shape, device="cuda") * 1e-2 for shape in shapes]
+        for params, opt in ((many, opt_many), (one, opt_one)):
+            for p, g in zip(params, grads):
+                p.grad = g.clone()
+            opt.step()
+    torch.cuda.synchronize()
+    assert len(opt_many._streams[many[0].device]) == 4
+    for a, b in zip(many, one):
+        assert torch.equal(a, b)
+        for key in ("momentum_q", "momentum_scale", "exp_avg", "exp_avg_sq"):
+            if key in opt_many.state[a]:
+                assert torch.equal(opt_many.state[a][key], opt_one.state[b][key])

@@ -146,9 +146,16 @@ class FP8Muon(MatrixOptimizer):
 
     def _step_buckets(self, ready):
         devices = {bucket[0][0].device for bucket in ready}
+        # buckets of one shape and size (a shape split because it exceeds _BATCH_ELEMENTS) each keep their own pointer
+        # tables: a table must not be rewritten while another stream's launch still reads it
+        seen, ordinals = {}, []
+        for bucket in ready:
+            key = (_shape(bucket[0][0], bucket[0][3]), len(bucket))
+            ordinals.append(seen.get(key, 0))
+            seen[key] = ordinals[-1] + 1
         if len(ready) < 2 or self._LANES < 2 or len(devices) != 1 or not ready[0][0][0].is_cuda:
-            for bucket in ready:
-                self._step_bucket(bucket)
+            for bucket, ordinal in zip(ready, ordinals):
+                self._step_bucket(bucket, ordinal=ordinal)
             return
         device = ready[0][0][0].device
         lanes = self._streams.setdefault(device, [])
@@ -163,7 +170,7 @@ class FP8Muon(MatrixOptimizer):
             lane = slot % len(lanes)
             lanes[lane].wait_event(start)
             with torch.cuda.stream(lanes[lane]):
-                self._step_bucket(ready[i], lane=lane)
+                self._step_bucket(ready[i], lane=lane, ordinal=ordinals[i])
         for stream in lanes:
             done = torch.cuda.Event()
             done.record(stream)
@@ -193,14 +200,14 @@ class FP8Muon(MatrixOptimizer):
         for _, _, state, _, _ in bucket:
             state["step"] += 1
 
-    def _step_bucket(self, bucket, lane=0):
+    def _step_bucket(self, bucket, lane=0, ordinal=0):
         param, _, _, group, _ = bucket[0]
         shape = _shape(param, group)
         count = param.numel()
         work = self._workspace.get((param.device, lane))
         if work is None or work.numel() < len(bucket) * count:
             work = self._workspace[(param.device, lane)] = torch.empty(len(bucket) * count, device=param.device, dtype=torch.bfloat16)
-        tables = self._bucket_tables.setdefault((shape, param.device, len(bucket)), ({}, {}))
+        tables = self._bucket_tables.setdefault((shape, param.device, len(bucket), ordinal), ({}, {}))
         # one launch for the momentum of the whole bucket when its members share the recipe, else one per matrix
         uniform = lambda *names: all(all(item[3][name] == group[name] for name in names) for item in bucket)
         items = []
