@@ -91,7 +91,15 @@ def ptr(tensor):
     return tensor.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def stream():
+    """Handle of the current stream of the current device (the raw accessors cost a tenth of building a Stream object,
+    which matters with a dozen launches in a 0.2 ms step)."""
+    if _raw_stream is not None and _raw_device is not None:
+        return _raw_stream(_raw_device())
     return torch.cuda.current_stream().cuda_stream
 
 
