@@ -96,6 +96,12 @@ int viola_tensor_scale(const float* maxima, int64_t parts, float* history, int h
 int viola_tensor_amax_columns(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t slices, float* maxima,
                               float* column_partial, viola_stream_t stream);
 
+/* viola_tensor_amax_columns + viola_tensor_scale + viola_column_reduce behind one call (maxima: ceil(cols / piece / 256)
+ * * slices floats of scratch, column_partial: slices * cols floats of scratch, column_sum [cols] of sum_dtype). */
+int viola_tensor_amax_columns_scale(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t slices, float* maxima,
+                                    float* column_partial, float* history, int history_len, int64_t index, int delayed,
+                                    float limit, float* scale, void* column_sum, int sum_dtype, viola_stream_t stream);
+
 /* Both launches of `tensor_scale` behind one call. */
 int viola_tensor_amax_scale(const void* x, int x_dtype, int64_t n, float* maxima, int64_t parts, float* history,
                             int history_len, int64_t index, int delayed, float limit, float* scale, viola_stream_t stream);

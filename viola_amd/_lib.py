@@ -38,6 +38,7 @@ _SIGNATURES = {
     "viola_tensor_amax": [_p, _i, _l, _p, _l, _p],
     "viola_tensor_scale": [_p, _l, _p, _i, _l, _i, _f, _p, _p],
     "viola_tensor_amax_columns": [_p, _i, _l, _l, _l, _p, _p, _p],
+    "viola_tensor_amax_columns_scale": [_p, _i, _l, _l, _l, _p, _p, _p, _i, _l, _i, _f, _p, _p, _i, _p],
     "viola_tensor_amax_scale": [_p, _i, _l, _p, _l, _p, _i, _l, _i, _f, _p, _p],
     "viola_tensor_quantize": [_p, _i, _l, _l, _p, _p, _p, _i, _f, _p],
     "viola_rotation_amax": [_p, _i, _l, _l, _p, _l, _p],

@@ -374,6 +374,22 @@ extern "C" int viola_tensor_amax_columns(const void* x, int x_dtype, int64_t row
     return viola_launch_status();
 }
 
+// viola_tensor_amax_columns, viola_tensor_scale and viola_column_reduce behind one call: the per-tensor scale of a
+// [rows, cols] gradient and its column sums (the bias gradient) from one read, three launches, one trip from the host.
+extern "C" int viola_column_reduce(const float* partial, int64_t parts, int64_t cols, void* out, int out_dtype,
+                                   viola_stream_t stream);
+extern "C" int viola_tensor_amax_columns_scale(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t slices,
+                                               float* maxima, float* column_partial, float* history, int history_len,
+                                               int64_t index, int delayed, float limit, float* scale, void* column_sum,
+                                               int sum_dtype, viola_stream_t stream) {
+    int status = viola_tensor_amax_columns(x, x_dtype, rows, cols, slices, maxima, column_partial, stream);
+    if (status) return status;
+    const int piece = 16 / viola_dtype_size(x_dtype);
+    const int64_t parts = ((cols / piece + 255) / 256) * slices;
+    status = viola_tensor_scale(maxima, parts, history, history_len, index, delayed, limit, scale, stream);
+    return status ? status : viola_column_reduce(column_partial, slices, cols, column_sum, sum_dtype, stream);
+}
+
 extern "C" int viola_tensor_amax_scale(const void* x, int x_dtype, int64_t n, float* maxima, int64_t parts, float* history,
                                        int history_len, int64_t index, int delayed, float limit, float* scale,
                                        viola_stream_t stream) {

@@ -37,10 +37,9 @@ def tensor_scale_and_column_sum(x, sum_dtype, *, history=None, index=0, delayed=
     scale = torch.empty(1, device=x.device, dtype=torch.float32)
     total = torch.empty(cols, device=x.device, dtype=sum_dtype)
     limit = torch.finfo(fp8_dtype).max if quantization_limit is None else quantization_limit
-    _lib.call("viola_tensor_amax_columns", _lib.ptr(x), _lib.code(x.dtype), rows, cols, slices, _lib.ptr(maxima), _lib.ptr(partial))
-    _lib.call("viola_tensor_scale", _lib.ptr(maxima), parts, _lib.ptr(history), history.numel(), int(index), int(bool(delayed)),
-              float(limit), _lib.ptr(scale))
-    _lib.call("viola_column_reduce", _lib.ptr(partial), slices, cols, _lib.ptr(total), _lib.code(sum_dtype))
+    _lib.call("viola_tensor_amax_columns_scale", _lib.ptr(x), _lib.code(x.dtype), rows, cols, slices, _lib.ptr(maxima),
+              _lib.ptr(partial), _lib.ptr(history), history.numel(), int(index), int(bool(delayed)), float(limit), _lib.ptr(scale),
+              _lib.ptr(total), _lib.code(sum_dtype))
     return scale, total
 
 
