@@ -8,7 +8,7 @@ import warnings
 import torch
 
 from .matrix import MatrixOptimizer
-from ..precision import _dtype, settings
+from ..precision import _resolve as _dtype, settings
 from ._kernels import adam_update, adam_update_many, momentum_update, momentum_update_many, weight_update_many, state_sizes, weight_update
 from ._orthogonalize import METHODS
 
