@@ -228,3 +228,77 @@ def test_fp8muon_step_at_ditxl_block():
         opt.step()
     for a, b in zip(together, alone):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("recipe", ["tensor", "mxfp8"])
+@pytest.mark.parametrize("m,n,k,formats", [(4096, 12288, 256, (E4, E4)), (4100, 12300, 384, (torch.float8_e5m2, E4)),
+                                           (8192, 8192, 1024, (E4, torch.float8_e5m2))])
+def test_large_tile_gemm_of_the_fold_free_recipes(recipe, m, n, k, formats):
+    """Products with at least 768 tiles of 256 x 256 take the one-block-per-CU kernel of the per-tensor and MXFP8
+    recipes: held to an fp32 GPU matmul of the dequantized operands (ragged edges in m and n included), to the bias
+    and rounding identity, and to the 128 x 128 kernel's result on a row sample (same products, same K order)."""
+    from viola_amd.nn import _grouped_kernels as g, _linear_kernels as lk
+    torch.manual_seed(8)
+    a = (torch.randn(m, k, device="cuda") * torch.exp2(torch.randint(-3, 4, (m, 1), device="cuda").float())).bfloat16()
+    b = (torch.randn(n, k, device="cuda") * torch.exp2(torch.randint(-3, 4, (n, 1), device="cuda").float())).bfloat16()
+    bias = torch.randn(n, device="cuda")
+    if recipe == "mxfp8":
+        (qa, sa), (qb, sb) = g.quantize(a, formats[0], (1, 32), native=True), g.quantize(b, formats[1], (32, 32), native=True)
+        run = lambda qa_, sa_, **kw: g.gemm(qa_, qb, sa_, sb, (1, 32), (32, 32), native=True, **kw)
+        reference = g.dequantize(qa, sa, (1, 32)) @ g.dequantize(qb, sb, (32, 32)).T
+    else:
+        sa, sb = lk.tensor_scale(a, fp8_dtype=formats[0]), lk.tensor_scale(b, fp8_dtype=formats[1])
+        qa, qb = lk.quantize(a, sa, fp8_dtype=formats[0])[0], lk.quantize(b, sb, fp8_dtype=formats[1])[0]
+        run = lambda qa_, sa_, **kw: lk.gemm(qa_, qb, sa_, sb, **kw)
+        reference = (qa.float() * sa) @ (qb.float() * sb).T
+    out = run(qa, sa, out_dtype=torch.float32)
+    assert rel_l2(out, reference) < 2e-5
+    assert torch.equal(run(qa, sa, out_dtype=torch.bfloat16, bias=bias), (out + bias).bfloat16())
+    rows = torch.arange(0, m, 37, device="cuda")[:96]                         # 96 rows: far below the large-tile threshold
+    sample = run(qa[rows].contiguous(), sa[rows].contiguous() if recipe == "mxfp8" else sa, out_dtype=torch.float32)
+    assert torch.equal(sample, out[rows])
+
+
+@pytest.mark.parametrize("recipe", ["tensor", "mxfp8"])
+def test_large_tile_gated_gemms_equal_the_small_tile_kernels(recipe):
+    """m = 8256, h = 6208: the gated forward and backward GEMMs of the per-tensor recipe run on 256-row tiles (those
+    of the MXFP8 recipe stay on 128 x 128: their epilogues do not fit the large tile's registers); a 96-row sample of
+    the same operands runs on the 128 x 128 kernel. Same products in the same K order: bit-equal, for
+    h, [g, u] and dz, and for the MXFP8 codes of h handed to the down projection."""
+    import types
+    from viola_amd.nn import _grouped_kernels as g, _linear_kernels as lk, _mlp_kernels as mk
+    m, h, k, k2 = 8192 + 64, 6208, 256, 384
+    torch.manual_seed(12)
+    x = (torch.randn(m, k, device="cuda") * torch.exp2(torch.randint(-2, 3, (m, 1), device="cuda").float())).bfloat16()
+    w = torch.empty(2 * h, k, device="cuda").uniform_(-1 / 16, 1 / 16)
+    dy = torch.randn(m, k2, device="cuda").bfloat16()
+    w2 = torch.empty(h, k2, device="cuda").uniform_(-1 / 16, 1 / 16)
+    bias = torch.randn(2 * h, device="cuda").bfloat16()
+    rows = torch.arange(0, m, 83, device="cuda")[:96]
+    if recipe == "mxfp8":
+        layer = types.SimpleNamespace(_native_scaling=True, _grouped_scaling=True, input_group_shape=(1, 32), weight_group_shape=(32, 32),
+                                      fp8_dtype=E4, _group_limit=lambda *a, **kw: None)
+        (qx, sx), (qw, sw) = g.quantize(x, E4, (1, 32), native=True), g.quantize(w, E4, (32, 32), native=True)
+        (qg, sg), (qw2, sw2) = g.quantize(dy, E4, (1, 32), native=True), g.quantize(w2, E4, (32, 32), native=True)
+        pick = lambda q, s: (q[rows].contiguous(), s[rows].contiguous())
+        extra = dict(group_a=(1, 32), group_b=(32, 32))
+    else:
+        layer = types.SimpleNamespace(_native_scaling=False, _grouped_scaling=False)
+        sx, sw, sg, sw2 = (lk.tensor_scale(t) for t in (x, w, dy, w2))
+        qx, qw, qg, qw2 = (lk.quantize(t, s)[0] for t, s in ((x, sx), (w, sw), (dy, sg), (w2, sw2)))
+        pick = lambda q, s: (q[rows].contiguous(), s)
+        extra = {}
+    out, aux, _ = mk.gemm(qx, qw, sx, sw, layer=layer, out_dtype=torch.bfloat16, bias=bias, activation="gelu", save=True)
+    small_out, small_aux, _ = mk.gemm(*pick(qx, sx)[:1], qw, pick(qx, sx)[1], sw, layer=layer, out_dtype=torch.bfloat16, bias=bias,
+                                      activation="gelu", save=True)
+    assert torch.equal(out[rows], small_out) and torch.equal(aux[rows], small_aux)
+    dz, _, _ = mk.gemm(qg, qw2, sg, sw2, layer=layer, out_dtype=torch.bfloat16, activation="gelu", backward=True, aux=aux, **extra)
+    small_dz, _, _ = mk.gemm(pick(qg, sg)[0], qw2, pick(qg, sg)[1], sw2, layer=layer, out_dtype=torch.bfloat16, activation="gelu",
+                             backward=True, aux=small_aux, **extra)
+    assert torch.equal(dz[rows], small_dz)
+    if recipe == "mxfp8":
+        codes, _, (scale, codes_t, scale_t) = mk.gemm(qx, qw, sx, sw, layer=layer, out_dtype=torch.bfloat16, bias=bias, activation="gelu",
+                                                      save=False, encode_output=True, save_output_transpose=True)
+        want = g.quantize_dual(out, E4, (1, 32), native=True)
+        for got, expected in zip((codes, scale, codes_t, scale_t), want):
+            assert torch.equal(got.view(torch.uint8), expected.view(torch.uint8))

@@ -125,24 +125,33 @@ typedef int i32x8 __attribute__((ext_vector_type(8)));
 // group 1), so lane (row, half) hands over the scale byte of K group `half` of its row. Scales travel in blocks of 16
 // K groups (one 16-byte piece per tile row and operand), double-buffered behind the ring; k must be a multiple of 128.
 constexpr int MX_GROUPS = 16, MX_CHUNKS = MX_GROUPS / FKG, MX_BLOCK = 2 * BM * MX_GROUPS;   // bytes of one block, a then b
-template <int MODE, bool A_BF8, bool B_BF8, bool B_ROWSCALE, typename TO, int TN, bool TENSOR = false, bool MX = false>
-__global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(GemmArgs p, int bias_dtype) {
+// BIG (per-tensor and block-scaled recipes): a 256 x 256 tile per 512-thread block, 2 x 4 waves of 4 x 2
+// sub-tiles, one block per CU. Without the per-group fold these kernels are bound by the L2 -> LDS stream (taking the
+// global loads out of the 128 x 128 kernel brings it from 1.7 to 4.4 PFLOP/s on a 16384 x 22016 x 4096 product, taking
+// the LDS reads out changes nothing); the larger tile moves half the bytes per flop.
+template <int MODE, bool A_BF8, bool B_BF8, bool B_ROWSCALE, typename TO, int TN, bool TENSOR = false, bool MX = false, bool BIG = false>
+__global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) void group_gemm_fast(GemmArgs p, int bias_dtype) {
     static_assert(!TENSOR || !B_ROWSCALE, "per-tensor scaling has no row scales");
     static_assert(!MX || !TENSOR, "one scaling recipe per kernel");
+    static_assert(!BIG || ((TENSOR || MX) && TN == 2), "the large tile exists for the fold-free kernels");
     constexpr bool NOFOLD = TENSOR || MX;                                   // the products of a chunk go straight into the totals
+    constexpr int WAVES_N = BIG ? 4 : 2, THREADS = BIG ? 512 : FTHREADS;     // waves as 2 (m) x WAVES_N (n)
+    constexpr int TBM = BIG ? 2 * BM : BM;                                   // rows of a per tile
+    constexpr int K_TILE_A = BIG ? 2 * F_TILE : F_TILE, K_STAGE = BIG ? 4 * F_TILE : F_STAGE, K_RAW = FSTAGES * K_STAGE;
+    constexpr int K_MX_BLOCK = BIG ? 2 * MX_BLOCK : MX_BLOCK;
     // without scale blocks the ring plus the epilogue's bias row is all the LDS a block needs: three blocks share a CU
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[TENSOR ? F_RAW + 1024 : MX ? F_RAW + 2 * MX_BLOCK : F_LDS];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[TENSOR ? K_RAW + 1024 : MX ? K_RAW + 2 * K_MX_BLOCK : F_LDS];
 
     // wave grid 2 (m) x 2 (n), 2 x 2 sub-tiles each. Plain / gated backward: sub-tile i of wave wn covers b rows
     // 64 wn + 32 i. Gated forward: the tile's b rows are 64 gate rows then the 64 up rows of the same n, and
     // i = 0 / 1 is the gate / up sub-tile of columns 32 wn .. 32 wn + 31, so one lane holds g and u of the same n.
     constexpr bool GATED = MODE == MODE_GATED_FWD;
-    constexpr int TM = 2;
-    constexpr int PANEL = GATED ? BN / 2 : 64 * TN;
+    constexpr int TM = BIG ? 4 : 2;
+    constexpr int PANEL = GATED ? 32 * WAVES_N : 32 * TN * WAVES_N;
     static_assert(!GATED || TN == 2, "gated forward pairs a gate and an up sub-tile");
     const int tid = threadIdx.x, lane = tid % WAVE;
     const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
-    const int wm = wave / 2, wn = wave % 2;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int l32 = lane % 32, lhi = lane / 32;
 
     // ---- which problem / tile (uniform per block)
@@ -160,7 +169,7 @@ __global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(Gemm
         tile_m = first_m + t % group % rows;
         tile_n = t % group / rows;
     }
-    int64_t m_begin = (int64_t)tile_m * BM, m_end = p.m;
+    int64_t m_begin = (int64_t)tile_m * TBM, m_end = p.m;
     int64_t k_begin = 0, k_end = p.k;
     const uint8_t* bptr = p.b;
     const float* sbptr = p.sb;
@@ -211,7 +220,7 @@ __global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(Gemm
     int piece_k[2];
 #pragma unroll
     for (int it = 0; it < 2; ++it) {
-        const int unit = it * 256 + tid, r = unit >> 2, piece = (unit & 3) ^ ((r >> 2) & 3);
+        const int unit = it * THREADS + tid, r = unit >> 2, piece = (unit & 3) ^ ((r >> 2) & 3);
         goff_a[it] = (uint32_t)((a_global_row(r) - m_begin) * p.lda + piece * 16);
         goff_b[it] = (uint32_t)(b_global_row(r) * p.ldb + piece * 16);        // relative to bptr + k_begin (row span < 2 GiB)
         piece_k[it] = piece * 16;
@@ -228,11 +237,11 @@ __global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(Gemm
     // load instruction `which` (0, 1: a; 2, 3: b) of chunk c into ring stage `stage`
     auto issue_one = [&](int64_t c, int stage, int which) {
         const int64_t k0 = c * FBK;                                          // relative to k_begin
-        const uint32_t base = lds_base + (uint32_t)stage * F_STAGE + (uint32_t)wave * 1024;
+        const uint32_t base = lds_base + (uint32_t)stage * K_STAGE + (uint32_t)wave * 1024;
         const int it = which & 1;
         const bool inside = k0 + piece_k[it] < k_len;
-        if (which < 2) load16_to_lds(res_a, base + it * 4096, inside ? goff_a[it] : OUTSIDE, (uint32_t)k0);
-        else load16_to_lds(res_b, base + F_TILE + it * 4096, inside ? goff_b[it] : OUTSIDE, (uint32_t)k0);
+        if (which < 2) load16_to_lds(res_a, base + it * THREADS * 16, inside ? goff_a[it] : OUTSIDE, (uint32_t)k0);
+        else load16_to_lds(res_b, base + K_TILE_A + it * THREADS * 16, inside ? goff_b[it] : OUTSIDE, (uint32_t)k0);
     };
     constexpr int CHUNK_LOADS = 2 + B_LOADS;
     auto issue = [&](int64_t c, int stage) {
@@ -250,12 +259,12 @@ __global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(Gemm
     // MX: scale block `block` (K groups 16 block ..) -> buffer block & 1: waves 0, 1 fetch the a rows' pieces, waves 2, 3 the b rows'
     const i32x4 res_mxa = raw_resource(p.sa, (p.m + p.ar - 1) / p.ar * p.ldsa);
     const i32x4 res_mxb = raw_resource(sbptr, (b_rows_total + p.br - 1) / p.br * p.ldsb);
-    const uint32_t mx_off = tid < BM ? (uint32_t)(a_global_row(tid) / p.ar * p.ldsa + (k_begin >> 5))
-                                     : (uint32_t)(b_global_row(tid - BM) / p.br * p.ldsb + (k_begin >> 5));
+    const uint32_t mx_off = tid < TBM ? (uint32_t)(a_global_row(tid) / p.ar * p.ldsa + (k_begin >> 5))
+                                      : (uint32_t)(b_global_row(tid - TBM) / p.br * p.ldsb + (k_begin >> 5));
     auto issue_mx_scales = [&](int64_t block) {
         const bool inside = block * MX_GROUPS < groups_total;
-        const uint32_t at = lds_base + F_RAW + (uint32_t)(block & 1) * MX_BLOCK + (uint32_t)wave * 1024;
-        load16_to_lds(wave < 2 ? res_mxa : res_mxb, at, inside ? mx_off : OUTSIDE, (uint32_t)(block * MX_GROUPS));
+        const uint32_t at = lds_base + K_RAW + (uint32_t)(block & 1) * K_MX_BLOCK + (uint32_t)wave * 1024;
+        load16_to_lds(wave < TBM / 64 ? res_mxa : res_mxb, at, inside ? mx_off : OUTSIDE, (uint32_t)(block * MX_GROUPS));
     };
     // raw area -> [group][row] floats of scale buffer `block & 1`; groups past the k range become zero (their
     // products are zero too, and a neighbouring row's value must not meet them)
@@ -310,8 +319,8 @@ __global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(Gemm
         return reinterpret_cast<const float*>(lds + F_SCALE + ((c / F_SCHUNKS) & 1) * 2 * F_SBLOCK) + (c % F_SCHUNKS) * FKG * BM;
     };
     auto read_operands = [&](int stage, int64_t c, Operands& o) {
-        const uint8_t* tile_a = lds + stage * F_STAGE;
-        const uint8_t* tile_b = tile_a + F_TILE;
+        const uint8_t* tile_a = lds + stage * K_STAGE;
+        const uint8_t* tile_b = tile_a + K_TILE_A;
         const float* scale_a = scale_block(c);
         const float* scale_b = scale_a + F_SBLOCK / 4;
         if constexpr (NOFOLD) {
@@ -331,11 +340,11 @@ __global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(Gemm
                 o.wide_b[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
             }
             if constexpr (MX) {
-                const uint8_t* block = lds + F_RAW + ((c / MX_CHUNKS) & 1) * MX_BLOCK + (c % MX_CHUNKS) * FKG + lhi;
+                const uint8_t* block = lds + K_RAW + ((c / MX_CHUNKS) & 1) * K_MX_BLOCK + (c % MX_CHUNKS) * FKG + lhi;
 #pragma unroll
                 for (int j = 0; j < TM; ++j) o.mx_a[j] = block[(a_sub(j) + l32) * MX_GROUPS];
 #pragma unroll
-                for (int i = 0; i < TN; ++i) o.mx_b[i] = block[BM * MX_GROUPS + (b_sub(i) + l32) * MX_GROUPS];
+                for (int i = 0; i < TN; ++i) o.mx_b[i] = block[TBM * MX_GROUPS + (b_sub(i) + l32) * MX_GROUPS];
             }
             return;
         }
@@ -518,7 +527,7 @@ __global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(Gemm
         // stage ring is free now) and stores them as 16-byte pieces along the rows instead.
         constexpr int PER = 16 / (int)sizeof(TO);                            // values per piece
         constexpr int WCOLS = 32 * TN, PLD = WCOLS + PER, PIECES = WCOLS / PER;
-        static_assert(4 * 32 * PLD * (int)sizeof(TO) <= F_RAW, "parking area fits in the stage ring");
+        static_assert(2 * WAVES_N * 32 * PLD * (int)sizeof(TO) <= K_RAW, "parking area fits in the stage ring");
         if ((p.ldo * sizeof(TO)) % 16 == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
             __syncthreads();                                                 // every wave has left the ring
             TO* park = reinterpret_cast<TO*>(lds) + wave * 32 * PLD;
@@ -526,8 +535,8 @@ __global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(Gemm
             // the tile's bias as fp32 in the (now idle) raw scale area: one global load per column, not per element
             float4 bias_q[TN][4];
             if (p.bias) {
-                float* bias_lds = reinterpret_cast<float*>(lds + F_RAW);
-                if (tid < 64 * TN) bias_lds[tid] = n_begin + tid < p.n ? load_bias(p.bias, n_begin + tid, bias_dtype) : 0.0f;
+                float* bias_lds = reinterpret_cast<float*>(lds + K_RAW);
+                if (tid < PANEL) bias_lds[tid] = n_begin + tid < p.n ? load_bias(p.bias, n_begin + tid, bias_dtype) : 0.0f;
                 __syncthreads();
 #pragma unroll
                 for (int i = 0; i < TN; ++i)
@@ -574,7 +583,7 @@ __global__ __launch_bounds__(FTHREADS, TENSOR ? 3 : 2) void group_gemm_fast(Gemm
         // of the (idle) stage ring and move to and from global memory as 16-byte pieces along the rows; one lane = one
         // row and runs of four columns would touch 32 cache lines per instruction. Needs 16-byte aligned rows.
         constexpr int PER = 16 / (int)sizeof(TO), PLD = 32 + PER, PIECES = 32 / PER, AREA = 32 * PLD;
-        static_assert(4 * 2 * AREA * (int)sizeof(TO) <= F_RAW, "parking areas fit in the stage ring");
+        static_assert(2 * WAVES_N * 2 * AREA * (int)sizeof(TO) <= K_RAW, "parking areas fit in the stage ring");
         TO* aux = static_cast<TO*>(p.aux);
         if ((p.n * sizeof(TO)) % 16 == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0 && (reinterpret_cast<uintptr_t>(aux) & 15) == 0) {
             __syncthreads();                                                 // every wave has left the ring

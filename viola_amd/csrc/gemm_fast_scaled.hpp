@@ -16,10 +16,48 @@ static void launch_scaled_formats(const GemmArgs& p, int a_dtype, int b_dtype, i
     else hipLaunchKernelGGL((group_gemm_fast<MODE, true, true, false, TO, TN, TENSOR, MX>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
 }
 
+// The 256 x 256 tile (one 512-thread block per CU) for products with at least three rounds of such tiles.
+template <int MODE, typename TO, bool TENSOR, bool MX>
+static void launch_big_formats(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, dim3 grid, hipStream_t stream) {
+    const bool a5 = a_dtype == VIOLA_E5M2, b5 = b_dtype == VIOLA_E5M2;
+    if (!a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE, false, false, false, TO, 2, TENSOR, MX, true>), grid, dim3(512), 0, stream, p, bias_dtype);
+    else if (a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE, true, false, false, TO, 2, TENSOR, MX, true>), grid, dim3(512), 0, stream, p, bias_dtype);
+    else if (!a5 && b5) hipLaunchKernelGGL((group_gemm_fast<MODE, false, true, false, TO, 2, TENSOR, MX, true>), grid, dim3(512), 0, stream, p, bias_dtype);
+    else hipLaunchKernelGGL((group_gemm_fast<MODE, true, true, false, TO, 2, TENSOR, MX, true>), grid, dim3(512), 0, stream, p, bias_dtype);
+}
+
+template <typename TO, bool TENSOR, bool MX>
+static void launch_big_modes(const GemmArgs& p, int mode, int a_dtype, int b_dtype, int bias_dtype, dim3 grid, hipStream_t stream) {
+    if (mode == MODE_PLAIN) launch_big_formats<MODE_PLAIN, TO, TENSOR, MX>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
+    else if constexpr (!MX) {
+        if (mode == MODE_GATED_FWD) launch_big_formats<MODE_GATED_FWD, TO, TENSOR, MX>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
+        else launch_big_formats<MODE_GATED_BWD, TO, TENSOR, MX>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
+    }
+}
+
 template <bool TENSOR, bool MX>
 static int launch_scaled_gemm_fast(const GemmArgs& args, int mode, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, dim3 grid,
                                    hipStream_t stream) {
     GemmArgs p = args;
+#ifndef VIOLA_BIG_TILES_FROM
+#define VIOLA_BIG_TILES_FROM (3 * 256)
+#endif
+    // a gated forward tile is 128 columns of h wide (its 256 b rows are 128 gate and 128 up rows)
+    const int64_t big_width = mode == MODE_GATED_FWD ? 128 : 256;
+    const int64_t big_m = (p.m + 255) / 256, big_n = (p.n + big_width - 1) / big_width;
+    // (the block-scaled gated kernels do not fit the large tile's register budget: their epilogues spill)
+    if ((mode == MODE_PLAIN || !MX) && big_m * big_n >= VIOLA_BIG_TILES_FROM && big_m * big_n < (1 << 30) && 256 * p.k < (1ll << 31)) {
+        p.tiles_n = (int)big_n;
+        p.tiles_m = (int)big_m;
+        const dim3 big_grid((unsigned)((big_m * big_n + 7) / 8 * 8), 1, 1);
+        switch (out_dtype) {
+            case VIOLA_F32: launch_big_modes<float, TENSOR, MX>(p, mode, a_dtype, b_dtype, bias_dtype, big_grid, stream); break;
+            case VIOLA_BF16: launch_big_modes<bf16_t, TENSOR, MX>(p, mode, a_dtype, b_dtype, bias_dtype, big_grid, stream); break;
+            case VIOLA_F16: launch_big_modes<f16_t, TENSOR, MX>(p, mode, a_dtype, b_dtype, bias_dtype, big_grid, stream); break;
+            default: return VIOLA_EINVAL;
+        }
+        return viola_launch_status();
+    }
     const bool narrow = mode == MODE_PLAIN && (int64_t)grid.x * grid.y < 512 && p.n > 64;
     if (narrow) grid.x = (unsigned)((p.n + 63) / 64);
     if ((int64_t)grid.x * grid.y < (1 << 30)) {
