@@ -234,7 +234,7 @@ def test_fp8muon_step_at_ditxl_block():
 @pytest.mark.parametrize("m,n,k,formats", [(4096, 12288, 256, (E4, E4)), (4100, 12300, 384, (torch.float8_e5m2, E4)),
                                            (8192, 8192, 1024, (E4, torch.float8_e5m2))])
 def test_large_tile_gemm_of_the_fold_free_recipes(recipe, m, n, k, formats):
-    """Products with at least 768 tiles of 256 x 256 take the one-block-per-CU kernel of the per-tensor and MXFP8
+    """Products with at least 512 tiles of 256 x 256 take the one-block-per-CU kernel of the per-tensor and MXFP8
     recipes: held to an fp32 GPU matmul of the dequantized operands (ragged edges in m and n included), to the bias
     and rounding identity, and to the 128 x 128 kernel's result on a row sample (same products, same K order)."""
     from viola_amd.nn import _grouped_kernels as g, _linear_kernels as lk
