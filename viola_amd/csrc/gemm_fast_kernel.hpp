@@ -313,7 +313,7 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
         uint4 a[FKG][TM], b[FKG][TN];
         float sa[FKG][TM], sb[FKG][TN];
         i32x8 wide_a[TM], wide_b[TN];                                        // TENSOR / MX: 16 k of either K group of a sub-tile row
-        int mx_a[TM], mx_b[TN];                                              // MX: the row's scale byte of K group lhi
+        int mx_a[(TM + 1) / 2], mx_b[(TN + 1) / 2];                          // MX: the rows' scale bytes of K group lhi, sub-tile t in byte 2 (t & 1) of word t / 2
     };
     auto scale_block = [&](int64_t c) -> const float* {                      // a scales of chunk c: [kg][row]; b scales F_SBLOCK later
         return reinterpret_cast<const float*>(lds + F_SCALE + ((c / F_SCHUNKS) & 1) * 2 * F_SBLOCK) + (c % F_SCHUNKS) * FKG * BM;
@@ -342,9 +342,15 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
             if constexpr (MX) {
                 const uint8_t* block = lds + K_RAW + ((c / MX_CHUNKS) & 1) * K_MX_BLOCK + (c % MX_CHUNKS) * FKG + lhi;
 #pragma unroll
-                for (int j = 0; j < TM; ++j) o.mx_a[j] = block[(a_sub(j) + l32) * MX_GROUPS];
+                for (int j = 0; j < TM; j += 2) {
+                    o.mx_a[j / 2] = block[(a_sub(j) + l32) * MX_GROUPS];
+                    if (j + 1 < TM) o.mx_a[j / 2] |= block[(a_sub(j + 1) + l32) * MX_GROUPS] << 16;
+                }
 #pragma unroll
-                for (int i = 0; i < TN; ++i) o.mx_b[i] = block[TBM * MX_GROUPS + (b_sub(i) + l32) * MX_GROUPS];
+                for (int i = 0; i < TN; i += 2) {
+                    o.mx_b[i / 2] = block[TBM * MX_GROUPS + (b_sub(i) + l32) * MX_GROUPS];
+                    if (i + 1 < TN) o.mx_b[i / 2] |= block[TBM * MX_GROUPS + (b_sub(i + 1) + l32) * MX_GROUPS] << 16;
+                }
             }
             return;
         }
@@ -361,6 +367,17 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
         }
     };
 
+    // the block-scaled MFMA with the scale bytes picked out of their words (the byte index is an immediate)
+    auto mx_mfma = [](i32x8 b, i32x8 a, f32x16 c, int scale_b, int scale_a, int which) -> f32x16 {
+        constexpr int FB = B_BF8 ? 1 : 0, FA = A_BF8 ? 1 : 0;
+        switch (which) {
+            case 0: return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b, a, c, FB, FA, 0, scale_b, 0, scale_a);
+            case 1: return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b, a, c, FB, FA, 0, scale_b, 2, scale_a);
+            case 2: return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b, a, c, FB, FA, 2, scale_b, 0, scale_a);
+            default: return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b, a, c, FB, FA, 2, scale_b, 2, scale_a);
+        }
+    };
+
     // Math of chunk c on the operands in `o`; `between(step)` runs after MFMA number `step` of the chunk (the
     // caller's global loads and LDS reads for later chunks go there, spread over the chunk).
     auto compute = [&](const Operands& o, int64_t c, auto&& between) {
@@ -373,7 +390,7 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
                     // both operands give a lane the same 32 of the chunk's 64 k (16 of each K group), so every product
                     // meets its partner whatever order the instruction walks them in
                     if constexpr (MX)
-                        total[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(o.wide_b[i], o.wide_a[j], total[i][j], B_BF8 ? 1 : 0, A_BF8 ? 1 : 0, 0, o.mx_b[i], 0, o.mx_a[j]);
+                        total[i][j] = mx_mfma(o.wide_b[i], o.wide_a[j], total[i][j], o.mx_b[i / 2], o.mx_a[j / 2], (i & 1) * 2 + (j & 1));
                     else
                         total[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(o.wide_b[i], o.wide_a[j], total[i][j], B_BF8 ? 1 : 0, A_BF8 ? 1 : 0, 0, 0, 0, 0);
                     __builtin_amdgcn_sched_barrier(0);

@@ -26,12 +26,19 @@ static void launch_big_formats(const GemmArgs& p, int a_dtype, int b_dtype, int 
     else hipLaunchKernelGGL((group_gemm_fast<MODE, true, true, false, TO, 2, TENSOR, MX, true>), grid, dim3(512), 0, stream, p, bias_dtype);
 }
 
+#ifndef VIOLA_MX_BIG_GATED
+#define VIOLA_MX_BIG_GATED 0
+#endif
+// which gated kernels exist on the large tile: all per-tensor ones; of the block-scaled ones those whose registers fit
+constexpr bool big_gated(bool mx, int mode) { return !mx || (VIOLA_MX_BIG_GATED >> (mode == MODE_GATED_FWD ? 0 : 1) & 1); }
+
 template <typename TO, bool TENSOR, bool MX>
 static void launch_big_modes(const GemmArgs& p, int mode, int a_dtype, int b_dtype, int bias_dtype, dim3 grid, hipStream_t stream) {
     if (mode == MODE_PLAIN) launch_big_formats<MODE_PLAIN, TO, TENSOR, MX>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
-    else if constexpr (!MX) {
-        if (mode == MODE_GATED_FWD) launch_big_formats<MODE_GATED_FWD, TO, TENSOR, MX>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
-        else launch_big_formats<MODE_GATED_BWD, TO, TENSOR, MX>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
+    else if (mode == MODE_GATED_FWD) {
+        if constexpr (big_gated(MX, MODE_GATED_FWD)) launch_big_formats<MODE_GATED_FWD, TO, TENSOR, MX>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
+    } else {
+        if constexpr (big_gated(MX, MODE_GATED_BWD)) launch_big_formats<MODE_GATED_BWD, TO, TENSOR, MX>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
     }
 }
 
@@ -46,7 +53,7 @@ static int launch_scaled_gemm_fast(const GemmArgs& args, int mode, int a_dtype, 
     const int64_t big_width = mode == MODE_GATED_FWD ? 128 : 256;
     const int64_t big_m = (p.m + 255) / 256, big_n = (p.n + big_width - 1) / big_width;
     // (the block-scaled gated kernels do not fit the large tile's register budget: their epilogues spill)
-    if ((mode == MODE_PLAIN || !MX) && big_m * big_n >= VIOLA_BIG_TILES_FROM && big_m * big_n < (1 << 30) && 256 * p.k < (1ll << 31)) {
+    if ((mode == MODE_PLAIN || big_gated(MX, mode)) && big_m * big_n >= VIOLA_BIG_TILES_FROM && big_m * big_n < (1 << 30) && 256 * p.k < (1ll << 31)) {
         p.tiles_n = (int)big_n;
         p.tiles_m = (int)big_m;
         const dim3 big_grid((unsigned)((big_m * big_n + 7) / 8 * 8), 1, 1);
