@@ -59,6 +59,14 @@ int viola_group_quantize_dual(const void* x, int x_dtype, int64_t rows, int64_t 
                               void* q, void* scale, void* qt, void* scale_t, int q_dtype, int gc,
                               float limit, float* column_partial, int scale_format, viola_stream_t stream);
 
+/* viola_group_quantize_dual of h = act(g) * u [rows, cols], rounded to z_dtype, read from the stored projection
+ * z = [g | u] [rows, 2 cols] (bf16 / fp16) instead of from a stored h: what the MXFP8 MLP hands from its gate/up
+ * projection to its down projection (viola/nn/_mlp_kernels.py:195-230 encode h in the GEMM's epilogue; this is the
+ * same result from the saved [g | u]). VIOLA_EUNSUPPORTED for fp32 z, gc != 32, cols % 8 != 0 or unaligned z / q. */
+int viola_gated_quantize_dual(const void* z, int z_dtype, int64_t rows, int64_t cols, int activation,
+                              void* q, void* scale, void* qt, void* scale_t, int q_dtype, int gc,
+                              float limit, int scale_format, viola_stream_t stream);
+
 /* column_partial (nullable) of viola_group_quantize_dual receives [ceil(rows/32), cols] fp32 sums of x over
  * each 32-row group, taken from the same read; viola_column_reduce adds the parts in a fixed order:
  * out[c] = sum_p partial[p][c], stored as out_dtype. Together they are the bias gradient dy.sum(0)

@@ -214,3 +214,25 @@ def test_block_transpose_moves_codes_and_scale_grid_in_one_launch(shape, group, 
     assert qt.shape == (shape[1], shape[0]) and st.dtype == s.dtype
     assert torch.equal(qt.cpu().view(torch.uint8), want_q.view(torch.uint8)) and torch.equal(st.cpu(), want_s)
     assert torch.equal(st.cpu(), s.T) and torch.equal(qt.cpu().view(torch.uint8), q.view(torch.uint8).T)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("activation", ["silu", "gelu", "relu"])
+@pytest.mark.parametrize("native", [False, True])
+def test_gated_quantize_dual_equals_activation_then_quantize(dtype, activation, native):
+    """h = act(g) * u quantized in both layouts straight from [g | u] is, bit for bit, the dual quantizer run on the
+    stored h of the activation kernel; ragged rows and a width that is not a multiple of the 64-column tile."""
+    from viola_amd.nn import _gated_kernels as gk, _grouped_kernels as g
+    torch.manual_seed(5)
+    for rows, h in ((100, 72), (256, 128), (33, 8)):
+        z = (torch.randn(rows, 2 * h, device="cuda") * torch.exp2(torch.randint(-6, 5, (rows, 1), device="cuda").float())).to(dtype)
+        z[3, 5] = float("nan")
+        for fp8 in (torch.float8_e4m3fn, torch.float8_e5m2):
+            got = g.gated_quantize_dual(z, activation, fp8, native=native)
+            assert got is not None
+            _, hidden = gk.gated_forward(z, activation)
+            want = g.quantize_dual(hidden, fp8, (1, 32), native=native)
+            for a, b in zip(got, want):
+                assert torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+    assert g.gated_quantize_dual(torch.zeros(4, 2 * 12, device="cuda", dtype=dtype), activation, torch.float8_e4m3fn) is None
+    assert g.gated_quantize_dual(torch.zeros(4, 64, device="cuda"), activation, torch.float8_e4m3fn) is None

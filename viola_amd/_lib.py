@@ -21,6 +21,7 @@ _i, _l, _f, _p = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 _SIGNATURES = {
     "viola_group_quantize": [_p, _i, _l, _l, _p, _i, _p, _i, _i, _f, _i, _p, _i, _i, _i, _p],
     "viola_group_quantize_dual": [_p, _i, _l, _l, _p, _p, _p, _p, _i, _i, _f, _p, _i, _p],
+    "viola_gated_quantize_dual": [_p, _i, _l, _l, _i, _p, _p, _p, _p, _i, _i, _f, _i, _p],
     "viola_column_reduce": [_p, _l, _l, _p, _i, _p],
     "viola_group_dequantize": [_p, _i, _p, _l, _l, _i, _i, _p, _p],
     "viola_fp8_transpose": [_p, _p, _l, _l, _l, _p],

@@ -290,4 +290,21 @@ __device__ __forceinline__ T round_store(float v, uint64_t element, uint64_t ste
     return from_f32<T>(v);
 }
 
+// act(g) and act'(g) of a gated MLP (viola/nn/_mlp_kernels.py:158-194): one formula for every kernel that applies it,
+// so the fused epilogues and the stand-alone passes give the same bits.
+__device__ __forceinline__ void gate_math(int activation, float g, float& act, float& derivative) {
+    if (activation == VIOLA_SILU) {
+        const float s = 1.0f / (1.0f + expf(-g));
+        act = g * s;
+        derivative = s * (1.0f + g * (1.0f - s));
+    } else if (activation == VIOLA_GELU) {
+        const float t = tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g));
+        act = 0.5f * g * (1.0f + t);
+        derivative = 0.5f * (1.0f + t) + 0.5f * g * (1.0f - t * t) * 0.7978845608028654f * (1.0f + 0.134145f * g * g);
+    } else {
+        act = fmaxf(g, 0.0f);
+        derivative = g > 0.0f ? 1.0f : 0.0f;
+    }
+}
+
 }  // namespace viola

@@ -45,4 +45,15 @@ int launch_tensor_gemm_fast(const GemmArgs& p, int mode, int a_dtype, int b_dtyp
 int launch_mx_gemm_fast(const GemmArgs& p, int mode, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, dim3 grid,
                         hipStream_t stream);
 
+// misc.hip: the gated activation as a pass of its own, in 16-byte pieces (false: alignment does not allow them)
+bool launch_gated_pieces(const void* z, const void* dy, int64_t dy_stride, void* out, int64_t rows, int64_t h, int dtype,
+                         int activation, bool backward, hipStream_t stream);
+
+// Per-tensor and block-scaled products with at least this many 256 x 256 output tiles (two rounds of the 256 CUs)
+// run on the large tile.
+#ifndef VIOLA_BIG_TILES_FROM
+#define VIOLA_BIG_TILES_FROM (2 * 256)
+#endif
+inline bool takes_large_tiles(int64_t m, int64_t n) { return ((m + 255) / 256) * ((n + 255) / 256) >= VIOLA_BIG_TILES_FROM; }
+
 }  // namespace viola

@@ -67,21 +67,6 @@ __device__ __forceinline__ float load_bias(const void* p, int64_t i, int dtype) 
     return (float)static_cast<const _Float16*>(p)[i];
 }
 
-__device__ __forceinline__ void gate_math(int activation, float g, float& act, float& derivative) {
-    if (activation == VIOLA_SILU) {
-        const float s = 1.0f / (1.0f + expf(-g));
-        act = g * s;
-        derivative = s * (1.0f + g * (1.0f - s));
-    } else if (activation == VIOLA_GELU) {
-        const float t = tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g));
-        act = 0.5f * g * (1.0f + t);
-        derivative = 0.5f * (1.0f + t) + 0.5f * g * (1.0f - t * t) * 0.7978845608028654f * (1.0f + 0.134145f * g * g);
-    } else {
-        act = fmaxf(g, 0.0f);
-        derivative = g > 0.0f ? 1.0f : 0.0f;
-    }
-}
-
 // Four consecutive outputs of one row.
 template <typename TO> struct Quad;
 template <> struct Quad<float> {
@@ -665,6 +650,9 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
                         float act, derivative;
                         gate_math(p.activation, g[r], act, derivative);
                         h[r] = act * u[r];
+                        // an FP32 value of its own: folded into a narrowing conversion (a mixed-precision FMA with a +0
+                        // addend) the product would round once instead of twice and -0 would become +0
+                        asm volatile("" : "+v"(h[r]));
                     }
                     const int64_t row0 = m_begin + a_sub(j);
                     put(park_a, h);

@@ -156,10 +156,8 @@ __global__ __launch_bounds__(256) void gated_forward_kernel(const void* __restri
     for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
         const int64_t r = idx / h, c = idx % h;
         const float g = load_half(z, r * 2 * h + c, dtype), u = load_half(z, r * 2 * h + h + c, dtype);
-        float a;
-        if (activation == VIOLA_SILU) a = g / (1.0f + expf(-g));
-        else if (activation == VIOLA_GELU) a = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
-        else a = fmaxf(g, 0.0f);
+        float a, derivative;
+        gate_math(activation, g, a, derivative);
         store_half(out, idx, dtype, a * u);
     }
 }
@@ -222,18 +220,17 @@ __global__ __launch_bounds__(256) void gated_forward_pieces(const T* __restrict_
     Piece<T>::load(z + r * 2 * h + h + c, u);
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-        float a;
-        if constexpr (ACT == VIOLA_SILU) a = g[i] / (1.0f + expf(-g[i]));
-        else if constexpr (ACT == VIOLA_GELU) a = 0.5f * g[i] * (1.0f + tanhf(0.7978845608028654f * (g[i] + 0.044715f * g[i] * g[i] * g[i])));
-        else a = fmaxf(g[i], 0.0f);
+        float a, derivative;
+        gate_math(ACT, g[i], a, derivative);
         o[i] = a * u[i];
     }
     Piece<T>::store(out + r * h + c, o);
 }
 
 template <typename T, int ACT>
-__global__ __launch_bounds__(256) void gated_backward_pieces(const T* __restrict__ z, const T* __restrict__ dy, T* __restrict__ dz,
+__global__ __launch_bounds__(256) void gated_backward_pieces(const T* __restrict__ z, const T* dy, int64_t dy_stride, T* dz,
                                                               int64_t pieces, int64_t per_row) {
+    // dy may be the up half of dz itself (dy = dz + h, dy_stride = 2 h): a thread reads its piece before it writes there
     constexpr int N = Piece<T>::N;
     const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (id >= pieces) return;
@@ -241,22 +238,11 @@ __global__ __launch_bounds__(256) void gated_backward_pieces(const T* __restrict
     float g[N], u[N], d[N], dg[N], du[N];
     Piece<T>::load(z + r * 2 * h + c, g);
     Piece<T>::load(z + r * 2 * h + h + c, u);
-    Piece<T>::load(dy + r * h + c, d);
+    Piece<T>::load(dy + r * dy_stride + c, d);
 #pragma unroll
     for (int i = 0; i < N; ++i) {
         float a, derivative;
-        if constexpr (ACT == VIOLA_SILU) {
-            const float s = 1.0f / (1.0f + expf(-g[i]));
-            a = g[i] * s;
-            derivative = s * (1.0f + g[i] * (1.0f - s));
-        } else if constexpr (ACT == VIOLA_GELU) {
-            const float t = tanhf(0.7978845608028654f * (g[i] + 0.044715f * g[i] * g[i] * g[i]));
-            a = 0.5f * g[i] * (1.0f + t);
-            derivative = 0.5f * (1.0f + t) + 0.5f * g[i] * (1.0f - t * t) * 0.7978845608028654f * (1.0f + 0.134145f * g[i] * g[i]);
-        } else {
-            a = fmaxf(g[i], 0.0f);
-            derivative = g[i] > 0.0f ? 1.0f : 0.0f;
-        }
+        gate_math(ACT, g[i], a, derivative);
         dg[i] = d[i] * u[i] * derivative;
         du[i] = d[i] * a;
     }
@@ -265,11 +251,11 @@ __global__ __launch_bounds__(256) void gated_backward_pieces(const T* __restrict
 }
 
 template <typename T>
-static bool launch_gated_pieces(const void* z, const void* dy, void* out, int64_t rows, int64_t h, int activation, bool backward,
-                                hipStream_t stream) {
+static bool launch_gated_pieces(const void* z, const void* dy, int64_t dy_stride, void* out, int64_t rows, int64_t h, int activation,
+                                bool backward, hipStream_t stream) {
     constexpr int N = Piece<T>::N;
     const auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
-    if (h % N != 0 || !aligned(z) || !aligned(out) || (backward && !aligned(dy))) return false;
+    if (h % N != 0 || !aligned(z) || !aligned(out) || (backward && (!aligned(dy) || dy_stride % N != 0))) return false;
     const int64_t per_row = h / N, pieces = rows * per_row, blocks = (pieces + 255) / 256;
     if (blocks > 0x7fffffff) return false;
     const dim3 grid((unsigned)blocks);
@@ -277,7 +263,7 @@ static bool launch_gated_pieces(const void* z, const void* dy, void* out, int64_
     const T* dp = static_cast<const T*>(dy);
     T* op = static_cast<T*>(out);
 #define VIOLA_GATED(ACT)                                                                                                   \
-    if (backward) hipLaunchKernelGGL((gated_backward_pieces<T, ACT>), grid, dim3(256), 0, stream, zp, dp, op, pieces, per_row); \
+    if (backward) hipLaunchKernelGGL((gated_backward_pieces<T, ACT>), grid, dim3(256), 0, stream, zp, dp, dy_stride, op, pieces, per_row); \
     else hipLaunchKernelGGL((gated_forward_pieces<T, ACT>), grid, dim3(256), 0, stream, zp, op, pieces, per_row);
     if (activation == VIOLA_SILU) { VIOLA_GATED(VIOLA_SILU) }
     else if (activation == VIOLA_GELU) { VIOLA_GATED(VIOLA_GELU) }
@@ -286,11 +272,13 @@ static bool launch_gated_pieces(const void* z, const void* dy, void* out, int64_
     return true;
 }
 
-static bool launch_gated_pieces(const void* z, const void* dy, void* out, int64_t rows, int64_t h, int dtype, int activation,
-                                bool backward, hipStream_t stream) {
-    if (dtype == VIOLA_F32) return launch_gated_pieces<float>(z, dy, out, rows, h, activation, backward, stream);
-    if (dtype == VIOLA_BF16) return launch_gated_pieces<bf16_t>(z, dy, out, rows, h, activation, backward, stream);
-    return launch_gated_pieces<f16_t>(z, dy, out, rows, h, activation, backward, stream);
+// The gated activation in 16-byte pieces: forward out [rows, h] = act(g) * u from z = [g | u]; backward out [rows, 2 h] from
+// z and dy (row stride dy_stride elements). False, and nothing launched, when alignment does not allow the pieces.
+bool launch_gated_pieces(const void* z, const void* dy, int64_t dy_stride, void* out, int64_t rows, int64_t h, int dtype,
+                         int activation, bool backward, hipStream_t stream) {
+    if (dtype == VIOLA_F32) return launch_gated_pieces<float>(z, dy, dy_stride, out, rows, h, activation, backward, stream);
+    if (dtype == VIOLA_BF16) return launch_gated_pieces<bf16_t>(z, dy, dy_stride, out, rows, h, activation, backward, stream);
+    return launch_gated_pieces<f16_t>(z, dy, dy_stride, out, rows, h, activation, backward, stream);
 }
 
 // ------------------------------------------------------------------ self checks
@@ -393,7 +381,7 @@ extern "C" int viola_gated_forward(const void* z, void* out, int64_t rows, int64
     VIOLA_CHECK_ARG(viola_is_float(dtype) && rows >= 0 && h >= 0 && activation >= VIOLA_SILU && activation <= VIOLA_RELU);
     if (rows == 0 || h == 0) return 0;
     VIOLA_CHECK_ARG(z && out);
-    if (launch_gated_pieces(z, nullptr, out, rows, h, dtype, activation, false, stream)) return viola_launch_status();
+    if (launch_gated_pieces(z, nullptr, 0, out, rows, h, dtype, activation, false, stream)) return viola_launch_status();
     hipLaunchKernelGGL(gated_forward_kernel, dim3(grid_for(rows * h)), dim3(256), 0, stream, z, out, rows, h, dtype, activation);
     return viola_launch_status();
 }
@@ -404,7 +392,7 @@ extern "C" int viola_gated_backward(const void* z, const void* dy, void* dz, int
     VIOLA_CHECK_ARG(viola_is_float(dtype) && rows >= 0 && h >= 0 && activation >= VIOLA_SILU && activation <= VIOLA_RELU);
     if (rows == 0 || h == 0) return 0;
     VIOLA_CHECK_ARG(z && dy && dz);
-    if (launch_gated_pieces(z, dy, dz, rows, h, dtype, activation, true, stream)) return viola_launch_status();
+    if (launch_gated_pieces(z, dy, h, dz, rows, h, dtype, activation, true, stream)) return viola_launch_status();
     hipLaunchKernelGGL(gated_backward_kernel, dim3(grid_for(rows * h)), dim3(256), 0, stream, z, dy, dz, rows, h, dtype, activation);
     return viola_launch_status();
 }

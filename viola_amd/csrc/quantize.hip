@@ -212,11 +212,18 @@ template <> __device__ __forceinline__ float widen16<f16_t>(uint32_t bits) {
     return (float)__builtin_bit_cast(_Float16, b);
 }
 
-template <typename TIn, typename TOut, bool ROWWISE>
+template <typename TIn> __device__ __forceinline__ uint32_t narrow16(float v);
+template <> __device__ __forceinline__ uint32_t narrow16<bf16_t>(float v) { return f32_to_bf16_bits(v); }
+template <> __device__ __forceinline__ uint32_t narrow16<f16_t>(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+
+// GATED: x is [rows, 2 cols] = [gate | up] and the tile quantized is act(gate) * up [rows, cols]
+// (viola/nn/_mlp_kernels.py:195-230 hands h over as codes; here from the stored projection instead of the accumulators).
+template <typename TIn, typename TOut, bool ROWWISE, bool GATED = false>
 __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x, uint8_t* __restrict__ q,
                                                         float* __restrict__ scale, uint8_t* __restrict__ qt,
                                                         float* __restrict__ scale_t, int64_t rows, int64_t cols,
-                                                        float limit, float* __restrict__ column_partial, int e8m0) {
+                                                        float limit, float* __restrict__ column_partial, int e8m0,
+                                                        int activation = 0) {
     constexpr int LD = 64 + 32;
     typedef short s16x4 __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
@@ -235,12 +242,39 @@ __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x
     const int64_t col8 = c0 + ch * 8;
 
     // all four loads first, without control flow: a raw buffer over the wavefront's 32 rows returns zero past its end
-    const int64_t span = (rows - r0 < 32 ? rows - r0 : 32) * cols * 2;
-    const __amdgpu_buffer_rsrc_t res = __builtin_amdgcn_make_buffer_rsrc(const_cast<TIn*>(x + r0 * cols), 0, (int)span, 0x00020000);
+    constexpr int WIDTH = GATED ? 2 : 1;                                     // x rows are [gate | up] when GATED
+    const int64_t span = (rows - r0 < 32 ? rows - r0 : 32) * cols * 2 * WIDTH;
+    const __amdgpu_buffer_rsrc_t res = __builtin_amdgcn_make_buffer_rsrc(const_cast<TIn*>(x + r0 * cols * WIDTH), 0, (int)span, 0x00020000);
     u32x4 raw[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-        raw[i] = __builtin_amdgcn_raw_buffer_load_b128(res, col8 < cols ? (int)(((lr + 8 * i) * cols + col8) * 2) : (int)0x80000000u, 0, 0);
+        raw[i] = __builtin_amdgcn_raw_buffer_load_b128(res, col8 < cols ? (int)(((lr + 8 * i) * cols * WIDTH + col8) * 2) : (int)0x80000000u, 0, 0);
+    if constexpr (GATED) {
+        // the tile quantized is h = act(gate) * up, rounded to TIn as the activation kernels store it
+        u32x4 up[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            up[i] = __builtin_amdgcn_raw_buffer_load_b128(res, col8 < cols ? (int)(((lr + 8 * i) * cols * 2 + cols + col8) * 2) : (int)0x80000000u, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                uint32_t packed = 0;
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const float g = widen16<TIn>(e ? raw[i][w] >> 16 : raw[i][w] & 0xffffu);
+                    const float u = widen16<TIn>(e ? up[i][w] >> 16 : up[i][w] & 0xffffu);
+                    float a, derivative;
+                    gate_math(activation, g, a, derivative);
+                    float hv = a * u;
+                    // keep the product an FP32 value of its own: folded into the narrowing conversion (a mixed-precision
+                    // FMA with a +0 addend) it rounds once instead of twice and turns -0 into +0
+                    asm volatile("" : "+v"(hv));
+                    packed |= narrow16<TIn>(hv) << (16 * e);
+                }
+                raw[i][w] = packed;
+            }
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(&mine[(lr + 8 * i) * LD + ch * 8]) = raw[i];
 
@@ -831,6 +865,36 @@ extern "C" int viola_group_quantize_dual(const void* x, int x_dtype, int64_t row
     if (x_dtype == VIOLA_BF16) VIOLA_DUAL(bf16_t, e5m2_t);
     VIOLA_DUAL(f16_t, e5m2_t);
 #undef VIOLA_DUAL
+}
+
+extern "C" int viola_gated_quantize_dual(const void* z, int z_dtype, int64_t rows, int64_t cols, int activation, void* q,
+                                         void* scale, void* qt, void* scale_t, int q_dtype, int gc, float limit,
+                                         int scale_format, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(scale_format == VIOLA_SCALE_F32 || scale_format == VIOLA_SCALE_E8M0);
+    VIOLA_CHECK_ARG(activation == VIOLA_SILU || activation == VIOLA_GELU || activation == VIOLA_RELU);
+    VIOLA_CHECK_ARG(viola_is_fp8(q_dtype) && viola_is_float(z_dtype) && rows >= 0 && cols >= 0 && limit > 0.0f);
+    if (gc != 32 || z_dtype == VIOLA_F32 || cols % 8 != 0) return VIOLA_EUNSUPPORTED;
+    if (rows == 0 || cols == 0) return 0;
+    VIOLA_CHECK_ARG(z && q && scale && qt && scale_t);
+    if (reinterpret_cast<uintptr_t>(z) % 16 != 0 || reinterpret_cast<uintptr_t>(q) % 8 != 0) return VIOLA_EUNSUPPORTED;
+    if (64 * cols * 2 >= (1ll << 31)) return VIOLA_EUNSUPPORTED;            // a wavefront's 32 rows are one buffer
+    const int e8m0 = scale_format == VIOLA_SCALE_E8M0;
+    const int64_t tiles16 = ((cols + 63) / 64) * ((rows + 127) / 128);
+    const dim3 grid16((unsigned)(tiles16 < 256 * 6 ? tiles16 : 256 * 6));
+#define VIOLA_GATED_DUAL(TI, TO)                                                                                            \
+    hipLaunchKernelGGL((quantize_dual16<TI, TO, true, true>), grid16, dim3(256), 0, stream, static_cast<const TI*>(z),       \
+                       static_cast<uint8_t*>(q), static_cast<float*>(scale), static_cast<uint8_t*>(qt),                      \
+                       static_cast<float*>(scale_t), rows, cols, limit, (float*)nullptr, e8m0, activation)
+    if (q_dtype == VIOLA_E4M3) {
+        if (z_dtype == VIOLA_BF16) VIOLA_GATED_DUAL(bf16_t, e4m3_t);
+        else VIOLA_GATED_DUAL(f16_t, e4m3_t);
+    } else {
+        if (z_dtype == VIOLA_BF16) VIOLA_GATED_DUAL(bf16_t, e5m2_t);
+        else VIOLA_GATED_DUAL(f16_t, e5m2_t);
+    }
+#undef VIOLA_GATED_DUAL
+    return viola_launch_status();
 }
 
 extern "C" int viola_column_reduce(const float* partial, int64_t parts, int64_t cols, void* out, int out_dtype,

@@ -85,6 +85,23 @@ def quantize_dual(x, dtype, group, *, limit=None, column_sum_dtype=None, native=
     return q, s, qt, st, total
 
 
+def gated_quantize_dual(z, activation, dtype, *, limit=None, native=False):
+    """quantize_dual of h = act(g) * u (rounded to z's dtype) straight from z = [g | u] [rows, 2 h], bf16 / fp16:
+    the codes an MLP's down projection reads (viola/nn/_mlp_kernels.py:195-230) without h ever being stored.
+    Returns (q, s, qt, st), or None for shapes the kernel does not take."""
+    assert z.is_cuda and z.dim() == 2 and z.shape[1] % 2 == 0
+    z = z.contiguous()
+    rows, h = z.shape[0], z.shape[1] // 2
+    limit = torch.finfo(dtype).max if limit is None else limit
+    q = torch.empty((rows, h), device=z.device, dtype=dtype)
+    s = torch.empty(scale_shape((rows, h), (1, 32)), device=z.device, dtype=_scale_dtype(native))
+    qt = torch.empty((h, rows), device=z.device, dtype=dtype)
+    st = torch.empty(scale_shape((h, rows), (1, 32)), device=z.device, dtype=_scale_dtype(native))
+    status = _lib.call("viola_gated_quantize_dual", _lib.ptr(z), _lib.code(z.dtype), rows, h, _lib.ACTIVATION[activation], _lib.ptr(q),
+                       _lib.ptr(s), _lib.ptr(qt), _lib.ptr(st), _lib.code(dtype), 32, float(limit), int(bool(native)), unsupported_ok=True)
+    return (q, s, qt, st) if status == 0 else None
+
+
 def transpose_group(group):
     """A 2-D block (>= 32 rows) transposes exactly; a 1-D row group keeps its shape and needs new K groups."""
     return tuple(group[::-1]) if group[0] >= 32 else tuple(group)
