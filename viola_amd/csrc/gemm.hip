@@ -359,8 +359,8 @@ extern "C" int viola_group_gemm(const void* a, int a_dtype, const void* b, int b
 }
 
 // Large gated products run as the plain GEMM on 256 x 256 tiles plus one elementwise pass over its output: with one
-// block per CU nothing covers a block's gated epilogue, and the pass costs less than that (16384 x 4096 -> 11008:
-// forward 1.46 ms against 1.72 ms, backward 0.96 ms against 1.26 ms under per-tensor scales). No extra memory: forward
+// block per CU nothing covers a block's gated epilogue, and the pass costs less than that (MLP step at 16384 x 4096 ->
+// 11008: 7.55 ms against 7.90 ms under per-tensor scales, 8.41 ms against 9.06 ms under MXFP8). No extra memory: forward
 // the plain product is the [g | u] the caller keeps anyway, backward it lands in the up half of dz and is replaced there.
 static bool gated_in_two_passes(int64_t m, int64_t n_plain, int64_t h, const void* aux, const void* out, int out_dtype) {
     const int64_t piece = out_dtype == VIOLA_F32 ? 4 : 8;
@@ -558,7 +558,7 @@ extern "C" int viola_mx_gated_gemm_encode(const void* a, int a_dtype, const void
         return VIOLA_EUNSUPPORTED;
     if (aux && enc_t && aux_dtype != VIOLA_F32 && takes_large_tiles(m, 2 * h) && 128 * h < (1ll << 31)) {
         // large products: the plain GEMM on 256 x 256 tiles writes [g | u], one pass over it writes the codes of h
-        // in both layouts (the encoding epilogue does not fit the large tile's registers; 1.7 ms against 2.5 ms at
+        // in both layouts (the encoding epilogue does not fit the large tile's registers; 2.0 ms against 2.5 ms at
         // 16384 x 4096 -> 11008)
         const int status = mx_gemm(a, a_dtype, b, b_dtype, sa, sb, m, 2 * h, k, ar, br, bias, bias_dtype, aux, 2 * h, aux_dtype, stream);
         if (status) return status;
