@@ -28,6 +28,9 @@ typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int FBK = 64, FKG = FBK / 32;                           // k bytes and K groups per LDS stage
 constexpr int FTHREADS = 256, FSTAGES = 3;
+#ifndef VIOLA_BIG_STAGES
+#define VIOLA_BIG_STAGES 3                                         // ring depth of the 256 x 256 tile kernels (4 measured the same)
+#endif
 constexpr int F_TILE = BM * FBK;                                  // bytes of one operand tile
 constexpr int F_STAGE = 2 * F_TILE;
 // Scales travel in blocks of 8 K groups (4 chunks): 32 bytes per row and operand, fetched as two 16-byte pieces
@@ -122,7 +125,8 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
     constexpr bool NOFOLD = TENSOR || MX;                                   // the products of a chunk go straight into the totals
     constexpr int WAVES_N = BIG ? 4 : 2, THREADS = BIG ? 512 : FTHREADS;     // waves as 2 (m) x WAVES_N (n)
     constexpr int TBM = BIG ? 2 * BM : BM;                                   // rows of a per tile
-    constexpr int K_TILE_A = BIG ? 2 * F_TILE : F_TILE, K_STAGE = BIG ? 4 * F_TILE : F_STAGE, K_RAW = FSTAGES * K_STAGE;
+    constexpr int K_TILE_A = BIG ? 2 * F_TILE : F_TILE, K_STAGE = BIG ? 4 * F_TILE : F_STAGE;
+    constexpr int K_STAGES = BIG ? VIOLA_BIG_STAGES : FSTAGES, K_RAW = K_STAGES * K_STAGE;   // ring depth: loads run K_STAGES chunks ahead
     constexpr int K_MX_BLOCK = BIG ? 2 * MX_BLOCK : MX_BLOCK;
     // without scale blocks the ring plus the epilogue's bias row is all the LDS a block needs: three blocks share a CU
     __shared__ __attribute__((aligned(1024))) uint8_t lds[TENSOR ? K_RAW + 1024 : MX ? K_RAW + 2 * K_MX_BLOCK : F_LDS];
@@ -453,7 +457,7 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
         }
     };
 
-    // Ring of three stages, chunk c in stage c % 3. At the top of iteration c the wave waits for its own loads of
+    // Ring of K_STAGES (three in what follows) stages, chunk c in stage c % 3. At the top of iteration c the wave waits for its own loads of
     // chunk c+1 (issued two iterations ago) and for its LDS reads of chunk c; after the barrier chunk c+1 is in LDS
     // for everybody and nobody reads chunk c's stage any more. Then: the loads of chunk c+3 into that stage (one
     // instruction every few MFMAs, so the waves of a CU do not queue up at the memory pipe), the LDS reads of chunk
@@ -463,9 +467,11 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
     constexpr int STEPS = FKG * TN * TM * 2, STRIDE = STEPS / CHUNK_LOADS;
     int stage_now = 0, stage_next = 1;
     auto chunk_step = [&](int64_t c, const Operands& now, Operands& next) {
-        if (!NOFOLD && c % F_SCHUNKS == 1) __builtin_amdgcn_s_waitcnt(0x0070 | (CHUNK_LOADS + 2));
-        else if (MX && c % MX_CHUNKS == 1) __builtin_amdgcn_s_waitcnt(0x0070 | (CHUNK_LOADS + 1));
-        else __builtin_amdgcn_s_waitcnt(0x0070 | CHUNK_LOADS);
+        constexpr int AHEAD = (K_STAGES - 2) * CHUNK_LOADS;                  // loads of the chunks after c + 1 may still be in flight
+        static_assert(AHEAD + 2 < 16 && (K_STAGES - 1) * CHUNK_LOADS < 16, "the counts fit the wait instruction's low field");
+        if (!NOFOLD && c % F_SCHUNKS == 1) __builtin_amdgcn_s_waitcnt(0x0070 | (AHEAD + 2));
+        else if (MX && c % MX_CHUNKS == 1) __builtin_amdgcn_s_waitcnt(0x0070 | (AHEAD + 1));
+        else __builtin_amdgcn_s_waitcnt(0x0070 | AHEAD);
         __syncthreads();
         if constexpr (!NOFOLD) {
             if (c % F_SCHUNKS == 0) issue_scales(c / F_SCHUNKS + 1);
@@ -477,17 +483,16 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
         if (c + 1 < chunks) read_operands(stage_next, c + 1, next);
         const int fill = stage_now;
         compute(now, c, [&](int step) {
-            if (step % STRIDE == 0 && step / STRIDE < CHUNK_LOADS) issue_one(c + 3, fill, step / STRIDE);
+            if (step % STRIDE == 0 && step / STRIDE < CHUNK_LOADS) issue_one(c + K_STAGES, fill, step / STRIDE);
         });
         stage_now = stage_next;
-        stage_next = stage_next == FSTAGES - 1 ? 0 : stage_next + 1;
+        stage_next = stage_next == K_STAGES - 1 ? 0 : stage_next + 1;
     };
     if constexpr (MX) issue_mx_scales(0);
     else if constexpr (!TENSOR) issue_scales(0);
-    issue(0, 0);
-    issue(1, 1);
-    issue(2, 2);
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * CHUNK_LOADS));                   // scale block 0 and chunk 0 are in LDS
+#pragma unroll
+    for (int s = 0; s < K_STAGES; ++s) issue(s, s);
+    __builtin_amdgcn_s_waitcnt(0x0F70 | ((K_STAGES - 1) * CHUNK_LOADS));                   // scale block 0 and chunk 0 are in LDS
     __syncthreads();
     if constexpr (!NOFOLD) {
         arrange_scales(0);
