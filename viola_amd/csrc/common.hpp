@@ -290,8 +290,9 @@ __device__ __forceinline__ T round_store(float v, uint64_t element, uint64_t ste
     return from_f32<T>(v);
 }
 
-// act(g) and act'(g) of a gated MLP (viola/nn/_mlp_kernels.py:158-194): one formula for every kernel that applies it,
-// so the fused epilogues and the stand-alone passes give the same bits.
+// act(g) and act'(g) of a gated MLP as the gated GEMM epilogues write them (viola/nn/_mlp_kernels.py:158-194), shared by
+// the epilogues and by the passes that stand in for them, so both give the same bits. (The stand-alone forward operator
+// writes silu as g / (1 + exp(-g)), viola/nn/_gated_kernels.py:29-35, which differs in the last place.)
 __device__ __forceinline__ void gate_math(int activation, float g, float& act, float& derivative) {
     if (activation == VIOLA_SILU) {
         const float s = 1.0f / (1.0f + expf(-g));

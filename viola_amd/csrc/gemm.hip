@@ -430,13 +430,13 @@ static int gated_two_passes(Plain&& plain, int64_t m, int64_t h, const void* bia
     if (!backward) {
         const int status = plain(2 * h, bias, aux, 2 * h);                  // [g | u], biased
         if (status) return status;
-        launch_gated_pieces(aux, nullptr, 0, out, m, h, out_dtype, activation, false, stream);
+        launch_gated_pieces(aux, nullptr, 0, out, m, h, out_dtype, activation, false, true, stream);
         return viola_launch_status();
     }
     uint8_t* up_half = static_cast<uint8_t*>(out) + h * (out_dtype == VIOLA_F32 ? 4 : 2);
     const int status = plain(h, nullptr, up_half, 2 * h);                   // dh, where d u will stand
     if (status) return status;
-    launch_gated_pieces(aux, up_half, 2 * h, out, m, h, out_dtype, activation, true, stream);
+    launch_gated_pieces(aux, up_half, 2 * h, out, m, h, out_dtype, activation, true, true, stream);
     return viola_launch_status();
 }
 

@@ -45,9 +45,10 @@ int launch_tensor_gemm_fast(const GemmArgs& p, int mode, int a_dtype, int b_dtyp
 int launch_mx_gemm_fast(const GemmArgs& p, int mode, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, dim3 grid,
                         hipStream_t stream);
 
-// misc.hip: the gated activation as a pass of its own, in 16-byte pieces (false: alignment does not allow them)
+// misc.hip: the gated activation as a pass of its own, in 16-byte pieces (false: alignment does not allow them);
+// epilogue_form: forward silu in the gated GEMM epilogue's expression instead of the stand-alone operator's
 bool launch_gated_pieces(const void* z, const void* dy, int64_t dy_stride, void* out, int64_t rows, int64_t h, int dtype,
-                         int activation, bool backward, hipStream_t stream);
+                         int activation, bool backward, bool epilogue_form, hipStream_t stream);
 
 // Per-tensor and block-scaled products with at least this many 256 x 256 output tiles (two rounds of the 256 CUs)
 // run on the large tile.

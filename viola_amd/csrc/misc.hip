@@ -157,7 +157,9 @@ __global__ __launch_bounds__(256) void gated_forward_kernel(const void* __restri
         const int64_t r = idx / h, c = idx % h;
         const float g = load_half(z, r * 2 * h + c, dtype), u = load_half(z, r * 2 * h + h + c, dtype);
         float a, derivative;
-        gate_math(activation, g, a, derivative);
+        // the stand-alone operator divides (viola/nn/_gated_kernels.py:29-35); the GEMM epilogues multiply by 1 / (1 + exp(-g))
+        if (activation == VIOLA_SILU) a = g / (1.0f + expf(-g));
+        else gate_math(activation, g, a, derivative);
         store_half(out, idx, dtype, a * u);
     }
 }
@@ -209,7 +211,9 @@ template <typename T> struct Piece {
     }
 };
 
-template <typename T, int ACT>
+// EPILOGUE_FORM: silu as g * (1 / (1 + exp(-g))), the gated GEMM epilogue's expression (viola/nn/_mlp_kernels.py:163-175),
+// for the pass that stands in for that epilogue; otherwise the stand-alone operator's g / (1 + exp(-g)).
+template <typename T, int ACT, bool EPILOGUE_FORM>
 __global__ __launch_bounds__(256) void gated_forward_pieces(const T* __restrict__ z, T* __restrict__ out, int64_t pieces, int64_t per_row) {
     constexpr int N = Piece<T>::N;
     const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -221,7 +225,8 @@ __global__ __launch_bounds__(256) void gated_forward_pieces(const T* __restrict_
 #pragma unroll
     for (int i = 0; i < N; ++i) {
         float a, derivative;
-        gate_math(ACT, g[i], a, derivative);
+        if constexpr (ACT == VIOLA_SILU && !EPILOGUE_FORM) a = g[i] / (1.0f + expf(-g[i]));
+        else gate_math(ACT, g[i], a, derivative);
         o[i] = a * u[i];
     }
     Piece<T>::store(out + r * h + c, o);
@@ -252,7 +257,7 @@ __global__ __launch_bounds__(256) void gated_backward_pieces(const T* __restrict
 
 template <typename T>
 static bool launch_gated_pieces(const void* z, const void* dy, int64_t dy_stride, void* out, int64_t rows, int64_t h, int activation,
-                                bool backward, hipStream_t stream) {
+                                bool backward, bool epilogue_form, hipStream_t stream) {
     constexpr int N = Piece<T>::N;
     const auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
     if (h % N != 0 || !aligned(z) || !aligned(out) || (backward && (!aligned(dy) || dy_stride % N != 0))) return false;
@@ -264,7 +269,8 @@ static bool launch_gated_pieces(const void* z, const void* dy, int64_t dy_stride
     T* op = static_cast<T*>(out);
 #define VIOLA_GATED(ACT)                                                                                                   \
     if (backward) hipLaunchKernelGGL((gated_backward_pieces<T, ACT>), grid, dim3(256), 0, stream, zp, dp, dy_stride, op, pieces, per_row); \
-    else hipLaunchKernelGGL((gated_forward_pieces<T, ACT>), grid, dim3(256), 0, stream, zp, op, pieces, per_row);
+    else if (epilogue_form) hipLaunchKernelGGL((gated_forward_pieces<T, ACT, true>), grid, dim3(256), 0, stream, zp, op, pieces, per_row); \
+    else hipLaunchKernelGGL((gated_forward_pieces<T, ACT, false>), grid, dim3(256), 0, stream, zp, op, pieces, per_row);
     if (activation == VIOLA_SILU) { VIOLA_GATED(VIOLA_SILU) }
     else if (activation == VIOLA_GELU) { VIOLA_GATED(VIOLA_GELU) }
     else { VIOLA_GATED(VIOLA_RELU) }
@@ -275,10 +281,10 @@ static bool launch_gated_pieces(const void* z, const void* dy, int64_t dy_stride
 // The gated activation in 16-byte pieces: forward out [rows, h] = act(g) * u from z = [g | u]; backward out [rows, 2 h] from
 // z and dy (row stride dy_stride elements). False, and nothing launched, when alignment does not allow the pieces.
 bool launch_gated_pieces(const void* z, const void* dy, int64_t dy_stride, void* out, int64_t rows, int64_t h, int dtype,
-                         int activation, bool backward, hipStream_t stream) {
-    if (dtype == VIOLA_F32) return launch_gated_pieces<float>(z, dy, dy_stride, out, rows, h, activation, backward, stream);
-    if (dtype == VIOLA_BF16) return launch_gated_pieces<bf16_t>(z, dy, dy_stride, out, rows, h, activation, backward, stream);
-    return launch_gated_pieces<f16_t>(z, dy, dy_stride, out, rows, h, activation, backward, stream);
+                         int activation, bool backward, bool epilogue_form, hipStream_t stream) {
+    if (dtype == VIOLA_F32) return launch_gated_pieces<float>(z, dy, dy_stride, out, rows, h, activation, backward, epilogue_form, stream);
+    if (dtype == VIOLA_BF16) return launch_gated_pieces<bf16_t>(z, dy, dy_stride, out, rows, h, activation, backward, epilogue_form, stream);
+    return launch_gated_pieces<f16_t>(z, dy, dy_stride, out, rows, h, activation, backward, epilogue_form, stream);
 }
 
 // ------------------------------------------------------------------ self checks
@@ -381,7 +387,7 @@ extern "C" int viola_gated_forward(const void* z, void* out, int64_t rows, int64
     VIOLA_CHECK_ARG(viola_is_float(dtype) && rows >= 0 && h >= 0 && activation >= VIOLA_SILU && activation <= VIOLA_RELU);
     if (rows == 0 || h == 0) return 0;
     VIOLA_CHECK_ARG(z && out);
-    if (launch_gated_pieces(z, nullptr, 0, out, rows, h, dtype, activation, false, stream)) return viola_launch_status();
+    if (launch_gated_pieces(z, nullptr, 0, out, rows, h, dtype, activation, false, false, stream)) return viola_launch_status();
     hipLaunchKernelGGL(gated_forward_kernel, dim3(grid_for(rows * h)), dim3(256), 0, stream, z, out, rows, h, dtype, activation);
     return viola_launch_status();
 }
@@ -392,7 +398,7 @@ extern "C" int viola_gated_backward(const void* z, const void* dy, void* dz, int
     VIOLA_CHECK_ARG(viola_is_float(dtype) && rows >= 0 && h >= 0 && activation >= VIOLA_SILU && activation <= VIOLA_RELU);
     if (rows == 0 || h == 0) return 0;
     VIOLA_CHECK_ARG(z && dy && dz);
-    if (launch_gated_pieces(z, dy, h, dz, rows, h, dtype, activation, true, stream)) return viola_launch_status();
+    if (launch_gated_pieces(z, dy, h, dz, rows, h, dtype, activation, true, false, stream)) return viola_launch_status();
     hipLaunchKernelGGL(gated_backward_kernel, dim3(grid_for(rows * h)), dim3(256), 0, stream, z, dy, dz, rows, h, dtype, activation);
     return viola_launch_status();
 }
