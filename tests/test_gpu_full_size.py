@@ -259,7 +259,8 @@ def test_large_tile_gemm_of_the_fold_free_recipes(recipe, m, n, k, formats):
     assert torch.equal(sample, out[rows])
 
 
-@pytest.mark.parametrize("out_dtype,activation", [(torch.bfloat16, "gelu"), (torch.float16, "gelu"), (torch.bfloat16, "silu"), (torch.float16, "relu")])
+@pytest.mark.parametrize("out_dtype,activation", [(torch.bfloat16, "gelu"), (torch.float16, "gelu"), (torch.bfloat16, "silu"), (torch.float16, "relu"),
+                                                  (torch.float32, "silu")])
 @pytest.mark.parametrize("recipe", ["tensor", "mxfp8"])
 def test_large_tile_gated_gemms_equal_the_small_tile_kernels(recipe, out_dtype, activation):
     """m = 8256, h = 6208: with [g, u] kept, the gated forward and backward products run as the plain GEMM on 256-row
