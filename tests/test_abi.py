@@ -97,5 +97,13 @@ def test_rejected_calls_return_codes_and_launch_nothing():
     assert lib.viola_gated_forward(P, P, 8, 8, E4M3, 0, None) == -1
     assert lib.viola_gated_forward(None, P, 8, 8, BF16, 0, None) == -1
     assert lib.viola_gated_forward(P, P, 0, 8, BF16, 0, None) == 0
+    # the dual quantizer fed from [g | u]
+    assert lib.viola_gated_quantize_dual(None, BF16, 64, 64, 0, P, P, P, P, E4M3, 32, 448.0, 0, None) == -1          # no input
+    assert lib.viola_gated_quantize_dual(P, BF16, 64, 64, 9, P, P, P, P, E4M3, 32, 448.0, 0, None) == -1             # no such activation
+    assert lib.viola_gated_quantize_dual(P, BF16, 64, 64, 0, P, P, P, P, BF16, 32, 448.0, 0, None) == -1             # codes must be FP8
+    assert lib.viola_gated_quantize_dual(P, F32, 64, 64, 0, P, P, P, P, E4M3, 32, 448.0, 0, None) == -2              # 16-bit [g | u] only
+    assert lib.viola_gated_quantize_dual(P, BF16, 64, 60, 0, P, P, P, P, E4M3, 32, 448.0, 0, None) == -2             # rows of h not 16-byte pieces
+    assert lib.viola_gated_quantize_dual(P, BF16, 64, 64, 0, P, P, P, P, E4M3, 64, 448.0, 0, None) == -2             # groups of 32 only
+    assert lib.viola_gated_quantize_dual(P, BF16, 0, 64, 0, P, P, P, P, E4M3, 32, 448.0, 0, None) == 0               # empty: done
     for status in (-1, -2):
         assert lib.viola_error_string(status)

@@ -364,7 +364,8 @@ extern "C" int viola_group_gemm(const void* a, int a_dtype, const void* b, int b
 // the plain product is the [g | u] the caller keeps anyway, backward it lands in the up half of dz and is replaced there.
 static bool gated_in_two_passes(int64_t m, int64_t n_plain, int64_t h, const void* aux, const void* out, int out_dtype) {
     const int64_t piece = out_dtype == VIOLA_F32 ? 4 : 8;
-    return aux && takes_large_tiles(m, n_plain) && h % piece == 0 && aligned16(aux) && aligned16(out);
+    return aux && takes_large_tiles(m, n_plain) && h % piece == 0 && aligned16(aux) && aligned16(out) &&
+           m * (h / piece) / 256 < 0x7fffffff;                               // the pass is one launch of 256-thread blocks
 }
 
 static int tensor_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb, int64_t m,
