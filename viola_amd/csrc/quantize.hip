@@ -229,6 +229,12 @@ __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x
     typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     __shared__ __attribute__((aligned(16))) uint16_t park[4][32 * LD];
+    // Transposed codes leave as whole 128-byte lines: the block's four wavefronts hold rows 32 w .. 32 w + 31 of the same
+    // 64 columns, so each has a 32-byte run of every column's line; the runs meet here ([column][128 + 16 bytes]) and
+    // go out as 16-byte pieces, eight lanes to a line, instead of 64 lines touched per store instruction.
+    constexpr int XLD = 128 + 16;
+    __shared__ __attribute__((aligned(16))) uint8_t lines[64 * XLD];
+    const bool by_lines = rows % 16 == 0 && (reinterpret_cast<uintptr_t>(qt) & 15) == 0;   // pieces are whole and aligned
     const int lane = threadIdx.x % WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);   // uniform: so is the buffer descriptor
     uint16_t* mine = park[wave];
     const int lr = lane / 8, ch = lane % 8;
@@ -237,13 +243,14 @@ __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x
     // resident, so the SIMDs keep several of them in flight instead of waiting for new workgroups to be dispatched
     const int64_t tiles_x = (cols + 63) / 64, tiles = tiles_x * ((rows + 127) / 128);
     for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-    const int64_t r0 = tile / tiles_x * 128 + wave * 32, c0 = tile % tiles_x * 64;
-    if (r0 >= rows) continue;                                                // whole wavefront skips together
+    const int64_t block_r0 = tile / tiles_x * 128;
+    const int64_t r0 = block_r0 + wave * 32, c0 = tile % tiles_x * 64;
+    const bool active = r0 < rows;                                           // a wavefront past the last row reads zeros and stores nothing
     const int64_t col8 = c0 + ch * 8;
 
     // all four loads first, without control flow: a raw buffer over the wavefront's 32 rows returns zero past its end
     constexpr int WIDTH = GATED ? 2 : 1;                                     // x rows are [gate | up] when GATED
-    const int64_t span = (rows - r0 < 32 ? rows - r0 : 32) * cols * 2 * WIDTH;
+    const int64_t span = active ? (rows - r0 < 32 ? rows - r0 : 32) * cols * 2 * WIDTH : 0;
     const __amdgpu_buffer_rsrc_t res = __builtin_amdgcn_make_buffer_rsrc(const_cast<TIn*>(x + r0 * cols * WIDTH), 0, (int)span, 0x00020000);
     u32x4 raw[4];
 #pragma unroll
@@ -356,7 +363,7 @@ __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x
             }
         }
     }
-    if (col < cols) {
+    if (active && col < cols) {
         const int64_t nr = (rows + 31) / 32;
         put_scale(scale_t, col * nr + r0 / 32, s_col, e8m0);
         if (column_partial) {
@@ -366,12 +373,30 @@ __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x
             column_partial[(r0 / 32) * cols + col] = sum;
         }
         uint8_t* dst = qt + col * rows + r0;
-        if (rows - r0 >= 32 && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+        if (by_lines) {
+            // stored below, by the whole block
+        } else if (rows - r0 >= 32 && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
             reinterpret_cast<uint4*>(dst)[0] = make_uint4(col_codes[0], col_codes[1], col_codes[2], col_codes[3]);
             reinterpret_cast<uint4*>(dst)[1] = make_uint4(col_codes[4], col_codes[5], col_codes[6], col_codes[7]);
         } else {
             const int count = (int)(rows - r0 < 32 ? rows - r0 : 32);
             for (int i = 0; i < count; ++i) dst[i] = (uint8_t)(col_codes[i >> 2] >> (8 * (i & 3)));
+        }
+    }
+    if (by_lines) {
+        __syncthreads();                                                     // the pieces of the tile before have been read
+        if (active) {
+            uint4* run = reinterpret_cast<uint4*>(&lines[lane * XLD + wave * 32]);
+            run[0] = make_uint4(col_codes[0], col_codes[1], col_codes[2], col_codes[3]);
+            run[1] = make_uint4(col_codes[4], col_codes[5], col_codes[6], col_codes[7]);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int id = it * 256 + (int)threadIdx.x, c = id >> 3, piece = id & 7;
+            const int64_t row = block_r0 + piece * 16;                       // rows % 16 == 0: a piece is inside or outside as a whole
+            if (c0 + c < cols && row < rows)
+                *reinterpret_cast<uint4*>(qt + (c0 + c) * rows + row) = *reinterpret_cast<const uint4*>(&lines[c * XLD + piece * 16]);
         }
     }
     }
