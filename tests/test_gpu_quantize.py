@@ -78,7 +78,7 @@ def test_quantize_transposed(in_dtype, fp8, group, shape):
 
 
 @pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float16, torch.float32])
-@pytest.mark.parametrize("shape", [(65, 128), (128, 64), (300, 200), (1, 32), (129, 72), (8192, 1024)])
+@pytest.mark.parametrize("shape", [(65, 128), (128, 64), (300, 200), (1, 32), (129, 72), (8192, 1024), (176, 200), (16, 64), (144, 72), (272, 136)])
 def test_quantize_dual_equals_two_passes(in_dtype, shape):
     g = _gpu()
     x = _input(shape, in_dtype, seed=11)
@@ -124,7 +124,7 @@ def test_quantize_rounding_ties_over_all_magnitudes(fp8, limit):
 
 
 @pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float16, torch.float32])
-@pytest.mark.parametrize("shape", [(65, 128), (300, 200), (129, 72), (8192, 1024), (32, 64)])
+@pytest.mark.parametrize("shape", [(65, 128), (300, 200), (129, 72), (8192, 1024), (32, 64), (176, 200), (144, 72)])
 def test_quantize_dual_column_sums(in_dtype, shape):
     """x.sum(0) from the quantizer's own read: fp32 accumulation in a fixed order, same codes as without it."""
     g = _gpu()
@@ -227,7 +227,7 @@ def test_gated_quantize_dual_equals_activation_then_quantize(dtype, activation, 
     test of the gated GEMMs.)"""
     from viola_amd.nn import _gated_kernels as gk, _grouped_kernels as g
     torch.manual_seed(5)
-    for rows, h in ((100, 72), (256, 128), (33, 8)):
+    for rows, h in ((100, 72), (256, 128), (33, 8), (176, 72)):
         z = (torch.randn(rows, 2 * h, device="cuda") * torch.exp2(torch.randint(-6, 5, (rows, 1), device="cuda").float())).to(dtype)
         z[3, 5] = float("nan")
         for fp8 in (torch.float8_e4m3fn, torch.float8_e5m2):
