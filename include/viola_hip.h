@@ -170,7 +170,10 @@ int viola_gated_gemm(const void* a, int a_dtype, const void* b, int b_dtype, con
 /* The same two gated projections under the other recipes of viola/nn/_mlp_kernels.py:16-231 (`grouped` false:
  * value *= sa[0] * sb[0], :157-166; native E8M0 scales, :120-127). viola_tensor_gated_gemm: one FP32 scale per
  * operand. viola_mx_gated_gemm: E8M0 bytes per 32 k as in viola_mx_gemm (ar, br = rows per scale row); returns
- * VIOLA_EUNSUPPORTED where viola_mx_gemm does, and in forward when h is not a multiple of br. */
+ * VIOLA_EUNSUPPORTED where viola_mx_gemm does, and in forward when h is not a multiple of br.
+ * Large products (at least 512 output tiles of 256 x 256) with aux given run as the plain GEMM followed by one
+ * elementwise pass on the same stream, with the same results and no memory beyond aux and out: forward the GEMM
+ * writes aux, backward it writes d into out[:, h:2h], which the pass then replaces (so out is also read there). */
 int viola_tensor_gated_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,
                             int64_t m, int64_t h, int64_t k, const void* bias, int bias_dtype, void* aux, void* out,
                             int out_dtype, int activation, int backward, viola_stream_t stream);
@@ -182,7 +185,8 @@ int viola_mx_gated_gemm(const void* a, int a_dtype, const void* b, int b_dtype, 
  * whose h = act(g) * u, rounded to aux_dtype, leaves the kernel as FP8 codes with E8M0 scales per 32 values: along its
  * rows (enc [m, h], enc_scale [m, h / 32]) for the down projection's forward GEMM and, when enc_t is not NULL, along
  * its columns (enc_t [h, m], enc_t_scale [h, m / 32]) for its wgrad. aux [m, 2h] (NULL allowed) receives [g, u].
- * VIOLA_EUNSUPPORTED where viola_mx_gated_gemm returns it, and when m or h is not a multiple of 32. */
+ * VIOLA_EUNSUPPORTED where viola_mx_gated_gemm returns it, and when m or h is not a multiple of 32. Large products
+ * with aux and enc_t given run as viola_mx_gemm into aux followed by viola_gated_quantize_dual (same results). */
 int viola_mx_gated_gemm_encode(const void* a, int a_dtype, const void* b, int b_dtype, const uint8_t* sa, const uint8_t* sb,
                                int64_t m, int64_t h, int64_t k, int ar, int br, const void* bias, int bias_dtype, void* aux,
                                int aux_dtype, void* enc, uint8_t* enc_scale, void* enc_t, uint8_t* enc_t_scale, int enc_dtype,
