@@ -115,11 +115,9 @@ __device__ __forceinline__ void load_tile(const TIn* __restrict__ x, float* tile
     }
 }
 
-// Encode 32 values held by one lane and store them at dst (a run of `count` <= 32 valid bytes).
+// Encode 32 values held by one lane into eight words of codes.
 template <typename TOut>
-__device__ __forceinline__ void store_group32(const float (&v)[32], float s, float poison, float limit, uint8_t* dst, int count,
-                                              bool aligned16) {
-    uint32_t w[8];
+__device__ __forceinline__ void encode_group32(const float (&v)[32], float s, float poison, float limit, uint32_t (&w)[8]) {
     const SharedDivisor divisor(s, poison);
     if (divisor.fast) {
 #pragma unroll
@@ -132,6 +130,14 @@ __device__ __forceinline__ void store_group32(const float (&v)[32], float s, flo
             for (int j = 0; j < 4; ++j) w[i] |= (uint32_t)encode_clamped<TOut>(v[4 * i + j], s, limit) << (8 * j);
         }
     }
+}
+
+// Encode 32 values held by one lane and store them at dst (a run of `count` <= 32 valid bytes).
+template <typename TOut>
+__device__ __forceinline__ void store_group32(const float (&v)[32], float s, float poison, float limit, uint8_t* dst, int count,
+                                              bool aligned16) {
+    uint32_t w[8];
+    encode_group32<TOut>(v, s, poison, limit, w);
     if (count == 32 && aligned16) {
         reinterpret_cast<uint4*>(dst)[0] = make_uint4(w[0], w[1], w[2], w[3]);
         reinterpret_cast<uint4*>(dst)[1] = make_uint4(w[4], w[5], w[6], w[7]);
@@ -660,15 +666,16 @@ __global__ __launch_bounds__(256) void quantize_segmented16(const TIn* __restric
     const int lr = lane / 8, ch = lane % 8;
     const int64_t nc = (cols + 31) / 32;
     const int64_t tiles_x = (cols + 63) / 64, slots = t_total / 32;
-    const int64_t work = ((int64_t)blockIdx.x * 4 + wave);                    // one (slot, column tile) per wavefront
-    if (work >= slots * tiles_x) return;
-    const int64_t slot = work / tiles_x, c0 = work % tiles_x * 64;
+    // a block takes four consecutive slots of one column tile, one per wavefront: their 32-byte runs of transposed
+    // codes are the four quarters of 128-byte lines (see quantize_dual16)
+    const int64_t first_slot = (int64_t)blockIdx.x / tiles_x * 4, slot = first_slot + wave, c0 = (int64_t)blockIdx.x % tiles_x * 64;
+    const bool active = slot < slots;                                        // a wavefront past the last slot reads zeros and stores nothing
     const int64_t token = slot * 32;
     int g = 0;
     while (g + 1 < groups && poffsets[g + 1] <= token) ++g;
     const int64_t first = offsets[g] + (token - poffsets[g]);
     const int64_t left = offsets[g + 1] - first;                               // valid rows of this slot (may be <= 0)
-    const int valid = (int)(left < 0 ? 0 : left > 32 ? 32 : left);
+    const int valid = !active ? 0 : (int)(left < 0 ? 0 : left > 32 ? 32 : left);
     const int64_t col8 = c0 + ch * 8;
 
     const __amdgpu_buffer_rsrc_t res = __builtin_amdgcn_make_buffer_rsrc(const_cast<TIn*>(x + first * cols), 0, (int)(valid * cols * 2), 0x00020000);
@@ -718,11 +725,28 @@ __global__ __launch_bounds__(256) void quantize_segmented16(const TIn* __restric
             poison = poison_of(poison, vc[4 * t + e]);
         }
     }
-    if (col < cols) {
-        const float s = group_scale(amax, limit);
-        scale_t[col * slots + slot] = s;
-        uint8_t* dst = qt + col * t_total + token;
-        store_group32<TOut>(vc, s, poison, limit, dst, 32, (reinterpret_cast<uintptr_t>(dst) & 15) == 0);
+    const float s = group_scale(amax, limit);
+    if (active && col < cols) scale_t[col * slots + slot] = s;
+    if ((reinterpret_cast<uintptr_t>(qt) & 15) != 0) {                        // (uniform) odd base: each wavefront stores its own runs
+        if (active && col < cols) store_group32<TOut>(vc, s, poison, limit, qt + col * t_total + token, 32, false);
+        return;
+    }
+    constexpr int XLD = 128 + 16;
+    __shared__ __attribute__((aligned(16))) uint8_t lines[64 * XLD];
+    if (active) {
+        uint32_t w[8];
+        encode_group32<TOut>(vc, s, poison, limit, w);
+        uint4* run = reinterpret_cast<uint4*>(&lines[lane * XLD + wave * 32]);
+        run[0] = make_uint4(w[0], w[1], w[2], w[3]);
+        run[1] = make_uint4(w[4], w[5], w[6], w[7]);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+        const int id = it * 256 + (int)threadIdx.x, c = id >> 3, piece = id & 7;
+        const int64_t at_token = first_slot * 32 + piece * 16;               // t_total is a multiple of 32: whole pieces only
+        if (c0 + c < cols && at_token < t_total)
+            *reinterpret_cast<uint4*>(qt + (c0 + c) * t_total + at_token) = *reinterpret_cast<const uint4*>(&lines[c * XLD + piece * 16]);
     }
 }
 
@@ -821,9 +845,9 @@ static int launch_segmented(const void* x, int64_t cols, const int64_t* offsets,
                             int64_t t_total, void* qt, float* scale_t, void* q, float* scale, float limit, hipStream_t stream) {
     if constexpr (sizeof(TIn) == 2) {
         const bool aligned = cols % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && (!q || reinterpret_cast<uintptr_t>(q) % 8 == 0);
-        const int64_t waves = (t_total / 32) * ((cols + 63) / 64);
-        if (aligned && (waves + 3) / 4 < (1ll << 31)) {
-            const dim3 grid16((unsigned)((waves + 3) / 4));
+        const int64_t blocks = ((t_total / 32 + 3) / 4) * ((cols + 63) / 64);   // four slots x one column tile each
+        if (aligned && blocks < (1ll << 31)) {
+            const dim3 grid16((unsigned)blocks);
             if (q) hipLaunchKernelGGL((quantize_segmented16<TIn, TOut, true>), grid16, dim3(256), 0, stream, static_cast<const TIn*>(x), offsets, poffsets, groups, cols, t_total, static_cast<uint8_t*>(qt), scale_t, static_cast<uint8_t*>(q), scale, limit);
             else hipLaunchKernelGGL((quantize_segmented16<TIn, TOut, false>), grid16, dim3(256), 0, stream, static_cast<const TIn*>(x), offsets, poffsets, groups, cols, t_total, static_cast<uint8_t*>(qt), scale_t, nullptr, nullptr, limit);
             return viola_launch_status();
