@@ -247,10 +247,16 @@ __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x
     const int64_t nc = (cols + 31) / 32;
     // a block walks tiles of 128 rows x 64 columns (column tiles fastest) with the grid's stride: the wavefronts stay
     // resident, so the SIMDs keep several of them in flight instead of waiting for new workgroups to be dispatched
-    const int64_t tiles_x = (cols + 63) / 64, tiles = tiles_x * ((rows + 127) / 128);
+    const int64_t tiles_x = (cols + 63) / 64, tiles_y = (rows + 127) / 128, tiles = tiles_x * tiles_y;
     for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-    const int64_t block_r0 = tile / tiles_x * 128;
-    const int64_t r0 = block_r0 + wave * 32, c0 = tile % tiles_x * 64;
+    // tiles in flight together (consecutive indices) should form a compact patch: 16 row tiles of one column tile, then
+    // the next column tile, so that a row of x is read in long runs and a row of the transposed output (2 KB per 16
+    // row tiles) is written in long runs too, however wide the matrix is
+    constexpr int64_t BAND = 16;                                            // 8 .. 32 measure the same, 64 slower
+    const int64_t patch = tile / (BAND * tiles_x), within = tile % (BAND * tiles_x);
+    const int64_t tall = tiles_y - patch * BAND < BAND ? tiles_y - patch * BAND : BAND;
+    const int64_t block_r0 = (patch * BAND + within % tall) * 128;
+    const int64_t r0 = block_r0 + wave * 32, c0 = within / tall * 64;
     const bool active = r0 < rows;                                           // a wavefront past the last row reads zeros and stores nothing
     const int64_t col8 = c0 + ch * 8;
 
