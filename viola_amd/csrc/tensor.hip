@@ -274,7 +274,13 @@ __global__ __launch_bounds__(256) void tensor_quantize_kernel(const TIn* __restr
     constexpr int LD = 64 + 16;                                         // padded row of the parking tile (bytes)
     __shared__ __attribute__((aligned(16))) uint8_t park[64 * LD];
     const int tid = threadIdx.x, lr = tid / 4, lc = (tid % 4) * 16;
-    const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+    // blocks are dispatched in index order: those in flight together take a patch of 32 row tiles per column tile, then
+    // the next column tile, so the transposed output is written in 2 KB runs per row however wide the matrix is
+    constexpr int64_t BAND = 32;
+    const int64_t tiles_x = gridDim.x, tiles_y = gridDim.y, id = (int64_t)blockIdx.y * tiles_x + blockIdx.x;
+    const int64_t patch = id / (BAND * tiles_x), within = id % (BAND * tiles_x);
+    const int64_t tall = tiles_y - patch * BAND < BAND ? tiles_y - patch * BAND : BAND;
+    const int64_t r0 = (patch * BAND + within % tall) * 64, c0 = within / tall * 64;
     const int64_t row = r0 + lr, col = c0 + lc;
     const float s = scale[0];
     float v[16];
