@@ -10,8 +10,8 @@
  *   - the library never allocates or frees device memory and never synchronises:
  *     each call enqueues kernels on `stream` (a hipStream_t) and returns;
  *   - a null pointer means "absent" (no bias, no aux, no source scale ...);
- *   - return 0 on success, VIOLA_EINVAL / VIOLA_EUNSUPPORTED for rejected arguments
- *     (nothing was launched), or a positive hipError_t from the launch;
+ *   - return 0 on success, a negative VIOLA_E* code for rejected arguments (nothing was
+ *     launched), or the positive hipError_t that hipLaunchKernel returned for a launch;
  *   - matrices are row-major and contiguous unless a stride is passed.
  */
 #ifndef VIOLA_HIP_H
@@ -295,14 +295,20 @@ int viola_momentum_dequantize(const void* q, const float* scale, float* out, int
  * out_diag (nullable) receives a second copy of the result with add_diag added to its diagonal after
  * rounding (Q = Z + 3.4445 I, viola/optim/_orthogonalize.py:45-47). transpose_out = 1 stores out and
  * out_diag as [batch, n, m] (the un-transposition of a tall matrix at the end of the chain,
- * viola/optim/_orthogonalize.py:20-21,52-53); residual stays [batch, m, n]. */
+ * viola/optim/_orthogonalize.py:20-21,52-53); residual stays [batch, m, n].
+ * With transpose_b = 1, bmat == a and m == n (a . a^T) only the tiles on and above the diagonal are multiplied
+ * and each is stored a second time transposed: out[i, j] and out[j, i] carry the same rounded product, and each
+ * takes the epilogue with its own residual element, so the result is what the full product gives for any
+ * residual, symmetric or not. The caller decides whether a . a^T is the product it wants: for a matrix that is
+ * symmetric only up to rounding, a . a differs from it and is requested with transpose_b = 0. */
 int viola_ns_gemm(const void* a, const void* bmat, const void* residual, void* out, int dtype,
                   int transpose_b, int epilogue, int64_t batch, int64_t m, int64_t n, int64_t k,
                   float add_diag, void* out_diag, int transpose_out, viola_stream_t stream);
 
 /* viola/optim/_orthogonalize.py:12-16 / _orthogonalize_kernels.py:80-84: x = dtype(matrix), optionally
  * transposed so rows <= cols, divided by (Frobenius norm + 1e-7), all in the working dtype.
- * in [batch, rows, cols] of in_dtype; out [batch, min, max] of dtype; workspace: batch floats. */
+ * in [batch, rows, cols] of in_dtype; out [batch, min, max] of dtype; workspace: 256 * batch floats (partial
+ * sums of squares; every slot is written before it is read, so it needs no clearing). */
 int viola_ns_prepare(const void* in, int in_dtype, void* out, int dtype, int64_t batch, int64_t rows, int64_t cols,
                      float* workspace, viola_stream_t stream);
 

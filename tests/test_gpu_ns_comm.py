@@ -65,6 +65,58 @@ def test_ns_gram_product_is_mirrored(dtype, batch, m, k, epilogue):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("batch,m,k", [(2, 384, 200), (1, 576, 384), (1, 1152, 64), (2, 256, 128)])
+@pytest.mark.parametrize("epilogue", [1, 2])
+def test_ns_gram_product_with_an_asymmetric_residual(dtype, batch, m, k, epilogue):
+    """a . a^T from one buffer (the mirrored path) with a residual that is NOT symmetric: every element, above and
+    below the diagonal, takes the epilogue with its own residual element, so the result equals the same product
+    taken with b as a separate copy of a (the full, un-mirrored kernel) bit for bit, and the oracle's contract."""
+    from viola_amd.optim import _orthogonalize_kernels as nk
+    torch.manual_seed(23)
+    a = (torch.randn(batch, m, k) / math.sqrt(k)).to(dtype).cuda()
+    residual = torch.randn(batch, m, m).to(dtype).cuda()
+    assert not torch.equal(residual, residual.mT)
+    same = nk._matmul(a, a, transpose_b=True, residual=residual, epilogue=epilogue)
+    other = nk._matmul(a, a.clone(), transpose_b=True, residual=residual, epilogue=epilogue)
+    assert torch.equal(same, other)
+    ref = ons.matmul(a.cpu(), a.cpu(), transpose_b=True, residual=residual.cpu(), epilogue=epilogue)
+    assert rel_l2(same, ref) < (2e-3 if dtype == torch.bfloat16 else 3e-4)
+    assert (same.cpu() == ref).float().mean() > .9
+
+
+def test_gram_chain_multiplies_r_by_r_past_the_first_iteration():
+    """viola/optim/_orthogonalize.py:44: z = -4.7750 r + 2.0315 (r @ r). After the first iteration of a segment r is
+    symmetric only up to fp16 rounding, so r @ r^T is a different product; the chain's GEMMs, replayed one by one
+    through the oracle's contract from the device's own intermediates, must be r @ r."""
+    from viola_amd.optim import _orthogonalize_kernels as nk
+    torch.manual_seed(24)
+    x = nk.prepare(torch.randn(1, 192, 640).cuda(), torch.float16)
+    r = nk._matmul(x, x, transpose_b=True)
+    z, q = nk._matmul(r, r, transpose_b=True, residual=r, epilogue=1, add_diag=nk.A_COEFF)
+    rz = nk._matmul(z, r, residual=r, epilogue=2)
+    r2 = nk._matmul(z, rz, residual=rz, epilogue=2)
+    assert not torch.equal(r2, r2.mT)                                          # the premise
+    calls = []
+    real = nk._matmul
+    def spy(a, b, **kw):
+        calls.append((a.data_ptr() == b.data_ptr(), kw.get("transpose_b", False), kw.get("epilogue", 0)))
+        return real(a, b, **kw)
+    nk._matmul = spy
+    try:
+        out = nk.run(torch.randn(1, 192, 640).cuda(), 5, "gram")
+    finally:
+        nk._matmul = real
+    grams = [c for c in calls if c[0] and c[2] == 1]
+    # segments of 2 and 3 iterations: the first z of each segment may use r r^T (r = x x^T is symmetric bit for bit),
+    # the other three must be r @ r
+    assert [c[1] for c in grams] == [True, False, True, False, False]
+    z2 = nk._matmul(r2, r2, residual=r2, epilogue=1)
+    ref = ons.matmul(r2.cpu(), r2.cpu(), residual=r2.cpu(), epilogue=1)
+    assert rel_l2(z2, ref) < 3e-4 and (z2.cpu() == ref).float().mean() > .9
+    assert torch.isfinite(out).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("batch,m,n,k", [(2, 192, 384, 192), (1, 130, 72, 96), (2, 64, 200, 136), (1, 33, 47, 65)])
 @pytest.mark.parametrize("transpose_b,epilogue", [(False, 2), (False, 0), (True, 0)])
 def test_ns_gemm_transposed_output(dtype, batch, m, n, k, transpose_b, epilogue):

@@ -33,8 +33,8 @@ def test_hardware_fp8_conversions_vs_software():
     counts = torch.zeros(4, dtype=torch.int64, device="cuda")
     _lib.call("viola_selftest_fp8", _lib.ptr(counts))
     torch.cuda.synchronize()
-    print("hw-vs-sw mismatches [e4m3 enc, e5m2 enc, e4m3 dec, e5m2 dec]:", counts.tolist())
-    assert counts[2:].tolist() == [0, 0]
+    # [e4m3 encode, e5m2 encode, e4m3 decode, e5m2 decode]: every fast quantizer path relies on all four being zero
+    assert counts.tolist() == [0, 0, 0, 0], f"hardware vs software FP8 conversion mismatches {counts.tolist()}"
 
 
 def test_software_codecs_all_codes():

@@ -340,6 +340,115 @@ def test_linear_oracle_against_float_math():
         assert rel_l2(dg, gg.grad) < 1e-5 and rel_l2(du, uu.grad) < 1e-6
 
 
+def _fake_quantize_rows(x, dtype=E4):
+    """Row-wise (1, 32) fake quantization written out with scalar loops over tiles: amax -> scale -> torch cast."""
+    limit = torch.finfo(dtype).max
+    out = torch.zeros(x.shape)
+    for r in range(x.shape[0]):
+        for c0 in range(0, x.shape[1], 32):
+            tile = x[r, c0:c0 + 32].float()
+            scale = tile.abs().max().clamp_min(1e-30) / limit
+            out[r, c0:c0 + 32] = (tile / scale).clamp(-limit, limit).to(dtype).float() * scale
+    return out
+
+
+@pytest.mark.parametrize("name", ["silu", "gelu", "relu"])
+def test_mlp_oracle_against_float_autograd_and_hand_composition(name):
+    """oracle.linear.mlp, pinned two ways. (1) Autograd of the float model down(act(gate(x)) * up(x))
+    (checks/mlp.py:12-16): a swapped gate/up half, dy used where the down projection's dx belongs, or a missing
+    term moves y / dx / a weight gradient by far more than FP8 quantization noise. (2) Every intermediate rebuilt by
+    hand from per-tile scalar-loop fake quantization and plain matmuls, bit for bit: z = [g | u] in that column order
+    and rounded to bf16, h = bf16(act(g) * u) from the ROUNDED g and u, dz = bf16([d*u*act'(g) | d*act(g)]) from the
+    rounded dH."""
+    torch.manual_seed(131)
+    rows, d_in, hidden, d_out = 33, 64, 96, 64
+    x = torch.randn(rows, d_in).bfloat16()
+    dy = torch.randn(rows, d_out).bfloat16()
+    w_gu = (torch.randn(2 * hidden, d_in) / d_in ** .5)
+    w_dn = (torch.randn(d_out, hidden) / hidden ** .5)
+    b_gu, b_dn = torch.randn(2 * hidden) * .1, torch.randn(d_out) * .1
+    # the oracle takes dequantized weights: put them on the (32, 32) FP8 grid first
+    w_gu = grouped.dequantize(*grouped.quantize(w_gu, E4, (32, 32)), (32, 32))
+    w_dn = grouped.dequantize(*grouped.quantize(w_dn, E4, (32, 32)), (32, 32))
+    r = linear.mlp(x, w_gu, b_gu, w_dn, b_dn, dy, name=name)
+
+    # (1) float autograd
+    xf = x.float().requires_grad_()
+    wg, wd = w_gu.clone().requires_grad_(), w_dn.clone().requires_grad_()
+    bg, bd = b_gu.clone().requires_grad_(), b_dn.clone().requires_grad_()
+    zf = xf @ wg.T + bg
+    yf = (linear.activation(name)(zf[:, :hidden]) * zf[:, hidden:]) @ wd.T + bd
+    yf.backward(dy.float())
+    bar = .12                                                        # two to three FP8 + bf16 roundings in a row (relu: kinks flip)
+    assert rel_l2(r["y"], yf.detach()) < bar and rel_l2(r["dx"], xf.grad) < bar
+    assert rel_l2(r["dw_gate_up"], wg.grad) < bar and rel_l2(r["dw_down"], wd.grad) < bar
+    assert rel_l2(r["db_gate_up"], bg.grad) < bar and torch.equal(r["db_down"], dy.sum(0, dtype=torch.bfloat16))
+    # the two halves are not interchangeable: the swapped model is far outside the bar
+    swapped = (linear.activation(name)(zf[:, hidden:]) * zf[:, :hidden]) @ wd.T + bd
+    assert rel_l2(r["y"], swapped.detach()) > 3 * bar
+
+    # (2) by hand
+    z = (_fake_quantize_rows(x) @ w_gu.T + b_gu).bfloat16()
+    assert r["z"].dtype == torch.bfloat16 and torch.equal(r["z"], z)
+    g, u = z[:, :hidden].float(), z[:, hidden:].float()
+    act = {"silu": lambda t: t * (1 / (1 + torch.exp(-t))), "relu": lambda t: t.clamp_min(0),
+           "gelu": lambda t: .5 * t * (1 + torch.tanh(0.7978845608028654 * (t + 0.044715 * t * t * t)))}[name]
+    h = (act(g) * u).bfloat16()
+    assert r["h"].dtype == torch.bfloat16 and torch.equal(r["h"], h)
+    assert torch.equal(r["y"], (_fake_quantize_rows(h) @ w_dn.T + b_dn).bfloat16())
+    dh = (_fake_quantize_rows(dy) @ w_dn).bfloat16().float()          # dgrad of the down projection, rounded
+    gg = g.clone().requires_grad_()
+    act(gg).sum().backward()
+    dz = torch.cat([dh * u * gg.grad, dh * act(g)], 1).bfloat16()
+    assert rel_l2(r["dz"], dz) < 2e-3                                  # autograd's derivative vs the closed form: last-place
+    assert (r["dz"].float() - dz.float()).abs().max() <= 2 ** -7 * dz.float().abs().max()
+    assert torch.equal(r["dx"], (_fake_quantize_rows(r["dz"]) @ w_gu).bfloat16())
+    # weight gradients contract over tokens: groups of 32 along the token axis of the transposed operands
+    gt, ht = _fake_quantize_rows(dy.T.contiguous()), _fake_quantize_rows(h.T.contiguous())
+    assert torch.equal(r["dw_down"], (gt @ ht.T).bfloat16())
+    zt, xt = _fake_quantize_rows(r["dz"].T.contiguous()), _fake_quantize_rows(x.T.contiguous())
+    assert torch.equal(r["dw_gate_up"], (zt @ xt.T).bfloat16())
+    assert torch.equal(r["db_gate_up"], r["dz"].sum(0, dtype=torch.bfloat16))
+
+
+def test_varlen_linear_oracle_against_brute_force():
+    """oracle.linear.varlen_linear on tiny inputs (groups of 0, 1, 37 and 3 rows), against loops that know nothing of
+    oracle.linear: rows of group g see weight g only, token tiles of the weight gradient restart at each group's first
+    row, an empty group contributes no rows and a zero gradient."""
+    torch.manual_seed(77)
+    counts, d_in, d_out = [0, 1, 37, 3, 0], 64, 32
+    total = sum(counts)
+    x = torch.randn(total, d_in).bfloat16()
+    dy = (torch.randn(total, d_out) * .1).bfloat16()
+    weights = [grouped.dequantize(*grouped.quantize(torch.randn(d_out, d_in) / 8, E4, (32, 32)), (32, 32)) for _ in counts]
+    r = linear.varlen_linear(x, weights, counts, dy)
+    assert r["y"].shape == (total, d_out) and r["dx"].shape == (total, d_in) and r["dw"].shape == (len(counts), d_out, d_in)
+    fx, fg = _fake_quantize_rows(x).double(), _fake_quantize_rows(dy).double()
+    offset = 0
+    for group, count in enumerate(counts):
+        w = weights[group].double()
+        for row in range(offset, offset + count):
+            y_row = torch.tensor([sum(fx[row, k] * w[n, k] for k in range(d_in)) for n in range(d_out)])
+            dx_row = torch.tensor([sum(fg[row, n] * w[n, k] for n in range(d_out)) for k in range(d_in)])
+            assert torch.equal(r["y"][row], y_row.float().bfloat16()) or rel_l2(r["y"][row], y_row) < 4e-3
+            assert torch.equal(r["dx"][row], dx_row.float().bfloat16()) or rel_l2(r["dx"][row], dx_row) < 4e-3
+        if count == 0:
+            assert r["dw"][group].abs().max() == 0
+        else:
+            # tiles of 32 tokens counted from the group's own first row
+            gt = _fake_quantize_rows(dy[offset:offset + count].T.contiguous()).double()
+            xt = _fake_quantize_rows(x[offset:offset + count].T.contiguous()).double()
+            assert rel_l2(r["dw"][group], gt @ xt.T) < 4e-3
+            if count > 1:                                            # tiles counted from row 0 of the batch differ
+                wrong = _fake_quantize_rows(dy.T.contiguous())[:, offset:offset + count].double() @ _fake_quantize_rows(x.T.contiguous())[:, offset:offset + count].double().T
+                assert rel_l2(wrong, gt @ xt.T) > 1e-3 or count % 32 == 0 and offset % 32 == 0
+        offset += count
+    # a group's rows depend on no other group: recomputing with the other weights zeroed changes nothing for group 2
+    zeroed = [w if g == 2 else torch.zeros_like(w) for g, w in enumerate(weights)]
+    r2 = linear.varlen_linear(x, zeroed, counts, dy)
+    assert torch.equal(r2["y"][1:38], r["y"][1:38]) and torch.equal(r2["dw"][2], r["dw"][2]) and r2["y"][0].abs().max() == 0
+
+
 # ----------------------------------------------------------------------------- per-tensor scaling
 @pytest.mark.parametrize("dtype", [E4, E5])
 def test_tensor_oracle_matches_the_reference_cpu_definitions(dtype):

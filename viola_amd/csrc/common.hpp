@@ -12,9 +12,28 @@
         if (!(cond)) return VIOLA_EINVAL; \
     } while (0)
 
+// Launches go through hipLaunchKernel, whose return value is the launch's own status; the first failure of an
+// entry point's launches is kept per thread and handed out (and cleared) by viola_launch_status(). The runtime's
+// last-error slot is never read or cleared: it may hold another library's error, and reading it is a call an
+// entry point has no need to make while a stream is being captured.
+inline thread_local int viola_first_launch_error = 0;
+
+template <typename... Params, typename... Args>
+static inline void viola_launch(void (*kernel)(Params...), dim3 grid, dim3 block, unsigned lds_bytes, hipStream_t stream,
+                                Args&&... args) {
+    static_assert(sizeof...(Params) == sizeof...(Args), "one argument per kernel parameter");
+    [&](Params... values) {
+        void* slots[] = {const_cast<void*>(static_cast<const void*>(&values))...};
+        const hipError_t e = hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, slots, lds_bytes, stream);
+        if (e != hipSuccess && viola_first_launch_error == 0) viola_first_launch_error = (int)e;
+    }(static_cast<Params>(args)...);
+}
+#define VIOLA_LAUNCH(kernel, grid, block, lds_bytes, stream, ...) viola_launch(kernel, grid, block, lds_bytes, stream, __VA_ARGS__)
+
 static inline int viola_launch_status() {
-    hipError_t e = hipGetLastError();
-    return e == hipSuccess ? 0 : (int)e;
+    const int e = viola_first_launch_error;
+    viola_first_launch_error = 0;
+    return e;
 }
 
 static inline bool viola_is_fp8(int dtype) { return dtype == VIOLA_E4M3 || dtype == VIOLA_E5M2; }

@@ -298,10 +298,10 @@ static int shift_of(int v) {
 template <int MODE, bool B_ROWSCALE, bool VEC, typename TO>
 static void launch_formats(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, dim3 grid, hipStream_t stream) {
     const bool a5 = a_dtype == VIOLA_E5M2, b5 = b_dtype == VIOLA_E5M2;
-    if (!a5 && !b5) hipLaunchKernelGGL((group_gemm_kernel<MODE, false, false, B_ROWSCALE, VEC, TO>), grid, dim3(256), 0, stream, p, bias_dtype);
-    else if (a5 && !b5) hipLaunchKernelGGL((group_gemm_kernel<MODE, true, false, B_ROWSCALE, VEC, TO>), grid, dim3(256), 0, stream, p, bias_dtype);
-    else if (!a5 && b5) hipLaunchKernelGGL((group_gemm_kernel<MODE, false, true, B_ROWSCALE, VEC, TO>), grid, dim3(256), 0, stream, p, bias_dtype);
-    else hipLaunchKernelGGL((group_gemm_kernel<MODE, true, true, B_ROWSCALE, VEC, TO>), grid, dim3(256), 0, stream, p, bias_dtype);
+    if (!a5 && !b5) VIOLA_LAUNCH((group_gemm_kernel<MODE, false, false, B_ROWSCALE, VEC, TO>), grid, dim3(256), 0, stream, p, bias_dtype);
+    else if (a5 && !b5) VIOLA_LAUNCH((group_gemm_kernel<MODE, true, false, B_ROWSCALE, VEC, TO>), grid, dim3(256), 0, stream, p, bias_dtype);
+    else if (!a5 && b5) VIOLA_LAUNCH((group_gemm_kernel<MODE, false, true, B_ROWSCALE, VEC, TO>), grid, dim3(256), 0, stream, p, bias_dtype);
+    else VIOLA_LAUNCH((group_gemm_kernel<MODE, true, true, B_ROWSCALE, VEC, TO>), grid, dim3(256), 0, stream, p, bias_dtype);
 }
 
 template <int MODE, typename TO>

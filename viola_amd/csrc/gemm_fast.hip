@@ -7,10 +7,10 @@ namespace viola {
 template <int MODE, bool B_ROWSCALE, typename TO, int TN>
 static void launch_formats(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, dim3 grid, hipStream_t stream) {
     const bool a5 = a_dtype == VIOLA_E5M2, b5 = b_dtype == VIOLA_E5M2;
-    if (!a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE, false, false, B_ROWSCALE, TO, TN>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else if (a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE, true, false, B_ROWSCALE, TO, TN>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else if (!a5 && b5) hipLaunchKernelGGL((group_gemm_fast<MODE, false, true, B_ROWSCALE, TO, TN>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else hipLaunchKernelGGL((group_gemm_fast<MODE, true, true, B_ROWSCALE, TO, TN>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    if (!a5 && !b5) VIOLA_LAUNCH((group_gemm_fast<MODE, false, false, B_ROWSCALE, TO, TN>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    else if (a5 && !b5) VIOLA_LAUNCH((group_gemm_fast<MODE, true, false, B_ROWSCALE, TO, TN>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    else if (!a5 && b5) VIOLA_LAUNCH((group_gemm_fast<MODE, false, true, B_ROWSCALE, TO, TN>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    else VIOLA_LAUNCH((group_gemm_fast<MODE, true, true, B_ROWSCALE, TO, TN>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
 }
 
 template <int MODE, int TN>

@@ -10,20 +10,20 @@ namespace viola {
 template <int MODE, typename TO, int TN, bool TENSOR, bool MX>
 static void launch_scaled_formats(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, dim3 grid, hipStream_t stream) {
     const bool a5 = a_dtype == VIOLA_E5M2, b5 = b_dtype == VIOLA_E5M2;
-    if (!a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE, false, false, false, TO, TN, TENSOR, MX>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else if (a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE, true, false, false, TO, TN, TENSOR, MX>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else if (!a5 && b5) hipLaunchKernelGGL((group_gemm_fast<MODE, false, true, false, TO, TN, TENSOR, MX>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else hipLaunchKernelGGL((group_gemm_fast<MODE, true, true, false, TO, TN, TENSOR, MX>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    if (!a5 && !b5) VIOLA_LAUNCH((group_gemm_fast<MODE, false, false, false, TO, TN, TENSOR, MX>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    else if (a5 && !b5) VIOLA_LAUNCH((group_gemm_fast<MODE, true, false, false, TO, TN, TENSOR, MX>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    else if (!a5 && b5) VIOLA_LAUNCH((group_gemm_fast<MODE, false, true, false, TO, TN, TENSOR, MX>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    else VIOLA_LAUNCH((group_gemm_fast<MODE, true, true, false, TO, TN, TENSOR, MX>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
 }
 
 // The 256 x 256 tile (one 512-thread block per CU) for products with at least two rounds of such tiles (8192 x 4096 x 1024: 52.9 us against 58.5; with fewer tiles the 128 x 128 kernel wins).
 template <int MODE, typename TO, bool TENSOR, bool MX>
 static void launch_big_formats(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, dim3 grid, hipStream_t stream) {
     const bool a5 = a_dtype == VIOLA_E5M2, b5 = b_dtype == VIOLA_E5M2;
-    if (!a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE, false, false, false, TO, 2, TENSOR, MX, true>), grid, dim3(512), 0, stream, p, bias_dtype);
-    else if (a5 && !b5) hipLaunchKernelGGL((group_gemm_fast<MODE, true, false, false, TO, 2, TENSOR, MX, true>), grid, dim3(512), 0, stream, p, bias_dtype);
-    else if (!a5 && b5) hipLaunchKernelGGL((group_gemm_fast<MODE, false, true, false, TO, 2, TENSOR, MX, true>), grid, dim3(512), 0, stream, p, bias_dtype);
-    else hipLaunchKernelGGL((group_gemm_fast<MODE, true, true, false, TO, 2, TENSOR, MX, true>), grid, dim3(512), 0, stream, p, bias_dtype);
+    if (!a5 && !b5) VIOLA_LAUNCH((group_gemm_fast<MODE, false, false, false, TO, 2, TENSOR, MX, true>), grid, dim3(512), 0, stream, p, bias_dtype);
+    else if (a5 && !b5) VIOLA_LAUNCH((group_gemm_fast<MODE, true, false, false, TO, 2, TENSOR, MX, true>), grid, dim3(512), 0, stream, p, bias_dtype);
+    else if (!a5 && b5) VIOLA_LAUNCH((group_gemm_fast<MODE, false, true, false, TO, 2, TENSOR, MX, true>), grid, dim3(512), 0, stream, p, bias_dtype);
+    else VIOLA_LAUNCH((group_gemm_fast<MODE, true, true, false, TO, 2, TENSOR, MX, true>), grid, dim3(512), 0, stream, p, bias_dtype);
 }
 
 #ifndef VIOLA_MX_BIG_GATED

@@ -268,9 +268,9 @@ static bool launch_gated_pieces(const void* z, const void* dy, int64_t dy_stride
     const T* dp = static_cast<const T*>(dy);
     T* op = static_cast<T*>(out);
 #define VIOLA_GATED(ACT)                                                                                                   \
-    if (backward) hipLaunchKernelGGL((gated_backward_pieces<T, ACT>), grid, dim3(256), 0, stream, zp, dp, dy_stride, op, pieces, per_row); \
-    else if (epilogue_form) hipLaunchKernelGGL((gated_forward_pieces<T, ACT, true>), grid, dim3(256), 0, stream, zp, op, pieces, per_row); \
-    else hipLaunchKernelGGL((gated_forward_pieces<T, ACT, false>), grid, dim3(256), 0, stream, zp, op, pieces, per_row);
+    if (backward) VIOLA_LAUNCH((gated_backward_pieces<T, ACT>), grid, dim3(256), 0, stream, zp, dp, dy_stride, op, pieces, per_row); \
+    else if (epilogue_form) VIOLA_LAUNCH((gated_forward_pieces<T, ACT, true>), grid, dim3(256), 0, stream, zp, op, pieces, per_row); \
+    else VIOLA_LAUNCH((gated_forward_pieces<T, ACT, false>), grid, dim3(256), 0, stream, zp, op, pieces, per_row);
     if (activation == VIOLA_SILU) { VIOLA_GATED(VIOLA_SILU) }
     else if (activation == VIOLA_GELU) { VIOLA_GATED(VIOLA_GELU) }
     else { VIOLA_GATED(VIOLA_RELU) }
@@ -331,11 +331,11 @@ static int launch_pack(const float* x, int64_t n, uint8_t* packet, int64_t rows,
                        hipStream_t stream) {
     const int64_t units = rows * groups;
     if (tile == 256 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(packet) % 4 == 0) {
-        hipLaunchKernelGGL(comm_pack256_kernel<TQ>, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x, n, packet, rows, groups, stride);
+        VIOLA_LAUNCH(comm_pack256_kernel<TQ>, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x, n, packet, rows, groups, stride);
     } else if (tile >= 64) {
-        hipLaunchKernelGGL((comm_pack_kernel<TQ, 64>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x, n, packet, rows, groups, tile, stride);
+        VIOLA_LAUNCH((comm_pack_kernel<TQ, 64>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x, n, packet, rows, groups, tile, stride);
     } else {
-        hipLaunchKernelGGL((comm_pack_kernel<TQ, 32>), dim3((unsigned)((units + 7) / 8)), dim3(256), 0, stream, x, n, packet, rows, groups, tile, stride);
+        VIOLA_LAUNCH((comm_pack_kernel<TQ, 32>), dim3((unsigned)((units + 7) / 8)), dim3(256), 0, stream, x, n, packet, rows, groups, tile, stride);
     }
     return viola_launch_status();
 }
@@ -370,14 +370,14 @@ extern "C" int viola_comm_unpack(const void* packet, float* out, int64_t n, int6
         const int64_t width = groups * tile;
         const int shift = __builtin_ctz((unsigned)tile);
         const dim3 grid(grid_for(total / 4));
-#define VIOLA_UNPACK(TQ, REDUCE) hipLaunchKernelGGL((comm_unpack_quads_kernel<TQ, REDUCE>), grid, dim3(256), 0, stream, pk, out, n, rows, width, shift, stride)
+#define VIOLA_UNPACK(TQ, REDUCE) VIOLA_LAUNCH((comm_unpack_quads_kernel<TQ, REDUCE>), grid, dim3(256), 0, stream, pk, out, n, rows, width, shift, stride)
         if (fp8_dtype == VIOLA_E4M3) { if (reduce) VIOLA_UNPACK(e4m3_t, true); else VIOLA_UNPACK(e4m3_t, false); }
         else { if (reduce) VIOLA_UNPACK(e5m2_t, true); else VIOLA_UNPACK(e5m2_t, false); }
 #undef VIOLA_UNPACK
         return viola_launch_status();
     }
-    if (fp8_dtype == VIOLA_E4M3) hipLaunchKernelGGL(comm_unpack_kernel<e4m3_t>, dim3(grid_for(total)), dim3(256), 0, stream, pk, out, n, rows, groups, tile, stride, reduce);
-    else hipLaunchKernelGGL(comm_unpack_kernel<e5m2_t>, dim3(grid_for(total)), dim3(256), 0, stream, pk, out, n, rows, groups, tile, stride, reduce);
+    if (fp8_dtype == VIOLA_E4M3) VIOLA_LAUNCH(comm_unpack_kernel<e4m3_t>, dim3(grid_for(total)), dim3(256), 0, stream, pk, out, n, rows, groups, tile, stride, reduce);
+    else VIOLA_LAUNCH(comm_unpack_kernel<e5m2_t>, dim3(grid_for(total)), dim3(256), 0, stream, pk, out, n, rows, groups, tile, stride, reduce);
     return viola_launch_status();
 }
 
@@ -388,7 +388,7 @@ extern "C" int viola_gated_forward(const void* z, void* out, int64_t rows, int64
     if (rows == 0 || h == 0) return 0;
     VIOLA_CHECK_ARG(z && out);
     if (launch_gated_pieces(z, nullptr, 0, out, rows, h, dtype, activation, false, false, stream)) return viola_launch_status();
-    hipLaunchKernelGGL(gated_forward_kernel, dim3(grid_for(rows * h)), dim3(256), 0, stream, z, out, rows, h, dtype, activation);
+    VIOLA_LAUNCH(gated_forward_kernel, dim3(grid_for(rows * h)), dim3(256), 0, stream, z, out, rows, h, dtype, activation);
     return viola_launch_status();
 }
 
@@ -399,14 +399,14 @@ extern "C" int viola_gated_backward(const void* z, const void* dy, void* dz, int
     if (rows == 0 || h == 0) return 0;
     VIOLA_CHECK_ARG(z && dy && dz);
     if (launch_gated_pieces(z, dy, h, dz, rows, h, dtype, activation, true, false, stream)) return viola_launch_status();
-    hipLaunchKernelGGL(gated_backward_kernel, dim3(grid_for(rows * h)), dim3(256), 0, stream, z, dy, dz, rows, h, dtype, activation);
+    VIOLA_LAUNCH(gated_backward_kernel, dim3(grid_for(rows * h)), dim3(256), 0, stream, z, dy, dz, rows, h, dtype, activation);
     return viola_launch_status();
 }
 
 extern "C" int viola_selftest_fp8(uint64_t* counts, viola_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     VIOLA_CHECK_ARG(counts);
-    hipLaunchKernelGGL(selftest_fp8_kernel, dim3(4096), dim3(256), 0, stream, reinterpret_cast<unsigned long long*>(counts));
+    VIOLA_LAUNCH(selftest_fp8_kernel, dim3(4096), dim3(256), 0, stream, reinterpret_cast<unsigned long long*>(counts));
     return viola_launch_status();
 }
 
@@ -415,7 +415,7 @@ extern "C" int viola_selftest_philox(const uint64_t* triples, uint32_t* out, int
     VIOLA_CHECK_ARG(count >= 0);
     if (count == 0) return 0;
     VIOLA_CHECK_ARG(triples && out);
-    hipLaunchKernelGGL(selftest_philox_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, triples, out, count);
+    VIOLA_LAUNCH(selftest_philox_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, triples, out, count);
     return viola_launch_status();
 }
 

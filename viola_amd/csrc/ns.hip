@@ -396,9 +396,9 @@ static int launch_ns(const void* a, const void* b, const void* residual, void* o
     const uint16_t* rp = static_cast<const uint16_t*>(residual);
     uint16_t* op = static_cast<uint16_t*>(out);
     uint16_t* dp = static_cast<uint16_t*>(out_diag);
-    if (epilogue == 0) hipLaunchKernelGGL((ns_gemm_kernel<IS_BF16, TRANSPOSE_B, 0, VEC>), grid, dim3(256), 0, stream, ap, bp, rp, op, dp, m, n, k, add_diag, transpose_out);
-    else if (epilogue == 1) hipLaunchKernelGGL((ns_gemm_kernel<IS_BF16, TRANSPOSE_B, 1, VEC>), grid, dim3(256), 0, stream, ap, bp, rp, op, dp, m, n, k, add_diag, transpose_out);
-    else hipLaunchKernelGGL((ns_gemm_kernel<IS_BF16, TRANSPOSE_B, 2, VEC>), grid, dim3(256), 0, stream, ap, bp, rp, op, dp, m, n, k, add_diag, transpose_out);
+    if (epilogue == 0) VIOLA_LAUNCH((ns_gemm_kernel<IS_BF16, TRANSPOSE_B, 0, VEC>), grid, dim3(256), 0, stream, ap, bp, rp, op, dp, m, n, k, add_diag, transpose_out);
+    else if (epilogue == 1) VIOLA_LAUNCH((ns_gemm_kernel<IS_BF16, TRANSPOSE_B, 1, VEC>), grid, dim3(256), 0, stream, ap, bp, rp, op, dp, m, n, k, add_diag, transpose_out);
+    else VIOLA_LAUNCH((ns_gemm_kernel<IS_BF16, TRANSPOSE_B, 2, VEC>), grid, dim3(256), 0, stream, ap, bp, rp, op, dp, m, n, k, add_diag, transpose_out);
     return viola_launch_status();
 }
 
@@ -409,22 +409,22 @@ static int launch_prepare(const void* in, void* out, int64_t batch, int64_t rows
     if constexpr (sizeof(TIn) == 2) {
         const bool aligned = reinterpret_cast<uintptr_t>(in) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
         if (aligned && cols % 8 == 0 && (rows * cols) % 8 == 0 && (rows + 127) / 128 <= 65535) {
-            hipLaunchKernelGGL((ns_sumsq16_kernel<TIn, IS_BF16>), dim3(PARTS, (unsigned)batch), dim3(256), 0, stream, src, workspace, rows * cols);
+            VIOLA_LAUNCH((ns_sumsq16_kernel<TIn, IS_BF16>), dim3(PARTS, (unsigned)batch), dim3(256), 0, stream, src, workspace, rows * cols);
             if (rows > cols) {
                 const dim3 tgrid((unsigned)((cols + 63) / 64), (unsigned)((rows + 127) / 128), (unsigned)batch);
-                hipLaunchKernelGGL((ns_scale16_transposed_kernel<TIn, IS_BF16>), tgrid, dim3(256), 0, stream, src, static_cast<uint16_t*>(out), workspace, rows, cols);
+                VIOLA_LAUNCH((ns_scale16_transposed_kernel<TIn, IS_BF16>), tgrid, dim3(256), 0, stream, src, static_cast<uint16_t*>(out), workspace, rows, cols);
             } else {
                 const int64_t octets = rows * cols / 8;
                 const unsigned bx = (unsigned)(octets / 256 / 4 < 1 ? 1 : octets / 256 / 4 > 4096 ? 4096 : octets / 256 / 4);
-                hipLaunchKernelGGL((ns_scale16_kernel<TIn, IS_BF16>), dim3(bx, (unsigned)batch), dim3(256), 0, stream, src, static_cast<uint16_t*>(out), workspace, rows * cols);
+                VIOLA_LAUNCH((ns_scale16_kernel<TIn, IS_BF16>), dim3(bx, (unsigned)batch), dim3(256), 0, stream, src, static_cast<uint16_t*>(out), workspace, rows * cols);
             }
             return viola_launch_status();
         }
     }
-    hipLaunchKernelGGL((ns_sumsq_kernel<TIn, IS_BF16>), dim3(PARTS, (unsigned)batch), dim3(256), 0, stream, src, workspace, rows * cols);
+    VIOLA_LAUNCH((ns_sumsq_kernel<TIn, IS_BF16>), dim3(PARTS, (unsigned)batch), dim3(256), 0, stream, src, workspace, rows * cols);
     const dim3 grid((unsigned)((cols + 31) / 32), (unsigned)((rows + 31) / 32), (unsigned)batch);
-    if (rows > cols) hipLaunchKernelGGL((ns_scale_kernel<TIn, IS_BF16, true>), grid, dim3(256), 0, stream, src, static_cast<uint16_t*>(out), workspace, rows, cols);
-    else hipLaunchKernelGGL((ns_scale_kernel<TIn, IS_BF16, false>), grid, dim3(256), 0, stream, src, static_cast<uint16_t*>(out), workspace, rows, cols);
+    if (rows > cols) VIOLA_LAUNCH((ns_scale_kernel<TIn, IS_BF16, true>), grid, dim3(256), 0, stream, src, static_cast<uint16_t*>(out), workspace, rows, cols);
+    else VIOLA_LAUNCH((ns_scale_kernel<TIn, IS_BF16, false>), grid, dim3(256), 0, stream, src, static_cast<uint16_t*>(out), workspace, rows, cols);
     return viola_launch_status();
 }
 

@@ -19,7 +19,8 @@
 //   * the b matrix is the MFMA "A" source, so a lane owns one output row m and runs of four
 //     consecutive n: 8-byte stores, per-row residual loads.
 //   * a Gram-type product (b == a, square output) computes only the tiles on and above the diagonal and
-//     stores each off-diagonal tile a second time transposed; transpose_out stores [n, m] only.
+//     stores each off-diagonal tile a second time transposed, its epilogue applied with the residual of the
+//     transposed position (exact for any residual); transpose_out stores [n, m] only.
 //   * work order: the 1-D grid is cut into eight contiguous ranges, one per XCD (blockIdx % 8), and
 //     inside a range tiles walk n fastest, so the tiles that share an a panel meet in one L2.
 #include "ns_args.hpp"
@@ -301,8 +302,19 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void ns_gemm_fast(NsArgs
                     // instruction still fills 64-byte segments
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        out[(col + e) * m + row] = o[e];
-                        if (out_diag) out_diag[(col + e) * m + row] = od[e];
+                        uint16_t flipped = o[e], flipped_diag = od[e];
+                        if (EPILOGUE && mirror) {
+                            // element [col + e, row] of a . a^T has this element's product (the sums run over the same
+                            // terms in the same order) but its own residual, which need not be symmetric; an
+                            // off-diagonal tile holds no diagonal element
+                            float value = ns_widen<IS_BF16>(ns_narrow<IS_BF16>(acc[i][j][r4 * 4 + e]));
+                            const float r = ns_widen<IS_BF16>(residual[(col + e) * n + row]);
+                            if (EPILOGUE == 1) value = -4.7750f * r + 2.0315f * value;
+                            if (EPILOGUE == 2) value = value + 3.4445f * r;
+                            flipped = flipped_diag = ns_narrow<IS_BF16>(value);
+                        }
+                        out[(col + e) * m + row] = flipped;
+                        if (out_diag) out_diag[(col + e) * m + row] = flipped_diag;
                     }
                 }
             }
@@ -317,9 +329,9 @@ static void launch_tiles(NsArgs p, int epilogue, hipStream_t stream) {
     p.tiles_n = (int)((p.n + BN - 1) / BN);
     p.tiles = p.batch * (p.symmetric ? (int64_t)p.tiles_n * (p.tiles_n + 1) / 2 : (int64_t)p.tiles_m * p.tiles_n);
     const unsigned grid = (unsigned)((p.tiles + 7) / 8 * 8);
-    if (epilogue == 0) hipLaunchKernelGGL((ns_gemm_fast<IS_BF16, B_KN, 0, WM, WN, WAVES_M, WAVES_N, SBK, STAGES>), dim3(grid), dim3(THREADS), 0, stream, p);
-    else if (epilogue == 1) hipLaunchKernelGGL((ns_gemm_fast<IS_BF16, B_KN, 1, WM, WN, WAVES_M, WAVES_N, SBK, STAGES>), dim3(grid), dim3(THREADS), 0, stream, p);
-    else hipLaunchKernelGGL((ns_gemm_fast<IS_BF16, B_KN, 2, WM, WN, WAVES_M, WAVES_N, SBK, STAGES>), dim3(grid), dim3(THREADS), 0, stream, p);
+    if (epilogue == 0) VIOLA_LAUNCH((ns_gemm_fast<IS_BF16, B_KN, 0, WM, WN, WAVES_M, WAVES_N, SBK, STAGES>), dim3(grid), dim3(THREADS), 0, stream, p);
+    else if (epilogue == 1) VIOLA_LAUNCH((ns_gemm_fast<IS_BF16, B_KN, 1, WM, WN, WAVES_M, WAVES_N, SBK, STAGES>), dim3(grid), dim3(THREADS), 0, stream, p);
+    else VIOLA_LAUNCH((ns_gemm_fast<IS_BF16, B_KN, 2, WM, WN, WAVES_M, WAVES_N, SBK, STAGES>), dim3(grid), dim3(THREADS), 0, stream, p);
 }
 
 template <bool IS_BF16, bool B_KN>

@@ -400,8 +400,8 @@ extern "C" int viola_momentum_update(const void* grad, int grad_dtype, const voi
         if (quads) {
             const dim3 qgrid((unsigned)((whole + 3) / 4));
 #define VIOLA_MQ(TG, EPL)                                                                                                   \
-    if (rounding) hipLaunchKernelGGL((momentum_1d_quads<TG, EPL, true>), qgrid, dim3(256), 0, stream, static_cast<const TG*>(grad), oq, old_scale, nq, new_scale, up, whole, beta, inv_loss_scale, nesterov, step, key); \
-    else hipLaunchKernelGGL((momentum_1d_quads<TG, EPL, false>), qgrid, dim3(256), 0, stream, static_cast<const TG*>(grad), oq, old_scale, nq, new_scale, up, whole, beta, inv_loss_scale, nesterov, step, key);
+    if (rounding) VIOLA_LAUNCH((momentum_1d_quads<TG, EPL, true>), qgrid, dim3(256), 0, stream, static_cast<const TG*>(grad), oq, old_scale, nq, new_scale, up, whole, beta, inv_loss_scale, nesterov, step, key); \
+    else VIOLA_LAUNCH((momentum_1d_quads<TG, EPL, false>), qgrid, dim3(256), 0, stream, static_cast<const TG*>(grad), oq, old_scale, nq, new_scale, up, whole, beta, inv_loss_scale, nesterov, step, key);
 #define VIOLA_MQT(EPL)                                                          \
     if (grad_dtype == VIOLA_F32) { VIOLA_MQ(float, EPL) }                        \
     else if (grad_dtype == VIOLA_BF16) { VIOLA_MQ(bf16_t, EPL) }                 \
@@ -414,8 +414,8 @@ extern "C" int viola_momentum_update(const void* grad, int grad_dtype, const voi
             const dim3 grid((unsigned)((blocks - first + 3) / 4));
 #define VIOLA_M1(EPL)                                                                                                        \
     case EPL * 64:                                                                                                           \
-        if (rounding) hipLaunchKernelGGL((momentum_1d_kernel<EPL, true>), grid, dim3(256), 0, stream, grad, grad_dtype, oq, old_scale, nq, new_scale, up, n, first, blocks, beta, inv_loss_scale, nesterov, step, key); \
-        else hipLaunchKernelGGL((momentum_1d_kernel<EPL, false>), grid, dim3(256), 0, stream, grad, grad_dtype, oq, old_scale, nq, new_scale, up, n, first, blocks, beta, inv_loss_scale, nesterov, step, key); \
+        if (rounding) VIOLA_LAUNCH((momentum_1d_kernel<EPL, true>), grid, dim3(256), 0, stream, grad, grad_dtype, oq, old_scale, nq, new_scale, up, n, first, blocks, beta, inv_loss_scale, nesterov, step, key); \
+        else VIOLA_LAUNCH((momentum_1d_kernel<EPL, false>), grid, dim3(256), 0, stream, grad, grad_dtype, oq, old_scale, nq, new_scale, up, n, first, blocks, beta, inv_loss_scale, nesterov, step, key); \
         break;
             switch (tile_size) { VIOLA_M1(1) VIOLA_M1(2) VIOLA_M1(4) VIOLA_M1(8) VIOLA_M1(16) }
 #undef VIOLA_M1
@@ -425,8 +425,8 @@ extern "C" int viola_momentum_update(const void* grad, int grad_dtype, const voi
     VIOLA_CHECK_ARG(planes > 0 && rows > 0 && cols > 0 && planes * rows * cols == n && tr > 0 && tc > 0 && tr * tc <= 4096);
     const int64_t tiles = planes * ((rows + tr - 1) / tr) * ((cols + tc - 1) / tc);
     const dim3 grid((unsigned)((tiles + 3) / 4));
-    if (rounding) hipLaunchKernelGGL((momentum_2d_kernel<true>), grid, dim3(256), 0, stream, grad, grad_dtype, oq, old_scale, nq, new_scale, up, planes, rows, cols, tr, tc, beta, inv_loss_scale, nesterov, step, key);
-    else hipLaunchKernelGGL((momentum_2d_kernel<false>), grid, dim3(256), 0, stream, grad, grad_dtype, oq, old_scale, nq, new_scale, up, planes, rows, cols, tr, tc, beta, inv_loss_scale, nesterov, step, key);
+    if (rounding) VIOLA_LAUNCH((momentum_2d_kernel<true>), grid, dim3(256), 0, stream, grad, grad_dtype, oq, old_scale, nq, new_scale, up, planes, rows, cols, tr, tc, beta, inv_loss_scale, nesterov, step, key);
+    else VIOLA_LAUNCH((momentum_2d_kernel<false>), grid, dim3(256), 0, stream, grad, grad_dtype, oq, old_scale, nq, new_scale, up, planes, rows, cols, tr, tc, beta, inv_loss_scale, nesterov, step, key);
     return viola_launch_status();
 }
 
@@ -441,8 +441,8 @@ extern "C" int viola_momentum_update_table(const int64_t* table, int64_t tensors
     VIOLA_CHECK_ARG(table);
     const dim3 grid((unsigned)((tiles + 3) / 4), (unsigned)tensors);
 #define VIOLA_MT(TG, EPL)                                                                                                   \
-    if (rounding) hipLaunchKernelGGL((momentum_table_quads<TG, EPL, true>), grid, dim3(256), 0, stream, table, tiles, beta, inv_loss_scale, nesterov, (uint64_t)rounding_step); \
-    else hipLaunchKernelGGL((momentum_table_quads<TG, EPL, false>), grid, dim3(256), 0, stream, table, tiles, beta, inv_loss_scale, nesterov, (uint64_t)rounding_step);
+    if (rounding) VIOLA_LAUNCH((momentum_table_quads<TG, EPL, true>), grid, dim3(256), 0, stream, table, tiles, beta, inv_loss_scale, nesterov, (uint64_t)rounding_step); \
+    else VIOLA_LAUNCH((momentum_table_quads<TG, EPL, false>), grid, dim3(256), 0, stream, table, tiles, beta, inv_loss_scale, nesterov, (uint64_t)rounding_step);
 #define VIOLA_MTT(EPL)                                                          \
     if (grad_dtype == VIOLA_F32) { VIOLA_MT(float, EPL) }                        \
     else if (grad_dtype == VIOLA_BF16) { VIOLA_MT(bf16_t, EPL) }                 \
@@ -462,9 +462,9 @@ extern "C" int viola_weight_update_table(const int64_t* table, int64_t tensors, 
     const int64_t quads = count / 4;
     const int64_t blocks = (quads + 255) / 256;
     const dim3 grid((unsigned)(blocks > 4096 ? 4096 : blocks), (unsigned)tensors);
-    if (grad_dtype == VIOLA_F32) hipLaunchKernelGGL(weight_table_quads_kernel<float>, grid, dim3(256), 0, stream, table, quads, lr, decay, update_scale);
-    else if (grad_dtype == VIOLA_BF16) hipLaunchKernelGGL(weight_table_quads_kernel<bf16_t>, grid, dim3(256), 0, stream, table, quads, lr, decay, update_scale);
-    else hipLaunchKernelGGL(weight_table_quads_kernel<f16_t>, grid, dim3(256), 0, stream, table, quads, lr, decay, update_scale);
+    if (grad_dtype == VIOLA_F32) VIOLA_LAUNCH(weight_table_quads_kernel<float>, grid, dim3(256), 0, stream, table, quads, lr, decay, update_scale);
+    else if (grad_dtype == VIOLA_BF16) VIOLA_LAUNCH(weight_table_quads_kernel<bf16_t>, grid, dim3(256), 0, stream, table, quads, lr, decay, update_scale);
+    else VIOLA_LAUNCH(weight_table_quads_kernel<f16_t>, grid, dim3(256), 0, stream, table, quads, lr, decay, update_scale);
     return viola_launch_status();
 }
 
@@ -480,18 +480,18 @@ extern "C" int viola_weight_update(void* weight, int weight_dtype, const void* g
         reinterpret_cast<uintptr_t>(grad) % (4 * grad_bytes) == 0) {
         const int64_t quads = n / 4, rest = n % 4;
         float* wp = static_cast<float*>(weight);
-        if (grad_dtype == VIOLA_F32) hipLaunchKernelGGL(weight_quads_kernel<float>, dim3(grid_for(quads)), dim3(256), 0, stream, wp, static_cast<const float*>(grad), quads, lr, decay, update_scale);
-        else if (grad_dtype == VIOLA_BF16) hipLaunchKernelGGL(weight_quads_kernel<bf16_t>, dim3(grid_for(quads)), dim3(256), 0, stream, wp, static_cast<const bf16_t*>(grad), quads, lr, decay, update_scale);
-        else hipLaunchKernelGGL(weight_quads_kernel<f16_t>, dim3(grid_for(quads)), dim3(256), 0, stream, wp, static_cast<const f16_t*>(grad), quads, lr, decay, update_scale);
+        if (grad_dtype == VIOLA_F32) VIOLA_LAUNCH(weight_quads_kernel<float>, dim3(grid_for(quads)), dim3(256), 0, stream, wp, static_cast<const float*>(grad), quads, lr, decay, update_scale);
+        else if (grad_dtype == VIOLA_BF16) VIOLA_LAUNCH(weight_quads_kernel<bf16_t>, dim3(grid_for(quads)), dim3(256), 0, stream, wp, static_cast<const bf16_t*>(grad), quads, lr, decay, update_scale);
+        else VIOLA_LAUNCH(weight_quads_kernel<f16_t>, dim3(grid_for(quads)), dim3(256), 0, stream, wp, static_cast<const f16_t*>(grad), quads, lr, decay, update_scale);
         if (rest)
-            hipLaunchKernelGGL(weight_kernel<false>, dim3(1), dim3(256), 0, stream, wp + 4 * quads, weight_dtype,
+            VIOLA_LAUNCH(weight_kernel<false>, dim3(1), dim3(256), 0, stream, wp + 4 * quads, weight_dtype,
                                static_cast<const uint8_t*>(grad) + 4 * quads * grad_bytes, grad_dtype, rest, lr, decay, update_scale, 0ull, 0ull, 0ull);
         return viola_launch_status();
     }
     if (rounding && weight_dtype != VIOLA_F32)
-        hipLaunchKernelGGL(weight_kernel<true>, dim3(grid_for(n)), dim3(256), 0, stream, weight, weight_dtype, grad, grad_dtype, n, lr, decay, update_scale, (uint64_t)rounding_step, (uint64_t)rounding_key, (uint64_t)offset);
+        VIOLA_LAUNCH(weight_kernel<true>, dim3(grid_for(n)), dim3(256), 0, stream, weight, weight_dtype, grad, grad_dtype, n, lr, decay, update_scale, (uint64_t)rounding_step, (uint64_t)rounding_key, (uint64_t)offset);
     else
-        hipLaunchKernelGGL(weight_kernel<false>, dim3(grid_for(n)), dim3(256), 0, stream, weight, weight_dtype, grad, grad_dtype, n, lr, decay, update_scale, (uint64_t)rounding_step, (uint64_t)rounding_key, (uint64_t)offset);
+        VIOLA_LAUNCH(weight_kernel<false>, dim3(grid_for(n)), dim3(256), 0, stream, weight, weight_dtype, grad, grad_dtype, n, lr, decay, update_scale, (uint64_t)rounding_step, (uint64_t)rounding_key, (uint64_t)offset);
     return viola_launch_status();
 }
 
@@ -505,9 +505,9 @@ extern "C" int viola_adam_update(void* weight, int weight_dtype, const void* gra
     VIOLA_CHECK_ARG(weight && grad && first && second);
     const AdamConstants c{lr, decay, b1, b2, inv_c1, inv_c2, eps, adamw, maximize};
     if (rounding && weight_dtype != VIOLA_F32)
-        hipLaunchKernelGGL(adam_kernel<true>, dim3(grid_for(n)), dim3(256), 0, stream, weight, weight_dtype, grad, grad_dtype, first, second, state_dtype, n, c, (uint64_t)rounding_step, (uint64_t)rounding_key, (uint64_t)offset);
+        VIOLA_LAUNCH(adam_kernel<true>, dim3(grid_for(n)), dim3(256), 0, stream, weight, weight_dtype, grad, grad_dtype, first, second, state_dtype, n, c, (uint64_t)rounding_step, (uint64_t)rounding_key, (uint64_t)offset);
     else
-        hipLaunchKernelGGL(adam_kernel<false>, dim3(grid_for(n)), dim3(256), 0, stream, weight, weight_dtype, grad, grad_dtype, first, second, state_dtype, n, c, (uint64_t)rounding_step, (uint64_t)rounding_key, (uint64_t)offset);
+        VIOLA_LAUNCH(adam_kernel<false>, dim3(grid_for(n)), dim3(256), 0, stream, weight, weight_dtype, grad, grad_dtype, first, second, state_dtype, n, c, (uint64_t)rounding_step, (uint64_t)rounding_key, (uint64_t)offset);
     return viola_launch_status();
 }
 
@@ -524,9 +524,9 @@ extern "C" int viola_adam_update_table(const int64_t* table, int64_t tensors, in
     const int64_t blocks = (max_count + 255) / 256;
     const dim3 grid((unsigned)(blocks > 1024 ? 1024 : blocks), (unsigned)tensors);
     if (rounding && weight_dtype != VIOLA_F32)
-        hipLaunchKernelGGL(adam_table_kernel<true>, grid, dim3(256), 0, stream, table, weight_dtype, grad_dtype, state_dtype, c, (uint64_t)rounding_step);
+        VIOLA_LAUNCH(adam_table_kernel<true>, grid, dim3(256), 0, stream, table, weight_dtype, grad_dtype, state_dtype, c, (uint64_t)rounding_step);
     else
-        hipLaunchKernelGGL(adam_table_kernel<false>, grid, dim3(256), 0, stream, table, weight_dtype, grad_dtype, state_dtype, c, (uint64_t)rounding_step);
+        VIOLA_LAUNCH(adam_table_kernel<false>, grid, dim3(256), 0, stream, table, weight_dtype, grad_dtype, state_dtype, c, (uint64_t)rounding_step);
     return viola_launch_status();
 }
 
@@ -536,7 +536,7 @@ extern "C" int viola_copy_scaled(const void* update, int update_dtype, void* out
     VIOLA_CHECK_ARG(viola_is_float(update_dtype) && viola_is_float(out_dtype) && src >= 0 && dst >= 0 && count >= 0);
     if (count == 0) return 0;
     VIOLA_CHECK_ARG(update && out);
-    hipLaunchKernelGGL(copy_scaled_kernel, dim3(grid_for(count)), dim3(256), 0, stream, update, update_dtype, out, out_dtype, src, dst, count, scale);
+    VIOLA_LAUNCH(copy_scaled_kernel, dim3(grid_for(count)), dim3(256), 0, stream, update, update_dtype, out, out_dtype, src, dst, count, scale);
     return viola_launch_status();
 }
 
@@ -547,6 +547,6 @@ extern "C" int viola_momentum_dequantize(const void* q, const float* scale, floa
     VIOLA_CHECK_ARG(n >= 0 && (granularity == 0 ? tile_size > 0 : (rows > 0 && cols > 0 && tr > 0 && tc > 0 && planes * rows * cols == n)));
     if (n == 0) return 0;
     VIOLA_CHECK_ARG(q && scale && out);
-    hipLaunchKernelGGL(momentum_dequantize_kernel, dim3(grid_for(n)), dim3(256), 0, stream, static_cast<const uint8_t*>(q), scale, out, n, granularity, tile_size, rows, cols, tr, tc);
+    VIOLA_LAUNCH(momentum_dequantize_kernel, dim3(grid_for(n)), dim3(256), 0, stream, static_cast<const uint8_t*>(q), scale, out, n, granularity, tile_size, rows, cols, tr, tc);
     return viola_launch_status();
 }

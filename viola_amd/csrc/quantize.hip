@@ -768,7 +768,7 @@ static int launch_quantize(const void* x, int64_t rows, int64_t cols, void* q, f
         const int64_t chunks = rows * nc * (gc / 8);
         const dim3 grid((unsigned)((chunks + 255) / 256));
 #define VIOLA_ROWWISE(GC) \
-    case GC: hipLaunchKernelGGL((quantize_rowwise<TIn, TOut, GC>), grid, dim3(256), 0, stream, xp, qp, scale, rows, cols, nc, limit, e8m0); break;
+    case GC: VIOLA_LAUNCH((quantize_rowwise<TIn, TOut, GC>), grid, dim3(256), 0, stream, xp, qp, scale, rows, cols, nc, limit, e8m0); break;
         switch (gc) {
             VIOLA_ROWWISE(32) VIOLA_ROWWISE(64) VIOLA_ROWWISE(128) VIOLA_ROWWISE(256) VIOLA_ROWWISE(512)
             default: return VIOLA_EINVAL;
@@ -780,26 +780,26 @@ static int launch_quantize(const void* x, int64_t rows, int64_t cols, void* q, f
         if (gr == 1 && gc == 32 && transposed && vec) {
             const int64_t tiles16 = ((cols + 63) / 64) * ((rows + 127) / 128);
             const dim3 grid16((unsigned)(tiles16 < 256 * 6 ? tiles16 : 256 * 6));
-            hipLaunchKernelGGL((quantize_dual16<TIn, TOut, false>), grid16, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit, nullptr, e8m0);
+            VIOLA_LAUNCH((quantize_dual16<TIn, TOut, false>), grid16, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit, nullptr, e8m0, 0);
             return viola_launch_status();
         }
     }
     if (gr == 1 && gc == 32 && transposed) {
         const dim3 grid((unsigned)((cols + TILE_C - 1) / TILE_C), (unsigned)((rows + TILE_R - 1) / TILE_R));
-        if (vec) hipLaunchKernelGGL((quantize_tile<TIn, TOut, false, true, true>), grid, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit, nullptr, e8m0);
-        else hipLaunchKernelGGL((quantize_tile<TIn, TOut, false, true, false>), grid, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit, nullptr, e8m0);
+        if (vec) VIOLA_LAUNCH((quantize_tile<TIn, TOut, false, true, true>), grid, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit, nullptr, e8m0);
+        else VIOLA_LAUNCH((quantize_tile<TIn, TOut, false, true, false>), grid, dim3(256), 0, stream, xp, nullptr, nullptr, qp, scale, rows, cols, limit, nullptr, e8m0);
         return viola_launch_status();
     }
     if (gr == 32 && gc == 32 && !transposed && cols % 4 == 0 && reinterpret_cast<uintptr_t>(x) % (4 * sizeof(TIn)) == 0 &&
         reinterpret_cast<uintptr_t>(q) % 4 == 0) {
         const int64_t units = (rows + 31) / 32 * ((cols + 127) / 128);
-        hipLaunchKernelGGL((quantize_block32<TIn, TOut>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, xp, qp, scale,
+        VIOLA_LAUNCH((quantize_block32<TIn, TOut>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, xp, qp, scale,
                            rows, cols, (cols + 31) / 32, limit, e8m0);
         return viola_launch_status();
     }
     const int64_t out_rows = transposed ? cols : rows, out_cols = transposed ? rows : cols;
     const int64_t ngroups = ((out_rows + gr - 1) / gr) * ((out_cols + gc - 1) / gc);
-    hipLaunchKernelGGL((quantize_generic<TIn, TOut, false>), dim3((unsigned)((ngroups + 3) / 4)), dim3(256), 0, stream,
+    VIOLA_LAUNCH((quantize_generic<TIn, TOut, false>), dim3((unsigned)((ngroups + 3) / 4)), dim3(256), 0, stream,
                        xp, nullptr, qp, scale, rows, cols, gr, gc, transposed, 1, 32, limit, e8m0);
     return viola_launch_status();
 }
@@ -820,7 +820,7 @@ static int launch_reencode(const void* x, const float* source_scale, int64_t row
                            int gr, int gc, float limit, int transposed, int sgr, int sgc, int e8m0, hipStream_t stream) {
     const int64_t out_rows = transposed ? cols : rows, out_cols = transposed ? rows : cols;
     const int64_t ngroups = ((out_rows + gr - 1) / gr) * ((out_cols + gc - 1) / gc);
-    hipLaunchKernelGGL((quantize_generic<TIn, TOut, true>), dim3((unsigned)((ngroups + 3) / 4)), dim3(256), 0, stream,
+    VIOLA_LAUNCH((quantize_generic<TIn, TOut, true>), dim3((unsigned)((ngroups + 3) / 4)), dim3(256), 0, stream,
                        static_cast<const TIn*>(x), source_scale, static_cast<uint8_t*>(q), scale, rows, cols, gr, gc,
                        transposed, sgr, sgc, limit, e8m0);
     return viola_launch_status();
@@ -836,13 +836,13 @@ static int launch_dual(const void* x, int64_t rows, int64_t cols, void* q, float
         if (vec && reinterpret_cast<uintptr_t>(q) % 8 == 0) {
             const int64_t tiles16 = ((cols + 63) / 64) * ((rows + 127) / 128);
             const dim3 grid16((unsigned)(tiles16 < 256 * 6 ? tiles16 : 256 * 6));
-            hipLaunchKernelGGL((quantize_dual16<TIn, TOut, true>), grid16, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale,
-                               static_cast<uint8_t*>(qt), scale_t, rows, cols, limit, column_partial, e8m0);
+            VIOLA_LAUNCH((quantize_dual16<TIn, TOut, true>), grid16, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale,
+                               static_cast<uint8_t*>(qt), scale_t, rows, cols, limit, column_partial, e8m0, 0);
             return viola_launch_status();
         }
     }
-    if (vec) hipLaunchKernelGGL((quantize_tile<TIn, TOut, true, true, true>), grid, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale, static_cast<uint8_t*>(qt), scale_t, rows, cols, limit, column_partial, e8m0);
-    else hipLaunchKernelGGL((quantize_tile<TIn, TOut, true, true, false>), grid, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale, static_cast<uint8_t*>(qt), scale_t, rows, cols, limit, column_partial, e8m0);
+    if (vec) VIOLA_LAUNCH((quantize_tile<TIn, TOut, true, true, true>), grid, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale, static_cast<uint8_t*>(qt), scale_t, rows, cols, limit, column_partial, e8m0);
+    else VIOLA_LAUNCH((quantize_tile<TIn, TOut, true, true, false>), grid, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale, static_cast<uint8_t*>(qt), scale_t, rows, cols, limit, column_partial, e8m0);
     return viola_launch_status();
 }
 
@@ -854,14 +854,14 @@ static int launch_segmented(const void* x, int64_t cols, const int64_t* offsets,
         const int64_t blocks = ((t_total / 32 + 3) / 4) * ((cols + 63) / 64);   // four slots x one column tile each
         if (aligned && blocks < (1ll << 31)) {
             const dim3 grid16((unsigned)blocks);
-            if (q) hipLaunchKernelGGL((quantize_segmented16<TIn, TOut, true>), grid16, dim3(256), 0, stream, static_cast<const TIn*>(x), offsets, poffsets, groups, cols, t_total, static_cast<uint8_t*>(qt), scale_t, static_cast<uint8_t*>(q), scale, limit);
-            else hipLaunchKernelGGL((quantize_segmented16<TIn, TOut, false>), grid16, dim3(256), 0, stream, static_cast<const TIn*>(x), offsets, poffsets, groups, cols, t_total, static_cast<uint8_t*>(qt), scale_t, nullptr, nullptr, limit);
+            if (q) VIOLA_LAUNCH((quantize_segmented16<TIn, TOut, true>), grid16, dim3(256), 0, stream, static_cast<const TIn*>(x), offsets, poffsets, groups, cols, t_total, static_cast<uint8_t*>(qt), scale_t, static_cast<uint8_t*>(q), scale, limit);
+            else VIOLA_LAUNCH((quantize_segmented16<TIn, TOut, false>), grid16, dim3(256), 0, stream, static_cast<const TIn*>(x), offsets, poffsets, groups, cols, t_total, static_cast<uint8_t*>(qt), scale_t, nullptr, nullptr, limit);
             return viola_launch_status();
         }
     }
     if (q) return VIOLA_EUNSUPPORTED;                                      // the row-wise by-product needs the 16-bit aligned path
     const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)(t_total / 32));
-    hipLaunchKernelGGL((quantize_transposed_segmented<TIn, TOut>), grid, dim3(64), 0, stream, static_cast<const TIn*>(x),
+    VIOLA_LAUNCH((quantize_transposed_segmented<TIn, TOut>), grid, dim3(64), 0, stream, static_cast<const TIn*>(x),
                        offsets, poffsets, groups, cols, t_total, static_cast<uint8_t*>(qt), scale_t, limit);
     return viola_launch_status();
 }
@@ -938,7 +938,7 @@ extern "C" int viola_gated_quantize_dual(const void* z, int z_dtype, int64_t row
     const int64_t tiles16 = ((cols + 63) / 64) * ((rows + 127) / 128);
     const dim3 grid16((unsigned)(tiles16 < 256 * 6 ? tiles16 : 256 * 6));
 #define VIOLA_GATED_DUAL(TI, TO)                                                                                            \
-    hipLaunchKernelGGL((quantize_dual16<TI, TO, true, true>), grid16, dim3(256), 0, stream, static_cast<const TI*>(z),       \
+    VIOLA_LAUNCH((quantize_dual16<TI, TO, true, true>), grid16, dim3(256), 0, stream, static_cast<const TI*>(z),       \
                        static_cast<uint8_t*>(q), static_cast<float*>(scale), static_cast<uint8_t*>(qt),                      \
                        static_cast<float*>(scale_t), rows, cols, limit, (float*)nullptr, e8m0, activation)
     if (q_dtype == VIOLA_E4M3) {
@@ -959,9 +959,9 @@ extern "C" int viola_column_reduce(const float* partial, int64_t parts, int64_t 
     if (cols == 0) return 0;
     VIOLA_CHECK_ARG(out && (parts == 0 || partial));
     const dim3 grid((unsigned)((cols + 31) / 32));
-    if (out_dtype == VIOLA_F32) hipLaunchKernelGGL(column_reduce_kernel<float>, grid, dim3(256), 0, stream, partial, parts, cols, static_cast<float*>(out));
-    else if (out_dtype == VIOLA_BF16) hipLaunchKernelGGL(column_reduce_kernel<bf16_t>, grid, dim3(256), 0, stream, partial, parts, cols, static_cast<bf16_t*>(out));
-    else hipLaunchKernelGGL(column_reduce_kernel<f16_t>, grid, dim3(256), 0, stream, partial, parts, cols, static_cast<f16_t*>(out));
+    if (out_dtype == VIOLA_F32) VIOLA_LAUNCH(column_reduce_kernel<float>, grid, dim3(256), 0, stream, partial, parts, cols, static_cast<float*>(out));
+    else if (out_dtype == VIOLA_BF16) VIOLA_LAUNCH(column_reduce_kernel<bf16_t>, grid, dim3(256), 0, stream, partial, parts, cols, static_cast<bf16_t*>(out));
+    else VIOLA_LAUNCH(column_reduce_kernel<f16_t>, grid, dim3(256), 0, stream, partial, parts, cols, static_cast<f16_t*>(out));
     return viola_launch_status();
 }
 
@@ -995,9 +995,9 @@ extern "C" int viola_group_dequantize(const void* q, int q_dtype, const float* s
     const int64_t total = rows * cols;
     const unsigned blocks = (unsigned)((total + 255) / 256 < 65536 * 16 ? (total + 255) / 256 : 65536 * 16);
     if (q_dtype == VIOLA_E4M3)
-        hipLaunchKernelGGL(dequantize_kernel<e4m3_t>, dim3(blocks), dim3(256), 0, stream, static_cast<const e4m3_t*>(q), scale, out, rows, cols, gr, gc);
+        VIOLA_LAUNCH(dequantize_kernel<e4m3_t>, dim3(blocks), dim3(256), 0, stream, static_cast<const e4m3_t*>(q), scale, out, rows, cols, gr, gc);
     else
-        hipLaunchKernelGGL(dequantize_kernel<e5m2_t>, dim3(blocks), dim3(256), 0, stream, static_cast<const e5m2_t*>(q), scale, out, rows, cols, gr, gc);
+        VIOLA_LAUNCH(dequantize_kernel<e5m2_t>, dim3(blocks), dim3(256), 0, stream, static_cast<const e5m2_t*>(q), scale, out, rows, cols, gr, gc);
     return viola_launch_status();
 }
 
@@ -1012,8 +1012,8 @@ extern "C" int viola_block_transpose(const void* x, void* out, int64_t rows, int
     const int64_t srows = (rows + gr - 1) / gr, scols = (cols + gc - 1) / gc;
     const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64), 1);
     const bool words = rows % 4 == 0 && cols % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 4 == 0;
-    if (words) hipLaunchKernelGGL(transpose_bytes<true>, grid, dim3(256), 0, stream, static_cast<const uint8_t*>(x), static_cast<uint8_t*>(out), rows, cols, static_cast<const uint8_t*>(scale), static_cast<uint8_t*>(scale_out), srows, scols, scale_bytes);
-    else hipLaunchKernelGGL(transpose_bytes<false>, grid, dim3(256), 0, stream, static_cast<const uint8_t*>(x), static_cast<uint8_t*>(out), rows, cols, static_cast<const uint8_t*>(scale), static_cast<uint8_t*>(scale_out), srows, scols, scale_bytes);
+    if (words) VIOLA_LAUNCH(transpose_bytes<true>, grid, dim3(256), 0, stream, static_cast<const uint8_t*>(x), static_cast<uint8_t*>(out), rows, cols, static_cast<const uint8_t*>(scale), static_cast<uint8_t*>(scale_out), srows, scols, scale_bytes);
+    else VIOLA_LAUNCH(transpose_bytes<false>, grid, dim3(256), 0, stream, static_cast<const uint8_t*>(x), static_cast<uint8_t*>(out), rows, cols, static_cast<const uint8_t*>(scale), static_cast<uint8_t*>(scale_out), srows, scols, scale_bytes);
     return viola_launch_status();
 }
 
@@ -1024,7 +1024,7 @@ extern "C" int viola_fp8_transpose(const void* x, void* out, int64_t batch, int6
     VIOLA_CHECK_ARG(x && out && (rows + 63) / 64 <= 65535 && batch <= 65535);
     const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64), (unsigned)batch);
     const bool words = rows % 4 == 0 && cols % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 4 == 0;
-    if (words) hipLaunchKernelGGL(transpose_bytes<true>, grid, dim3(256), 0, stream, static_cast<const uint8_t*>(x), static_cast<uint8_t*>(out), rows, cols, nullptr, nullptr, 0, 0, 0);
-    else hipLaunchKernelGGL(transpose_bytes<false>, grid, dim3(256), 0, stream, static_cast<const uint8_t*>(x), static_cast<uint8_t*>(out), rows, cols, nullptr, nullptr, 0, 0, 0);
+    if (words) VIOLA_LAUNCH(transpose_bytes<true>, grid, dim3(256), 0, stream, static_cast<const uint8_t*>(x), static_cast<uint8_t*>(out), rows, cols, nullptr, nullptr, 0, 0, 0);
+    else VIOLA_LAUNCH(transpose_bytes<false>, grid, dim3(256), 0, stream, static_cast<const uint8_t*>(x), static_cast<uint8_t*>(out), rows, cols, nullptr, nullptr, 0, 0, 0);
     return viola_launch_status();
 }

@@ -339,7 +339,7 @@ static int launch_tensor_quantize(const void* x, const float* scale, void* q, vo
     const int vector_q = q && reinterpret_cast<uintptr_t>(q) % 16 == 0 && cols % 16 == 0;
     const int vector_qt = qt && reinterpret_cast<uintptr_t>(qt) % 16 == 0 && rows % 16 == 0;
     const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64));
-    hipLaunchKernelGGL((tensor_quantize_kernel<TIn, TOut, ROTATE>), grid, dim3(256), 0, stream, static_cast<const TIn*>(x), scale,
+    VIOLA_LAUNCH((tensor_quantize_kernel<TIn, TOut, ROTATE>), grid, dim3(256), 0, stream, static_cast<const TIn*>(x), scale,
                        static_cast<uint8_t*>(q), static_cast<uint8_t*>(qt), rows, cols, limit, vector_in, vector_q, vector_qt);
     return viola_launch_status();
 }
@@ -352,9 +352,9 @@ extern "C" int viola_tensor_amax(const void* x, int x_dtype, int64_t n, float* m
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     VIOLA_CHECK_ARG(viola_is_float(x_dtype) && n >= 0 && parts > 0 && parts <= 65535 && maxima && (n == 0 || x));
     const dim3 grid((unsigned)parts);
-    if (x_dtype == VIOLA_F32) hipLaunchKernelGGL(tensor_amax_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(x), n, maxima);
-    else if (x_dtype == VIOLA_BF16) hipLaunchKernelGGL(tensor_amax_kernel<bf16_t>, grid, dim3(256), 0, stream, static_cast<const bf16_t*>(x), n, maxima);
-    else hipLaunchKernelGGL(tensor_amax_kernel<f16_t>, grid, dim3(256), 0, stream, static_cast<const f16_t*>(x), n, maxima);
+    if (x_dtype == VIOLA_F32) VIOLA_LAUNCH(tensor_amax_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(x), n, maxima);
+    else if (x_dtype == VIOLA_BF16) VIOLA_LAUNCH(tensor_amax_kernel<bf16_t>, grid, dim3(256), 0, stream, static_cast<const bf16_t*>(x), n, maxima);
+    else VIOLA_LAUNCH(tensor_amax_kernel<f16_t>, grid, dim3(256), 0, stream, static_cast<const f16_t*>(x), n, maxima);
     return viola_launch_status();
 }
 
@@ -362,7 +362,7 @@ extern "C" int viola_tensor_scale(const float* maxima, int64_t parts, float* his
                                   int delayed, float limit, float* scale, viola_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     VIOLA_CHECK_ARG(maxima && parts > 0 && history && history_len > 0 && index >= 0 && limit > 0.0f && scale);
-    hipLaunchKernelGGL(tensor_scale_kernel, dim3(1), dim3(256), 0, stream, maxima, parts, history, history_len, index, delayed, limit, scale);
+    VIOLA_LAUNCH(tensor_scale_kernel, dim3(1), dim3(256), 0, stream, maxima, parts, history, history_len, index, delayed, limit, scale);
     return viola_launch_status();
 }
 
@@ -374,9 +374,9 @@ extern "C" int viola_tensor_amax_columns(const void* x, int x_dtype, int64_t row
     VIOLA_CHECK_ARG(cols % piece == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(column_partial) % 16 == 0);
     const int64_t slice_rows = (rows + slices - 1) / slices;
     const dim3 grid((unsigned)((cols / piece + 255) / 256), (unsigned)slices);
-    if (x_dtype == VIOLA_F32) hipLaunchKernelGGL(tensor_amax_columns_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(x), rows, cols, slice_rows, maxima, column_partial);
-    else if (x_dtype == VIOLA_BF16) hipLaunchKernelGGL(tensor_amax_columns_kernel<bf16_t>, grid, dim3(256), 0, stream, static_cast<const bf16_t*>(x), rows, cols, slice_rows, maxima, column_partial);
-    else hipLaunchKernelGGL(tensor_amax_columns_kernel<f16_t>, grid, dim3(256), 0, stream, static_cast<const f16_t*>(x), rows, cols, slice_rows, maxima, column_partial);
+    if (x_dtype == VIOLA_F32) VIOLA_LAUNCH(tensor_amax_columns_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(x), rows, cols, slice_rows, maxima, column_partial);
+    else if (x_dtype == VIOLA_BF16) VIOLA_LAUNCH(tensor_amax_columns_kernel<bf16_t>, grid, dim3(256), 0, stream, static_cast<const bf16_t*>(x), rows, cols, slice_rows, maxima, column_partial);
+    else VIOLA_LAUNCH(tensor_amax_columns_kernel<f16_t>, grid, dim3(256), 0, stream, static_cast<const f16_t*>(x), rows, cols, slice_rows, maxima, column_partial);
     return viola_launch_status();
 }
 
@@ -438,9 +438,9 @@ extern "C" int viola_rotation_amax(const void* x, int x_dtype, int64_t rows, int
     const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64));
     VIOLA_CHECK_ARG(parts == (int64_t)grid.x * grid.y);
     const int vector_in = reinterpret_cast<uintptr_t>(x) % 16 == 0 && (cols * viola_dtype_size(x_dtype)) % 16 == 0;
-    if (x_dtype == VIOLA_F32) hipLaunchKernelGGL(rotation_amax_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(x), rows, cols, vector_in, maxima);
-    else if (x_dtype == VIOLA_BF16) hipLaunchKernelGGL(rotation_amax_kernel<bf16_t>, grid, dim3(256), 0, stream, static_cast<const bf16_t*>(x), rows, cols, vector_in, maxima);
-    else hipLaunchKernelGGL(rotation_amax_kernel<f16_t>, grid, dim3(256), 0, stream, static_cast<const f16_t*>(x), rows, cols, vector_in, maxima);
+    if (x_dtype == VIOLA_F32) VIOLA_LAUNCH(rotation_amax_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(x), rows, cols, vector_in, maxima);
+    else if (x_dtype == VIOLA_BF16) VIOLA_LAUNCH(rotation_amax_kernel<bf16_t>, grid, dim3(256), 0, stream, static_cast<const bf16_t*>(x), rows, cols, vector_in, maxima);
+    else VIOLA_LAUNCH(rotation_amax_kernel<f16_t>, grid, dim3(256), 0, stream, static_cast<const f16_t*>(x), rows, cols, vector_in, maxima);
     return viola_launch_status();
 }
 
@@ -451,8 +451,8 @@ extern "C" int viola_rotation_inverse(void* x, int x_dtype, int64_t rows, int64_
     VIOLA_CHECK_ARG(x && (rows + 63) / 64 <= 65535);
     const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64));
     const int vector_in = reinterpret_cast<uintptr_t>(x) % 16 == 0 && (cols * viola_dtype_size(x_dtype)) % 16 == 0;
-    if (x_dtype == VIOLA_F32) hipLaunchKernelGGL(rotation_inplace_kernel<float>, grid, dim3(256), 0, stream, static_cast<float*>(x), rows, cols, vector_in);
-    else if (x_dtype == VIOLA_BF16) hipLaunchKernelGGL(rotation_inplace_kernel<bf16_t>, grid, dim3(256), 0, stream, static_cast<bf16_t*>(x), rows, cols, vector_in);
-    else hipLaunchKernelGGL(rotation_inplace_kernel<f16_t>, grid, dim3(256), 0, stream, static_cast<f16_t*>(x), rows, cols, vector_in);
+    if (x_dtype == VIOLA_F32) VIOLA_LAUNCH(rotation_inplace_kernel<float>, grid, dim3(256), 0, stream, static_cast<float*>(x), rows, cols, vector_in);
+    else if (x_dtype == VIOLA_BF16) VIOLA_LAUNCH(rotation_inplace_kernel<bf16_t>, grid, dim3(256), 0, stream, static_cast<bf16_t*>(x), rows, cols, vector_in);
+    else VIOLA_LAUNCH(rotation_inplace_kernel<f16_t>, grid, dim3(256), 0, stream, static_cast<f16_t*>(x), rows, cols, vector_in);
     return viola_launch_status();
 }

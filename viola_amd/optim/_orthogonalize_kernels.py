@@ -43,7 +43,7 @@ def run(matrix, steps, method):
     if method == "standard" or x.shape[-2] == x.shape[-1]:
         for step in range(steps):
             r = _matmul(x, x, transpose_b=True)
-            z = _matmul(r, r, transpose_b=True, residual=r, epilogue=1)      # r is symmetric: r r = r r^T
+            z = _matmul(r, r, transpose_b=True, residual=r, epilogue=1)      # r = x x^T is symmetric bit for bit: r r = r r^T
             x = _matmul(z, x, residual=x, epilogue=2, transpose_out=tall and step == steps - 1)
     else:
         segments = [length for length in (min(steps, 2), max(steps - 2, 0)) if length]
@@ -55,7 +55,8 @@ def run(matrix, steps, method):
                     # Z and Q = Z + 3.4445 I from the one product
                     z, q = _matmul(r, r, transpose_b=True, residual=r, epilogue=1, add_diag=A_COEFF)
                 else:
-                    z = _matmul(r, r, transpose_b=True, residual=r, epilogue=1)
+                    # past the first iteration r = 3.4445 rz + z rz is symmetric only up to rounding: r @ r as written
+                    z = _matmul(r, r, residual=r, epilogue=1)
                     q = _matmul(z, q, residual=q, epilogue=2)
                 if i + 1 < length:
                     rz = _matmul(z, r, residual=r, epilogue=2)
