@@ -30,7 +30,7 @@ enum { VIOLA_SILU = 0, VIOLA_GELU = 1, VIOLA_RELU = 2 };
 enum { VIOLA_NEAREST = 0, VIOLA_STOCHASTIC = 1 };
 /* group scales: FP32 values, or E8M0 bytes (power-of-two scale 2^(byte - 127), the `native` / mxfp8 recipe) */
 enum { VIOLA_SCALE_F32 = 0, VIOLA_SCALE_E8M0 = 1 };
-enum { VIOLA_EINVAL = -1, VIOLA_EUNSUPPORTED = -2 };
+enum { VIOLA_EINVAL = -1, VIOLA_EUNSUPPORTED = -2, VIOLA_ETOOLARGE = -3 };
 
 int viola_abi_version(void);
 const char* viola_error_string(int code);
@@ -311,6 +311,17 @@ int viola_ns_gemm(const void* a, const void* bmat, const void* residual, void* o
  * sums of squares; every slot is written before it is read, so it needs no clearing). */
 int viola_ns_prepare(const void* in, int in_dtype, void* out, int dtype, int64_t batch, int64_t rows, int64_t cols,
                      float* workspace, viola_stream_t stream);
+
+/* No counterpart in the reference. viola_ns_prepare for callers that cannot allocate device memory (code under
+ * HIP-graph capture, serving loops, harnesses that forbid hipMalloc): the same kernels and results, with the
+ * partial sums in a 1 MiB array built into the library (one copy per GPU, held until the process ends) instead
+ * of a caller's workspace. batch <= 1024, otherwise VIOLA_ETOOLARGE and nothing is launched. The array's address
+ * on the current device is looked up on the first call there (batch = 0 is accepted as a set-up call that does
+ * only this); `stream` must belong to the current device. Calls on one GPU share the array: two that overlap in
+ * time (different streams, or threads) race; calls on one stream are ordered and safe. Calls no hipMalloc /
+ * hipFree and no allocating library routine. */
+int viola_ns_prepare_static(const void* in, int in_dtype, void* out, int dtype, int64_t batch, int64_t rows,
+                            int64_t cols, viola_stream_t stream);
 
 /* ---------------------------------------------------------------- FP8 gradient wire codec
  * viola/distributed/_fp8_kernels.py:84-87 `pack` (_pack :18-43) and :90-93 `unpack` (_unpack :46-69).

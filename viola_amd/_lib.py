@@ -57,6 +57,7 @@ _SIGNATURES = {
     "viola_momentum_dequantize": [_p, _p, _p, _l, _i, _i, _l, _l, _l, _i, _i, _p],
     "viola_ns_gemm": [_p, _p, _p, _p, _i, _i, _i, _l, _l, _l, _l, _f, _p, _i, _p],
     "viola_ns_prepare": [_p, _i, _p, _i, _l, _l, _l, _p, _p],
+    "viola_ns_prepare_static": [_p, _i, _p, _i, _l, _l, _l, _p],
     "viola_comm_pack": [_p, _l, _p, _l, _l, _i, _i, _p],
     "viola_comm_unpack": [_p, _p, _l, _l, _l, _i, _i, _i, _p],
     "viola_selftest_fp8": [_p, _p],

@@ -425,5 +425,6 @@ extern "C" const char* viola_error_string(int code) {
     if (code == 0) return "success";
     if (code == VIOLA_EINVAL) return "invalid argument (nothing launched)";
     if (code == VIOLA_EUNSUPPORTED) return "unsupported configuration (nothing launched)";
+    if (code == VIOLA_ETOOLARGE) return "size beyond the library's built-in scratch buffer (nothing launched)";
     return hipGetErrorString(static_cast<hipError_t>(code));
 }

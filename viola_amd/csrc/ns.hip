@@ -7,6 +7,9 @@
 // consecutive n. b may be given as [n, k] (transpose_b) or [k, n]; the latter is transposed on
 // its way into LDS.
 #include <type_traits>
+#include <atomic>
+#include <mutex>
+
 #include "ns_args.hpp"
 
 namespace viola {
@@ -428,6 +431,37 @@ static int launch_prepare(const void* in, void* out, int64_t batch, int64_t rows
     return viola_launch_status();
 }
 
+// Scratch of viola_ns_prepare_static: the partial sums of squares that viola_ns_prepare keeps in its caller's
+// workspace. One copy per GPU, held until the process ends; its address on a device is looked up once, with that
+// device current, and only that address (never the array's name, which on the host is a stand-in) reaches kernels.
+constexpr int64_t NS_STATIC_BATCH = 1024;
+static __device__ __align__(256) float ns_static_scratch[NS_STATIC_BATCH * PARTS];
+constexpr int NS_STATIC_DEVICES = 64;
+static std::atomic<float*> ns_static_address[NS_STATIC_DEVICES];
+static std::mutex ns_static_mutex;
+
+static int ns_static_workspace(float** workspace) {
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) return (int)e;
+    if (device < 0 || device >= NS_STATIC_DEVICES) return VIOLA_EUNSUPPORTED;
+    float* address = ns_static_address[device].load(std::memory_order_acquire);
+    if (address == nullptr) {
+        std::lock_guard<std::mutex> guard(ns_static_mutex);
+        address = ns_static_address[device].load(std::memory_order_relaxed);
+        if (address == nullptr) {
+            void* found = nullptr;
+            e = hipGetSymbolAddress(&found, HIP_SYMBOL(ns_static_scratch));
+            if (e != hipSuccess) return (int)e;
+            if (found == nullptr) return (int)hipErrorInvalidSymbol;
+            address = static_cast<float*>(found);
+            ns_static_address[device].store(address, std::memory_order_release);
+        }
+    }
+    *workspace = address;
+    return 0;
+}
+
 }  // namespace viola
 
 using namespace viola;
@@ -480,4 +514,14 @@ extern "C" int viola_ns_prepare(const void* in, int in_dtype, void* out, int dty
     if (in_dtype == VIOLA_BF16) VIOLA_PREP(bf16_t, false);
     VIOLA_PREP(f16_t, false);
 #undef VIOLA_PREP
+}
+
+extern "C" int viola_ns_prepare_static(const void* in, int in_dtype, void* out, int dtype, int64_t batch, int64_t rows,
+                                       int64_t cols, viola_stream_t stream) {
+    VIOLA_CHECK_ARG(batch >= 0);
+    if (batch > NS_STATIC_BATCH) return VIOLA_ETOOLARGE;             // beyond the built-in scratch: use viola_ns_prepare
+    float* workspace = nullptr;
+    const int status = ns_static_workspace(&workspace);              // also for batch == 0: a set-up call
+    if (status != 0) return status;
+    return viola_ns_prepare(in, in_dtype, out, dtype, batch, rows, cols, workspace, stream);
 }
