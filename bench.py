@@ -5,8 +5,10 @@ parameter set, the wire codec and quantizer bandwidths, a roofline object for th
 
     python bench.py --gpus 1 --steps 200 --warmup 50
 
-The defaults are long enough (tens of milliseconds of back-to-back launches) for the GPU to settle at its sustained
-clock: a 20-step run reads some 15 % slower than the steady state a training loop sees.
+Before a leg is sampled the device runs that leg's own step back to back for about 100 ms, outside the step and
+warm-up counts (the reference's benchmarks warm for about 30 ms before sampling, checks/benchmark_linear.py:41-52): a
+GPU that has idled through set-up needs some tens of milliseconds of work to reach its sustained clock, and a
+20-step run would otherwise read that ramp instead of the steady state a training loop sees.
 
 A step is one `y = layer(x); y.backward(dy)` including every quantize / transpose launch, inputs
 resident in HBM. TFLOP/s = 6*M*K*N / t (the reference's definition, checks/benchmark_linear.py:165).
@@ -14,6 +16,7 @@ resident in HBM. TFLOP/s = 6*M*K*N / t (the reference's definition, checks/bench
 
 import argparse
 import json
+import math
 import os
 import statistics
 import sys
@@ -30,10 +33,39 @@ PEAK = {"fp8_tflops": 5000.0, "bf16_tflops": 2500.0, "hbm_gbs": 8000.0}
 # dispatch), each scaled by the same counter's reading for the 256 MiB copy_scaled_kernel launch (factors 2.00 and 1.00):
 # fetch (2 * 62.2 + 124.7) / 3 MB, write (2 * 41.9 + 8.4) / 3 MB. The algorithmic figure is 65 MB per launch.
 GEMM_TRAFFIC_BYTES = 83.0e6 + 30.8e6
+# What the grouped-scale recipe can reach at all on this part: per 32-k group and 32 x 32 sub-tile the SIMD issues two
+# K = 16 FP8 MFMAs (64 matrix-pipe cycles) and 16 FP32 FMAs; MFMA and VALU share the issue port, >= 72 issue cycles per
+# 64 of matrix work, on MFMAs that run at half the f8f6f4 rate: 2.5 PFLOP/s x 64 / 72 at the 2.4 GHz boost clock.
+GEMM_ATTAINABLE_TFLOPS = 2500.0 * 64 / 72
 
 
-def timed(fn, steps, warmup):
+WARM_MS = 100.0
+
+
+def log(message):
+    """Progress on stderr (the JSON line is the only thing on stdout)."""
+    print(f"[bench] {message}", file=sys.stderr, flush=True)
+
+
+def device_warm(fn, target_ms=WARM_MS):
+    """Run fn back to back for about target_ms of device time (probe one call, then repeat; at most 4096 calls)."""
     import torch
+    fn()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    fn()
+    end.record()
+    end.synchronize()
+    for _ in range(min(4096, math.ceil(target_ms / max(start.elapsed_time(end), 1e-3)))):
+        fn()
+    torch.cuda.synchronize()
+
+
+def timed(fn, steps, warmup, warm=True):
+    import torch
+    if warm:
+        device_warm(fn)
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -98,10 +130,32 @@ def muon_case(method="standard", rounding="nearest", blocks=28, d=1152):
     return opt, params, elements
 
 
+def _median_time(fn, repeats=3):
+    fn()                                                                          # warm-up
+    times = []
+    for _ in range(repeats):
+        begin = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - begin)
+    return statistics.median(times)
+
+
+def _bounded(fn, seconds):
+    """fn() in a daemon thread; its result, or None when it has not returned after `seconds`."""
+    import threading
+    box = []
+    worker = threading.Thread(target=lambda: box.append(fn()), daemon=True)
+    worker.start()
+    worker.join(seconds)
+    return box[0] if box else None
+
+
 def cpu_baseline():
-    """The oracle's Linear forward+backward (dequantized-FP32 matmuls) on this host's cores, one full C2 step."""
+    """The oracle's Linear forward+backward (dequantized-FP32 matmuls) on this host's cores, one full C2 step, plus
+    the other CPU legs (eager Newton-Schulz on one 1024 x 4096 matrix, the wire codec on one 25 MB bucket, the momentum
+    codec on one qkv-sized matrix) under `others`."""
     import torch
-    from oracle import grouped as og, linear as ol
+    from oracle import comm as oc, grouped as og, linear as ol, ns as ons, optim as oo
     torch.manual_seed(20261125)
     cores = min(os.cpu_count() or 1, 16)
     torch.set_num_threads(cores)
@@ -110,15 +164,86 @@ def cpu_baseline():
     w = torch.empty(N, K).uniform_(-1 / 32, 1 / 32)
     qw, sw = og.quantize(w, torch.float8_e4m3fn, (32, 32))
     w_real = og.dequantize(qw, sw, (32, 32))
-    times = []
-    for _ in range(3):
-        begin = time.perf_counter()
-        ol.linear(x, w_real, torch.zeros(N), dy)
-        times.append(time.perf_counter() - begin)
-    best = statistics.median(times[1:])
+    best = _median_time(lambda: ol.linear(x, w_real, torch.zeros(N), dy), repeats=2)
+    log(f"cpu linear: {best * 1e3:.0f} ms")
+    others = {}
+    n = 6553600
+    bucket = torch.randn(n) * 1e-3
+    t_pack = _median_time(lambda: oc.pack(bucket, 1, n // 256, 256, torch.float8_e4m3fn))
+    packet = oc.pack(bucket, 1, n // 256, 256, torch.float8_e4m3fn)
+    t_unpack = _median_time(lambda: oc.unpack(packet, n, 256, torch.float8_e4m3fn))
+    others["comm_codec_25MB"] = dict(pack_ms=t_pack * 1e3, unpack_ms=t_unpack * 1e3, pack_gbs=5.016 * n / t_pack / 1e9,
+                                     unpack_gbs=5.016 * n / t_unpack / 1e9, sample="one 6 553 600-element fp32 bucket, tile 256")
+    shape = (3456, 1152)
+    grad = torch.randn(shape) * 1e-3
+    count = shape[0] * shape[1]
+    q0, s0 = torch.zeros(count, dtype=torch.uint8), torch.ones(count // 256)
+    t_mom = _median_time(lambda: oo.momentum_update(grad, q0, s0, beta=.95, shape=shape))
+    others["momentum_3456x1152"] = dict(ms=t_mom * 1e3, gbs=8.03 * count / t_mom / 1e9, sample="one qkv-sized matrix, tile 256, nearest")
+    # the eager Newton-Schulz recipes last, each under a time limit: a host without fast half-precision matmuls
+    # can take minutes (or not come back) on them; a leg that misses its limit is reported as such
+    g = torch.randn(1024, 4096)
+    for method, flops in (("standard", NS_C1_FLOPS["standard"]), ("gram", NS_C1_FLOPS["gram"])):
+        t = _bounded(lambda: _median_time(lambda: ons.METHODS[method](g, steps=5)), 30.0)
+        log(f"cpu ns {method}: {'no result within 30 s' if t is None else f'{t * 1e3:.0f} ms'}")
+        if t is None:
+            others[f"ns_{method}_1024x4096"] = dict(ms=None, tflops=None, sample="one matrix, 5 steps, eager torch on the host: not finished within 30 s")
+            break                                                                 # its threads may still be busy
+        others[f"ns_{method}_1024x4096"] = dict(ms=t * 1e3, tflops=flops / t / 1e12, sample="one matrix, 5 steps, eager torch on the host")
     return dict(value=6 * M * K * N / best / 1e12, unit="TFLOP/s", cores=cores, kind="port",
                 sample=f"one full {M}x{K}->{N} forward+backward per run, median of 2 after 1 warm-up "
-                       f"({best * 1e3:.0f} ms per step)")
+                       f"({best * 1e3:.0f} ms per step)", others=others)
+
+
+# Newton-Schulz on one 1024 x 4096 matrix, 5 steps: standard 5 (4 m^2 n + 2 m^3), gram 8 m^2 n + 28 m^3
+NS_C1_FLOPS = {"standard": 5 * (4 * 1024 ** 2 * 4096 + 2 * 1024 ** 3), "gram": 8 * 1024 ** 2 * 4096 + 28 * 1024 ** 3}
+
+
+def ns_single_case(steps, warmup):
+    """Config 1: one [1024, 4096] fp32 gradient through each Newton-Schulz method, with the per-launch breakdown."""
+    import torch
+    from viola_amd.optim._orthogonalize import METHODS
+    torch.manual_seed(1)
+    g = torch.randn(1024, 4096, device="cuda")
+    out = {}
+    for method in ("standard", "gram"):
+        fn = lambda: METHODS[method](g, steps=5)
+        ms, _ = timed(fn, steps, warmup)
+        b = kernel_breakdown(fn, min(steps, 20))
+        gemm_ms = b["viola_ns_gemm"]["avg_ms"] * b["viola_ns_gemm"]["launches_per_step"]
+        out[method] = dict(ms=ms, tflops=NS_C1_FLOPS[method] / (ms * 1e-3) / 1e12, gemm_launches=b["viola_ns_gemm"]["launches_per_step"],
+                           gemm_ms=gemm_ms, gemm_tflops=NS_C1_FLOPS[method] / (gemm_ms * 1e-3) / 1e12,
+                           gemm_frac_peak=NS_C1_FLOPS[method] / (gemm_ms * 1e-3) / 1e12 / PEAK["bf16_tflops"])
+    return out
+
+
+def varlen_case(steps, warmup):
+    """Config 4: 16 groups sharing K = 4096, N = 1024, 32768 rows split by a seeded multinomial with one empty and
+    one 3-row group; forward + backward of the variable-group linear, 3 x 2 x 32768 x 4096 x 1024 flop."""
+    import torch
+    from viola_amd.nn import _varlen as v
+    groups, k, n, total = 16, 4096, 1024, 32768
+    generator = torch.Generator().manual_seed(6)
+    counts = torch.bincount(torch.multinomial(torch.ones(groups) / groups, total, replacement=True, generator=generator), minlength=groups)
+    counts[3] += counts[5] - 3
+    counts[5] = 3
+    counts[7] += counts[9]
+    counts[9] = 0
+    counts = counts.tolist()
+    torch.manual_seed(7)
+    x = torch.randn(total, k, device="cuda").bfloat16().requires_grad_()
+    dy = torch.randn(total, n, device="cuda").bfloat16()
+    experts = v.GroupedExperts(groups, k, n, device="cuda")
+
+    def step():
+        x.grad = experts.weight.grad = None
+        experts(x, counts).backward(dy)
+    ms, wall = timed(step, steps, warmup)
+    flops = 3 * 2 * total * k * n
+    b = kernel_breakdown(step, min(steps, 10))
+    gemm_ms = sum(v_["avg_ms"] * v_["launches_per_step"] for name, v_ in b.items() if "gemm" in name)
+    return dict(step_ms=ms, wall_ms=wall, flops=flops, tflops=flops / (ms * 1e-3) / 1e12, counts=counts, kernels=b,
+                gemm_ms=gemm_ms, gemm_tflops=flops / (gemm_ms * 1e-3) / 1e12, gemm_frac_fp8_peak=flops / (gemm_ms * 1e-3) / 1e12 / PEAK["fp8_tflops"])
 
 
 def main():
@@ -129,6 +254,7 @@ def main():
     parser.add_argument("--skip-cpu", action="store_true", help="leave out the CPU baseline leg")
     parser.add_argument("--skip-muon", action="store_true", help="leave out the FP8Muon / codec legs")
     parser.add_argument("--skip-mlp", action="store_true", help="leave out the gated MLP leg")
+    parser.add_argument("--skip-varlen", action="store_true", help="leave out the variable-group (MoE) leg")
     parser.add_argument("--muon-streams", type=int, default=0, help="streams FP8Muon.step spreads its shape buckets over "
                         "(0: the optimizer's default; 1 keeps a kernel trace free of overlapping launches)")
     parser.add_argument("--calibrate", action="store_true",
@@ -142,6 +268,7 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     _lib.library()
 
+    log("linear step")
     layer, x, dy, step = linear_case()
     ms, wall_ms = timed(step, args.steps, args.warmup)
     flops = 6 * M * K * N
@@ -151,7 +278,11 @@ def main():
     gemm_tflops = 2 * M * K * N / (gemm["avg_ms"] * 1e-3) / 1e12
     roofline = dict(bound="mfma", kernel="group_gemm_fast (viola_group_gemm: fwd, dgrad, wgrad)",
                     achieved=gemm_tflops, peak=PEAK["fp8_tflops"], unit="TFLOP/s", frac=gemm_tflops / PEAK["fp8_tflops"],
-                    avg_launch_ms=gemm["avg_ms"], traffic=GEMM_TRAFFIC_BYTES)
+                    avg_launch_ms=gemm["avg_ms"], traffic=GEMM_TRAFFIC_BYTES,
+                    traffic_source="stored calibration (two rocprofv3 --pmc runs, profiles/linear_step_8192x1024x4096_hbm_traffic.txt), not read in this run",
+                    attainable=GEMM_ATTAINABLE_TFLOPS,
+                    attainable_note="issue-bound ceiling of an FP32 scale per 32 k: the K = 16 FP8 MFMAs (half the f8f6f4 rate) plus one "
+                                    "FP32 FMA per accumulator and K group through the same issue port; frac stays against the 5 PFLOP/s peak")
     quant = {}
     if "viola_group_quantize_dual" in breakdown:
         # X [M, K] and dY [M, N] each once per step: 4.25 B per element (bf16 in, two FP8 layouts + scales out)
@@ -163,6 +294,7 @@ def main():
     extra = {}
     if not args.skip_muon:
         for method in ("standard", "gram"):
+            log(f"FP8Muon step, {method}")
             opt, params, elements = muon_case(method)
             if args.muon_streams:
                 opt._LANES = args.muon_streams
@@ -193,6 +325,7 @@ def main():
             del opt, params
             torch.cuda.empty_cache()
         from viola_amd.distributed import _fp8_kernels as codec, packet_bytes
+        log("comm codec")
         n = 6553600
         bucket = torch.randn(n, device="cuda") * 1e-3
         packet = torch.empty((1, packet_bytes(n // 256, 256)), dtype=torch.uint8, device="cuda")
@@ -207,6 +340,7 @@ def main():
         # forward + backward + FP8Muon step + write-back of the master as FP8 codes and (32, 32) scales
         import viola_amd
         from viola_amd.nn import _grouped_kernels as gk
+        log("bound training step")
         viola_amd.set_master_weight_dtype("fp32")
         viola_amd.set_gradient_dtype("bf16")
         torch.manual_seed(1)
@@ -232,6 +366,7 @@ def main():
         # the reference's default recipe on the same layer: one scale per tensor, epilogue scaling (the GEMM runs on
         # the K = 64 f8f6f4 MFMA, the kernel the 5 PFLOP/s figure belongs to)
         import viola_amd
+        log("per-tensor and MXFP8 linear steps")
         viola_amd.set_gradient_dtype("bf16")
         torch.manual_seed(2)
         current = viola_amd.nn.Linear(K, N, device="cuda", dtype=torch.bfloat16, scaling="current", forward_dtype="e4m3",
@@ -276,6 +411,7 @@ def main():
         dym = torch.randn(Mm, Dm, device="cuda").bfloat16()
         extra["mlp_step"] = {"shape": [Mm, Dm, Hm], "flops": mlp_flops}
         for scaling in ("grouped", "current", "mxfp8"):
+            log(f"MLP step, {scaling}")
             viola_amd.set_gradient_dtype("bf16")
             torch.manual_seed(4)
             mlp = viola_amd.nn.MLP(Dm, Hm, activation="silu", weight_dtype="fp8", scaling=scaling, mode="memory", backward_dtype="e4m3",
@@ -292,6 +428,13 @@ def main():
             extra["mlp_step"][scaling] = dict(step_ms=mlp_ms, tflops=mlp_flops / (mlp_ms * 1e-3) / 1e12, gated_gemm=gated)
             del mlp
         del xm, dym
+
+    if not args.skip_muon:
+        log("Newton-Schulz, one 1024 x 4096 matrix")
+        extra["ns_1024x4096"] = ns_single_case(min(args.steps, 50), min(args.warmup, 10))
+    if not args.skip_varlen:
+        log("variable-group step")
+        extra["varlen_step"] = varlen_case(min(args.steps, 20), min(args.warmup, 5))
 
     if args.calibrate:
         from viola_amd.optim import _kernels as ok
@@ -311,8 +454,11 @@ def main():
         "roofline": roofline, "quantize": quant, "kernels": breakdown, **extra,
     }
     if not args.skip_cpu:
+        log("CPU baselines")
         result["cpu_baseline"] = cpu_baseline()
-    print(json.dumps(result))
+    print(json.dumps(result), flush=True)
+    if any(leg.get("ms", 0) is None for leg in result.get("cpu_baseline", {}).get("others", {}).values()):
+        os._exit(0)                                                  # a CPU leg is still running in its thread: do not wait for it
 
 
 if __name__ == "__main__":
