@@ -19,6 +19,11 @@ REFERENCE = Path("/root/reference/viola/optim/_orthogonalize.py")
 CASES = [("standard", (64, 256), 5), ("standard", (192, 64), 5), ("standard", (96, 96), 3),
          ("gram", (64, 256), 5), ("gram", (192, 64), 5), ("gram", (96, 96), 5), ("gram", (64, 160), 2),
          ("standard", (2, 48, 80), 5), ("gram", (2, 48, 80), 5)]
+# The benchmark's single-matrix configuration: one 1024 x 4096 fp32 Gaussian matrix, seed 1, 5 steps. The 4 M-element
+# input is regenerated from its seed by the tests (its sum and a strided sample are stored to make sure of that);
+# of the output a strided sample and all singular values are stored.
+LARGE = (1024, 4096)
+LARGE_STRIDE = 16
 
 
 def main():
@@ -34,6 +39,17 @@ def main():
     path = Path(__file__).with_name("ns_golden.pt")
     torch.save(rows, path)
     print(path, sum(r["input"].numel() for r in rows), "input elements")
+    torch.manual_seed(1)
+    matrix = torch.randn(*LARGE)
+    large = dict(shape=LARGE, seed=1, steps=5, stride=LARGE_STRIDE, input_sum=matrix.double().sum(),
+                 input_sample=matrix[::LARGE_STRIDE, ::LARGE_STRIDE].contiguous())
+    for method in ("standard", "gram"):
+        out = module.METHODS[method](matrix, steps=5)
+        large[method] = dict(sample=out[::LARGE_STRIDE, ::LARGE_STRIDE].contiguous(),
+                             singular_values=torch.linalg.svdvals(out.float()))
+    path = Path(__file__).with_name("ns_golden_1024x4096.pt")
+    torch.save(large, path)
+    print(path)
 
 
 if __name__ == "__main__":

@@ -85,6 +85,86 @@ def test_gated_mlp_gemms_at_16384x4096x11008():
     # the fused forward equals the plain GEMM followed by the elementwise kernel
     plain = g.gemm(qx, qw, sx, sw, (1, 32), (32, 32), out_dtype=torch.bfloat16)
     assert torch.equal(plain, aux)
+    del plain, z, qx, sx, qw, sw
+    # the gated backward at the same size: dz = [d u act'(g) | d act(g)] with d = dY . W_down (a = dY codes, b = the down
+    # projection's W^T [hidden, out]); bit-equal to the plain dgrad GEMM followed by the elementwise backward kernel, and
+    # on the row sample within bf16 rounding of fp32 math on the dequantized operands
+    from viola_amd.nn import _gated_kernels as gk
+    _, qg, sg = _quantized(m, d, (1, 32), 6)
+    torch.manual_seed(7)
+    w2 = torch.empty(h, d, device="cuda").uniform_(-1 / 64, 1 / 64)
+    qw2, sw2 = g.quantize(w2, E4, (32, 32))
+    del w2
+    dz, _, _ = mk.gemm(qg, qw2, sg, sw2, layer=recipe, out_dtype=torch.bfloat16, activation="silu", backward=True, aux=aux,
+                       group_a=(1, 32), group_b=(32, 32))
+    assert dz.shape == (m, 2 * h)
+    dh = g.gemm(qg, qw2, sg, sw2, (1, 32), (32, 32), out_dtype=torch.bfloat16)
+    assert torch.equal(dz, gk.gated_backward(aux, dh, "silu"))
+    d_ref = (g.dequantize(qg[rows].contiguous(), sg[rows].contiguous(), (1, 32)) @ g.dequantize(qw2, sw2, (32, 32)).T).bfloat16().float()
+    sig = torch.sigmoid(gate)
+    expect = torch.cat([d_ref * up * (sig * (1 + gate * (1 - sig))), d_ref * gate * sig], 1).bfloat16()
+    assert rel_l2(dz[rows], expect) < 6e-3
+
+
+def test_mlp_module_at_16384x4096x11008():
+    """The whole viola_amd.nn.MLP forward + backward at the benchmark's size (grouped recipe, FP8 weight storage, memory
+    mode) against fp32 GPU math on dequantized operands: y and dx on a row sample (row-wise quantization is per row, so
+    a sample of rows stands alone), the two weight gradients on a sample of their rows with the full token contraction,
+    the bias gradients as fp32 column sums."""
+    import viola_amd
+    from viola_amd.nn import _grouped_kernels as g
+    m, d, h = 16384, 4096, 11008
+    viola_amd.set_gradient_dtype("bf16")
+    try:
+        torch.manual_seed(11)
+        mlp = viola_amd.nn.MLP(d, h, activation="silu", weight_dtype="fp8", scaling="grouped", mode="memory", backward_dtype="e4m3",
+                               device="cuda", dtype=torch.bfloat16)
+    finally:
+        viola_amd.precision._settings["gradient_dtype"] = None
+    x = torch.randn(m, d, device="cuda").bfloat16().requires_grad_()
+    dy = torch.randn(m, d, device="cuda").bfloat16()
+    y = mlp(x)
+    y.backward(dy)
+    fake = lambda t, transposed=False: g.dequantize(*g.quantize(t.contiguous(), E4, (1, 32), transposed=transposed), (1, 32))
+    w_gu = g.dequantize(mlp.gate_up.weight.detach(), mlp.gate_up.weight_scale, (32, 32))
+    w_dn = g.dequantize(mlp.down.weight.detach(), mlp.down.weight_scale, (32, 32))
+    b_gu, b_dn = mlp.gate_up.bias.detach().float(), mlp.down.bias.detach().float()
+
+    def hidden(x_rows):
+        z = (fake(x_rows) @ w_gu.T + b_gu).bfloat16().float()
+        gate, up = z[:, :h], z[:, h:]
+        sig = 1 / (1 + torch.exp(-gate))
+        return gate, up, sig, (gate * sig * up).bfloat16()
+
+    def hidden_grad(dy_rows, gate, up, sig):
+        dh = (fake(dy_rows) @ w_dn).bfloat16().float()
+        return torch.cat([dh * up * (sig * (1 + gate * (1 - sig))), dh * gate * sig], 1).bfloat16()
+
+    rows = torch.arange(0, m, 61, device="cuda")
+    gate, up, sig, h_rows = hidden(x.detach()[rows])
+    assert rel_l2(y[rows], (fake(h_rows) @ w_dn.T + b_dn).bfloat16()) < 4e-3
+    dz_rows = hidden_grad(dy[rows], gate, up, sig)
+    assert rel_l2(x.grad[rows], (fake(dz_rows) @ w_gu).bfloat16()) < 6e-3
+    del gate, up, sig, h_rows, dz_rows
+    # weight gradients contract over all 16384 tokens: rebuild h and dz in full (in slices of 2048 tokens)
+    h_full = torch.empty(m, h, device="cuda", dtype=torch.bfloat16)
+    dz_full = torch.empty(m, 2 * h, device="cuda", dtype=torch.bfloat16)
+    for start in range(0, m, 2048):
+        part = slice(start, start + 2048)
+        gate, up, sig, h_full[part] = hidden(x.detach()[part])
+        dz_full[part] = hidden_grad(dy[part], gate, up, sig)
+    del gate, up, sig
+    assert rel_l2(mlp.down.bias.grad, dy.float().sum(0)) < 3e-3                    # fp32 column sums in another order, one bf16 rounding
+    assert rel_l2(mlp.gate_up.bias.grad, dz_full.float().sum(0)) < 4e-3
+    out_rows = torch.arange(0, d, 97, device="cuda")
+    got = mlp.down.weight.grad[out_rows]
+    want = fake(dy[:, out_rows], transposed=True) @ fake(h_full, transposed=True).T
+    assert rel_l2(got, want.bfloat16()) < 5e-3, rel_l2(got, want)
+    del want, h_full
+    hidden_rows = torch.arange(0, 2 * h, 501, device="cuda")
+    got = mlp.gate_up.weight.grad[hidden_rows]
+    want = fake(dz_full[:, hidden_rows], transposed=True) @ fake(x.detach(), transposed=True).T
+    assert rel_l2(got, want.bfloat16()) < 6e-3, rel_l2(got, want)
 
 
 @pytest.mark.parametrize("recipe", ["tensor", "mxfp8"])
@@ -206,8 +286,11 @@ def test_newton_schulz_batched_equals_single_at_ditxl_shapes(method):
         assert sigma.max() < 1.3 and (shape[0] == shape[1] or sigma.min() > .3), (shape, float(sigma.min()), float(sigma.max()))
 
 
-def test_fp8muon_step_at_ditxl_block():
-    """One transformer block of the DiT-XL set: the batched step equals stepping each parameter in its own optimizer."""
+@pytest.mark.parametrize("method,rounding", [("standard", "nearest"), ("gram", "nearest"), ("standard", "stochastic"), ("gram", "stochastic")])
+def test_fp8muon_step_at_ditxl_block(method, rounding):
+    """One transformer block of the DiT-XL set, two steps: the batched step equals stepping each parameter in its own
+    optimizer, bit for bit, for both Newton-Schulz methods and both roundings of the momentum state (the stochastic
+    rounding key depends on the parameter's index only, which the stand-alone optimizers are given)."""
     import viola_amd
     d = 1152
     shapes = ((3 * d, d), (d, d), (4 * d, d), (d, 4 * d), (d,), (3 * d,))
@@ -219,15 +302,31 @@ def test_fp8muon_step_at_ditxl_block():
             p.grad = torch.randn_like(p) * 1e-3
         return params
 
+    options = dict(lr=1e-3, weight_decay=.01, adjust_lr_fn="match_rms_adamw", mode="balanced", tile_size=256, ns_method=method,
+                   rounding=rounding, rounding_seed=42)
     together = build(9)
-    viola_amd.optim.FP8Muon(together, lr=1e-3, weight_decay=.01, adjust_lr_fn="match_rms_adamw").step()
+    batched = viola_amd.optim.FP8Muon(together, **options)
+    batched.step()
+    batched.step()
     alone = build(9)
+    singles = []
     for index, p in enumerate(alone):
-        opt = viola_amd.optim.FP8Muon([{"params": [p], "viola_parameter_indices": [index]}], lr=1e-3, weight_decay=.01,
-                                      adjust_lr_fn="match_rms_adamw")
-        opt.step()
-    for a, b in zip(together, alone):
-        assert torch.equal(a, b)
+        singles.append(viola_amd.optim.FP8Muon([{"params": [p], "viola_parameter_indices": [index]}], **options))
+        singles[-1].step()
+        singles[-1].step()
+    for a, b, opt in zip(together, alone, singles):
+        assert torch.equal(a, b) and torch.isfinite(a).all()
+        if a.ndim == 2:
+            assert torch.equal(batched.state[a]["momentum_q"], opt.state[b]["momentum_q"])
+            assert torch.equal(batched.state[a]["momentum_scale"], opt.state[b]["momentum_scale"])
+    if rounding == "stochastic":
+        nearest = build(9)
+        viola_amd.optim.FP8Muon(nearest, **{**options, "rounding": "nearest"}).step()
+        again = build(9)
+        first = viola_amd.optim.FP8Muon(again, **options)
+        first.step()
+        # one step: the update itself does not depend on the rounding of the state that is stored for the next one
+        assert all(torch.equal(a, b) for a, b in zip(nearest, again))
 
 
 @pytest.mark.parametrize("recipe", ["tensor", "mxfp8"])

@@ -293,6 +293,23 @@ def test_ns_matches_reference_golden(golden_dir):
 
 
 @pytest.mark.parametrize("method", ["standard", "gram"])
+def test_ns_matches_reference_golden_at_1024x4096(method, golden_dir):
+    """The benchmark's single-matrix configuration (viola/optim/_orthogonalize.py:10-54 on one 1024 x 4096 Gaussian
+    matrix, seed 1, 5 steps): a strided sample of the reference's output and its singular values, written by
+    tests/golden/make_ns_golden.py. The input is regenerated from the seed and checked against the stored sample."""
+    golden = torch.load(golden_dir / "ns_golden_1024x4096.pt", weights_only=True)
+    torch.manual_seed(golden["seed"])
+    matrix = torch.randn(*golden["shape"])
+    stride = golden["stride"]
+    assert torch.equal(matrix[::stride, ::stride], golden["input_sample"]) and matrix.double().sum() == golden["input_sum"]
+    out = ns.METHODS[method](matrix, steps=golden["steps"])
+    assert torch.equal(out[::stride, ::stride], golden[method]["sample"])
+    sigma = torch.linalg.svdvals(out.float())
+    assert torch.allclose(sigma, golden[method]["singular_values"], atol=1e-4)
+    assert sigma.max() < 1.25 and sigma.min() > .6                                  # the quintic's band
+
+
+@pytest.mark.parametrize("method", ["standard", "gram"])
 @pytest.mark.parametrize("shape", [(64, 256), (192, 64), (96, 96)])
 def test_ns_invariants_and_chain(method, shape):
     torch.manual_seed(1)

@@ -247,6 +247,9 @@ class Linear(nn.Module):
             x = x.to(torch.get_autocast_dtype("cuda"))
         if self._pending_refresh:
             self.refresh_weight(self._master())
+            assert not self._pending_refresh, \
+                "The FP8 weight has not been quantized yet: its master is still on the host. Move the model to the GPU " \
+                "before binding an optimizer (the quantizer runs on the GPU only)."
         need_backward = torch.is_grad_enabled() and (
             x.requires_grad or self.weight.requires_grad or (self.bias is not None and self.bias.requires_grad))
         if self._grouped_scaling:
@@ -284,6 +287,11 @@ class Linear(nn.Module):
         if self._pending_refresh and weight.is_cuda and self._master() is not None and self._master().is_cuda:
             self.refresh_weight(self._master())
         return self
+
+    def _save_to_state_dict(self, destination, prefix, keep_vars):
+        assert not self._pending_refresh, \
+            "This Linear was built on the host and its FP8 codes do not exist yet: move it to the GPU before saving."
+        super()._save_to_state_dict(destination, prefix, keep_vars)
 
     def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
         expected = self.fp8_dtype if self.weight_dtype == "fp8" else _STORAGE[self.weight_dtype]

@@ -207,7 +207,8 @@ class FP8Muon(MatrixOptimizer):
         work = self._workspace.get((param.device, lane))
         if work is None or work.numel() < len(bucket) * count:
             work = self._workspace[(param.device, lane)] = torch.empty(len(bucket) * count, device=param.device, dtype=torch.bfloat16)
-        tables = self._bucket_tables.setdefault((shape, param.device, len(bucket), ordinal), ({}, {}))
+        # keyed by lane as well: a table is only ever rewritten on the stream whose launches read it
+        tables = self._bucket_tables.setdefault((shape, param.device, len(bucket), ordinal, lane), ({}, {}))
         # one launch for the momentum of the whole bucket when its members share the recipe, else one per matrix
         uniform = lambda *names: all(all(item[3][name] == group[name] for name in names) for item in bucket)
         items = []
