@@ -260,7 +260,16 @@ def main():
     parser.add_argument("--calibrate", action="store_true",
                         help="also launch copy_scaled_kernel once over 64 Mi floats (256 MiB read, 256 MiB written): "
                              "the known-size kernel that FETCH_SIZE / WRITE_SIZE readings are scaled by")
+    parser.add_argument("--only", default="", help="comma-separated legs to run besides the Linear step (muon, bound, recipes, mlp, "
+                        "ns1, varlen); default: all that are not skipped. For profiling one leg at a time")
     args = parser.parse_args()
+    skipped = {"muon": args.skip_muon, "bound": args.skip_muon, "recipes": args.skip_muon, "ns1": args.skip_muon,
+               "mlp": args.skip_mlp, "varlen": args.skip_varlen}
+    only = {leg for leg in args.only.split(",") if leg}
+    assert only <= set(skipped), f"unknown leg in --only: {sorted(only - set(skipped))}"
+
+    def want(leg):
+        return leg in only if only else not skipped[leg]
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
     import torch
@@ -292,7 +301,7 @@ def main():
                      gbs=per_step / (q["avg_ms"] * 1e-3) / 1e9, frac_hbm=per_step / (q["avg_ms"] * 1e-3) / 1e9 / PEAK["hbm_gbs"])
 
     extra = {}
-    if not args.skip_muon:
+    if want("muon"):
         for method in ("standard", "gram"):
             log(f"FP8Muon step, {method}")
             opt, params, elements = muon_case(method)
@@ -335,7 +344,7 @@ def main():
         extra["comm_codec"] = dict(bucket_elements=n, pack_ms=pack_ms, unpack_ms=unpack_ms,
                                    pack_gbs=5.016 * n / (pack_ms * 1e-3) / 1e9, unpack_gbs=5.016 * n / (unpack_ms * 1e-3) / 1e9)
 
-    if not args.skip_muon:
+    if want("bound"):
         # the training loop closed: the same Linear under bind_optimizer (fp32 master, bf16 gradients), one
         # forward + backward + FP8Muon step + write-back of the master as FP8 codes and (32, 32) scales
         import viola_amd
@@ -362,7 +371,7 @@ def main():
                                             refresh_gbs=(4 + 1 + 4 / 1024) * K * N / (refresh_ms * 1e-3) / 1e9)
         viola_amd.precision._settings.update(master_weight_dtype=torch.float32, gradient_dtype=None)
 
-    if not args.skip_muon:
+    if want("recipes"):
         # the reference's default recipe on the same layer: one scale per tensor, epilogue scaling (the GEMM runs on
         # the K = 64 f8f6f4 MFMA, the kernel the 5 PFLOP/s figure belongs to)
         import viola_amd
@@ -401,7 +410,7 @@ def main():
                                                gemm_frac_fp8_peak=2 * M * K * N / (cg["avg_ms"] * 1e-3) / 1e12 / PEAK["fp8_tflops"],
                                                launches_per_step=sum(v["launches_per_step"] for v in cb.values()))
 
-    if not args.skip_mlp:
+    if want("mlp"):
         # the gated MLP of the reference's MLP benchmark shape (16384 tokens, 4096 -> 11008 -> 4096, SwiGLU), forward +
         # backward, under the three recipes: gating fused into the gate/up GEMM's and the down dgrad GEMM's epilogues
         import viola_amd
@@ -429,10 +438,10 @@ def main():
             del mlp
         del xm, dym
 
-    if not args.skip_muon:
+    if want("ns1"):
         log("Newton-Schulz, one 1024 x 4096 matrix")
         extra["ns_1024x4096"] = ns_single_case(min(args.steps, 50), min(args.warmup, 10))
-    if not args.skip_varlen:
+    if want("varlen"):
         log("variable-group step")
         extra["varlen_step"] = varlen_case(min(args.steps, 20), min(args.warmup, 5))
 

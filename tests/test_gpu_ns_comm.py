@@ -14,10 +14,13 @@ E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("batch,m,n,k", [(1, 64, 64, 256), (2, 130, 72, 96), (1, 256, 384, 128), (3, 33, 47, 65), (2, 384, 576, 200)])
+@pytest.mark.parametrize("batch,m,n,k", [(1, 64, 64, 256), (2, 130, 72, 96), (1, 256, 384, 128), (3, 33, 47, 65), (2, 384, 576, 200),
+                                         (1, 1024, 1024, 520), (300, 64, 64, 256), (130, 130, 72, 96), (50, 256, 384, 128), (30, 384, 576, 200)])
 @pytest.mark.parametrize("transpose_b,epilogue", [(True, 0), (False, 0), (False, 1), (True, 1), (False, 2)])
 def test_ns_gemm_contract(dtype, batch, m, n, k, transpose_b, epilogue):
-    """One chain GEMM against its contract: fp32 accumulate -> round -> fp32 epilogue -> round."""
+    """One chain GEMM against its contract: fp32 accumulate -> round -> fp32 epilogue -> round. A product with fewer
+    than 40 tiles of 128 x 128 per matrix runs on 64 x 64 tiles with k split over the wavefronts of a block, a larger
+    one (1024 x 1024 here) on the 128- or 192-wide tiles; shapes that are not multiples of 8 on the generic kernel."""
     from viola_amd.optim import _orthogonalize_kernels as nk
     torch.manual_seed(9)
     a = (torch.randn(batch, m, k) / math.sqrt(k)).to(dtype)
@@ -29,10 +32,11 @@ def test_ns_gemm_contract(dtype, batch, m, n, k, transpose_b, epilogue):
     # identical except where a different fp32 summation order flips the final rounding (one ulp of the output dtype)
     ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
     diff = (out.cpu().float() - ref.float()).abs()
-    # second term: the rounded product may flip by one ulp before the epilogue scales it (by 2.0315 at most),
-    # which is not small next to a result that cancels towards zero
+    # second term: the rounded product may flip by one grid step before the epilogue scales it (by 2.0315 at most),
+    # which is not small next to a result that cancels towards zero; a grid step is up to 2 ulp of a value at the
+    # bottom of its binade
     product = ons.matmul(a, b, transpose_b=transpose_b).float().abs()
-    bound = 4 * ulp * ref.float().abs() + 2.1 * ulp * product + 1e-4 * ref.float().abs().max()
+    bound = 4 * ulp * ref.float().abs() + 4.2 * ulp * product + 1e-4 * ref.float().abs().max()
     assert (diff <= bound).all()
     assert rel_l2(out, ref) < (2e-3 if dtype == torch.bfloat16 else 3e-4)
     assert (diff == 0).float().mean() > .9
@@ -45,7 +49,7 @@ def test_ns_gemm_contract(dtype, batch, m, n, k, transpose_b, epilogue):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("batch,m,k", [(2, 384, 200), (1, 576, 96), (3, 200, 72), (1, 1152, 64)])
+@pytest.mark.parametrize("batch,m,k", [(2, 384, 200), (1, 576, 96), (3, 200, 72), (1, 1152, 64), (50, 384, 200), (6, 1152, 64), (1, 1024, 4096)])
 @pytest.mark.parametrize("epilogue", [0, 1])
 def test_ns_gram_product_is_mirrored(dtype, batch, m, k, epilogue):
     """a . a^T (same buffer for both operands) computes the upper tiles only and mirrors them: the result
@@ -57,15 +61,17 @@ def test_ns_gram_product_is_mirrored(dtype, batch, m, k, epilogue):
     residual = r if epilogue else None
     same = nk._matmul(a, a, transpose_b=True, residual=residual, epilogue=epilogue, add_diag=3.4445 if epilogue else None)
     other = nk._matmul(a, a.clone(), transpose_b=True, residual=residual, epilogue=epilogue, add_diag=3.4445 if epilogue else None)
+    # at 1024 rows the Gram product (36 tiles of its own) and the two-buffer product (64 tiles) run on different tile
+    # shapes: equal to rounding there, bit for bit everywhere else
     for x, y in zip(same if epilogue else (same,), other if epilogue else (other,)):
-        assert torch.equal(x, y)
+        assert torch.equal(x, y) if m != 1024 else rel_l2(x, y) < (2e-3 if dtype == torch.bfloat16 else 3e-4)
         assert torch.equal(x, x.mT)
     ref = ons.matmul(a.cpu(), a.cpu(), transpose_b=True, residual=residual.cpu() if epilogue else None, epilogue=epilogue)
     assert rel_l2(same[0] if epilogue else same, ref) < (2e-3 if dtype == torch.bfloat16 else 3e-4)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("batch,m,k", [(2, 384, 200), (1, 576, 384), (1, 1152, 64), (2, 256, 128)])
+@pytest.mark.parametrize("batch,m,k", [(2, 384, 200), (1, 576, 384), (1, 1152, 64), (2, 256, 128), (50, 384, 200), (6, 1152, 64)])
 @pytest.mark.parametrize("epilogue", [1, 2])
 def test_ns_gram_product_with_an_asymmetric_residual(dtype, batch, m, k, epilogue):
     """a . a^T from one buffer (the mirrored path) with a residual that is NOT symmetric: every element, above and
@@ -117,7 +123,8 @@ def test_gram_chain_multiplies_r_by_r_past_the_first_iteration():
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("batch,m,n,k", [(2, 192, 384, 192), (1, 130, 72, 96), (2, 64, 200, 136), (1, 33, 47, 65)])
+@pytest.mark.parametrize("batch,m,n,k", [(2, 192, 384, 192), (1, 130, 72, 96), (2, 64, 200, 136), (1, 33, 47, 65), (1, 100, 72, 96),
+                                         (60, 192, 384, 192), (140, 64, 200, 136)])
 @pytest.mark.parametrize("transpose_b,epilogue", [(False, 2), (False, 0), (True, 0)])
 def test_ns_gemm_transposed_output(dtype, batch, m, n, k, transpose_b, epilogue):
     from viola_amd.optim import _orthogonalize_kernels as nk

@@ -335,6 +335,64 @@ __global__ __launch_bounds__(256) void ns_scale16_kernel(const TIn* __restrict__
     }
 }
 
+// FP32 inputs (a gradient handed over as it is) in 16-byte accesses: four loads in flight per thread for the sum of
+// squares, eight values per thread and step for the scaling.
+template <bool IS_BF16>
+__global__ __launch_bounds__(256) void ns_sumsq32_kernel(const float* __restrict__ in, float* __restrict__ workspace, int64_t count) {
+    const int64_t bz = blockIdx.y;
+    const float4* src = reinterpret_cast<const float4*>(in + bz * count);
+    const int64_t quads = count / 4;
+    const int64_t per = (quads + PARTS - 1) / PARTS;
+    const int64_t begin = (int64_t)blockIdx.x * per;
+    const int64_t end = begin + per < quads ? begin + per : quads;
+    float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    auto add = [](float& sum, const float4& q) {
+        const float v[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float w = half_to_f32<IS_BF16>(f32_to_half<IS_BF16>(v[e]));
+            sum += w * w;
+        }
+    };
+    int64_t i = begin + threadIdx.x;
+    for (; i + 768 < end; i += 1024) {
+        const float4 q0 = src[i], q1 = src[i + 256], q2 = src[i + 512], q3 = src[i + 768];
+        add(part[0], q0); add(part[1], q1); add(part[2], q2); add(part[3], q3);
+    }
+    for (; i < end; i += 256) add(part[0], src[i]);
+    float sum = (part[0] + part[1]) + (part[2] + part[3]);
+    __shared__ float partial[4];
+    sum = wave_sum(sum);
+    if (threadIdx.x % WAVE == 0) partial[threadIdx.x / WAVE] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) workspace[bz * PARTS + blockIdx.x] = (partial[0] + partial[1]) + (partial[2] + partial[3]);
+}
+
+template <bool IS_BF16>
+__global__ __launch_bounds__(256) void ns_scale32_kernel(const float* __restrict__ in, uint16_t* __restrict__ out,
+                                                          const float* __restrict__ workspace, int64_t count) {
+    __shared__ float denom_s;
+    const int64_t bz = blockIdx.y;
+    const float denom = ns_denominator(workspace, bz, IS_BF16, &denom_s);
+    const SharedDivisor divisor(denom, 0.0f);
+    const float4* src = reinterpret_cast<const float4*>(in + bz * count);
+    uint4* dst = reinterpret_cast<uint4*>(out + bz * count);
+    const int64_t octets = count / 8;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < octets; i += (int64_t)gridDim.x * 256) {
+        const float4 q0 = src[2 * i], q1 = src[2 * i + 1];
+        const float v[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float lo = half_to_f32<IS_BF16>(f32_to_half<IS_BF16>(v[2 * e])), hi = half_to_f32<IS_BF16>(f32_to_half<IS_BF16>(v[2 * e + 1]));
+            const bool plain = !(fabsf(lo) < INFINITY) || !(fabsf(hi) < INFINITY);
+            const SharedDivisor use = plain ? SharedDivisor(denom, __uint_as_float(0x7fc00000u)) : divisor;
+            o[e] = ns_scaled<IS_BF16>(lo, denom, use) | (ns_scaled<IS_BF16>(hi, denom, use) << 16);
+        }
+        dst[i] = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+}
+
 // Transposed: a wavefront parks 32 rows x 64 columns of raw 16-bit values in LDS and reads them back with
 // ds_read_b64_tr_b16, so each lane ends up with the 32 rows of one column = 64 contiguous bytes of the output.
 template <typename TIn, bool IS_BF16>
@@ -421,6 +479,16 @@ static int launch_prepare(const void* in, void* out, int64_t batch, int64_t rows
                 const unsigned bx = (unsigned)(octets / 256 / 4 < 1 ? 1 : octets / 256 / 4 > 4096 ? 4096 : octets / 256 / 4);
                 VIOLA_LAUNCH((ns_scale16_kernel<TIn, IS_BF16>), dim3(bx, (unsigned)batch), dim3(256), 0, stream, src, static_cast<uint16_t*>(out), workspace, rows * cols);
             }
+            return viola_launch_status();
+        }
+    }
+    if constexpr (sizeof(TIn) == 4) {
+        const bool aligned = reinterpret_cast<uintptr_t>(in) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+        if (aligned && (rows * cols) % 8 == 0 && rows <= cols) {
+            VIOLA_LAUNCH((ns_sumsq32_kernel<IS_BF16>), dim3(PARTS, (unsigned)batch), dim3(256), 0, stream, src, workspace, rows * cols);
+            const int64_t octets = rows * cols / 8;
+            const unsigned bx = (unsigned)(octets / 256 / 4 < 1 ? 1 : octets / 256 / 4 > 4096 ? 4096 : octets / 256 / 4);
+            VIOLA_LAUNCH((ns_scale32_kernel<IS_BF16>), dim3(bx, (unsigned)batch), dim3(256), 0, stream, src, static_cast<uint16_t*>(out), workspace, rows * cols);
             return viola_launch_status();
         }
     }

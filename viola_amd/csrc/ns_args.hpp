@@ -15,6 +15,7 @@ struct NsArgs {
     int transpose_out;          // store out (and out_diag) as [batch, n, m]
     int symmetric;              // b == a, m == n: compute tiles with tn >= tm only and mirror them
     int tiles_m, tiles_n;
+    int group_m;                // tile rows per band of the work order (ns_fast.hip)
     int64_t tiles;              // batch * tiles_m * tiles_n
 };
 

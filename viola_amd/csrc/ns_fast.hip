@@ -20,7 +20,8 @@
 //     consecutive n: 8-byte stores, per-row residual loads.
 //   * a Gram-type product (b == a, square output) computes only the tiles on and above the diagonal and
 //     stores each off-diagonal tile a second time transposed, its epilogue applied with the residual of the
-//     transposed position (exact for any residual); transpose_out stores [n, m] only.
+//     transposed position (exact for any residual); transpose_out stores [n, m] only. Both placements leave
+//     LDS as 16-byte pieces.
 //   * work order: the 1-D grid is cut into eight contiguous ranges, one per XCD (blockIdx % 8), and
 //     inside a range tiles walk n fastest, so the tiles that share an a panel meet in one L2.
 #include "ns_args.hpp"
@@ -35,6 +36,13 @@ typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 
 constexpr uint32_t NS_OUTSIDE = 0x80000000u;
+#ifndef NS_FILL
+#define NS_FILL 200                                            // blocks that count as one per compute unit (256 units)
+#endif
+#ifndef NS_SMALL_SBK
+#define NS_SMALL_SBK 64
+#define NS_SMALL_STAGES 4
+#endif
 
 template <bool IS_BF16>
 __device__ __forceinline__ f32x16 ns_mfma(uint4 x, uint4 y, f32x16 c) {
@@ -64,6 +72,66 @@ __device__ __forceinline__ i32x4 make_rsrc(const void* base) {
     return r;
 }
 
+// Which output tile a block works on. The blocks of an XCD take a contiguous range of `work` numbers; inside a matrix the
+// numbers walk the tile grid in bands of p.group_m tile rows, column by column inside a band (rows fastest), so that
+// the tiles in flight on one XCD share p.group_m panels of a and a few panels of b and its L2 holds them. A Gram
+// product walks the tiles on and above the diagonal in the same banded order.
+__device__ __forceinline__ void ns_tile_of(const NsArgs& p, int64_t work, int& tm, int& tn, int64_t& bz) {
+    const int band = p.group_m;
+    if (p.symmetric) {
+        const int t = p.tiles_n;
+        const int64_t upper = (int64_t)t * (t + 1) / 2;
+        bz = work / upper;
+        int rest = (int)(work % upper);
+        int first = 0;
+        for (;;) {                                               // the band: rows first .. first + rows - 1, columns first .. t - 1
+            const int rows = t - first < band ? t - first : band;
+            const int in_band = rows * (t - first) - rows * (rows - 1) / 2;
+            if (rest < in_band) break;
+            rest -= in_band;
+            first += rows;
+        }
+        const int rows = t - first < band ? t - first : band;
+        int col = first;
+        for (;;) {                                               // column col holds rows first .. min(col, first + rows - 1)
+            const int here = col - first + 1 < rows ? col - first + 1 : rows;
+            if (rest < here) break;
+            rest -= here;
+            ++col;
+        }
+        tm = first + rest;
+        tn = col;
+    } else {
+        const int64_t per = (int64_t)p.tiles_n * p.tiles_m;
+        bz = work / per;
+        const int t = (int)(work % per);
+        const int group = band * p.tiles_n;
+        const int first = t / group * band;
+        const int rows = p.tiles_m - first < band ? p.tiles_m - first : band;
+        tm = first + t % group % rows;
+        tn = t % group / rows;
+    }
+    // the coordinates come out of divisions the compiler carries in vector registers; pin them to scalars so
+    // everything derived from them (buffer resources, LDS bases) is wave-uniform
+    tm = __builtin_amdgcn_readfirstlane(tm);
+    tn = __builtin_amdgcn_readfirstlane(tn);
+    bz = __builtin_amdgcn_readfirstlane((int)bz);
+}
+
+// Band height for ns_tile_of: an XCD works on about an eighth of the tiles at a time (of one matrix at most); a band of
+// g rows by w columns with g w = that many tiles touches g panels of a and w of b, least when g : w = their sizes.
+static int ns_band(const NsArgs& p, int bm, int bn) {
+#ifdef NS_BAND
+    return NS_BAND;
+#endif
+    const int64_t own = p.symmetric ? (int64_t)p.tiles_n * (p.tiles_n + 1) / 2 : (int64_t)p.tiles_m * p.tiles_n;
+    const int64_t share = p.tiles / 8 < own ? (p.tiles / 8 > 0 ? p.tiles / 8 : 1) : own;
+    int band = 1;
+    while ((int64_t)(band + 1) * (band + 1) * bm <= share * bn) ++band;
+    const int rows = p.symmetric ? p.tiles_n : p.tiles_m;
+    return band < rows ? band : rows;
+}
+
 // Shape: WAVES_M x WAVES_N wavefronts of WM x WN accumulators; SBK k per stage, STAGES stages (loads run
 // STAGES - 1 chunks ahead). Small: 2 x 2 waves, 32 k, 3 stages, two blocks per CU. Big: 4 x 2 waves of 3 x 3
 // (384 x 192), 64 k (whole 128-byte lines per row and load), 2 stages, one block per CU.
@@ -88,24 +156,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void ns_gemm_fast(NsArgs
     if (work >= p.tiles) return;
     int tm, tn;
     int64_t bz;
-    if (p.symmetric) {
-        // upper triangle of the tile grid, row by row: row tm holds tiles_n - tm tiles
-        const int64_t upper = (int64_t)p.tiles_n * (p.tiles_n + 1) / 2;
-        bz = work / upper;
-        int rest = (int)(work % upper);
-        tm = 0;
-        while (rest >= p.tiles_n - tm) { rest -= p.tiles_n - tm; ++tm; }
-        tn = tm + rest;
-    } else {
-        tn = (int)(work % p.tiles_n);
-        tm = (int)((work / p.tiles_n) % p.tiles_m);
-        bz = work / ((int64_t)p.tiles_n * p.tiles_m);
-    }
-    // the tile coordinates come out of 64-bit divisions the compiler carries in vector registers; pin them
-    // to scalars so everything derived from them (buffer resources, LDS bases) is wave-uniform
-    tm = __builtin_amdgcn_readfirstlane(tm);
-    tn = __builtin_amdgcn_readfirstlane(tn);
-    bz = __builtin_amdgcn_readfirstlane((int)bz);
+    ns_tile_of(p, work, tm, tn, bz);
     const bool mirror = p.symmetric && tn != tm;
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
     const int64_t m = p.m, n = p.n, k = p.k;
@@ -210,7 +261,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void ns_gemm_fast(NsArgs
     int cur = 0, fill = AHEAD;
     for (int64_t c = 0; c < chunks; ++c) {
         // all loads but those of the newest AHEAD - 1 chunks have landed: chunk c is in LDS for this wave ...
-        __builtin_amdgcn_s_waitcnt(0x0F70 | ((AHEAD - 1) * (A_LOADS + B_LOADS)));
+        constexpr int IN_FLIGHT = (AHEAD - 1) * (A_LOADS + B_LOADS);  // vmcnt: low four bits, two more in bits 14..15
+        static_assert(IN_FLIGHT < 64, "the count fits the wait instruction");
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (IN_FLIGHT & 15) | ((IN_FLIGHT >> 4) << 14));
         __syncthreads();                    // ... and for every wave; stage `fill` was last read in chunk c-1
         issue((c + AHEAD) * SBK, fill);     // past the end: zeros into a stage nobody reads
         compute(lds + cur * STAGE_EL);
@@ -222,30 +275,39 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void ns_gemm_fast(NsArgs
     const uint16_t* residual = EPILOGUE ? p.residual + bz * m * n : nullptr;
     uint16_t* out = p.out + bz * m * n;
     uint16_t* out_diag = p.out_diag ? p.out_diag + bz * m * n : nullptr;
-    if (!p.transpose_out && !mirror) {
-        // Row-major output: the accumulators hold one row per lane in runs of four columns, which as stores would touch
-        // 32 cache lines per instruction. Each wavefront instead parks its rounded products, 32 rows at a time, in LDS
-        // (the stage ring is free now) and picks them up as 16-byte pieces along the rows, so that the residual loads,
-        // the epilogue arithmetic and the stores all run on 8 consecutive columns of one row.
-        constexpr int WCOLS = 32 * WN, PLD = WCOLS + 8, PIECES = WCOLS / 8;   // parked row: 16 bytes of padding
-        static_assert(WAVES_M * WAVES_N * 32 * PLD * 2 <= (int)sizeof(lds), "parking area fits in the stage ring");
-        __syncthreads();                                                  // every wave has left the ring
-        uint16_t* park = lds + wave * 32 * PLD;
+    // The accumulators hold one row per lane in runs of four columns, which as stores would touch 32 cache lines per
+    // instruction. Each wavefront instead parks its rounded products, 32 rows at a time, in LDS (the stage ring is free
+    // now) and picks them up as 16-byte pieces: along the rows for the [m, n] placement, so that the residual loads, the
+    // epilogue arithmetic and the stores all run on 8 consecutive columns of one row, and down the columns for the
+    // [n, m] placement (the mirrored copy of an off-diagonal Gram tile, or a transposed result), 8 consecutive m of one n.
+    constexpr int WCOLS = 32 * WN, PLD = WCOLS + 8, PIECES = WCOLS / 8;       // parked row: 16 bytes of padding
+    static_assert(WAVES_M * WAVES_N * 32 * PLD * 2 <= (int)sizeof(lds), "parking area fits in the stage ring");
+    __syncthreads();                                                      // every wave has left the ring
+    uint16_t* park = lds + wave * 32 * PLD;
+    auto finish = [&](uint16_t product, float r, bool diagonal, uint32_t& bits, uint32_t& dbits) {
+        float value = ns_widen<IS_BF16>(product);
+        if (EPILOGUE == 1) value = -4.7750f * r + 2.0315f * value;
+        if (EPILOGUE == 2) value = value + 3.4445f * r;
+        bits = ns_narrow<IS_BF16>(value);
+        dbits = diagonal ? ns_narrow<IS_BF16>(ns_widen<IS_BF16>((uint16_t)bits) + p.add_diag) : bits;
+    };
 #pragma unroll
-        for (int j = 0; j < WM; ++j) {
+    for (int j = 0; j < WM; ++j) {
 #pragma unroll
-            for (int i = 0; i < WN; ++i)
+        for (int i = 0; i < WN; ++i)
 #pragma unroll
-                for (int r4 = 0; r4 < 4; ++r4) {
-                    uint32_t h[4];
+            for (int r4 = 0; r4 < 4; ++r4) {
+                uint32_t h[4];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) h[e] = ns_narrow<IS_BF16>(acc[i][j][r4 * 4 + e]);
-                    *reinterpret_cast<uint2*>(&park[l32 * PLD + i * 32 + r4 * 8 + lhi * 4]) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
-                }
+                for (int e = 0; e < 4; ++e) h[e] = ns_narrow<IS_BF16>(acc[i][j][r4 * 4 + e]);
+                *reinterpret_cast<uint2*>(&park[l32 * PLD + i * 32 + r4 * 8 + lhi * 4]) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+            }
+        const int64_t row0 = m0 + wm * 32 * WM + j * 32, col0 = n0 + wn * WCOLS;   // of the parked 32 x WCOLS block
+        if (!p.transpose_out) {
 #pragma unroll
             for (int it = 0; it < 32 * PIECES / WAVE; ++it) {
                 const int id = it * WAVE + lane, pr = id / PIECES, pc = id % PIECES;
-                const int64_t row = m0 + wm * 32 * WM + j * 32 + pr, col = n0 + wn * WCOLS + pc * 8;
+                const int64_t row = row0 + pr, col = col0 + pc * 8;
                 const uint4 raw = *reinterpret_cast<const uint4*>(&park[pr * PLD + pc * 8]);
                 if (row >= m || col >= n) continue;                       // n is a multiple of 8: whole pieces
                 uint4 res = make_uint4(0, 0, 0, 0);
@@ -254,12 +316,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void ns_gemm_fast(NsArgs
                 uint32_t o[4], od[4];
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    float value = ns_widen<IS_BF16>((uint16_t)(pw[e / 2] >> (16 * (e % 2))));
-                    const float r = ns_widen<IS_BF16>((uint16_t)(rw[e / 2] >> (16 * (e % 2))));
-                    if (EPILOGUE == 1) value = -4.7750f * r + 2.0315f * value;
-                    if (EPILOGUE == 2) value = value + 3.4445f * r;
-                    const uint32_t bits = ns_narrow<IS_BF16>(value);
-                    const uint32_t dbits = col + e == row ? ns_narrow<IS_BF16>(ns_widen<IS_BF16>((uint16_t)bits) + p.add_diag) : bits;
+                    uint32_t bits, dbits;
+                    finish((uint16_t)(pw[e / 2] >> (16 * (e % 2))), ns_widen<IS_BF16>((uint16_t)(rw[e / 2] >> (16 * (e % 2)))), col + e == row, bits, dbits);
                     if (e % 2 == 0) { o[e / 2] = bits; od[e / 2] = dbits; }
                     else { o[e / 2] |= bits << 16; od[e / 2] |= dbits << 16; }
                 }
@@ -267,54 +325,43 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void ns_gemm_fast(NsArgs
                 if (out_diag) *reinterpret_cast<uint4*>(out_diag + row * n + col) = make_uint4(od[0], od[1], od[2], od[3]);
             }
         }
-        return;
-    }
+        if (p.transpose_out || mirror) {
+            // element [n, m] of the placement has the product parked at [m][n]. A mirrored element takes the residual of
+            // its own position (a . a^T is symmetric, its residual need not be; an off-diagonal tile holds no diagonal
+            // element), a transposed result the residual of the position it was computed for.
+            const bool whole = m % 8 == 0;
+#pragma unroll 1
+            for (int it = 0; it < WCOLS * 4 / WAVE; ++it) {                   // not unrolled: the accumulators of the later j are still live
+                const int id = it * WAVE + lane, ln = id / 4, lm = id % 4 * 8;
+                const int64_t orow = col0 + ln, ocol = row0 + lm;         // row and first column in the [n, m] placement
+                uint16_t product[8];
 #pragma unroll
-    for (int j = 0; j < WM; ++j) {
-        const int64_t row = m0 + wm * 32 * WM + j * 32 + l32;
-        if (row >= m) continue;
+                for (int e = 0; e < 8; ++e) product[e] = park[(lm + e) * PLD + ln];
+                if (orow >= n || ocol >= m) continue;
+                uint32_t rw[4] = {0, 0, 0, 0};
+                if (EPILOGUE && mirror) {                                 // m == n, a multiple of 8: a whole piece of residual row orow
+                    const uint4 res = *reinterpret_cast<const uint4*>(residual + orow * n + ocol);
+                    rw[0] = res.x; rw[1] = res.y; rw[2] = res.z; rw[3] = res.w;
+                } else if (EPILOGUE) {
 #pragma unroll
-        for (int i = 0; i < WN; ++i) {
-#pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                const int64_t col = n0 + wn * 32 * WN + i * 32 + r4 * 8 + lhi * 4;
-                if (col >= n) continue;                               // n is a multiple of 8: whole quads
-                uint16_t res[4] = {0, 0, 0, 0}, o[4], od[4];
-                if (EPILOGUE) {
-                    const uint2 raw = *reinterpret_cast<const uint2*>(residual + row * n + col);
-                    res[0] = (uint16_t)raw.x; res[1] = (uint16_t)(raw.x >> 16); res[2] = (uint16_t)raw.y; res[3] = (uint16_t)(raw.y >> 16);
+                    for (int e = 0; e < 8; ++e)
+                        if (ocol + e < m) rw[e / 2] |= (uint32_t)residual[(ocol + e) * n + orow] << (16 * (e % 2));
                 }
+                uint32_t o[4], od[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float value = ns_widen<IS_BF16>(ns_narrow<IS_BF16>(acc[i][j][r4 * 4 + e]));
-                    if (EPILOGUE == 1) value = -4.7750f * ns_widen<IS_BF16>(res[e]) + 2.0315f * value;
-                    if (EPILOGUE == 2) value = value + 3.4445f * ns_widen<IS_BF16>(res[e]);
-                    const uint16_t bits = ns_narrow<IS_BF16>(value);
-                    o[e] = bits;
-                    od[e] = col + e == row ? ns_narrow<IS_BF16>(ns_widen<IS_BF16>(bits) + p.add_diag) : bits;
+                for (int e = 0; e < 8; ++e) {
+                    uint32_t bits, dbits;
+                    finish(product[e], ns_widen<IS_BF16>((uint16_t)(rw[e / 2] >> (16 * (e % 2)))), !mirror && ocol + e == orow, bits, dbits);
+                    if (e % 2 == 0) { o[e / 2] = bits; od[e / 2] = dbits; }
+                    else { o[e / 2] |= bits << 16; od[e / 2] |= dbits << 16; }
                 }
-                if (!p.transpose_out) {
-                    *reinterpret_cast<uint2*>(out + row * n + col) = make_uint2((uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16));
-                    if (out_diag) *reinterpret_cast<uint2*>(out_diag + row * n + col) = make_uint2((uint32_t)od[0] | ((uint32_t)od[1] << 16), (uint32_t)od[2] | ((uint32_t)od[3] << 16));
-                }
-                if (p.transpose_out || mirror) {
-                    // [n, m] placement: 32 lanes hold 32 consecutive m of one n, so each 2-byte store
-                    // instruction still fills 64-byte segments
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        uint16_t flipped = o[e], flipped_diag = od[e];
-                        if (EPILOGUE && mirror) {
-                            // element [col + e, row] of a . a^T has this element's product (the sums run over the same
-                            // terms in the same order) but its own residual, which need not be symmetric; an
-                            // off-diagonal tile holds no diagonal element
-                            float value = ns_widen<IS_BF16>(ns_narrow<IS_BF16>(acc[i][j][r4 * 4 + e]));
-                            const float r = ns_widen<IS_BF16>(residual[(col + e) * n + row]);
-                            if (EPILOGUE == 1) value = -4.7750f * r + 2.0315f * value;
-                            if (EPILOGUE == 2) value = value + 3.4445f * r;
-                            flipped = flipped_diag = ns_narrow<IS_BF16>(value);
-                        }
-                        out[(col + e) * m + row] = flipped;
-                        if (out_diag) out_diag[(col + e) * m + row] = flipped_diag;
+                if (whole) {
+                    *reinterpret_cast<uint4*>(out + orow * m + ocol) = make_uint4(o[0], o[1], o[2], o[3]);
+                    if (out_diag) *reinterpret_cast<uint4*>(out_diag + orow * m + ocol) = make_uint4(od[0], od[1], od[2], od[3]);
+                } else {
+                    for (int e = 0; e < 8 && ocol + e < m; ++e) {
+                        out[orow * m + ocol + e] = (uint16_t)(o[e / 2] >> (16 * (e % 2)));
+                        if (out_diag) out_diag[orow * m + ocol + e] = (uint16_t)(od[e / 2] >> (16 * (e % 2)));
                     }
                 }
             }
@@ -328,6 +375,7 @@ static void launch_tiles(NsArgs p, int epilogue, hipStream_t stream) {
     p.tiles_m = (int)((p.m + BM - 1) / BM);
     p.tiles_n = (int)((p.n + BN - 1) / BN);
     p.tiles = p.batch * (p.symmetric ? (int64_t)p.tiles_n * (p.tiles_n + 1) / 2 : (int64_t)p.tiles_m * p.tiles_n);
+    p.group_m = ns_band(p, BM, BN);
     const unsigned grid = (unsigned)((p.tiles + 7) / 8 * 8);
     if (epilogue == 0) VIOLA_LAUNCH((ns_gemm_fast<IS_BF16, B_KN, 0, WM, WN, WAVES_M, WAVES_N, SBK, STAGES>), dim3(grid), dim3(THREADS), 0, stream, p);
     else if (epilogue == 1) VIOLA_LAUNCH((ns_gemm_fast<IS_BF16, B_KN, 1, WM, WN, WAVES_M, WAVES_N, SBK, STAGES>), dim3(grid), dim3(THREADS), 0, stream, p);
@@ -336,17 +384,25 @@ static void launch_tiles(NsArgs p, int epilogue, hipStream_t stream) {
 
 template <bool IS_BF16, bool B_KN>
 static void launch_shape(const NsArgs& p, int epilogue, hipStream_t stream) {
+    // Every tile shape of ns_gemm_fast gives an output element the same arithmetic (k walked in steps of 16 into one
+    // FP32 accumulator, rounded once), so the choice below is about filling the GPU only and may look at the batch.
+    auto area = [&](int64_t tm, int64_t tn) { return ((p.m + tm - 1) / tm) * ((p.n + tn - 1) / tn) * tm * tn; };
+    auto blocks = [&](int64_t tm, int64_t tn) {
+        const int64_t rows = (p.m + tm - 1) / tm, cols = (p.n + tn - 1) / tn;
+        return p.batch * (p.symmetric ? cols * (cols + 1) / 2 : rows * cols);
+    };
     // 192-wide tiles move a third less operand data per flop; take them unless their padding costs more
     // than that (1152 = 6 x 192 and its multiples fit exactly)
-    auto area = [&](int64_t tm, int64_t tn) { return ((p.m + tm - 1) / tm) * ((p.n + tn - 1) / tn) * tm * tn; };
-    const bool wide = area(192, 192) * 20 <= area(128, 128) * 21;
+    const bool wide = area(192, 192) * 20 <= area(128, 128) * 21 && blocks(192, 192) >= NS_FILL;
     // 384 x 192 blocks with whole-line loads when they fit as well as the 192s and still give every CU a few tiles
     // (a Gram product keeps square tiles for its mirrored stores)
-    const bool big = wide && !p.symmetric && area(384, 192) <= area(192, 192) &&
-                     p.batch * ((p.m + 383) / 384) * ((p.n + 191) / 192) >= 3 * 256;
+    const bool big = wide && !p.symmetric && area(384, 192) <= area(192, 192) && blocks(384, 192) >= 3 * 256;
     if (big) launch_tiles<IS_BF16, B_KN, 3, 3, 4, 2, 64, 2>(p, epilogue, stream);
     else if (wide) launch_tiles<IS_BF16, B_KN, 3, 3, 2, 2, 32, 3>(p, epilogue, stream);
-    else launch_tiles<IS_BF16, B_KN, 2, 2, 2, 2, 32, 3>(p, epilogue, stream);
+    else if (blocks(128, 128) >= NS_FILL) launch_tiles<IS_BF16, B_KN, 2, 2, 2, 2, 32, 3>(p, epilogue, stream);
+    // fewer 128 x 128 tiles than compute units (one matrix of a thousand rows): smaller tiles put more of the chip to work
+    else if (!p.symmetric && blocks(128, 64) >= NS_FILL) launch_tiles<IS_BF16, B_KN, 2, 1, 2, 2, 32, 3>(p, epilogue, stream);
+    else launch_tiles<IS_BF16, B_KN, 1, 1, 2, 2, NS_SMALL_SBK, NS_SMALL_STAGES>(p, epilogue, stream);
 }
 
 bool launch_ns_gemm_fast(const NsArgs& p, bool is_bf16, bool b_kn, int epilogue, hipStream_t stream) {
