@@ -199,6 +199,20 @@ __device__ __forceinline__ uint32_t fast_encode4(const SharedDivisor& d, float l
                          __builtin_amdgcn_fmed3f(d.quotient(c), -limit, limit), __builtin_amdgcn_fmed3f(d.quotient(e), -limit, limit));
 }
 
+// The same without the clamp, for groups whose scale is max |v| / limit with limit the format's largest finite value:
+// a quotient is then at most limit in all but its last place, and everything below the first value that rounds past
+// the largest code (464 for e4m3, 61440 for e5m2) converts to that code, which is what the clamp would give.
+template <typename T>
+__device__ __forceinline__ uint32_t fast_encode4_unclamped(const SharedDivisor& d, float a, float b, float c, float e) {
+    return hw_encode4<T>(d.quotient(a), d.quotient(b), d.quotient(c), d.quotient(e));
+}
+
+// max of two pairs of 16-bit unsigned values (one v_pk_max_u16)
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+    typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2_t, a), __builtin_bit_cast(u16x2_t, b)));
+}
+
 // ------------------------------------------------------------------ group scales and the clamped encoder
 template <typename TOut>
 __device__ __forceinline__ uint8_t encode_clamped(float v, float s, float limit) {

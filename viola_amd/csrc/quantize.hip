@@ -9,6 +9,8 @@
 //   quantize_generic   any (gr, gc), transposed or not, optional re-encode from codes+scales:
 //                      one wavefront per group, two passes over the group (second hits cache).
 //   dequantize, fp8 transpose, segmented transposed quantize for the variable-group path.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace viola {
@@ -301,21 +303,24 @@ __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x
     float vr[4][8], s_row[4];
     bool fast = true;
     SharedDivisor d_row[4] = {SharedDivisor(1.0f, 0.0f), SharedDivisor(1.0f, 0.0f), SharedDivisor(1.0f, 0.0f), SharedDivisor(1.0f, 0.0f)};
+    // The largest magnitude of a group is found on the raw 16-bit patterns, two to an instruction: with the sign bit
+    // masked off, bf16 and fp16 order as unsigned integers like their values, and anything at or above the pattern of
+    // infinity is an Inf or a NaN, which sends the wavefront down the exact path below (where the maximum is taken
+    // again the way the reference's kernel takes it, ignoring NaN).
+    constexpr uint32_t MAGNITUDE = 0x7fff7fffu, INF16 = sizeof(TIn) == 2 && std::is_same<TIn, bf16_t>::value ? 0x7f80u : 0x7c00u;
+    auto top16 = [](uint32_t pairs) -> uint32_t { const uint32_t lo = pairs & 0xffffu, hi = pairs >> 16; return lo > hi ? lo : hi; };
     if constexpr (ROWWISE) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            float amax = 0.0f, poison = 0.0f;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                vr[i][e] = widen16<TIn>(e % 2 ? raw[i][e / 2] >> 16 : raw[i][e / 2] & 0xffffu);
-                amax = fmaxf(amax, fabsf(vr[i][e]));
-                poison = poison_of(poison, vr[i][e]);
-            }
-            amax = group_max<4>(amax);
-            poison += quad_xor<1>(poison);
-            poison += quad_xor<2>(poison);
-            s_row[i] = group_scale(amax, limit, e8m0);
-            d_row[i] = SharedDivisor(s_row[i], poison);
+            for (int e = 0; e < 8; ++e) vr[i][e] = widen16<TIn>(e % 2 ? raw[i][e / 2] >> 16 : raw[i][e / 2] & 0xffffu);
+            uint32_t top = top16(pk_max_u16(pk_max_u16(raw[i][0] & MAGNITUDE, raw[i][1] & MAGNITUDE), pk_max_u16(raw[i][2] & MAGNITUDE, raw[i][3] & MAGNITUDE)));
+            const uint32_t other = (uint32_t)__builtin_amdgcn_mov_dpp((int)top, 0x4E, 0xf, 0xf, true);      // lanes 2 3 0 1 of the quad
+            top = top > other ? top : other;
+            const uint32_t next = (uint32_t)__builtin_amdgcn_mov_dpp((int)top, 0xB1, 0xf, 0xf, true);       // lanes 1 0 3 2
+            top = top > next ? top : next;
+            s_row[i] = group_scale(widen16<TIn>(top), limit, e8m0);
+            d_row[i] = SharedDivisor(s_row[i], top >= INF16 ? __uint_as_float(0x7fc00000u) : 0.0f);
             fast = fast && d_row[i].fast;
         }
     }
@@ -324,25 +329,33 @@ __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x
     const int strip = (lane / 16) * 16, sub = lane & 15;
     const uint16_t* at = &mine[(sub >> 2) * LD + strip + 4 * (sub & 3)];
     float vc[32];
-    float amax = 0.0f, poison = 0.0f;
+    uint32_t top_col = 0;
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
-        const s16x4 four = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at + 4 * t * LD));
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            vc[4 * t + e] = widen16<TIn>((uint16_t)four[e]);
-            amax = fmaxf(amax, fabsf(vc[4 * t + e]));
-            poison = poison_of(poison, vc[4 * t + e]);
-        }
+        const uint2 four = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at + 4 * t * LD)));
+        vc[4 * t] = widen16<TIn>(four.x & 0xffffu); vc[4 * t + 1] = widen16<TIn>(four.x >> 16);
+        vc[4 * t + 2] = widen16<TIn>(four.y & 0xffffu); vc[4 * t + 3] = widen16<TIn>(four.y >> 16);
+        top_col = pk_max_u16(top_col, pk_max_u16(four.x & MAGNITUDE, four.y & MAGNITUDE));
     }
-    const float s_col = group_scale(amax, limit, e8m0);
-    const SharedDivisor d_col(s_col, poison);
+    top_col = top16(top_col);
+    float s_col = group_scale(widen16<TIn>(top_col), limit, e8m0);
+    const SharedDivisor d_col(s_col, top_col >= INF16 ? __uint_as_float(0x7fc00000u) : 0.0f);
     fast = fast && d_col.fast;
 
     // one decision per wavefront: the common case runs without a single divergent branch
     uint2 row_codes[4];
     uint32_t col_codes[8];
-    if (__builtin_amdgcn_ballot_w64(!fast) == 0) {
+    if (__builtin_amdgcn_ballot_w64(!fast) == 0 && limit == fp8_traits<TOut>::max) {
+        // the scale is max |v| / (the format's largest value): no quotient can round past the largest code
+        if constexpr (ROWWISE) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                row_codes[i] = make_uint2(fast_encode4_unclamped<TOut>(d_row[i], vr[i][0], vr[i][1], vr[i][2], vr[i][3]),
+                                          fast_encode4_unclamped<TOut>(d_row[i], vr[i][4], vr[i][5], vr[i][6], vr[i][7]));
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) col_codes[k] = fast_encode4_unclamped<TOut>(d_col, vc[4 * k], vc[4 * k + 1], vc[4 * k + 2], vc[4 * k + 3]);
+    } else if (__builtin_amdgcn_ballot_w64(!fast) == 0) {
         if constexpr (ROWWISE) {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
@@ -352,11 +365,23 @@ __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x
 #pragma unroll
         for (int k = 0; k < 8; ++k) col_codes[k] = fast_encode4<TOut>(d_col, limit, vc[4 * k], vc[4 * k + 1], vc[4 * k + 2], vc[4 * k + 3]);
     } else {
-        const SharedDivisor exact(1.0f, __uint_as_float(0x7fc00000u));       // fast == false: true division, software encoder
+        // some group of the wavefront holds an Inf or a NaN, or a scale outside the quotient route's domain: the maxima
+        // again as the reference's kernel takes them (fmax ignores NaN), true division, software encoder
+        const SharedDivisor exact(1.0f, __uint_as_float(0x7fc00000u));
         if constexpr (ROWWISE) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) row_codes[i] = encode8<TOut>(vr[i], s_row[i], limit, exact);
+            for (int i = 0; i < 4; ++i) {
+                float amax = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(vr[i][e]));
+                s_row[i] = group_scale(group_max<4>(amax), limit, e8m0);
+                row_codes[i] = encode8<TOut>(vr[i], s_row[i], limit, exact);
+            }
         }
+        float amax = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(vc[i]));
+        s_col = group_scale(amax, limit, e8m0);
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
             col_codes[k] = 0;
