@@ -139,6 +139,16 @@ int viola_tensor_gemm(const void* a, int a_dtype, const void* b, int b_dtype, co
                       int64_t m, int64_t n, int64_t k, const void* bias, int bias_dtype, void* out, int out_dtype,
                       viola_stream_t stream);
 
+/* The same product under the reference's accum_dtype="fp16" options (viola/nn/_linear_kernels.py:139-155, :198-211):
+ * every 32 k the running FP16 partial becomes fp16(partial + the 32 products); after accum_block k (rounded down to
+ * whole 64-k chunks from 64 up; 0: never) the partial is added to a total kept in reduce_dtype (VIOLA_F32 or
+ * VIOLA_BF16, rounded after every addition) and cleared; out = (total * sa[0]) * sb[0] (+ bias). An ablation option:
+ * runs on the generic kernel. The 32 products are summed in FP32 and rounded once, the best case of a tensor-core
+ * instruction with an FP16 accumulator. */
+int viola_tensor_gemm_half(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,
+                           int64_t m, int64_t n, int64_t k, const void* bias, int bias_dtype, void* out, int out_dtype,
+                           int accum_block, int reduce_dtype, viola_stream_t stream);
+
 /* ---------------------------------------------------------------- MXFP8: E8M0 scales per 32 k
  * viola/nn/_grouped_kernels.py:310-328 `gemm` with native=True (gemm_kernel :195-293 on the block-scaled MMA of
  * :174-192): out[m, n] = sum_kg (sum_{k in kg} a[m, k] b[n, k]) * 2^(sa[m / ar, kg] - 127) * 2^(sb[n / br, kg] - 127)
@@ -156,6 +166,15 @@ int viola_mx_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const 
 int viola_group_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,
                      int64_t m, int64_t n, int64_t k, int ar, int ak, int br, int bk,
                      const void* bias, int bias_dtype, void* out, int out_dtype, viola_stream_t stream);
+
+/* viola_group_gemm under accum_dtype="fp16" (viola/nn/_grouped_kernels.py:268-292, :310-318): the raw products of
+ * gcd(ak, bk, accum_block) k (accum_block 0: gcd(ak, bk)) meet in an FP16 partial, fp16(partial + 32 products) per
+ * 32 k, which is then scaled, (partial * sa) * sb, added to a total kept in reduce_dtype (VIOLA_F32 or VIOLA_BF16,
+ * rounded after every addition) and cleared. Generic kernel; same FP32-sum-then-round model of the 32-k step. */
+int viola_group_gemm_half(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,
+                          int64_t m, int64_t n, int64_t k, int ar, int ak, int br, int bk,
+                          const void* bias, int bias_dtype, void* out, int out_dtype, int accum_block, int reduce_dtype,
+                          viola_stream_t stream);
 
 /* viola/nn/_mlp_kernels.py:243-277 `gemm` (kernel :16-231), grouped FP32-scale path.
  * forward (backward = 0): b is [2h, k]; g = a.b[0:h]^T, u = a.b[h:2h]^T (+bias), each rounded to

@@ -107,3 +107,38 @@ def gemm_kgroup_order(a, b, sa, sb, group_a, group_b, *, bias=None):
     if bias is not None:
         total = total + bias.float()
     return total
+
+
+def gemm_half(a, b, sa, sb, group_a, group_b, *, accum_block_size=0, reduce_dtype=torch.float32, bias=None,
+              out_dtype=torch.float32):
+    """gemm_kernel with accum_dtype='float16' (viola/nn/_grouped_kernels.py:268-292, :310-318).
+
+    `acc` is an FP16 fragment advanced by the 32-k tensor-core step `mma.mma(al, bl, acc)`: modelled as
+    acc = fp16(acc + the 32 products summed exactly), the best a unit with an FP16 accumulator can return (what the
+    reference's GPU does inside that step is not written in its source: parity with it is held to the bound of
+    checks/check_grouped_linear.py:41, not to the bit). Every partial_k = gcd(group K sizes, accum_block_size) k:
+    total = reduce_dtype(float(total) + float(acc) * sa * sb), acc = 0.
+    """
+    import math
+    m, k = a.shape
+    n = b.shape[0]
+    partial_k = math.gcd(group_a[1], group_b[1])
+    if accum_block_size:
+        partial_k = math.gcd(partial_k, accum_block_size)
+    total = torch.zeros(m, n, dtype=reduce_dtype)
+    acc = torch.zeros(m, n, dtype=torch.float16)
+    af, bf = a.double(), b.double()
+    rows = torch.arange(m) // group_a[0]
+    cols = torch.arange(n) // group_b[0]
+    for k0 in range(0, k, 32):
+        step = af[:, k0:k0 + 32] @ bf[:, k0:k0 + 32].T                    # exact in float64
+        acc = (acc.double() + step).to(torch.float16)
+        if (k0 + 32) % partial_k == 0 or k0 + 32 >= k:
+            scaled = (acc.float() * sa[rows, k0 // group_a[1]][:, None]) * sb[cols, k0 // group_b[1]][None, :]
+            total = (total.float() + scaled).to(reduce_dtype)
+            acc = torch.zeros_like(acc)
+    value = total.float()
+    if bias is not None:
+        value = value + bias.float()
+    return value.to(out_dtype)
+

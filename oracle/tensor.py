@@ -49,6 +49,32 @@ def gemm(a, b, sa, sb, *, bias=None, out_dtype=torch.float32):
     return value.to(out_dtype)
 
 
+def gemm_half(a, b, sa, sb, *, accum_block_size=0, reduce_dtype=torch.float32, bias=None, out_dtype=torch.float32):
+    """_gemm_kernel / _mixed_gemm_kernel with accum_dtype='float16' (viola/nn/_linear_kernels.py:139-161, :198-224).
+
+    The FP16 fragment advances by 32-k tensor-core steps, acc = fp16(acc + the 32 products summed exactly) (the
+    model of oracle.grouped.gemm_half). After whole chunks of bk k (bk = 64, or accum_block_size below that) that
+    complete accum_block_size // bk chunks, and after the last chunk, total = reduce_dtype(float(total) + float(acc))
+    and acc = 0; with accum_block_size = 0 the fragment runs over all of k. out = float(total) * sa * sb + bias."""
+    m, k = a.shape
+    n = b.shape[0]
+    bk = accum_block_size if 0 < accum_block_size < 64 else 64
+    acc = torch.zeros(m, n, dtype=torch.float16)
+    total = torch.zeros(m, n, dtype=reduce_dtype)
+    af, bf = a.double(), b.double()
+    chunks = -(-k // bk)
+    for chunk in range(chunks):
+        for k0 in range(chunk * bk, min((chunk + 1) * bk, k), 32):
+            acc = (acc.double() + af[:, k0:k0 + 32] @ bf[:, k0:k0 + 32].T).to(torch.float16)
+        if accum_block_size and ((chunk + 1) % (accum_block_size // bk) == 0 or chunk == chunks - 1):
+            total = (total.float() + acc.float()).to(reduce_dtype)
+            acc = torch.zeros_like(acc)
+    value = (total.float() if accum_block_size else acc.float()) * sa.float().reshape(()) * sb.float().reshape(())
+    if bias is not None:
+        value = value + bias.float()
+    return value.to(out_dtype)
+
+
 def linear(x, qw, sw, bias, dy, *, fp8=torch.float8_e4m3fn, bwd_fp8=torch.float8_e5m2, sx=None, sg=None,
            out_dtype=torch.bfloat16, grad_dtype=torch.bfloat16):
     """Expected y, dx, dw, db of Linear(scaling="current") from the stored weight codes (checks/linear.py:34-36):

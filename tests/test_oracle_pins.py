@@ -466,6 +466,47 @@ def test_varlen_linear_oracle_against_brute_force():
     assert torch.equal(r2["y"][1:38], r["y"][1:38]) and torch.equal(r2["dw"][2], r["dw"][2]) and r2["y"][0].abs().max() == 0
 
 
+def test_half_accumulator_oracles_by_hand():
+    """oracle.grouped.gemm_half / oracle.tensor.gemm_half (the reference's accum_dtype='fp16' loops) on cases worked out
+    by hand: 2049 is a tie between the FP16 neighbours 2048 and 2050 and goes to 2048; the partial is cleared per scale
+    group (grouped recipe) or runs on (per-tensor, no block); a bf16 total rounds after every addition; sums that FP16
+    holds exactly reproduce the FP32 product; and on the reference's test distribution with its half-sum limit the
+    result stays inside the bound of checks/check_grouped_linear.py:41 while differing from the FP32 sums."""
+    from oracle import tensor
+    a, b = torch.zeros(1, 64), torch.zeros(1, 64)
+    a[0, 0], b[0, 0], a[0, 1], b[0, 1] = 64, 32, 1, 1                              # first 32 k: 2048 + 1
+    a[0, 32], b[0, 32] = 2, 3                                                      # second 32 k: 6
+    qa, qb = a.to(E4), b.to(E4)
+    sa, sb = torch.tensor([[.5, 2.]]), torch.tensor([[1., 1.]])
+    assert grouped.gemm(qa, qb, sa, sb, (1, 32), (32, 32)).item() == 2049 * .5 + 12
+    assert grouped.gemm_half(qa, qb, sa, sb, (1, 32), (32, 32)).item() == 2048 * .5 + 12       # per group: fp16(2049) = 2048
+    one, half = torch.tensor([1.]), torch.tensor([.5])
+    assert tensor.gemm_half(qa, qb, half, one).item() == 2054 * .5                 # one running partial: fp16(2048 + 6) = 2054
+    assert tensor.gemm_half(qa, qb, half, one, accum_block_size=32).item() == 2054 * .5      # fp32 total of 2048 and 6
+    # a bf16 total: 2048 + 6 = 2054 rounds to 2048 (bf16 spacing 16 there)
+    assert tensor.gemm_half(qa, qb, half, one, accum_block_size=32, reduce_dtype=torch.bfloat16).item() == 2048 * .5
+    assert grouped.gemm_half(qa, qb, torch.ones(1, 2), sb, (1, 32), (32, 32), reduce_dtype=torch.bfloat16).item() == 2048
+    # (1, 64) groups: one partial spans both 32-k steps, fp16(2048 + 6); an accumulation block of 32 splits it again
+    wide = torch.tensor([[.5]])
+    assert grouped.gemm_half(qa, qb, wide, torch.ones(1, 1), (1, 64), (32, 64)).item() == 2054 * .5
+    assert grouped.gemm_half(qa, qb, wide, torch.ones(1, 1), (1, 64), (32, 64), accum_block_size=32).item() == 2054 * .5
+    # small integers: every partial sum is an integer below 2048, exact in FP16
+    torch.manual_seed(60)
+    ia, ib = torch.randint(-3, 4, (9, 96)).float().to(E4), torch.randint(-3, 4, (7, 96)).float().to(E4)
+    isa, isb = torch.exp2(torch.randint(-2, 3, (9, 3)).float()), torch.exp2(torch.randint(-2, 3, (1, 3)).float())
+    assert torch.equal(grouped.gemm_half(ia, ib, isa, isb, (1, 32), (32, 32)), grouped.gemm(ia, ib, isa, isb, (1, 32), (32, 32)))
+    assert torch.equal(tensor.gemm_half(ia, ib, one, one), tensor.gemm(ia, ib, one, one))
+    # the reference's own check (check_grouped_linear.py:23-46, half=True): limit 8, bound .01
+    torch.manual_seed(2041)
+    x = (torch.randn(65, 128) * torch.exp2(torch.randint(-5, 6, (65, 1)))).bfloat16()
+    w = (torch.randn(96, 128) * torch.exp2(torch.randint(-5, 6, (96, 1)))).bfloat16()
+    (qx, sx), (qw, sw) = grouped.quantize(x, E5, (1, 32), limit=8.0), grouped.quantize(w, E4, (32, 32), limit=8.0)
+    exact = grouped.gemm(qx, qw, sx, sw, (1, 32), (32, 32))
+    model = grouped.gemm_half(qx, qw, sx, sw, (1, 32), (32, 32))
+    assert 0 < rel_l2(model, exact) < .01
+    assert 0 < rel_l2(grouped.gemm_half(qx, qw, sx, sw, (1, 32), (32, 32), reduce_dtype=torch.bfloat16), exact) < .01
+
+
 # ----------------------------------------------------------------------------- per-tensor scaling
 @pytest.mark.parametrize("dtype", [E4, E5])
 def test_tensor_oracle_matches_the_reference_cpu_definitions(dtype):

@@ -27,6 +27,8 @@ _SIGNATURES = {
     "viola_fp8_transpose": [_p, _p, _l, _l, _l, _p],
     "viola_block_transpose": [_p, _p, _l, _l, _p, _p, _i, _i, _i, _p],
     "viola_group_gemm": [_p, _i, _p, _i, _p, _p, _l, _l, _l, _i, _i, _i, _i, _p, _i, _p, _i, _p],
+    "viola_group_gemm_half": [_p, _i, _p, _i, _p, _p, _l, _l, _l, _i, _i, _i, _i, _p, _i, _p, _i, _i, _i, _p],
+    "viola_tensor_gemm_half": [_p, _i, _p, _i, _p, _p, _l, _l, _l, _p, _i, _p, _i, _i, _i, _p],
     "viola_gated_gemm": [_p, _i, _p, _i, _p, _p, _l, _l, _l, _i, _i, _i, _i, _p, _i, _p, _p, _i, _i, _i, _p],
     "viola_varlen_group_gemm": [_p, _i, _p, _i, _p, _p, _p, _i, _l, _l, _l, _i, _i, _i, _i, _l, _l, _p, _i, _p],
     "viola_varlen_wgrad_gemm": [_p, _i, _p, _i, _p, _p, _p, _i, _l, _l, _l, _p, _i, _p],

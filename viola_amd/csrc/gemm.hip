@@ -57,8 +57,18 @@ template <typename TO> __device__ __forceinline__ float round_through(float v) {
 
 // A_BF8/B_BF8: operand formats (false = e4m3, true = e5m2). B_ROWSCALE: b scales vary inside a 32-row block.
 // VEC: 16-byte global loads are legal (k ranges and row strides multiples of 16, aligned bases).
-template <int MODE, bool A_BF8, bool B_BF8, bool B_ROWSCALE, bool VEC, typename TO>
+//
+// HALF models the reference's accum_dtype="fp16" (viola/nn/_grouped_kernels.py:268-292, _linear_kernels.py:139-155,
+// :198-211): its FP8 tensor-core instruction covers 32 k and, with an FP16 accumulator, returns
+// fp16(accumulator + the 32 products); the accumulator is cleared after `half_period` k, when it is added to a
+// running total held in FP32 or bf16 (rounded after every addition). HALF == 1 is the grouped recipe (a period is one
+// scale group: the partial is scaled by sa * sb as it is added, (partial * sa) * sb), HALF == 2 the per-tensor recipe
+// (scales applied to the finished total; half_period == 0: one partial over the whole k range and no total). Here the
+// 32 products are summed in FP32 by the MFMA and rounded once, which is that instruction's best case; where the
+// hardware's own sum is coarser the reference's results differ, inside the bound its checks allow (.01).
+template <int MODE, bool A_BF8, bool B_BF8, bool B_ROWSCALE, bool VEC, typename TO, int HALF = 0>
 __global__ __launch_bounds__(256, 2) void group_gemm_kernel(GemmArgs p, int bias_dtype) {
+    static_assert(HALF == 0 || MODE == MODE_PLAIN, "the FP16-accumulator model is built for the plain product");
     __shared__ __attribute__((aligned(16))) uint8_t lds_a[2][BM * LDK];
     __shared__ __attribute__((aligned(16))) uint8_t lds_b[2][BN * LDK];
     __shared__ __attribute__((aligned(16))) float lds_sa[2][KG][BM];
@@ -178,6 +188,19 @@ __global__ __launch_bounds__(256, 2) void group_gemm_kernel(GemmArgs p, int bias
 #pragma unroll
             for (int r = 0; r < 16; ++r) total[i][j][r] = 0.0f;
 
+    // HALF: the FP16 partial sums (kept as the floats they round to)
+    f32x16 partial[HALF ? 2 : 1][HALF ? 2 : 1];
+    if constexpr (HALF != 0) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) partial[i][j][r] = 0.0f;
+    }
+    auto to_half = [](float v) -> float { return (float)(_Float16)v; };
+    auto reduced = [&](float v) -> float { return p.reduce_bf16 ? bf16_bits_to_f32(f32_to_bf16_bits(v)) : v; };
+
     const int64_t chunks = (k_end - k_begin + BK - 1) / BK;
     if (chunks > 0) {
         fetch(k_begin);
@@ -209,6 +232,34 @@ __global__ __launch_bounds__(256, 2) void group_gemm_kernel(GemmArgs p, int bias
                             acc[i][j] = mfma32<A_BF8, B_BF8>(opb[i], opa[j], acc[i][j]);
                         }
                     }
+            }
+            if constexpr (HALF != 0) {
+                // this 32-k step joins the FP16 partial; at the end of a period (and of the k range) the partial joins the total
+                const int64_t done = chunk * BK + kg * 32 + 32;                  // k covered so far, relative to k_begin
+                const bool last = done >= k_end - k_begin;
+                const bool flush = p.half_period ? (done % p.half_period == 0 || last) : false;
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const float sa_l = lds_sa[s][kg][wm * 64 + j * 32 + l32];
+#pragma unroll
+                    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            const float h = to_half(partial[i][j][r] + acc[i][j][r]);
+                            partial[i][j][r] = h;
+                            if (flush) {
+                                float term = h;
+                                if constexpr (HALF == 1) {
+                                    const float sb_l = B_ROWSCALE ? lds_sb[s][kg][b_sub(i) + (r / 4) * 8 + lhi * 4 + r % 4] : lds_sb[s][kg][b_sub(i)];
+                                    term = (h * sa_l) * sb_l;
+                                }
+                                total[i][j][r] = reduced(total[i][j][r] + term);
+                                partial[i][j][r] = 0.0f;
+                            }
+                        }
+                    }
+                }
+                continue;
             }
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
@@ -270,6 +321,10 @@ __global__ __launch_bounds__(256, 2) void group_gemm_kernel(GemmArgs p, int bias
                     const int64_t ncol = n_begin + wn * 64 + i * 32 + (r / 4) * 8 + lhi * 4 + r % 4;
                     if (ncol >= p.n) continue;
                     float v = total[i][j][r];
+                    if constexpr (HALF == 2) {
+                        v = p.half_period ? v : partial[i][j][r];
+                        v = (v * p.sa[0]) * p.sb[0];
+                    }
                     if constexpr (MODE == MODE_PLAIN) {
                         if (p.bias) v += load_dtype(p.bias, ncol, bias_dtype);
                         out[mrow * p.ldo + ncol] = from_f32<TO>(v);
@@ -330,6 +385,32 @@ static int launch_out(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtyp
     return viola_launch_status();
 }
 
+// The FP16-accumulator model: always the generic kernel (an ablation option of the reference, not a fast path).
+template <int HALF, bool B_ROWSCALE, typename TO>
+static void launch_half_formats(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, dim3 grid, hipStream_t stream) {
+    const bool a5 = a_dtype == VIOLA_E5M2, b5 = b_dtype == VIOLA_E5M2;
+    if (!a5 && !b5) VIOLA_LAUNCH((group_gemm_kernel<MODE_PLAIN, false, false, B_ROWSCALE, false, TO, HALF>), grid, dim3(256), 0, stream, p, bias_dtype);
+    else if (a5 && !b5) VIOLA_LAUNCH((group_gemm_kernel<MODE_PLAIN, true, false, B_ROWSCALE, false, TO, HALF>), grid, dim3(256), 0, stream, p, bias_dtype);
+    else if (!a5 && b5) VIOLA_LAUNCH((group_gemm_kernel<MODE_PLAIN, false, true, B_ROWSCALE, false, TO, HALF>), grid, dim3(256), 0, stream, p, bias_dtype);
+    else VIOLA_LAUNCH((group_gemm_kernel<MODE_PLAIN, true, true, B_ROWSCALE, false, TO, HALF>), grid, dim3(256), 0, stream, p, bias_dtype);
+}
+
+template <int HALF>
+static int launch_half(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, bool rowscale, dim3 grid,
+                       hipStream_t stream) {
+#define VIOLA_HALF(TO)                                                                                        \
+    if (HALF == 1 && rowscale) launch_half_formats<HALF, HALF == 1, TO>(p, a_dtype, b_dtype, bias_dtype, grid, stream); \
+    else launch_half_formats<HALF, false, TO>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
+    switch (out_dtype) {
+        case VIOLA_F32: VIOLA_HALF(float) break;
+        case VIOLA_BF16: VIOLA_HALF(bf16_t) break;
+        case VIOLA_F16: VIOLA_HALF(f16_t) break;
+        default: return VIOLA_EINVAL;
+    }
+#undef VIOLA_HALF
+    return viola_launch_status();
+}
+
 static bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
 static bool pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
 
@@ -356,6 +437,54 @@ extern "C" int viola_group_gemm(const void* a, int a_dtype, const void* b, int b
     const bool vec = k % 16 == 0 && aligned16(a) && aligned16(b);
     const bool rowscale = br % 32 != 0;
     return launch_out<MODE_PLAIN>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, vec, dim3((unsigned)gx, (unsigned)gy), stream);
+}
+
+static int gcd_of(int a, int b) { while (b) { const int t = a % b; a = b; b = t; } return a; }
+
+extern "C" int viola_group_gemm_half(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,
+                                     int64_t m, int64_t n, int64_t k, int ar, int ak, int br, int bk, const void* bias,
+                                     int bias_dtype, void* out, int out_dtype, int accum_block, int reduce_dtype,
+                                     viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_fp8(a_dtype) && viola_is_fp8(b_dtype) && viola_is_float(out_dtype));
+    VIOLA_CHECK_ARG(m >= 0 && n >= 0 && k >= 0 && ar > 0 && br > 0 && pow2(ak) && pow2(bk) && ak >= 32 && bk >= 32);
+    VIOLA_CHECK_ARG((!bias || viola_is_float(bias_dtype)) && accum_block >= 0 && accum_block % 32 == 0);
+    VIOLA_CHECK_ARG(reduce_dtype == VIOLA_F32 || reduce_dtype == VIOLA_BF16);
+    if (m == 0 || n == 0) return 0;
+    VIOLA_CHECK_ARG(out && (k == 0 || (a && b && sa && sb)));
+    const int64_t gy = (m + BM - 1) / BM, gx = (n + BN - 1) / BN;
+    VIOLA_CHECK_ARG(gy <= 65535);
+    GemmArgs p = {};
+    p.a = static_cast<const uint8_t*>(a); p.b = static_cast<const uint8_t*>(b); p.sa = sa; p.sb = sb;
+    p.bias = bias; p.out = out; p.m = m; p.n = n; p.k = k; p.lda = k; p.ldb = k;
+    p.ldsa = (k + ak - 1) / ak; p.ldsb = (k + bk - 1) / bk; p.ldo = n;
+    p.ar = ar; p.br = br; p.ak_shift = shift_of(ak); p.bk_shift = shift_of(bk);
+    // the partial is cleared where the reference clears it: every gcd(a's K group, b's K group, accum_block) k
+    p.half_period = accum_block ? gcd_of(gcd_of(ak, bk), accum_block) : gcd_of(ak, bk);
+    p.reduce_bf16 = reduce_dtype == VIOLA_BF16;
+    return launch_half<1>(p, a_dtype, b_dtype, bias_dtype, out_dtype, br % 32 != 0, dim3((unsigned)gx, (unsigned)gy), stream);
+}
+
+extern "C" int viola_tensor_gemm_half(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,
+                                      int64_t m, int64_t n, int64_t k, const void* bias, int bias_dtype, void* out, int out_dtype,
+                                      int accum_block, int reduce_dtype, viola_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    VIOLA_CHECK_ARG(viola_is_fp8(a_dtype) && viola_is_fp8(b_dtype) && viola_is_float(out_dtype));
+    VIOLA_CHECK_ARG(m >= 0 && n >= 0 && k >= 0 && k < (1ll << 30) && (!bias || viola_is_float(bias_dtype)));
+    VIOLA_CHECK_ARG(accum_block >= 0 && accum_block % 32 == 0 && (reduce_dtype == VIOLA_F32 || reduce_dtype == VIOLA_BF16));
+    if (m == 0 || n == 0) return 0;
+    VIOLA_CHECK_ARG(out && sa && sb && (k == 0 || (a && b)));
+    const int64_t gy = (m + BM - 1) / BM, gx = (n + BN - 1) / BN;
+    VIOLA_CHECK_ARG(gy <= 65535);
+    GemmArgs p = {};
+    p.a = static_cast<const uint8_t*>(a); p.b = static_cast<const uint8_t*>(b); p.sa = sa; p.sb = sb;
+    p.bias = bias; p.out = out; p.m = m; p.n = n; p.k = k; p.lda = k; p.ldb = k; p.ldo = n;
+    p.ldsa = 0; p.ldsb = 0; p.ar = 1 << 30; p.br = 1 << 30; p.ak_shift = 30; p.bk_shift = 30;
+    // the reference's loop adds the partial to the total after whole chunks of 64 k (of accum_block k below that):
+    // viola/nn/_linear_kernels.py:150-153, :272-273
+    p.half_period = accum_block < 64 ? accum_block : accum_block / 64 * 64;
+    p.reduce_bf16 = reduce_dtype == VIOLA_BF16;
+    return launch_half<2>(p, a_dtype, b_dtype, bias_dtype, out_dtype, false, dim3((unsigned)gx, (unsigned)gy), stream);
 }
 
 // Large gated products run as the plain GEMM on 256 x 256 tiles plus one elementwise pass over its output: with one

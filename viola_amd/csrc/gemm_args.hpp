@@ -29,6 +29,9 @@ struct GemmArgs {
     // scales per 32 values, along its rows (enc [m, n], enc_scale [m, n / 32]) and along its columns
     // (enc_t [n, m], enc_t_scale [n, m / 32]; enc_t may be null); m and n are multiples of 32
     uint8_t* enc; uint8_t* enc_scale; uint8_t* enc_t; uint8_t* enc_t_scale; float enc_limit; int enc_bf8;
+    // FP16-accumulator model of the generic kernel (HALF != 0): k covered by one FP16 partial sum before it is added to
+    // the running total (0: the whole k range, no separate total), and whether that total is kept in bf16
+    int half_period; int reduce_bf16;
 };
 
 

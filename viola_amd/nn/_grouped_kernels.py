@@ -123,9 +123,11 @@ def transpose(q, scale, group, *, native=False, limit=None):
 
 def gemm(a, b, sa, sb, group_a, group_b, *, out_dtype, native=False, bias=None, autotune=False,
          accum_dtype="fp32", accum_block_size=0, accum_reduce_dtype="fp32"):
-    """out[m, n] = sum over 32-wide K groups of (a_codes . b_codes^T) * sa * sb (+ bias); a [m, k], b [n, k]."""
-    # the accumulation arguments select no other kernel: the FP8 MFMA sums in FP32, which meets the bound the
-    # reference holds its FP16 sums to (checks/check_grouped_linear.py:41)
+    """out[m, n] = sum over 32-wide K groups of (a_codes . b_codes^T) * sa * sb (+ bias); a [m, k], b [n, k].
+
+    accum_dtype="fp16" (FP32 scales only) takes the FP16-accumulator model of the reference's kernel: FP16 partial sums
+    per scale group, totals in accum_reduce_dtype. With FP32 accumulation the other two options change nothing (the
+    MFMA's sums are FP32 throughout)."""
     assert accum_dtype in ("fp32", "fp16") and accum_reduce_dtype in ("fp32", "bf16") and accum_block_size % 32 == 0
     assert a.is_cuda and b.is_cuda and a.shape[1] == b.shape[1]
     a, b, sa, sb = a.contiguous(), b.contiguous(), sa.contiguous(), sb.contiguous()
@@ -134,6 +136,13 @@ def gemm(a, b, sa, sb, group_a, group_b, *, out_dtype, native=False, bias=None, 
     assert tuple(sa.shape) == scale_shape((m, k), group_a) and tuple(sb.shape) == scale_shape((n, k), group_b)
     out = torch.empty((m, n), device=a.device, dtype=out_dtype)
     bias_c = bias.contiguous() if bias is not None else None
+    if accum_dtype == "fp16":
+        assert not native, "MXFP8 MMA uses FP32 accumulation."
+        _lib.call("viola_group_gemm_half", _lib.ptr(a), _lib.code(a.dtype), _lib.ptr(b), _lib.code(b.dtype), _lib.ptr(sa), _lib.ptr(sb),
+                  m, n, k, group_a[0], group_a[1], group_b[0], group_b[1], _lib.ptr(bias_c),
+                  _lib.code(bias_c.dtype) if bias_c is not None else 0, _lib.ptr(out), _lib.code(out_dtype), accum_block_size,
+                  _lib.BF16 if accum_reduce_dtype == "bf16" else _lib.F32)
+        return out
     if native:
         assert sa.dtype == torch.uint8 and sb.dtype == torch.uint8 and group_a[1] == 32 and group_b[1] == 32
         status = _lib.call("viola_mx_gemm", _lib.ptr(a), _lib.code(a.dtype), _lib.ptr(b), _lib.code(b.dtype), _lib.ptr(sa),

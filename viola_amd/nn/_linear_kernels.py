@@ -75,12 +75,18 @@ def quantize(x, scale, *, rowwise=True, transpose=False, fp8_dtype=torch.float8_
 
 def gemm(a, b, sa, sb, *, out_dtype, bias=None, autotune=False, accum_dtype="fp32", accum_block_size=0,
          accum_reduce_dtype="fp32"):
-    """(a * sa) @ (b * sb).T + bias with the scaling in the epilogue; a [m, k] and b [n, k] are FP8 codes."""
-    # the accumulation arguments select no other kernel: the FP8 MFMA sums in FP32
+    """(a * sa) @ (b * sb).T + bias with the scaling in the epilogue; a [m, k] and b [n, k] are FP8 codes.
+    accum_dtype="fp16" takes the FP16-accumulator model of the reference's kernel (FP16 partial sums over
+    accum_block_size k, totals in accum_reduce_dtype); with FP32 accumulation the other two options change nothing."""
     assert accum_dtype in ("fp32", "fp16") and accum_reduce_dtype in ("fp32", "bf16") and accum_block_size % 32 == 0
     assert a.is_cuda and a.is_contiguous() and b.is_contiguous() and a.shape[1] == b.shape[1]
     out = torch.empty((a.shape[0], b.shape[0]), device=a.device, dtype=out_dtype)
     has_bias = bias is not None and bias.numel() > 0
+    if accum_dtype == "fp16":
+        _lib.call("viola_tensor_gemm_half", _lib.ptr(a), _lib.code(a.dtype), _lib.ptr(b), _lib.code(b.dtype), _lib.ptr(sa), _lib.ptr(sb),
+                  a.shape[0], b.shape[0], a.shape[1], _lib.ptr(bias) if has_bias else None, _lib.code(bias.dtype) if has_bias else 0,
+                  _lib.ptr(out), _lib.code(out_dtype), accum_block_size, _lib.BF16 if accum_reduce_dtype == "bf16" else _lib.F32)
+        return out
     _lib.call("viola_tensor_gemm", _lib.ptr(a), _lib.code(a.dtype), _lib.ptr(b), _lib.code(b.dtype), _lib.ptr(sa), _lib.ptr(sb),
               a.shape[0], b.shape[0], a.shape[1], _lib.ptr(bias) if has_bias else None, _lib.code(bias.dtype) if has_bias else 0,
               _lib.ptr(out), _lib.code(out_dtype))

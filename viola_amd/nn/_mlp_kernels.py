@@ -25,6 +25,18 @@ def gemm(a, b, sa, sb, *, layer, out_dtype, activation, backward=False, aux=None
     a, b, sa, sb = a.contiguous(), b.contiguous(), sa.contiguous(), sb.contiguous()
     m, k = a.shape
     h = b.shape[0] if backward else b.shape[0] // 2
+    if getattr(layer, "accum_dtype", "fp32") == "fp16":
+        # the FP16-accumulator model exists for the plain product: the same values as a fused epilogue from the plain
+        # GEMM (which rounds g, u and d to out_dtype as the epilogue does) and the elementwise kernels
+        plain = (lambda bias_: layer._group_gemm(a, b, sa, sb, tuple(group_a or layer.input_group_shape),
+                                                 tuple(group_b or layer.weight_group_shape), out_dtype=out_dtype, bias=bias_)) \
+            if layer._grouped_scaling else (lambda bias_: layer._tensor_gemm(a, b, sa, sb, out_dtype=out_dtype, bias=bias_))
+        empty = torch.empty((0, 0), device=a.device, dtype=torch.uint8)
+        extra = (empty, a.new_empty((0, 0)), empty)
+        if backward:
+            return _gated_kernels.gated_backward(aux, plain(None), activation), aux, extra
+        z, out = _gated_kernels.gated_forward(plain(bias), activation)
+        return out, (z if save else z.new_empty((0, 0))), extra
     out = torch.empty((m, 2 * h if backward else h), device=a.device, dtype=out_dtype)
     if aux is None:
         aux = torch.empty((m, 2 * h) if save else (0, 0), device=a.device, dtype=out_dtype)

@@ -42,7 +42,7 @@ def forward_core(x, weight, bias, layer, need_backward, needs, *, gated=None):
     if gated:
         y, aux, _ = _mlp_kernels.gemm(qx, qw, sx, sw, layer=layer, out_dtype=x2.dtype, bias=bias, activation=gated, save=need_backward)
     else:
-        y = kernels.gemm(qx, qw, sx, sw, out_dtype=x2.dtype, bias=bias)
+        y = layer._tensor_gemm(qx, qw, sx, sw, out_dtype=x2.dtype, bias=bias)
     record = None
     if need_backward:
         if save_fp8:
@@ -89,7 +89,7 @@ def backward_core(record, tensors, dy, needs, *, gated=None, aux=None):
         if gated and not layer.rotation_size:
             dx, _, _ = _mlp_kernels.gemm(qg, wt, sg, sw, layer=layer, out_dtype=record.x_dtype, activation=gated, backward=True, aux=aux)
         else:
-            dx = kernels.gemm(qg, wt, sg, sw, out_dtype=record.x_dtype)
+            dx = layer._tensor_gemm(qg, wt, sg, sw, out_dtype=record.x_dtype)
             if layer.rotation_size:
                 rotation.inverse_(dx)
             if gated:
@@ -101,7 +101,7 @@ def backward_core(record, tensors, dy, needs, *, gated=None, aux=None):
             xt = saved_x
         else:
             _, xt = quantize(saved_x, sx, rowwise=False, transpose=True, fp8_dtype=fp8, quantization_limit=record.input_limit)
-        dw = kernels.gemm(qgt, xt, sg, sx, out_dtype=record.weight_grad_dtype)
+        dw = layer._tensor_gemm(qgt, xt, sg, sx, out_dtype=record.weight_grad_dtype)
         if layer.rotation_size:
             rotation.inverse_(dw)
     return dx, dw, db

@@ -5,13 +5,12 @@ gradient tile), `scaling="mxfp8"` (the same groups with E8M0 power-of-two scales
 MFMA) and the per-tensor recipes `scaling="current"` / `"delayed"` (one FP32 scale per tensor,
 delayed = the maximum of an amax history), e4m3 / e5m2 operand formats.
 
-Accumulation: the FP8 MFMA of gfx950 accumulates in FP32 and has no narrower accumulator, so
-`accum_dtype="fp16"`, `accum_block_size` and `accum_reduce_dtype="bf16"` (a speed / register knob of
-the reference's tensor-core kernels) change no GEMM here. What they change in the reference's DATA is
-kept: the quantization limits derived from them (linear.py:232-253), so codes and scales are the
-ones the reference stores, and the products are summed in FP32, inside the tolerance the reference
-checks its FP16 sums against (checks/check_grouped_linear.py:41,73). `rotation_size=64` (per-tensor recipes only)
-stores and multiplies Hadamard-rotated X and W.
+Accumulation: `accum_dtype="fp16"` (with `accum_block_size`, `accum_reduce_dtype`) is the reference's ablation of
+narrow accumulators. The quantization limits it implies (linear.py:232-253) are applied, so codes and scales are the
+ones the reference stores, and the GEMMs follow the FP16-accumulator model of its kernels: FP16 partial sums advanced
+every 32 k, cleared into an FP32 or BF16 total per scale group / accumulation block. The FP8 MFMA of gfx950 sums in
+FP32, so the model runs on the generic kernel with explicit roundings; with `accum_dtype="fp32"` the other two options
+change nothing. `rotation_size=64` (per-tensor recipes only) stores and multiplies Hadamard-rotated X and W.
 """
 
 import math
@@ -161,7 +160,13 @@ class Linear(nn.Module):
         return min(_half_sum_limit(self.accum_block_size or reduction), torch.finfo(fp8_dtype).max)
 
     def _group_gemm(self, a, b, sa, sb, ga, gb, *, out_dtype, bias=None):
-        return grouped.gemm(a, b, sa, sb, ga, gb, out_dtype=out_dtype, bias=bias, native=self._native_scaling)
+        return grouped.gemm(a, b, sa, sb, ga, gb, out_dtype=out_dtype, bias=bias, native=self._native_scaling,
+                            accum_dtype=self.accum_dtype, accum_block_size=self.accum_block_size,
+                            accum_reduce_dtype=self.accum_reduce_dtype)
+
+    def _tensor_gemm(self, a, b, sa, sb, *, out_dtype, bias=None):
+        return kernels.gemm(a, b, sa, sb, out_dtype=out_dtype, bias=bias, accum_dtype=self.accum_dtype,
+                            accum_block_size=self.accum_block_size, accum_reduce_dtype=self.accum_reduce_dtype)
 
     # ------------------------------------------------------------------ weights
     def _master(self):
