@@ -205,41 +205,60 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
     const i32x4 res_sa = raw_resource(p.sa, (p.m + p.ar - 1) / p.ar * p.ldsa * 4);
     const i32x4 res_sb = raw_resource(sbptr, (b_rows_total + p.br - 1) / p.br * p.ldsb * 4);
     constexpr uint32_t OUTSIDE = 0x80000000u;
-    uint32_t goff_a[2], goff_b[2];
-    int piece_k[2];
+    const int64_t k_len = k_end - k_begin;
+    const int groups_total = (int)((k_len + 31) / 32);
+    const int chunks = (int)((k_len + FBK - 1) / FBK);
+    const int full_chunks = (int)(k_len / FBK);                             // chunks wholly inside the k range
+    // Offsets of the thread's 16-byte pieces. Chunks wholly inside the k range use them as they are; for the one chunk
+    // that straddles the end of the range the pieces past it are redirected outside the buffer (they read zero), and
+    // for chunks past the range (issued to keep the load counts of the ring uniform) all of them are. `cur_*` holds
+    // what the next issue uses and is switched by retarget(), a wave-uniform branch taken at most twice per tile.
+    uint32_t goff_a[2], goff_b[2], tail_a[2], tail_b[2], cur_a[2], cur_b[2];
 #pragma unroll
     for (int it = 0; it < 2; ++it) {
         const int unit = it * THREADS + tid, r = unit >> 2, piece = (unit & 3) ^ ((r >> 2) & 3);
-        goff_a[it] = (uint32_t)((a_global_row(r) - m_begin) * p.lda + piece * 16);
-        goff_b[it] = (uint32_t)(b_global_row(r) * p.ldb + piece * 16);        // relative to bptr + k_begin (row span < 2 GiB)
-        piece_k[it] = piece * 16;
+        goff_a[it] = (uint32_t)(a_global_row(r) - m_begin) * (uint32_t)p.lda + piece * 16;   // tile rows x lda < 4 GiB (checked by the launcher)
+        goff_b[it] = (uint32_t)b_global_row(r) * (uint32_t)p.ldb + piece * 16;   // relative to bptr + k_begin (row span < 2 GiB)
+        const bool inside_tail = (int64_t)full_chunks * FBK + piece * 16 < k_len;
+        tail_a[it] = inside_tail ? goff_a[it] : OUTSIDE;
+        tail_b[it] = inside_tail ? goff_b[it] : OUTSIDE;
+        cur_a[it] = goff_a[it];
+        cur_b[it] = goff_b[it];
     }
+    auto retarget = [&](int c) {                                             // before the loads of chunk c are issued
+        if (__builtin_expect(c >= full_chunks, 0)) {
+            asm volatile("; end of the k range");                           // keeps this a branch, not per-chunk selects
+            const bool straddles = c == full_chunks;
+#pragma unroll
+            for (int it = 0; it < 2; ++it) {
+                cur_a[it] = straddles ? tail_a[it] : OUTSIDE;
+                cur_b[it] = straddles ? tail_b[it] : OUTSIDE;
+            }
+        }
+    };
     // scales: per block of 8 K groups the thread fetches groups 4 shalf .. 4 shalf + 3 of tile row srow
     const int srow = tid % BM, shalf = tid / BM;
     const uint32_t sa_off = (uint32_t)(a_global_row(srow) / p.ar * p.ldsa * 4 + ((k_begin >> 5) + shalf * 4) * 4);
     const uint32_t sb_off = (uint32_t)(b_global_row(srow) / p.br * p.ldsb * 4 + ((k_begin >> 5) + shalf * 4) * 4);
     constexpr int B_LOADS = TN;                                              // 64 b rows per load instruction
-    const int64_t k_len = k_end - k_begin;
-    const int groups_total = (int)((k_len + 31) / 32);
-    const int64_t chunks = (k_len + FBK - 1) / FBK;
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
     // load instruction `which` (0, 1: a; 2, 3: b) of chunk c into ring stage `stage`
-    auto issue_one = [&](int64_t c, int stage, int which) {
-        const int64_t k0 = c * FBK;                                          // relative to k_begin
+    auto issue_one = [&](int c, int stage, int which) {
+        const uint32_t k0 = (uint32_t)c * FBK;                               // relative to k_begin
         const uint32_t base = lds_base + (uint32_t)stage * K_STAGE + (uint32_t)wave * 1024;
         const int it = which & 1;
-        const bool inside = k0 + piece_k[it] < k_len;
-        if (which < 2) load16_to_lds(res_a, base + it * THREADS * 16, inside ? goff_a[it] : OUTSIDE, (uint32_t)k0);
-        else load16_to_lds(res_b, base + K_TILE_A + it * THREADS * 16, inside ? goff_b[it] : OUTSIDE, (uint32_t)k0);
+        if (which < 2) load16_to_lds(res_a, base + it * THREADS * 16, cur_a[it], k0);
+        else load16_to_lds(res_b, base + K_TILE_A + it * THREADS * 16, cur_b[it], k0);
     };
     constexpr int CHUNK_LOADS = 2 + B_LOADS;
-    auto issue = [&](int64_t c, int stage) {
+    auto issue = [&](int c, int stage) {
+        retarget(c);
 #pragma unroll
         for (int i = 0; i < CHUNK_LOADS; ++i) issue_one(c, stage, i);
     };
     // scale block `block` (K groups 8 block .. 8 block + 7 of the k range) -> raw area, one 16-byte piece per thread
     // and operand; a piece wholly past the k range is not fetched
-    auto issue_scales = [&](int64_t block) {
+    auto issue_scales = [&](int block) {
         const bool inside = block * F_SGROUPS + shalf * 4 < groups_total;
         const uint32_t at = lds_base + F_RAW + (uint32_t)wave * 1024;
         load16_to_lds(res_sa, at, inside ? sa_off : OUTSIDE, (uint32_t)(block * F_SGROUPS * 4));
@@ -250,14 +269,14 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
     const i32x4 res_mxb = raw_resource(sbptr, (b_rows_total + p.br - 1) / p.br * p.ldsb);
     const uint32_t mx_off = tid < TBM ? (uint32_t)(a_global_row(tid) / p.ar * p.ldsa + (k_begin >> 5))
                                       : (uint32_t)(b_global_row(tid - TBM) / p.br * p.ldsb + (k_begin >> 5));
-    auto issue_mx_scales = [&](int64_t block) {
+    auto issue_mx_scales = [&](int block) {
         const bool inside = block * MX_GROUPS < groups_total;
         const uint32_t at = lds_base + K_RAW + (uint32_t)(block & 1) * K_MX_BLOCK + (uint32_t)wave * 1024;
         load16_to_lds(wave < TBM / 64 ? res_mxa : res_mxb, at, inside ? mx_off : OUTSIDE, (uint32_t)(block * MX_GROUPS));
     };
     // raw area -> [group][row] floats of scale buffer `block & 1`; groups past the k range become zero (their
     // products are zero too, and a neighbouring row's value must not meet them)
-    auto arrange_scales = [&](int64_t block) {
+    auto arrange_scales = [&](int block) {
         const float4 va = *reinterpret_cast<const float4*>(lds + F_RAW + tid * 16);
         const float4 vb = *reinterpret_cast<const float4*>(lds + F_RAW + F_SBLOCK + tid * 16);
         float* ta = reinterpret_cast<float*>(lds + F_SCALE + (block & 1) * 2 * F_SBLOCK);
@@ -304,10 +323,10 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
         i32x8 wide_a[TM], wide_b[TN];                                        // TENSOR / MX: 16 k of either K group of a sub-tile row
         int mx_a[(TM + 1) / 2], mx_b[(TN + 1) / 2];                          // MX: the rows' scale bytes of K group lhi, sub-tile t in byte 2 (t & 1) of word t / 2
     };
-    auto scale_block = [&](int64_t c) -> const float* {                      // a scales of chunk c: [kg][row]; b scales F_SBLOCK later
+    auto scale_block = [&](int c) -> const float* {                      // a scales of chunk c: [kg][row]; b scales F_SBLOCK later
         return reinterpret_cast<const float*>(lds + F_SCALE + ((c / F_SCHUNKS) & 1) * 2 * F_SBLOCK) + (c % F_SCHUNKS) * FKG * BM;
     };
-    auto read_operands = [&](int stage, int64_t c, Operands& o) {
+    auto read_operands = [&](int stage, int c, Operands& o) {
         const uint8_t* tile_a = lds + stage * K_STAGE;
         const uint8_t* tile_b = tile_a + K_TILE_A;
         const float* scale_a = scale_block(c);
@@ -369,7 +388,7 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
 
     // Math of chunk c on the operands in `o`; `between(step)` runs after MFMA number `step` of the chunk (the
     // caller's global loads and LDS reads for later chunks go there, spread over the chunk).
-    auto compute = [&](const Operands& o, int64_t c, auto&& between) {
+    auto compute = [&](const Operands& o, int c, auto&& between) {
         if constexpr (NOFOLD) {
             constexpr int STEPS_PER = FKG * 2;
 #pragma unroll
@@ -466,7 +485,7 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
     // waits below cover it one iteration later.
     constexpr int STEPS = FKG * TN * TM * 2, STRIDE = STEPS / CHUNK_LOADS;
     int stage_now = 0, stage_next = 1;
-    auto chunk_step = [&](int64_t c, const Operands& now, Operands& next) {
+    auto chunk_step = [&](int c, const Operands& now, Operands& next) {
         constexpr int AHEAD = (K_STAGES - 2) * CHUNK_LOADS;                  // loads of the chunks after c + 1 may still be in flight
         static_assert(AHEAD + 2 < 16 && (K_STAGES - 1) * CHUNK_LOADS < 16, "the counts fit the wait instruction's low field");
         if (!NOFOLD && c % F_SCHUNKS == 1) __builtin_amdgcn_s_waitcnt(0x0070 | (AHEAD + 2));
@@ -481,6 +500,7 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
             if (c % MX_CHUNKS == 0) issue_mx_scales(c / MX_CHUNKS + 1);
         }
         if (c + 1 < chunks) read_operands(stage_next, c + 1, next);
+        retarget(c + K_STAGES);
         const int fill = stage_now;
         compute(now, c, [&](int step) {
             if (step % STRIDE == 0 && step / STRIDE < CHUNK_LOADS) issue_one(c + K_STAGES, fill, step / STRIDE);
@@ -500,7 +520,7 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
     }
     Operands set0, set1;
     read_operands(0, 0, set0);
-    for (int64_t c = 0; c < chunks; c += 2) {
+    for (int c = 0; c < chunks; c += 2) {
         chunk_step(c, set0, set1);
         if (c + 1 < chunks) chunk_step(c + 1, set1, set0);
     }
