@@ -33,10 +33,11 @@ PEAK = {"fp8_tflops": 5000.0, "bf16_tflops": 2500.0, "hbm_gbs": 8000.0}
 # dispatch), each scaled by the same counter's reading for the 256 MiB copy_scaled_kernel launch (factors 2.00 and 1.00):
 # fetch (2 * 62.2 + 124.7) / 3 MB, write (2 * 41.9 + 8.4) / 3 MB. The algorithmic figure is 65 MB per launch.
 GEMM_TRAFFIC_BYTES = 83.0e6 + 30.8e6
-# What the grouped-scale recipe can reach at all on this part: per 32-k group and 32 x 32 sub-tile the SIMD issues two
-# K = 16 FP8 MFMAs (64 matrix-pipe cycles) and 16 FP32 FMAs; MFMA and VALU share the issue port, >= 72 issue cycles per
-# 64 of matrix work, on MFMAs that run at half the f8f6f4 rate: 2.5 PFLOP/s x 64 / 72 at the 2.4 GHz boost clock.
-GEMM_ATTAINABLE_TFLOPS = 2500.0 * 64 / 72
+# Per 64-k chunk a wavefront of the grouped-scale GEMM issues 16 K = 16 FP8 MFMAs and, through the same port, the 128
+# FP32 FMAs that fold their sums into the totals (one FMA per accumulator and 32-k group). What that costs on the
+# machine is measured in the run itself by viola_probe_chunk_loop (chunk_loop_probe below).
+PROBE_PARTS = {"math": 0, "math_lds_reads": 1, "math_loads": 4, "all": 7}
+PROBE_CHUNKS, PROBE_BLOCKS, PROBE_LDA = 2048, 512, 4096
 
 
 WARM_MS = 100.0
@@ -78,6 +79,28 @@ def timed(fn, steps, warmup, warm=True):
     torch.cuda.synchronize()
     wall = (time.perf_counter() - begin) * 1e3
     return max(start.elapsed_time(end), 0.0) / steps, wall / steps
+
+
+def chunk_loop_probe():
+    """Time per 64-k chunk of the grouped-scale GEMM's instruction mix with nothing else in the way (two 256-thread
+    blocks per CU on all 256 CUs, like the GEMM), for the math alone, with the LDS operand reads, with the global ->
+    LDS loads, and with both plus the barrier. A 128 x 128 tile does 2 * 128 * 128 * 64 flops per chunk."""
+    import torch
+    from viola_amd import _lib
+    out = torch.empty(PROBE_BLOCKS * 256, device="cuda")
+    src = torch.randint(0, 255, (72 * 128 * PROBE_LDA,), device="cuda", dtype=torch.uint8)
+    result = {}
+    for name, parts in PROBE_PARTS.items():
+        def run():
+            _lib.call("viola_probe_chunk_loop", parts, _lib.ptr(out), _lib.ptr(src), src.numel(), PROBE_BLOCKS, PROBE_CHUNKS, PROBE_LDA)
+        ms, _ = timed(run, 5, 2, warm=False)
+        result[name + "_us_per_chunk"] = ms * 1e3 / PROBE_CHUNKS
+    flops_per_chunk = 2 * 128 * 128 * 64 * PROBE_BLOCKS
+    result["all_tflops"] = flops_per_chunk / (result["all_us_per_chunk"] * 1e-6) / 1e12
+    result["math_tflops"] = flops_per_chunk / (result["math_us_per_chunk"] * 1e-6) / 1e12
+    result["note"] = ("viola_probe_chunk_loop: the GEMM kernel's chunk loop (16 MFMA 32x32x16 fp8 + 128 FMA + 8 scale products per "
+                      "wavefront and chunk) without a GEMM around it, 512 blocks x 2048 chunks")
+    return result
 
 
 def kernel_breakdown(fn, steps):
@@ -285,13 +308,18 @@ def main():
     breakdown = kernel_breakdown(step, args.steps)
     gemm = breakdown["viola_group_gemm"]
     gemm_tflops = 2 * M * K * N / (gemm["avg_ms"] * 1e-3) / 1e12
+    log("chunk loop probe")
+    probe = chunk_loop_probe()
     roofline = dict(bound="mfma", kernel="group_gemm_fast (viola_group_gemm: fwd, dgrad, wgrad)",
                     achieved=gemm_tflops, peak=PEAK["fp8_tflops"], unit="TFLOP/s", frac=gemm_tflops / PEAK["fp8_tflops"],
                     avg_launch_ms=gemm["avg_ms"], traffic=GEMM_TRAFFIC_BYTES,
                     traffic_source="stored calibration (two rocprofv3 --pmc runs, profiles/linear_step_8192x1024x4096_hbm_traffic.txt), not read in this run",
-                    attainable=GEMM_ATTAINABLE_TFLOPS,
-                    attainable_note="issue-bound ceiling of an FP32 scale per 32 k: the K = 16 FP8 MFMAs (half the f8f6f4 rate) plus one "
-                                    "FP32 FMA per accumulator and K group through the same issue port; frac stays against the 5 PFLOP/s peak")
+                    attainable=probe["all_tflops"],
+                    attainable_note="measured in this run (chunk_loop_probe): the rate at which this machine runs the kernel's own "
+                                    "instruction mix (K = 16 FP8 MFMAs, one FP32 FMA per accumulator and 32-k group through the same issue "
+                                    "port, LDS operand reads, global -> LDS loads, one barrier per chunk) with nothing else in the way; "
+                                    "the math alone, without operand traffic, runs at chunk_loop_probe.math_tflops; frac stays against "
+                                    "the 5 PFLOP/s peak")
     quant = {}
     if "viola_group_quantize_dual" in breakdown:
         # X [M, K] and dY [M, N] each once per step: 4.25 B per element (bf16 in, two FP8 layouts + scales out)
@@ -460,7 +488,7 @@ def main():
         "config": {"workload": "viola.nn.Linear(1024, 4096, scaling='grouped', e4m3/e4m3, fp8 weight storage, mode='memory') "
                                "forward+backward on 8192 tokens, bf16 activations and gradients"},
         "frac_of_fp8_peak": value / PEAK["fp8_tflops"],
-        "roofline": roofline, "quantize": quant, "kernels": breakdown, **extra,
+        "roofline": roofline, "chunk_loop_probe": probe, "quantize": quant, "kernels": breakdown, **extra,
     }
     if not args.skip_cpu:
         log("CPU baselines")

@@ -360,6 +360,19 @@ int viola_selftest_fp8(uint64_t* counts, viola_stream_t stream);
 /* philox(element, step, key) word 0 for `count` triples (device arrays) -> out. */
 int viola_selftest_philox(const uint64_t* triples, uint32_t* out, int64_t count, viola_stream_t stream);
 
+
+/* ---------------------------------------------------------------- issue-rate probe (measurement support)
+ * No counterpart in the reference. Runs the chunk loop of the grouped-scale FP8 GEMM without a GEMM around it: per
+ * 64-k chunk and wavefront 16 v_mfma_f32_32x32x16_fp8_fp8, the 128 FP32 FMAs that fold them into the totals and 8
+ * scale products, in blocks of 256 threads, two to a CU. `parts` switches on what a real chunk adds: bit 0 the LDS
+ * reads of the next chunk's operands and scales, bit 1 the barrier, bit 2 the wavefront's four global -> LDS loads
+ * (src: a byte matrix of 72 x 128 rows with row stride lda, a multiple of 64; 16-byte aligned; may be NULL without
+ * bit 2). Timing a launch of `blocks` blocks over `chunks` (even) chunks gives the time per chunk this instruction mix
+ * needs when nothing else is in the way; bench.py derives the GEMM's attainable rate from it. out: blocks * 256 floats
+ * of no meaning. */
+int viola_probe_chunk_loop(int parts, float* out, const void* src, int64_t src_bytes, int blocks, int chunks, int lda,
+                           viola_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -64,6 +64,7 @@ _SIGNATURES = {
     "viola_comm_unpack": [_p, _p, _l, _l, _l, _i, _i, _i, _p],
     "viola_selftest_fp8": [_p, _p],
     "viola_selftest_philox": [_p, _p, _l, _p],
+    "viola_probe_chunk_loop": [_i, _p, _p, _l, _i, _i, _i, _p],
 }
 EXPORTS = tuple(_SIGNATURES) + ("viola_abi_version", "viola_error_string")
 
