@@ -98,6 +98,14 @@ template <> struct Quad<f16_t> {
     }
 };
 
+// A finished 16-byte piece of the output, stored with the streaming hint: nothing in this launch reads it again, and
+// kept out of the way it does not push the operand panels that the tiles of an XCD share out of its L2 (8192 x 4096 x
+// 1024 with a 64 MB output: 85 -> 80 us).
+__device__ __forceinline__ void store_streaming(void* p, uint4 piece) {
+    const i32x4 v = {(int)piece.x, (int)piece.y, (int)piece.z, (int)piece.w};
+    __builtin_nontemporal_store(v, static_cast<i32x4*>(p));
+}
+
 template <typename TO> __device__ __forceinline__ float rounded(float v) { return to_f32(from_f32<TO>(v)); }
 
 // TN: 32-column sub-tiles per wave; TN = 1 halves the tile to 128 x 64 for problems with too few 128 x 128 tiles to
@@ -594,7 +602,7 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
                     const uint4 piece = *reinterpret_cast<const uint4*>(&park[pr * PLD + pc * PER]);
                     if (mrow >= m_end || ncol >= p.n) continue;
                     if (ncol + PER <= p.n) {
-                        *reinterpret_cast<uint4*>(out + mrow * p.ldo + ncol) = piece;
+                        store_streaming(out + mrow * p.ldo + ncol, piece);
                     } else {
                         const TO* values = reinterpret_cast<const TO*>(&piece);
                         for (int e = 0; e < PER; ++e)
@@ -640,7 +648,7 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
                     const int id = it * WAVE + lane, pr = id / PIECES, pc = id % PIECES;
                     const int64_t mrow = row0 + pr, ncol = col0 + pc * PER;
                     const uint4 piece = *reinterpret_cast<const uint4*>(&park[pr * PLD + pc * PER]);
-                    if (mrow < m_end && ncol < p.n) *reinterpret_cast<uint4*>(dst + mrow * ld + ncol) = piece;
+                    if (mrow < m_end && ncol < p.n) store_streaming(dst + mrow * ld + ncol, piece);
                 }
             };
             auto fetch = [&](TO* park, const TO* src, int64_t ld, int64_t row0, int64_t col0) {
