@@ -237,6 +237,8 @@ def ns_single_case(steps, warmup):
         out[method] = dict(ms=ms, tflops=NS_C1_FLOPS[method] / (ms * 1e-3) / 1e12, gemm_launches=b["viola_ns_gemm"]["launches_per_step"],
                            gemm_ms=gemm_ms, gemm_tflops=NS_C1_FLOPS[method] / (gemm_ms * 1e-3) / 1e12,
                            gemm_frac_peak=NS_C1_FLOPS[method] / (gemm_ms * 1e-3) / 1e12 / PEAK["bf16_tflops"])
+    out["note"] = ("gemm_ms sums HIP-event pairs around 15-18 launches of 5-18 us each in a second, instrumented pass: the pairs' own "
+                   "cost makes it exceed ms, the chain timed without them")
     return out
 
 
