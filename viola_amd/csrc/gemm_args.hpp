@@ -25,6 +25,9 @@ struct GemmArgs {
     // fast kernel only: 1-D grid of tiles_m * tiles_n output tiles (rounded up to a multiple of 8) walked in an
     // XCD-aware order; tiles_m == 0 keeps the plain (blockIdx.x, blockIdx.y) = (n tile, m tile) mapping
     int tiles_m, tiles_n;
+    // fast kernel only, filled in by its launchers: bytes of the two scale arrays (a 16-byte piece may reach past the
+    // last scale row and must then read zero, so their buffer descriptors carry the true size)
+    int64_t sa_bytes, sb_bytes;
     // MX gated forward only: when enc is set, h is not written to out but quantized in the epilogue with E8M0
     // scales per 32 values, along its rows (enc [m, n], enc_scale [m, n / 32]) and along its columns
     // (enc_t [n, m], enc_t_scale [n, m / 32]; enc_t may be null); m and n are multiples of 32

@@ -32,6 +32,9 @@ static int launch_mode(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dty
 int launch_group_gemm_fast(const GemmArgs& args, int mode, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, bool rowscale,
                            dim3 grid, hipStream_t stream) {
     GemmArgs p = args;
+    const int64_t b_rows = mode == MODE_GATED_FWD ? 2 * p.n : p.n;
+    p.sa_bytes = (p.m + p.ar - 1) / p.ar * p.ldsa * 4;
+    p.sb_bytes = (b_rows + p.br - 1) / p.br * p.ldsb * 4;
     // Two blocks fit a CU: with fewer than 512 tiles of 128 x 128, halve the tile in n so that all 256 CUs get two.
     const bool narrow = mode == MODE_PLAIN && (int64_t)grid.x * grid.y * grid.z < 512 && p.n > 64;
     if (narrow) grid.x = (unsigned)((p.n + 63) / 64);

@@ -210,8 +210,8 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
     const i32x4 res_a = raw_resource(p.a + m_begin * p.lda + k_begin);
     const i32x4 res_b = raw_resource(bptr + k_begin);
     // scale buffers carry their true size: a 16-byte piece may reach past the last row, and must then read zero
-    const i32x4 res_sa = raw_resource(p.sa, (p.m + p.ar - 1) / p.ar * p.ldsa * 4);
-    const i32x4 res_sb = raw_resource(sbptr, (b_rows_total + p.br - 1) / p.br * p.ldsb * 4);
+    const i32x4 res_sa = raw_resource(p.sa, p.sa_bytes);
+    const i32x4 res_sb = raw_resource(sbptr, p.sb_bytes);
     constexpr uint32_t OUTSIDE = 0x80000000u;
     const int64_t k_len = k_end - k_begin;
     const int groups_total = (int)((k_len + 31) / 32);
@@ -246,8 +246,9 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
     };
     // scales: per block of 8 K groups the thread fetches groups 4 shalf .. 4 shalf + 3 of tile row srow
     const int srow = tid % BM, shalf = tid / BM;
-    const uint32_t sa_off = (uint32_t)(a_global_row(srow) / p.ar * p.ldsa * 4 + ((k_begin >> 5) + shalf * 4) * 4);
-    const uint32_t sb_off = (uint32_t)(b_global_row(srow) / p.br * p.ldsb * 4 + ((k_begin >> 5) + shalf * 4) * 4);
+    // (row indices and scale offsets fit 31 bits, the launcher sees to it: 32-bit division, not the 64-bit routine)
+    const uint32_t sa_off = (uint32_t)a_global_row(srow) / (uint32_t)p.ar * (uint32_t)p.ldsa * 4 + (uint32_t)((k_begin >> 5) + shalf * 4) * 4;
+    const uint32_t sb_off = (uint32_t)b_global_row(srow) / (uint32_t)p.br * (uint32_t)p.ldsb * 4 + (uint32_t)((k_begin >> 5) + shalf * 4) * 4;
     constexpr int B_LOADS = TN;                                              // 64 b rows per load instruction
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
     // load instruction `which` (0, 1: a; 2, 3: b) of chunk c into ring stage `stage`
@@ -273,10 +274,10 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
         load16_to_lds(res_sb, at + F_SBLOCK, inside ? sb_off : OUTSIDE, (uint32_t)(block * F_SGROUPS * 4));
     };
     // MX: scale block `block` (K groups 16 block ..) -> buffer block & 1: waves 0, 1 fetch the a rows' pieces, waves 2, 3 the b rows'
-    const i32x4 res_mxa = raw_resource(p.sa, (p.m + p.ar - 1) / p.ar * p.ldsa);
-    const i32x4 res_mxb = raw_resource(sbptr, (b_rows_total + p.br - 1) / p.br * p.ldsb);
-    const uint32_t mx_off = tid < TBM ? (uint32_t)(a_global_row(tid) / p.ar * p.ldsa + (k_begin >> 5))
-                                      : (uint32_t)(b_global_row(tid - TBM) / p.br * p.ldsb + (k_begin >> 5));
+    const i32x4 res_mxa = raw_resource(p.sa, p.sa_bytes);
+    const i32x4 res_mxb = raw_resource(sbptr, p.sb_bytes);
+    const uint32_t mx_off = tid < TBM ? (uint32_t)a_global_row(tid) / (uint32_t)p.ar * (uint32_t)p.ldsa + (uint32_t)(k_begin >> 5)
+                                      : (uint32_t)b_global_row(tid - TBM) / (uint32_t)p.br * (uint32_t)p.ldsb + (uint32_t)(k_begin >> 5);
     auto issue_mx_scales = [&](int block) {
         const bool inside = block * MX_GROUPS < groups_total;
         const uint32_t at = lds_base + K_RAW + (uint32_t)(block & 1) * K_MX_BLOCK + (uint32_t)wave * 1024;

@@ -46,6 +46,12 @@ template <bool TENSOR, bool MX>
 static int launch_scaled_gemm_fast(const GemmArgs& args, int mode, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, dim3 grid,
                                    hipStream_t stream) {
     GemmArgs p = args;
+    {
+        // MX: the scale arrays hold bytes; per-tensor scales are read directly, not through these descriptors
+        const int64_t b_rows = mode == MODE_GATED_FWD ? 2 * p.n : p.n;
+        p.sa_bytes = (p.m + p.ar - 1) / p.ar * p.ldsa;
+        p.sb_bytes = (b_rows + p.br - 1) / p.br * p.ldsb;
+    }
     // a gated forward tile is 128 columns of h wide (its 256 b rows are 128 gate and 128 up rows)
     const int64_t big_width = mode == MODE_GATED_FWD ? 128 : 256;
     const int64_t big_m = (p.m + 255) / 256, big_n = (p.n + big_width - 1) / big_width;
