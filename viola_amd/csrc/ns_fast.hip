@@ -291,6 +291,21 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void ns_gemm_fast(NsArgs
         bits = ns_narrow<IS_BF16>(value);
         dbits = diagonal ? ns_narrow<IS_BF16>(ns_widen<IS_BF16>((uint16_t)bits) + p.add_diag) : bits;
     };
+    // The residual pieces of the [m, n] placement are fetched one 32-row block ahead: the loads of block j + 1 leave
+    // before block j is finished and stored, so that a wavefront waits for memory once per block and not once per piece.
+    constexpr int ROW_ITERS = 32 * PIECES / WAVE;
+    uint4 ahead[2][ROW_ITERS];
+    auto fetch_residual = [&](int j, uint4 (&pieces)[ROW_ITERS]) {
+        const int64_t row0 = m0 + wm * 32 * WM + j * 32, col0 = n0 + wn * WCOLS;
+#pragma unroll
+        for (int it = 0; it < ROW_ITERS; ++it) {
+            const int id = it * WAVE + lane, pr = id / PIECES, pc = id % PIECES;
+            const int64_t row = row0 + pr, col = col0 + pc * 8;
+            // a piece outside the matrix reads the first one instead (its value is not used)
+            pieces[it] = *reinterpret_cast<const uint4*>(residual + (row < m && col < n ? row * n + col : 0));
+        }
+    };
+    if (EPILOGUE && !p.transpose_out) fetch_residual(0, ahead[0]);
 #pragma unroll
     for (int j = 0; j < WM; ++j) {
 #pragma unroll
@@ -304,14 +319,15 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void ns_gemm_fast(NsArgs
             }
         const int64_t row0 = m0 + wm * 32 * WM + j * 32, col0 = n0 + wn * WCOLS;   // of the parked 32 x WCOLS block
         if (!p.transpose_out) {
+            if (EPILOGUE && j + 1 < WM) fetch_residual(j + 1, ahead[(j + 1) & 1]);
 #pragma unroll
-            for (int it = 0; it < 32 * PIECES / WAVE; ++it) {
+            for (int it = 0; it < ROW_ITERS; ++it) {
                 const int id = it * WAVE + lane, pr = id / PIECES, pc = id % PIECES;
                 const int64_t row = row0 + pr, col = col0 + pc * 8;
                 const uint4 raw = *reinterpret_cast<const uint4*>(&park[pr * PLD + pc * 8]);
                 if (row >= m || col >= n) continue;                       // n is a multiple of 8: whole pieces
                 uint4 res = make_uint4(0, 0, 0, 0);
-                if (EPILOGUE) res = *reinterpret_cast<const uint4*>(residual + row * n + col);
+                if (EPILOGUE) res = ahead[j & 1][it];
                 const uint32_t pw[4] = {raw.x, raw.y, raw.z, raw.w}, rw[4] = {res.x, res.y, res.z, res.w};
                 uint32_t o[4], od[4];
 #pragma unroll
