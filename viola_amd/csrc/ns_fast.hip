@@ -57,6 +57,17 @@ template <bool IS_BF16> __device__ __forceinline__ uint16_t ns_narrow(float v) {
     if constexpr (IS_BF16) return f32_to_bf16_bits(v);
     else { _Float16 h = (_Float16)v; uint16_t bits; __builtin_memcpy(&bits, &h, 2); return bits; }
 }
+// the same conversions on two neighbouring elements packed in 32 bits (low half first)
+typedef _Float16 ns_f16x2 __attribute__((ext_vector_type(2)));
+typedef float ns_f32x2 __attribute__((ext_vector_type(2)));
+template <bool IS_BF16> __device__ __forceinline__ void ns_widen2(uint32_t pair, float& lo, float& hi) {
+    if constexpr (IS_BF16) { lo = __uint_as_float(pair << 16); hi = __uint_as_float(pair & 0xffff0000u); }
+    else { const ns_f16x2 h = __builtin_bit_cast(ns_f16x2, pair); lo = (float)h.x; hi = (float)h.y; }
+}
+template <bool IS_BF16> __device__ __forceinline__ uint32_t ns_narrow2(float lo, float hi) {
+    if constexpr (IS_BF16) return f32_to_bf16x2_bits(lo, hi);
+    else { const ns_f32x2 pair = {lo, hi}; return __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, ns_f16x2)); }
+}
 
 // 64 lanes x 16 bytes from a raw buffer straight into LDS at lds_addr + 16 * lane. The compiler is
 // not told that this touches LDS (it would drain every outstanding load before each LDS read); the
@@ -272,9 +283,18 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void ns_gemm_fast(NsArgs
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);     // drain the trailing loads before the LDS allocation is released
 
+    // Element offsets inside one matrix fit 32 bits (the launcher checks it): the pieces below are addressed as a
+    // per-matrix base, the same for every lane, plus a 32-bit byte offset.
     const uint16_t* residual = EPILOGUE ? p.residual + bz * m * n : nullptr;
     uint16_t* out = p.out + bz * m * n;
     uint16_t* out_diag = p.out_diag ? p.out_diag + bz * m * n : nullptr;
+    const uint32_t um = (uint32_t)m, un = (uint32_t)n;
+    auto load_piece = [](const uint16_t* base, uint32_t element) -> uint4 {
+        return *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(base) + (size_t)(element * 2u));
+    };
+    auto store_piece = [](uint16_t* base, uint32_t element, uint4 piece) {
+        *reinterpret_cast<uint4*>(reinterpret_cast<char*>(base) + (size_t)(element * 2u)) = piece;
+    };
     // The accumulators hold one row per lane in runs of four columns, which as stores would touch 32 cache lines per
     // instruction. Each wavefront instead parks its rounded products, 32 rows at a time, in LDS (the stage ring is free
     // now) and picks them up as 16-byte pieces: along the rows for the [m, n] placement, so that the residual loads, the
@@ -284,25 +304,39 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void ns_gemm_fast(NsArgs
     static_assert(WAVES_M * WAVES_N * 32 * PLD * 2 <= (int)sizeof(lds), "parking area fits in the stage ring");
     __syncthreads();                                                      // every wave has left the ring
     uint16_t* park = lds + wave * 32 * PLD;
-    auto finish = [&](uint16_t product, float r, bool diagonal, uint32_t& bits, uint32_t& dbits) {
-        float value = ns_widen<IS_BF16>(product);
-        if (EPILOGUE == 1) value = -4.7750f * r + 2.0315f * value;
-        if (EPILOGUE == 2) value = value + 3.4445f * r;
-        bits = ns_narrow<IS_BF16>(value);
-        dbits = diagonal ? ns_narrow<IS_BF16>(ns_widen<IS_BF16>((uint16_t)bits) + p.add_diag) : bits;
+    // two neighbouring elements at a time: the rounded products and the residual as packed pairs in, the result pair out
+    auto finish = [&](uint32_t products, uint32_t residuals) -> uint32_t {
+        if (EPILOGUE == 0) return products;                               // widening and narrowing a rounded value again changes nothing
+        float v0, v1, r0, r1;
+        ns_widen2<IS_BF16>(products, v0, v1);
+        ns_widen2<IS_BF16>(residuals, r0, r1);
+        if (EPILOGUE == 1) { v0 = -4.7750f * r0 + 2.0315f * v0; v1 = -4.7750f * r1 + 2.0315f * v1; }
+        if (EPILOGUE == 2) { v0 = v0 + 3.4445f * r0; v1 = v1 + 3.4445f * r1; }
+        return ns_narrow2<IS_BF16>(v0, v1);
+    };
+    // the second copy: element `at` of the piece (the one on the diagonal) gets add_diag
+    auto with_diagonal = [&](uint4 piece, uint32_t at) -> uint4 {
+        uint32_t w[4] = {piece.x, piece.y, piece.z, piece.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            if (at == (uint32_t)e) {
+                const uint32_t bits = ns_narrow<IS_BF16>(ns_widen<IS_BF16>((uint16_t)(w[e / 2] >> (16 * (e % 2)))) + p.add_diag);
+                w[e / 2] = (w[e / 2] & ~(0xffffu << (16 * (e % 2)))) | (bits << (16 * (e % 2)));
+            }
+        return make_uint4(w[0], w[1], w[2], w[3]);
     };
     // The residual pieces of the [m, n] placement are fetched one 32-row block ahead: the loads of block j + 1 leave
     // before block j is finished and stored, so that a wavefront waits for memory once per block and not once per piece.
     constexpr int ROW_ITERS = 32 * PIECES / WAVE;
     uint4 ahead[2][ROW_ITERS];
+    const uint32_t tile_row = (uint32_t)m0 + wm * 32 * WM, col0 = (uint32_t)n0 + wn * WCOLS;
     auto fetch_residual = [&](int j, uint4 (&pieces)[ROW_ITERS]) {
-        const int64_t row0 = m0 + wm * 32 * WM + j * 32, col0 = n0 + wn * WCOLS;
 #pragma unroll
         for (int it = 0; it < ROW_ITERS; ++it) {
             const int id = it * WAVE + lane, pr = id / PIECES, pc = id % PIECES;
-            const int64_t row = row0 + pr, col = col0 + pc * 8;
+            const uint32_t row = tile_row + j * 32 + pr, col = col0 + pc * 8;
             // a piece outside the matrix reads the first one instead (its value is not used)
-            pieces[it] = *reinterpret_cast<const uint4*>(residual + (row < m && col < n ? row * n + col : 0));
+            pieces[it] = load_piece(residual, row < um && col < un ? row * un + col : 0u);
         }
     };
     if (EPILOGUE && !p.transpose_out) fetch_residual(0, ahead[0]);
@@ -311,34 +345,22 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void ns_gemm_fast(NsArgs
 #pragma unroll
         for (int i = 0; i < WN; ++i)
 #pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                uint32_t h[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) h[e] = ns_narrow<IS_BF16>(acc[i][j][r4 * 4 + e]);
-                *reinterpret_cast<uint2*>(&park[l32 * PLD + i * 32 + r4 * 8 + lhi * 4]) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
-            }
-        const int64_t row0 = m0 + wm * 32 * WM + j * 32, col0 = n0 + wn * WCOLS;   // of the parked 32 x WCOLS block
+            for (int r4 = 0; r4 < 4; ++r4)
+                *reinterpret_cast<uint2*>(&park[l32 * PLD + i * 32 + r4 * 8 + lhi * 4]) =
+                    make_uint2(ns_narrow2<IS_BF16>(acc[i][j][r4 * 4], acc[i][j][r4 * 4 + 1]), ns_narrow2<IS_BF16>(acc[i][j][r4 * 4 + 2], acc[i][j][r4 * 4 + 3]));
+        const uint32_t row0 = tile_row + j * 32;                          // of the parked 32 x WCOLS block
         if (!p.transpose_out) {
             if (EPILOGUE && j + 1 < WM) fetch_residual(j + 1, ahead[(j + 1) & 1]);
 #pragma unroll
             for (int it = 0; it < ROW_ITERS; ++it) {
                 const int id = it * WAVE + lane, pr = id / PIECES, pc = id % PIECES;
-                const int64_t row = row0 + pr, col = col0 + pc * 8;
+                const uint32_t row = row0 + pr, col = col0 + pc * 8;
                 const uint4 raw = *reinterpret_cast<const uint4*>(&park[pr * PLD + pc * 8]);
-                if (row >= m || col >= n) continue;                       // n is a multiple of 8: whole pieces
-                uint4 res = make_uint4(0, 0, 0, 0);
-                if (EPILOGUE) res = ahead[j & 1][it];
-                const uint32_t pw[4] = {raw.x, raw.y, raw.z, raw.w}, rw[4] = {res.x, res.y, res.z, res.w};
-                uint32_t o[4], od[4];
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    uint32_t bits, dbits;
-                    finish((uint16_t)(pw[e / 2] >> (16 * (e % 2))), ns_widen<IS_BF16>((uint16_t)(rw[e / 2] >> (16 * (e % 2)))), col + e == row, bits, dbits);
-                    if (e % 2 == 0) { o[e / 2] = bits; od[e / 2] = dbits; }
-                    else { o[e / 2] |= bits << 16; od[e / 2] |= dbits << 16; }
-                }
-                *reinterpret_cast<uint4*>(out + row * n + col) = make_uint4(o[0], o[1], o[2], o[3]);
-                if (out_diag) *reinterpret_cast<uint4*>(out_diag + row * n + col) = make_uint4(od[0], od[1], od[2], od[3]);
+                if (row >= um || col >= un) continue;                     // n is a multiple of 8: whole pieces
+                const uint4 res = EPILOGUE ? ahead[j & 1][it] : make_uint4(0, 0, 0, 0);
+                const uint4 o = make_uint4(finish(raw.x, res.x), finish(raw.y, res.y), finish(raw.z, res.z), finish(raw.w, res.w));
+                store_piece(out, row * un + col, o);
+                if (out_diag) store_piece(out_diag, row * un + col, row - col < 8u ? with_diagonal(o, row - col) : o);
             }
         }
         if (p.transpose_out || mirror) {
@@ -349,35 +371,30 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 2) void ns_gemm_fast(NsArgs
 #pragma unroll 1
             for (int it = 0; it < WCOLS * 4 / WAVE; ++it) {                   // not unrolled: the accumulators of the later j are still live
                 const int id = it * WAVE + lane, ln = id / 4, lm = id % 4 * 8;
-                const int64_t orow = col0 + ln, ocol = row0 + lm;         // row and first column in the [n, m] placement
-                uint16_t product[8];
+                const uint32_t orow = col0 + ln, ocol = row0 + lm;        // row and first column in the [n, m] placement
+                uint32_t pw[4];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) product[e] = park[(lm + e) * PLD + ln];
-                if (orow >= n || ocol >= m) continue;
+                for (int e = 0; e < 8; e += 2) pw[e / 2] = (uint32_t)park[(lm + e) * PLD + ln] | ((uint32_t)park[(lm + e + 1) * PLD + ln] << 16);
+                if (orow >= un || ocol >= um) continue;
                 uint32_t rw[4] = {0, 0, 0, 0};
                 if (EPILOGUE && mirror) {                                 // m == n, a multiple of 8: a whole piece of residual row orow
-                    const uint4 res = *reinterpret_cast<const uint4*>(residual + orow * n + ocol);
+                    const uint4 res = load_piece(residual, orow * un + ocol);
                     rw[0] = res.x; rw[1] = res.y; rw[2] = res.z; rw[3] = res.w;
                 } else if (EPILOGUE) {
 #pragma unroll
                     for (int e = 0; e < 8; ++e)
-                        if (ocol + e < m) rw[e / 2] |= (uint32_t)residual[(ocol + e) * n + orow] << (16 * (e % 2));
+                        if (ocol + e < um) rw[e / 2] |= (uint32_t)residual[(size_t)((ocol + e) * un + orow)] << (16 * (e % 2));
                 }
-                uint32_t o[4], od[4];
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    uint32_t bits, dbits;
-                    finish(product[e], ns_widen<IS_BF16>((uint16_t)(rw[e / 2] >> (16 * (e % 2)))), !mirror && ocol + e == orow, bits, dbits);
-                    if (e % 2 == 0) { o[e / 2] = bits; od[e / 2] = dbits; }
-                    else { o[e / 2] |= bits << 16; od[e / 2] |= dbits << 16; }
-                }
+                uint4 o = make_uint4(finish(pw[0], rw[0]), finish(pw[1], rw[1]), finish(pw[2], rw[2]), finish(pw[3], rw[3]));
+                const uint4 od = !mirror && orow - ocol < 8u ? with_diagonal(o, orow - ocol) : o;
                 if (whole) {
-                    *reinterpret_cast<uint4*>(out + orow * m + ocol) = make_uint4(o[0], o[1], o[2], o[3]);
-                    if (out_diag) *reinterpret_cast<uint4*>(out_diag + orow * m + ocol) = make_uint4(od[0], od[1], od[2], od[3]);
+                    store_piece(out, orow * um + ocol, o);
+                    if (out_diag) store_piece(out_diag, orow * um + ocol, od);
                 } else {
-                    for (int e = 0; e < 8 && ocol + e < m; ++e) {
-                        out[orow * m + ocol + e] = (uint16_t)(o[e / 2] >> (16 * (e % 2)));
-                        if (out_diag) out_diag[orow * m + ocol + e] = (uint16_t)(od[e / 2] >> (16 * (e % 2)));
+                    const uint32_t ow[4] = {o.x, o.y, o.z, o.w}, dw[4] = {od.x, od.y, od.z, od.w};
+                    for (int e = 0; e < 8 && ocol + e < um; ++e) {
+                        out[(size_t)(orow * um + ocol + e)] = (uint16_t)(ow[e / 2] >> (16 * (e % 2)));
+                        if (out_diag) out_diag[(size_t)(orow * um + ocol + e)] = (uint16_t)(dw[e / 2] >> (16 * (e % 2)));
                     }
                 }
             }
@@ -426,7 +443,7 @@ bool launch_ns_gemm_fast(const NsArgs& p, bool is_bf16, bool b_kn, int epilogue,
     if (p.k % 8 || p.n % 8 || p.k == 0) return false;
     if (!aligned(p.a) || !aligned(p.b) || !aligned(p.out) || !aligned(p.residual) || !aligned(p.out_diag)) return false;
     const int64_t limit = (1ll << 31) - 65536;
-    if (p.m * p.k * 2 >= limit || p.n * p.k * 2 >= limit) return false;
+    if (p.m * p.k * 2 >= limit || p.n * p.k * 2 >= limit || p.m * p.n * 2 >= limit) return false;
     if (p.batch * ((p.m + 127) / 128) * ((p.n + 127) / 128) >= (1ll << 31) - 8) return false;
     if (is_bf16) { if (b_kn) launch_shape<true, true>(p, epilogue, stream); else launch_shape<true, false>(p, epilogue, stream); }
     else { if (b_kn) launch_shape<false, true>(p, epilogue, stream); else launch_shape<false, false>(p, epilogue, stream); }
