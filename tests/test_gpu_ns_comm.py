@@ -138,6 +138,32 @@ def test_ns_gemm_transposed_output(dtype, batch, m, n, k, transpose_b, epilogue)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("batch,m,k", [(2, 192, 192), (1, 136, 96), (1, 100, 72), (40, 192, 136), (3, 576, 64)])
+@pytest.mark.parametrize("epilogue", [0, 1])
+def test_ns_gemm_second_copy_with_the_diagonal_shifted(dtype, batch, m, k, epilogue):
+    """The second output (the result with add_diag on its diagonal) through every store path of a square product: the
+    plain placement, the transposed one, and the mirrored one of a product of a matrix with itself; it must be the
+    first output with the constant added to the diagonal elements in the output's own dtype, bit for bit."""
+    from viola_amd.optim import _orthogonalize_kernels as nk
+    torch.manual_seed(25)
+    a = (torch.randn(batch, m, k) / math.sqrt(k)).to(dtype).cuda()
+    b = (torch.randn(batch, m, k) / math.sqrt(k)).to(dtype).cuda()
+    residual = torch.randn(batch, m, m).to(dtype).cuda() if epilogue else None
+    def shifted(z):
+        expect = z.clone()
+        expect.diagonal(dim1=-2, dim2=-1).add_(3.4445)
+        return expect
+    plain = nk._matmul(a, b, transpose_b=True, residual=residual, epilogue=epilogue)
+    z, q = nk._matmul(a, b, transpose_b=True, residual=residual, epilogue=epilogue, add_diag=3.4445)
+    assert torch.equal(z, plain) and torch.equal(q, shifted(plain))
+    zt, qt = nk._matmul(a, b, transpose_b=True, residual=residual, epilogue=epilogue, add_diag=3.4445, transpose_out=True)
+    assert torch.equal(zt, plain.mT.contiguous()) and torch.equal(qt, shifted(plain.mT.contiguous()))
+    gram = nk._matmul(a, a, transpose_b=True, residual=residual, epilogue=epilogue)
+    zg, qg = nk._matmul(a, a, transpose_b=True, residual=residual, epilogue=epilogue, add_diag=3.4445)
+    assert torch.equal(zg, gram) and torch.equal(qg, shifted(gram))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("shape", [(1, 64, 256), (2, 192, 64), (1, 96, 96), (1, 33, 70)])
 @pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32])
 def test_ns_prepare(dtype, shape, in_dtype):
