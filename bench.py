@@ -33,13 +33,6 @@ PEAK = {"fp8_tflops": 5000.0, "bf16_tflops": 2500.0, "hbm_gbs": 8000.0}
 # dispatch), each scaled by the same counter's reading for the 256 MiB copy_scaled_kernel launch (factors 2.00 and 1.00):
 # fetch (2 * 58.0 + 122.0) / 3 MB, write (2 * 41.9 + 8.8) / 3 MB. The algorithmic figure is 65 MB per launch.
 GEMM_TRAFFIC_BYTES = 79.3e6 + 30.9e6
-# Per 64-k chunk a wavefront of the grouped-scale GEMM issues 16 K = 16 FP8 MFMAs and, through the same port, the 128
-# FP32 FMAs that fold their sums into the totals (one FMA per accumulator and 32-k group). What that costs on the
-# machine is measured in the run itself by viola_probe_chunk_loop (chunk_loop_probe below).
-PROBE_PARTS = {"math": 0, "math_lds_reads": 1, "math_loads": 4, "all": 7}
-PROBE_CHUNKS, PROBE_BLOCKS, PROBE_LDA = 2048, 512, 4096
-
-
 WARM_MS = 100.0
 
 
@@ -79,28 +72,6 @@ def timed(fn, steps, warmup, warm=True):
     torch.cuda.synchronize()
     wall = (time.perf_counter() - begin) * 1e3
     return max(start.elapsed_time(end), 0.0) / steps, wall / steps
-
-
-def chunk_loop_probe():
-    """Time per 64-k chunk of the grouped-scale GEMM's instruction mix with nothing else in the way (two 256-thread
-    blocks per CU on all 256 CUs, like the GEMM), for the math alone, with the LDS operand reads, with the global ->
-    LDS loads, and with both plus the barrier. A 128 x 128 tile does 2 * 128 * 128 * 64 flops per chunk."""
-    import torch
-    from viola_amd import _lib
-    out = torch.empty(PROBE_BLOCKS * 256, device="cuda")
-    src = torch.randint(0, 255, (72 * 128 * PROBE_LDA,), device="cuda", dtype=torch.uint8)
-    result = {}
-    for name, parts in PROBE_PARTS.items():
-        def run():
-            _lib.call("viola_probe_chunk_loop", parts, _lib.ptr(out), _lib.ptr(src), src.numel(), PROBE_BLOCKS, PROBE_CHUNKS, PROBE_LDA)
-        ms, _ = timed(run, 5, 2, warm=False)
-        result[name + "_us_per_chunk"] = ms * 1e3 / PROBE_CHUNKS
-    flops_per_chunk = 2 * 128 * 128 * 64 * PROBE_BLOCKS
-    result["all_tflops"] = flops_per_chunk / (result["all_us_per_chunk"] * 1e-6) / 1e12
-    result["math_tflops"] = flops_per_chunk / (result["math_us_per_chunk"] * 1e-6) / 1e12
-    result["note"] = ("viola_probe_chunk_loop: the GEMM kernel's chunk loop (16 MFMA 32x32x16 fp8 + 128 FMA + 8 scale products per "
-                      "wavefront and chunk) without a GEMM around it, 512 blocks x 2048 chunks")
-    return result
 
 
 def kernel_breakdown(fn, steps):
@@ -180,7 +151,10 @@ def cpu_baseline():
     import torch
     from oracle import comm as oc, grouped as og, linear as ol, ns as ons, optim as oo
     torch.manual_seed(20261125)
-    cores = min(os.cpu_count() or 1, 16)
+    # threads: this job's share of the host (the GPU boxes give a one-GPU job 16 of the host's cores, whatever
+    # os.cpu_count() reports for the whole machine); both numbers go into the record
+    host_cpus = os.cpu_count() or 1
+    cores = min(host_cpus, 16)
     torch.set_num_threads(cores)
     x = torch.randn(M, K).bfloat16()
     dy = (torch.randn(M, N) * 1e-2).bfloat16()
@@ -206,14 +180,33 @@ def cpu_baseline():
     # the eager Newton-Schulz recipes last, each under a time limit: a host without fast half-precision matmuls
     # can take minutes (or not come back) on them; a leg that misses its limit is reported as such
     g = torch.randn(1024, 4096)
-    for method, flops in (("standard", NS_C1_FLOPS["standard"]), ("gram", NS_C1_FLOPS["gram"])):
-        t = _bounded(lambda: _median_time(lambda: ons.METHODS[method](g, steps=5)), 30.0)
-        log(f"cpu ns {method}: {'no result within 30 s' if t is None else f'{t * 1e3:.0f} ms'}")
-        if t is None:
-            others[f"ns_{method}_1024x4096"] = dict(ms=None, tflops=None, sample="one matrix, 5 steps, eager torch on the host: not finished within 30 s")
+    small = torch.randn(256, 1024)
+    small_flops = {"standard": 5 * (4 * 256 ** 2 * 1024 + 2 * 256 ** 3), "gram": 8 * 256 ** 2 * 1024 + 28 * 256 ** 3}
+    for method in ("standard", "gram"):
+        # a 256 x 1024 matrix first (1/64 of the work): the fp16 chain of `gram` runs on the host's scalar half-precision
+        # matmul and does not finish the full matrix within the limit; its full-size figure is then this one scaled
+        t_small = _bounded(lambda: _median_time(lambda: ons.METHODS[method](small, steps=5)), 30.0)
+        if t_small is None:
+            others[f"ns_{method}_256x1024"] = dict(ms=None, tflops=None, sample="one 256 x 1024 matrix, 5 steps, eager torch on the host: not finished within 30 s")
             break                                                                 # its threads may still be busy
-        others[f"ns_{method}_1024x4096"] = dict(ms=t * 1e3, tflops=flops / t / 1e12, sample="one matrix, 5 steps, eager torch on the host")
-    return dict(value=6 * M * K * N / best / 1e12, unit="TFLOP/s", cores=cores, kind="port",
+        others[f"ns_{method}_256x1024"] = dict(ms=t_small * 1e3, tflops=small_flops[method] / t_small / 1e12,
+                                               sample="one 256 x 1024 matrix, 5 steps, eager torch on the host")
+        scaled_ms = t_small * 1e3 * NS_C1_FLOPS[method] / small_flops[method]
+        if scaled_ms > 20e3:
+            log(f"cpu ns {method}: 256 x 1024 in {t_small * 1e3:.0f} ms; full size not run (about {scaled_ms / 1e3:.0f} s by flop count)")
+            others[f"ns_{method}_1024x4096"] = dict(ms=scaled_ms, tflops=small_flops[method] / t_small / 1e12, scaled=True,
+                                                   sample="not run: the 256 x 1024 time scaled by the flop ratio (x%.1f)" % (NS_C1_FLOPS[method] / small_flops[method]))
+            continue
+        t = _bounded(lambda: _median_time(lambda: ons.METHODS[method](g, steps=5)), 60.0)
+        log(f"cpu ns {method}: {'no result within 60 s' if t is None else f'{t * 1e3:.0f} ms'}")
+        if t is None:
+            others[f"ns_{method}_1024x4096"] = dict(ms=scaled_ms, tflops=small_flops[method] / t_small / 1e12, scaled=True,
+                                                   sample="not finished within 60 s: the 256 x 1024 time scaled by the flop ratio")
+            break
+        others[f"ns_{method}_1024x4096"] = dict(ms=t * 1e3, tflops=NS_C1_FLOPS[method] / t / 1e12, scaled=False,
+                                               sample="one matrix, 5 steps, eager torch on the host")
+    return dict(value=6 * M * K * N / best / 1e12, unit="TFLOP/s", cores=cores, host_cpus=host_cpus,
+                cores_note=f"{cores} torch threads = this job's share of the host's {host_cpus} logical CPUs", kind="port",
                 sample=f"one full {M}x{K}->{N} forward+backward per run, median of 2 after 1 warm-up "
                        f"({best * 1e3:.0f} ms per step)", others=others)
 
@@ -310,18 +303,10 @@ def main():
     breakdown = kernel_breakdown(step, args.steps)
     gemm = breakdown["viola_group_gemm"]
     gemm_tflops = 2 * M * K * N / (gemm["avg_ms"] * 1e-3) / 1e12
-    log("chunk loop probe")
-    probe = chunk_loop_probe()
     roofline = dict(bound="mfma", kernel="group_gemm_fast (viola_group_gemm: fwd, dgrad, wgrad)",
                     achieved=gemm_tflops, peak=PEAK["fp8_tflops"], unit="TFLOP/s", frac=gemm_tflops / PEAK["fp8_tflops"],
                     avg_launch_ms=gemm["avg_ms"], traffic=GEMM_TRAFFIC_BYTES,
-                    traffic_source="stored calibration (two rocprofv3 --pmc runs, profiles/linear_step_8192x1024x4096_hbm_traffic.txt), not read in this run",
-                    attainable=probe["all_tflops"],
-                    attainable_note="measured in this run (chunk_loop_probe): the rate at which this machine runs the kernel's own "
-                                    "instruction mix (K = 16 FP8 MFMAs, one FP32 FMA per accumulator and 32-k group through the same issue "
-                                    "port, LDS operand reads, global -> LDS loads, one barrier per chunk) with nothing else in the way; "
-                                    "the math alone, without operand traffic, runs at chunk_loop_probe.math_tflops; frac stays against "
-                                    "the 5 PFLOP/s peak")
+                    traffic_source="stored calibration (two rocprofv3 --pmc runs, profiles/linear_step_8192x1024x4096_hbm_traffic.txt), not read in this run")
     quant = {}
     if "viola_group_quantize_dual" in breakdown:
         # X [M, K] and dY [M, N] each once per step: 4.25 B per element (bf16 in, two FP8 layouts + scales out)
@@ -373,6 +358,20 @@ def main():
         unpack_ms, _ = timed(lambda: codec.unpack(packet, out, 256, torch.float8_e4m3fn), 50, 5)
         extra["comm_codec"] = dict(bucket_elements=n, pack_ms=pack_ms, unpack_ms=unpack_ms,
                                    pack_gbs=5.016 * n / (pack_ms * 1e-3) / 1e9, unpack_gbs=5.016 * n / (unpack_ms * 1e-3) / 1e9)
+        # the DiT-XL gradients are 68 such buckets; 16 of them through the table entry points, one launch each way
+        many = 16
+        buckets = [torch.randn(n, device="cuda") * 1e-3 for _ in range(many)]
+        packets = [torch.empty((1, packet_bytes(n // 256, 256)), dtype=torch.uint8, device="cuda") for _ in range(many)]
+        outs = [torch.empty_like(b) for b in buckets]
+        tables = ({}, {})
+        pack_many_ms, _ = timed(lambda: codec.pack_many(buckets, packets, 256, torch.float8_e4m3fn, cache=tables[0]), 20, 5)
+        unpack_many_ms, _ = timed(lambda: codec.unpack_many(packets, outs, 256, torch.float8_e4m3fn, cache=tables[1]), 20, 5)
+        extra["comm_codec"].update(buckets_per_launch=many, pack_many_ms=pack_many_ms, unpack_many_ms=unpack_many_ms,
+                                   pack_many_gbs=5.016 * n * many / (pack_many_ms * 1e-3) / 1e9,
+                                   unpack_many_gbs=5.016 * n * many / (unpack_many_ms * 1e-3) / 1e9,
+                                   pack_many_frac_hbm=5.016 * n * many / (pack_many_ms * 1e-3) / 1e9 / PEAK["hbm_gbs"],
+                                   unpack_many_frac_hbm=5.016 * n * many / (unpack_many_ms * 1e-3) / 1e9 / PEAK["hbm_gbs"])
+        del buckets, packets, outs
 
     if want("bound"):
         # the training loop closed: the same Linear under bind_optimizer (fp32 master, bf16 gradients), one
@@ -490,13 +489,14 @@ def main():
         "config": {"workload": "viola.nn.Linear(1024, 4096, scaling='grouped', e4m3/e4m3, fp8 weight storage, mode='memory') "
                                "forward+backward on 8192 tokens, bf16 activations and gradients"},
         "frac_of_fp8_peak": value / PEAK["fp8_tflops"],
-        "roofline": roofline, "chunk_loop_probe": probe, "quantize": quant, "kernels": breakdown, **extra,
+        "roofline": roofline, "quantize": quant, "kernels": breakdown, **extra,
     }
     if not args.skip_cpu:
         log("CPU baselines")
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result), flush=True)
-    if any(leg.get("ms", 0) is None for leg in result.get("cpu_baseline", {}).get("others", {}).values()):
+    others = result.get("cpu_baseline", {}).get("others", {})
+    if any(leg.get("ms", 0) is None or "not finished" in leg.get("sample", "") for leg in others.values()):
         os._exit(0)                                                  # a CPU leg is still running in its thread: do not wait for it
 
 

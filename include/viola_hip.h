@@ -324,6 +324,17 @@ int viola_ns_gemm(const void* a, const void* bmat, const void* residual, void* o
                   int transpose_b, int epilogue, int64_t batch, int64_t m, int64_t n, int64_t k,
                   float add_diag, void* out_diag, int transpose_out, viola_stream_t stream);
 
+/* viola/optim/_orthogonalize_kernels.py:114-197 `plan` (the per-shape schedule the reference picks by timing its
+ * candidates: bm, bn): which tile shape viola_ns_gemm runs a product on. Host arithmetic only, nothing is launched and
+ * no GPU is needed. Operands are taken as 16-byte aligned; same_operand != 0 means a and bmat are one buffer.
+ * plan[0], plan[1]: rows and columns of output per block; plan[2]: 1 when only the tiles on and above the diagonal
+ * are multiplied and mirrored (a . a^T, not transposed on output); plan[3]: 0 for the generic kernel (shapes the tiled
+ * one does not take: k or n not a multiple of 8, a matrix of 2 GiB or more), 1..5 for the tiled kernel's shapes in
+ * growing size. Every shape computes an element with the same sequence of operations, so the plan never changes a
+ * result. */
+int viola_ns_plan(int64_t batch, int64_t m, int64_t n, int64_t k, int transpose_b, int same_operand, int transpose_out,
+                  int* plan);
+
 /* viola/optim/_orthogonalize.py:12-16 / _orthogonalize_kernels.py:80-84: x = dtype(matrix), optionally
  * transposed so rows <= cols, divided by (Frobenius norm + 1e-7), all in the working dtype.
  * in [batch, rows, cols] of in_dtype; out [batch, min, max] of dtype; workspace: 256 * batch floats (partial
@@ -352,6 +363,19 @@ int viola_comm_pack(const float* x, int64_t n, void* packet, int64_t rows, int64
 int viola_comm_unpack(const void* packet, float* out, int64_t n, int64_t rows, int64_t groups, int tile, int fp8_dtype,
                       int reduce, viola_stream_t stream);
 
+/* viola_comm_pack / viola_comm_unpack for many buckets in one launch: the reference drains its gradient buckets one
+ * pack and one unpack launch at a time (viola/distributed/gradients.py:101-125 -> fp8.py:49-85), and a 25 MB bucket
+ * is too short a launch to reach the memory system's streaming rate. table: device array of `buckets` rows of eight
+ * int64. pack: {x, n, packet, rows, groups, 0, 0, 0}, x 16-byte and packet 4-byte aligned, tile 256 only
+ * (VIOLA_EUNSUPPORTED otherwise: call viola_comm_pack per bucket); max_units = the largest rows * groups of a bucket.
+ * unpack: {packet, n, out, rows, groups, 0, 0, 0}, out 16-byte and packet 4-byte aligned, n <= (reduce ? 1 : rows) *
+ * groups * tile as for viola_comm_unpack (not checked here: the table lives on the device); max_elements = the
+ * largest (reduce ? 1 : rows) * groups * tile of a bucket. Bytes and values are those of the per-bucket entry points. */
+int viola_comm_pack_table(const int64_t* table, int64_t buckets, int64_t max_units, int tile, int fp8_dtype,
+                          viola_stream_t stream);
+int viola_comm_unpack_table(const int64_t* table, int64_t buckets, int64_t max_elements, int tile, int fp8_dtype,
+                            int reduce, viola_stream_t stream);
+
 /* ---------------------------------------------------------------- self checks (test support)
  * Compare the hardware FP8 conversion instructions with the software codecs over every fp32 bit
  * pattern of magnitude <= the format's clamp range (encode) and all 256 codes (decode); writes
@@ -360,18 +384,6 @@ int viola_selftest_fp8(uint64_t* counts, viola_stream_t stream);
 /* philox(element, step, key) word 0 for `count` triples (device arrays) -> out. */
 int viola_selftest_philox(const uint64_t* triples, uint32_t* out, int64_t count, viola_stream_t stream);
 
-
-/* ---------------------------------------------------------------- issue-rate probe (measurement support)
- * No counterpart in the reference. Runs the chunk loop of the grouped-scale FP8 GEMM without a GEMM around it: per
- * 64-k chunk and wavefront 16 v_mfma_f32_32x32x16_fp8_fp8, the 128 FP32 FMAs that fold them into the totals and 8
- * scale products, in blocks of 256 threads, two to a CU. `parts` switches on what a real chunk adds: bit 0 the LDS
- * reads of the next chunk's operands and scales, bit 1 the barrier, bit 2 the wavefront's four global -> LDS loads
- * (src: a byte matrix of 72 x 128 rows with row stride lda, a multiple of 64; 16-byte aligned; may be NULL without
- * bit 2). Timing a launch of `blocks` blocks over `chunks` (even) chunks gives the time per chunk this instruction mix
- * needs when nothing else is in the way; bench.py derives the GEMM's attainable rate from it. out: blocks * 256 floats
- * of no meaning. */
-int viola_probe_chunk_loop(int parts, float* out, const void* src, int64_t src_bytes, int blocks, int chunks, int lda,
-                           viola_stream_t stream);
 
 #ifdef __cplusplus
 }

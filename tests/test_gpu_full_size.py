@@ -329,6 +329,44 @@ def test_fp8muon_step_at_ditxl_block(method, rounding):
         assert all(torch.equal(a, b) for a, b in zip(nearest, again))
 
 
+@pytest.mark.parametrize("method", ["standard", "gram"])
+def test_fp8muon_step_at_the_ditxl_set(method):
+    """The optimizer benchmark's whole parameter set (28 transformer blocks of width 1152: 112 matrices in three shape
+    buckets of 28 and 56, plus the bias vectors), two steps: the batched step, whose Newton-Schulz products run on the
+    large tiles that only a batch of this size selects, equals stepping every parameter in an optimizer of its own,
+    bit for bit, weights and momentum state."""
+    import viola_amd
+    from viola_amd.optim import _orthogonalize_kernels as nk
+    d, blocks = 1152, 28
+    shapes = ((3 * d, d), (d, d), (4 * d, d), (d, 4 * d), (3 * d,), (d,), (4 * d,), (d,))
+    assert nk.plan(blocks, d, 3 * d, d)["kernel"] != nk.plan(1, d, 3 * d, d)["kernel"]
+
+    def build(seed):
+        torch.manual_seed(seed)
+        params = [torch.nn.Parameter(torch.randn(*s, device="cuda") * .02) for _ in range(blocks) for s in shapes]
+        for p in params:
+            p.grad = torch.randn_like(p) * 1e-3
+        return params
+
+    options = dict(lr=1e-3, weight_decay=.01, adjust_lr_fn="match_rms_adamw", mode="balanced", tile_size=256, ns_method=method,
+                   rounding="nearest", rounding_seed=42)
+    together = build(10)
+    batched = viola_amd.optim.FP8Muon(together, **options)
+    batched.step()
+    batched.step()
+    alone = build(10)
+    for index, (a, b) in enumerate(zip(together, alone)):
+        single = viola_amd.optim.FP8Muon([{"params": [b], "viola_parameter_indices": [index]}], **options)
+        single.step()
+        single.step()
+        assert torch.equal(a, b) and torch.isfinite(a).all(), (index, tuple(a.shape))
+        if a.ndim == 2:
+            assert torch.equal(batched.state[a]["momentum_q"], single.state[b]["momentum_q"]), index
+            assert torch.equal(batched.state[a]["momentum_scale"], single.state[b]["momentum_scale"]), index
+        b.grad = None
+        del single
+
+
 @pytest.mark.parametrize("recipe", ["tensor", "mxfp8"])
 @pytest.mark.parametrize("m,n,k,formats", [(4096, 12288, 256, (E4, E4)), (4100, 12300, 384, (torch.float8_e5m2, E4)),
                                            (8192, 8192, 1024, (E4, torch.float8_e5m2))])

@@ -13,23 +13,27 @@ pytestmark = pytest.mark.gpu
 E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("batch,m,n,k", [(1, 64, 64, 256), (2, 130, 72, 96), (1, 256, 384, 128), (3, 33, 47, 65), (2, 384, 576, 200),
-                                         (1, 1024, 1024, 520), (300, 64, 64, 256), (130, 130, 72, 96), (50, 256, 384, 128), (30, 384, 576, 200)])
-@pytest.mark.parametrize("transpose_b,epilogue", [(True, 0), (False, 0), (False, 1), (True, 1), (False, 2)])
-def test_ns_gemm_contract(dtype, batch, m, n, k, transpose_b, epilogue):
-    """One chain GEMM against its contract: fp32 accumulate -> round -> fp32 epilogue -> round. A product with fewer
-    than 40 tiles of 128 x 128 per matrix runs on 64 x 64 tiles with k split over the wavefronts of a block, a larger
-    one (1024 x 1024 here) on the 128- or 192-wide tiles; shapes that are not multiples of 8 on the generic kernel."""
-    from viola_amd.optim import _orthogonalize_kernels as nk
-    torch.manual_seed(9)
-    a = (torch.randn(batch, m, k) / math.sqrt(k)).to(dtype)
-    b = (torch.randn(batch, n, k) if transpose_b else torch.randn(batch, k, n)).to(dtype)
-    residual = torch.randn(batch, m, n).to(dtype) if epilogue else None
-    out = nk._matmul(a.cuda(), b.cuda(), transpose_b=transpose_b, residual=residual.cuda() if epilogue else None, epilogue=epilogue)
+# Shape tables at module level: tests/test_ns_plan.py replays them through the library's tile planner on the CPU and
+# fails when a tile shape of the kernel, or a product of the DiT-XL step, is left without a covering case.
+CONTRACT_SHAPES = [(1, 64, 64, 256), (2, 130, 72, 96), (1, 256, 384, 128), (3, 33, 47, 65), (2, 384, 576, 200),
+                   (1, 1024, 1024, 520), (300, 64, 64, 256), (130, 130, 72, 96), (50, 256, 384, 128), (30, 384, 576, 200),
+                   (11, 1152, 4608, 64)]
+CONTRACT_MODES = [(True, 0), (False, 0), (False, 1), (True, 1), (False, 2)]
+GRAM_SHAPES = [(2, 384, 200), (1, 576, 96), (3, 200, 72), (1, 1152, 64), (50, 384, 200), (6, 1152, 64), (1, 1024, 4096), (12, 1152, 64)]
+GRAM_ASYMMETRIC_SHAPES = [(2, 384, 200), (1, 576, 384), (1, 1152, 64), (2, 256, 128), (50, 384, 200), (6, 1152, 64), (12, 1152, 64)]
+TRANSPOSED_SHAPES = [(2, 192, 384, 192), (1, 130, 72, 96), (2, 64, 200, 136), (1, 33, 47, 65), (1, 100, 72, 96),
+                     (60, 192, 384, 192), (140, 64, 200, 136), (11, 1152, 4608, 64)]
+TRANSPOSED_MODES = [(False, 2), (False, 0), (True, 0)]
+DIAGONAL_SHAPES = [(2, 192, 192), (1, 136, 96), (1, 100, 72), (40, 192, 136), (3, 576, 64), (12, 1152, 64)]
+DITXL_BATCH = 28                                                           # transformer blocks of the DiT-XL parameter set
+DITXL_PRODUCTS = [(1152, 3456, 1152), (1152, 4608, 1152)]                  # z . x of the qkv and the MLP matrices: m, n, k
+DITXL_GRAM_K = [3456, 4608, 1152]                                          # x . x^T of the three shape buckets: k (m = 1152)
+
+
+def assert_ns_contract(out, a, b, residual, transpose_b, epilogue, dtype):
+    """`out` (device result) against the chain GEMM's contract evaluated on the CPU: identical except where a different
+    fp32 summation order flips the final rounding (one ulp of the output dtype)."""
     ref = ons.matmul(a, b, transpose_b=transpose_b, residual=residual, epilogue=epilogue)
-    assert out.dtype == dtype
-    # identical except where a different fp32 summation order flips the final rounding (one ulp of the output dtype)
     ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
     diff = (out.cpu().float() - ref.float()).abs()
     # second term: the rounded product may flip by one grid step before the epilogue scales it (by 2.0315 at most),
@@ -40,6 +44,23 @@ def test_ns_gemm_contract(dtype, batch, m, n, k, transpose_b, epilogue):
     assert (diff <= bound).all()
     assert rel_l2(out, ref) < (2e-3 if dtype == torch.bfloat16 else 3e-4)
     assert (diff == 0).float().mean() > .9
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("batch,m,n,k", CONTRACT_SHAPES)
+@pytest.mark.parametrize("transpose_b,epilogue", CONTRACT_MODES)
+def test_ns_gemm_contract(dtype, batch, m, n, k, transpose_b, epilogue):
+    """One chain GEMM against its contract: fp32 accumulate -> round -> fp32 epilogue -> round. A product with fewer
+    than 40 tiles of 128 x 128 per matrix runs on 64 x 64 tiles with k split over the wavefronts of a block, a larger
+    one (1024 x 1024 here) on the 128- or 192-wide tiles; shapes that are not multiples of 8 on the generic kernel."""
+    from viola_amd.optim import _orthogonalize_kernels as nk
+    torch.manual_seed(9)
+    a = (torch.randn(batch, m, k) / math.sqrt(k)).to(dtype)
+    b = (torch.randn(batch, n, k) if transpose_b else torch.randn(batch, k, n)).to(dtype)
+    residual = torch.randn(batch, m, n).to(dtype) if epilogue else None
+    out = nk._matmul(a.cuda(), b.cuda(), transpose_b=transpose_b, residual=residual.cuda() if epilogue else None, epilogue=epilogue)
+    assert out.dtype == dtype
+    assert_ns_contract(out, a, b, residual, transpose_b, epilogue, dtype)
     if epilogue == 1 and m == n:
         z, q = nk._matmul(a.cuda(), b.cuda(), transpose_b=transpose_b, residual=residual.cuda(), epilogue=1, add_diag=3.4445)
         assert torch.equal(z, out)
@@ -49,7 +70,7 @@ def test_ns_gemm_contract(dtype, batch, m, n, k, transpose_b, epilogue):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("batch,m,k", [(2, 384, 200), (1, 576, 96), (3, 200, 72), (1, 1152, 64), (50, 384, 200), (6, 1152, 64), (1, 1024, 4096)])
+@pytest.mark.parametrize("batch,m,k", GRAM_SHAPES)
 @pytest.mark.parametrize("epilogue", [0, 1])
 def test_ns_gram_product_is_mirrored(dtype, batch, m, k, epilogue):
     """a . a^T (same buffer for both operands) computes the upper tiles only and mirrors them: the result
@@ -71,7 +92,7 @@ def test_ns_gram_product_is_mirrored(dtype, batch, m, k, epilogue):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("batch,m,k", [(2, 384, 200), (1, 576, 384), (1, 1152, 64), (2, 256, 128), (50, 384, 200), (6, 1152, 64)])
+@pytest.mark.parametrize("batch,m,k", GRAM_ASYMMETRIC_SHAPES)
 @pytest.mark.parametrize("epilogue", [1, 2])
 def test_ns_gram_product_with_an_asymmetric_residual(dtype, batch, m, k, epilogue):
     """a . a^T from one buffer (the mirrored path) with a residual that is NOT symmetric: every element, above and
@@ -123,9 +144,8 @@ def test_gram_chain_multiplies_r_by_r_past_the_first_iteration():
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("batch,m,n,k", [(2, 192, 384, 192), (1, 130, 72, 96), (2, 64, 200, 136), (1, 33, 47, 65), (1, 100, 72, 96),
-                                         (60, 192, 384, 192), (140, 64, 200, 136)])
-@pytest.mark.parametrize("transpose_b,epilogue", [(False, 2), (False, 0), (True, 0)])
+@pytest.mark.parametrize("batch,m,n,k", TRANSPOSED_SHAPES)
+@pytest.mark.parametrize("transpose_b,epilogue", TRANSPOSED_MODES)
 def test_ns_gemm_transposed_output(dtype, batch, m, n, k, transpose_b, epilogue):
     from viola_amd.optim import _orthogonalize_kernels as nk
     torch.manual_seed(22)
@@ -138,7 +158,73 @@ def test_ns_gemm_transposed_output(dtype, batch, m, n, k, transpose_b, epilogue)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("batch,m,k", [(2, 192, 192), (1, 136, 96), (1, 100, 72), (40, 192, 136), (3, 576, 64)])
+@pytest.mark.parametrize("m,n,k", DITXL_PRODUCTS)
+@pytest.mark.parametrize("epilogue,transpose_out", [(0, False), (2, False), (2, True), (0, True)])
+def test_ns_gemm_at_the_ditxl_batch(dtype, m, n, k, epilogue, transpose_out):
+    """z . x of the optimizer benchmark's two large shape buckets at its batch of 28 matrices, where the launcher picks
+    its largest tile: every matrix of the batch must come out bit for bit as it does alone (a single matrix runs on the
+    small tiles that the contract test checks element by element), and three of them are held to the contract directly."""
+    from viola_amd.optim import _orthogonalize_kernels as nk
+    assert nk.plan(DITXL_BATCH, m, n, k)["kernel"] != nk.plan(1, m, n, k)["kernel"]
+    torch.manual_seed(31)
+    a = (torch.randn(DITXL_BATCH, m, k) / math.sqrt(k)).to(dtype)
+    b = torch.randn(DITXL_BATCH, k, n).to(dtype)
+    residual = torch.randn(DITXL_BATCH, m, n).to(dtype) if epilogue else None
+    ad, bd, rd = a.cuda(), b.cuda(), residual.cuda() if epilogue else None
+    out = nk._matmul(ad, bd, residual=rd, epilogue=epilogue, transpose_out=transpose_out)
+    assert out.shape == ((DITXL_BATCH, n, m) if transpose_out else (DITXL_BATCH, m, n))
+    for i in range(DITXL_BATCH):
+        alone = nk._matmul(ad[i:i + 1], bd[i:i + 1], residual=rd[i:i + 1] if epilogue else None, epilogue=epilogue,
+                           transpose_out=transpose_out)
+        assert torch.equal(alone[0], out[i]), i
+    if not transpose_out:
+        rows = [0, 13, DITXL_BATCH - 1]
+        assert_ns_contract(out[rows], a[rows], b[rows], residual[rows] if epilogue else None, False, epilogue, dtype)
+    else:
+        assert torch.equal(out, nk._matmul(ad, bd, residual=rd, epilogue=epilogue).mT.contiguous())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("k", DITXL_GRAM_K)
+@pytest.mark.parametrize("epilogue,residual_kind", [(0, None), (1, "symmetric"), (1, "asymmetric")])
+def test_ns_gram_product_at_the_ditxl_batch(dtype, k, epilogue, residual_kind):
+    """x . x^T (one buffer for both operands: upper tiles multiplied, lower ones mirrored) of 28 matrices of 1152 rows,
+    with the second output that carries the shifted diagonal: bit for bit what each matrix gives alone and what the
+    un-mirrored kernel gives from two buffers; three matrices against the contract."""
+    from viola_amd.optim import _orthogonalize_kernels as nk
+    m = 1152
+    assert nk.plan(DITXL_BATCH, m, m, k, transpose_b=True, same_operand=True) != nk.plan(1, m, m, k, transpose_b=True, same_operand=True)
+    torch.manual_seed(32)
+    a = (torch.randn(DITXL_BATCH, m, k) / math.sqrt(k)).to(dtype)
+    ad = a.cuda()
+    if residual_kind == "symmetric":
+        rd = nk._matmul(ad, ad, transpose_b=True)
+        assert torch.equal(rd, rd.mT)
+    elif residual_kind == "asymmetric":
+        rd = torch.randn(DITXL_BATCH, m, m).to(dtype).cuda()
+    else:
+        rd = None
+    diag = 3.4445 if epilogue else None
+    got = nk._matmul(ad, ad, transpose_b=True, residual=rd, epilogue=epilogue, add_diag=diag)
+    full = nk._matmul(ad, ad.clone(), transpose_b=True, residual=rd, epilogue=epilogue, add_diag=diag)
+    for x, y in zip(got if epilogue else (got,), full if epilogue else (full,)):
+        assert torch.equal(x, y)
+    out = got[0] if epilogue else got
+    if residual_kind != "asymmetric":
+        assert torch.equal(out, out.mT)
+    if epilogue:
+        expect = out.clone()
+        expect.diagonal(dim1=-2, dim2=-1).add_(3.4445)
+        assert torch.equal(got[1], expect)
+    for i in range(DITXL_BATCH):
+        alone = nk._matmul(ad[i:i + 1], ad[i:i + 1], transpose_b=True, residual=rd[i:i + 1] if epilogue else None, epilogue=epilogue)
+        assert torch.equal(alone[0], out[i]), i
+    rows = [0, 13, DITXL_BATCH - 1]
+    assert_ns_contract(out[rows], a[rows], a[rows], rd[rows].cpu() if epilogue else None, True, epilogue, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("batch,m,k", DIAGONAL_SHAPES)
 @pytest.mark.parametrize("epilogue", [0, 1])
 def test_ns_gemm_second_copy_with_the_diagonal_shifted(dtype, batch, m, k, epilogue):
     """The second output (the result with add_diag on its diagonal) through every store path of a square product: the
@@ -161,6 +247,15 @@ def test_ns_gemm_second_copy_with_the_diagonal_shifted(dtype, batch, m, k, epilo
     gram = nk._matmul(a, a, transpose_b=True, residual=residual, epilogue=epilogue)
     zg, qg = nk._matmul(a, a, transpose_b=True, residual=residual, epilogue=epilogue, add_diag=3.4445)
     assert torch.equal(zg, gram) and torch.equal(qg, shifted(gram))
+    # a matrix times its own transpose, stored transposed: every element of both outputs is written (the result is
+    # the transpose of the plain one for any residual, symmetric or not)
+    for poison in (0.0, float("nan")):
+        from viola_amd import _lib
+        zt = torch.full_like(gram, poison)
+        qt = torch.full_like(gram, poison)
+        _lib.call("viola_ns_gemm", _lib.ptr(a), _lib.ptr(a), _lib.ptr(residual), _lib.ptr(zt), _lib.code(dtype), 1, epilogue,
+                  batch, m, m, k, 3.4445, _lib.ptr(qt), 1)
+        assert torch.equal(zt, gram.mT.contiguous()) and torch.equal(qt, shifted(gram.mT.contiguous()))
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
@@ -273,3 +368,43 @@ def test_comm_nonfinite_and_roundtrip_object():
         x[3], x[600] = float("nan"), float("inf")
         FP8Communication(1025, None, torch.device("cuda"), mode="all_reduce", fp8_format=fmt).roundtrip(x)
         assert not torch.isfinite(x[3]) and not torch.isfinite(x[600]) and torch.isfinite(x[900])   # :80-92
+
+
+@pytest.mark.parametrize("dtype", [E4, E5])
+@pytest.mark.parametrize("tile", [256, 64])
+def test_comm_codec_many_buckets_in_one_launch(tile, dtype):
+    """pack_many / unpack_many (a device table of buckets, one launch each way) against the oracle and against the
+    bucket-by-bucket entry points, bit for bit: buckets of different lengths (one ragged, one shorter than a tile, one
+    with several rows), a NaN and an Inf, and the row-summing decode. tile 64 takes the bucket-by-bucket route for
+    pack (the table kernel is built for 256) and the table route for unpack."""
+    from viola_amd.distributed import _fp8_kernels as codec, packet_bytes
+    torch.manual_seed(301)
+    sizes = [(6553600 // 16, 1), (65539, 1), (100, 1), (8193, 3), (4096, 2)]
+    sources, packets, expected = [], [], []
+    for n, rows in sizes:
+        x = torch.randn(n) * torch.logspace(-4, 4, n)
+        x[::97] *= 32
+        if n > 700:
+            x[3], x[600] = float("nan"), float("inf")
+        groups = math.ceil(n / (rows * tile))
+        sources.append(x)
+        packets.append(torch.zeros((rows, packet_bytes(groups, tile)), dtype=torch.uint8, device="cuda"))
+        expected.append(oc.pack(x, rows, groups, tile, dtype))
+    cache = {}
+    device_sources = [x.cuda() for x in sources]
+    for _ in range(2):                                                         # the second call reuses the cached table
+        for packet in packets:
+            packet.zero_()
+        codec.pack_many(device_sources, packets, tile, dtype, cache=cache)
+        for packet, want in zip(packets, expected):
+            assert torch.equal(packet.cpu(), want)
+    outs = [torch.full((n,), float("nan"), device="cuda") for n, _ in sizes]
+    codec.unpack_many(packets, outs, tile, dtype)
+    for out, want, (n, rows) in zip(outs, expected, sizes):
+        ref = oc.unpack(want, n, tile, dtype)
+        assert torch.equal(out.cpu().view(torch.int32), ref.view(torch.int32))
+    sums = [torch.full((p.shape[1] // (tile + 4) * tile,), float("nan"), device="cuda") for p in packets]
+    codec.unpack_many(packets, sums, tile, dtype, reduce=True)
+    for out, want in zip(sums, expected):
+        ref = oc.unpack(want, out.numel(), tile, dtype, reduce=True)
+        assert torch.equal(out.cpu().view(torch.int32), ref.view(torch.int32))

@@ -36,6 +36,39 @@ def test_static_scratch_prepare_equals_the_workspace_entry_point(dtype, in_dtype
         assert torch.isfinite(out).all()
 
 
+def _device_free_bytes():
+    """Free device memory as the runtime reports it (hipMemGetInfo through torch's own HIP runtime)."""
+    return torch.cuda.mem_get_info()[0]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_static_scratch_prepare_allocates_nothing_and_matches_the_oracle(dtype):
+    """What the entry point is for: after its set-up call, calls with every buffer already in the caller's hands leave
+    torch's allocator counters and the device's free memory exactly where they were (a hipMalloc inside the call would
+    move the latter, an allocation through torch the former). One result is also held to the CPU oracle directly."""
+    from oracle import ns as ons
+    from conftest import rel_l2
+    from viola_amd import _lib
+    _lib.call("viola_ns_prepare_static", None, _lib.F32, None, _lib.code(dtype), 0, 0, 0)              # set-up call
+    torch.manual_seed(78)
+    matrices = [torch.randn(28, 192, 576, device="cuda"), torch.randn(3, 96, 40, device="cuda") * 1e-3]
+    outs = [torch.empty(m.shape[0], min(m.shape[1:]), max(m.shape[1:]), device="cuda", dtype=dtype) for m in matrices]
+    host = [m.cpu() for m in matrices]
+    torch.cuda.synchronize()
+    before = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), _device_free_bytes())
+    for _ in range(3):
+        for matrix, out in zip(matrices, outs):
+            _lib.call("viola_ns_prepare_static", _lib.ptr(matrix), _lib.F32, _lib.ptr(out), _lib.code(dtype), *matrix.shape)
+    torch.cuda.synchronize()
+    after = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), _device_free_bytes())
+    assert after == before, (before, after)
+    ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
+    for matrix, out in zip(host, outs):
+        ref, _ = ons._prepare(matrix, dtype)
+        # the norm is one dtype-rounded scalar; a different fp32 summation order can move it by one ulp at most
+        assert rel_l2(out, ref.contiguous()) < 2 * ulp
+
+
 def test_static_scratch_prepare_rejects_what_does_not_fit():
     from viola_amd import _lib
     x = torch.zeros(8, device="cuda")

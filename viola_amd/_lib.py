@@ -62,11 +62,12 @@ _SIGNATURES = {
     "viola_ns_prepare_static": [_p, _i, _p, _i, _l, _l, _l, _p],
     "viola_comm_pack": [_p, _l, _p, _l, _l, _i, _i, _p],
     "viola_comm_unpack": [_p, _p, _l, _l, _l, _i, _i, _i, _p],
+    "viola_comm_pack_table": [_p, _l, _l, _i, _i, _p],
+    "viola_comm_unpack_table": [_p, _l, _l, _i, _i, _i, _p],
     "viola_selftest_fp8": [_p, _p],
     "viola_selftest_philox": [_p, _p, _l, _p],
-    "viola_probe_chunk_loop": [_i, _p, _p, _l, _i, _i, _i, _p],
 }
-EXPORTS = tuple(_SIGNATURES) + ("viola_abi_version", "viola_error_string")
+EXPORTS = tuple(_SIGNATURES) + ("viola_abi_version", "viola_error_string", "viola_ns_plan")
 
 _lib = None
 
@@ -84,6 +85,7 @@ def library():
             fn.argtypes, fn.restype = argtypes, ctypes.c_int
         lib.viola_abi_version.restype = ctypes.c_int
         lib.viola_error_string.argtypes, lib.viola_error_string.restype = [ctypes.c_int], ctypes.c_char_p
+        lib.viola_ns_plan.argtypes, lib.viola_ns_plan.restype = [_l, _l, _l, _l, _i, _i, _i, ctypes.POINTER(ctypes.c_int)], ctypes.c_int
         assert lib.viola_abi_version() == 1
         _lib = lib
     return _lib

@@ -17,7 +17,7 @@ ARCH = "gfx950"
 # scale with an explicit fmaf.
 COMMON = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17", "-ffp-contract=off", "-fno-fast-math",
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
-SOURCES = ["quantize.hip", "gemm.hip", "gemm_fast.hip", "gemm_fast_tensor.hip", "gemm_fast_mx.hip", "ns.hip", "ns_fast.hip", "optim.hip", "misc.hip", "tensor.hip", "probe.hip"]
+SOURCES = ["quantize.hip", "gemm.hip", "gemm_fast.hip", "gemm_fast_tensor.hip", "gemm_fast_mx.hip", "ns.hip", "ns_fast.hip", "optim.hip", "misc.hip", "tensor.hip"]
 
 
 def hipcc():

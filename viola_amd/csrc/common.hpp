@@ -36,6 +36,13 @@ static inline int viola_launch_status() {
     return e;
 }
 
+// First statement of an entry point: the caller's stream, and a clean launch status. A call that launched and then
+// left through an argument check never collected its status; the next call on that thread must not inherit it.
+static inline hipStream_t viola_enter(viola_stream_t stream) {
+    viola_first_launch_error = 0;
+    return static_cast<hipStream_t>(stream);
+}
+
 static inline bool viola_is_fp8(int dtype) { return dtype == VIOLA_E4M3 || dtype == VIOLA_E5M2; }
 static inline bool viola_is_float(int dtype) { return dtype == VIOLA_F32 || dtype == VIOLA_BF16 || dtype == VIOLA_F16; }
 static inline int viola_dtype_size(int dtype) { return dtype == VIOLA_F32 ? 4 : (dtype == VIOLA_BF16 || dtype == VIOLA_F16) ? 2 : 1; }

@@ -421,7 +421,7 @@ using namespace viola;
 extern "C" int viola_group_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,
                                 int64_t m, int64_t n, int64_t k, int ar, int ak, int br, int bk, const void* bias,
                                 int bias_dtype, void* out, int out_dtype, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_fp8(a_dtype) && viola_is_fp8(b_dtype) && viola_is_float(out_dtype));
     VIOLA_CHECK_ARG(m >= 0 && n >= 0 && k >= 0 && ar > 0 && br > 0 && pow2(ak) && pow2(bk) && ak >= 32 && bk >= 32);
     VIOLA_CHECK_ARG(!bias || viola_is_float(bias_dtype));
@@ -445,7 +445,7 @@ extern "C" int viola_group_gemm_half(const void* a, int a_dtype, const void* b, 
                                      int64_t m, int64_t n, int64_t k, int ar, int ak, int br, int bk, const void* bias,
                                      int bias_dtype, void* out, int out_dtype, int accum_block, int reduce_dtype,
                                      viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_fp8(a_dtype) && viola_is_fp8(b_dtype) && viola_is_float(out_dtype));
     VIOLA_CHECK_ARG(m >= 0 && n >= 0 && k >= 0 && ar > 0 && br > 0 && pow2(ak) && pow2(bk) && ak >= 32 && bk >= 32);
     VIOLA_CHECK_ARG((!bias || viola_is_float(bias_dtype)) && accum_block >= 0 && accum_block % 32 == 0);
@@ -468,7 +468,7 @@ extern "C" int viola_group_gemm_half(const void* a, int a_dtype, const void* b, 
 extern "C" int viola_tensor_gemm_half(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,
                                       int64_t m, int64_t n, int64_t k, const void* bias, int bias_dtype, void* out, int out_dtype,
                                       int accum_block, int reduce_dtype, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_fp8(a_dtype) && viola_is_fp8(b_dtype) && viola_is_float(out_dtype));
     VIOLA_CHECK_ARG(m >= 0 && n >= 0 && k >= 0 && k < (1ll << 30) && (!bias || viola_is_float(bias_dtype)));
     VIOLA_CHECK_ARG(accum_block >= 0 && accum_block % 32 == 0 && (reduce_dtype == VIOLA_F32 || reduce_dtype == VIOLA_BF16));
@@ -575,7 +575,7 @@ static int gated_two_passes(Plain&& plain, int64_t m, int64_t h, const void* bia
 extern "C" int viola_tensor_gated_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const float* sa, const float* sb,
                                        int64_t m, int64_t h, int64_t k, const void* bias, int bias_dtype, void* aux, void* out,
                                        int out_dtype, int activation, int backward, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_fp8(a_dtype) && viola_is_fp8(b_dtype) && viola_is_float(out_dtype));
     VIOLA_CHECK_ARG(m >= 0 && h >= 0 && k >= 0 && k < (1ll << 30));
     VIOLA_CHECK_ARG(activation >= VIOLA_SILU && activation <= VIOLA_RELU && (!bias || viola_is_float(bias_dtype)));
@@ -610,7 +610,7 @@ extern "C" int viola_tensor_gated_gemm(const void* a, int a_dtype, const void* b
 extern "C" int viola_mx_gated_gemm(const void* a, int a_dtype, const void* b, int b_dtype, const uint8_t* sa, const uint8_t* sb,
                                    int64_t m, int64_t h, int64_t k, int ar, int br, const void* bias, int bias_dtype, void* aux,
                                    void* out, int out_dtype, int activation, int backward, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_fp8(a_dtype) && viola_is_fp8(b_dtype) && viola_is_float(out_dtype));
     VIOLA_CHECK_ARG(m >= 0 && h >= 0 && k >= 0 && ar > 0 && br > 0);
     VIOLA_CHECK_ARG(activation >= VIOLA_SILU && activation <= VIOLA_RELU && (!bias || viola_is_float(bias_dtype)));
@@ -643,7 +643,7 @@ extern "C" int viola_gated_gemm(const void* a, int a_dtype, const void* b, int b
                                 int64_t m, int64_t h, int64_t k, int ar, int ak, int br, int bk, const void* bias,
                                 int bias_dtype, void* aux, void* out, int out_dtype, int activation, int backward,
                                 viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_fp8(a_dtype) && viola_is_fp8(b_dtype) && viola_is_float(out_dtype));
     VIOLA_CHECK_ARG(m >= 0 && h >= 0 && k >= 0 && ar > 0 && br > 0 && pow2(ak) && pow2(bk) && ak >= 32 && bk >= 32);
     VIOLA_CHECK_ARG(activation >= VIOLA_SILU && activation <= VIOLA_RELU && (!bias || viola_is_float(bias_dtype)));
@@ -673,7 +673,7 @@ extern "C" int viola_mx_gated_gemm_encode(const void* a, int a_dtype, const void
                                           void* aux, int aux_dtype, void* enc, uint8_t* enc_scale, void* enc_t,
                                           uint8_t* enc_t_scale, int enc_dtype, float limit, int activation,
                                           viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_fp8(a_dtype) && viola_is_fp8(b_dtype) && viola_is_float(aux_dtype) && viola_is_fp8(enc_dtype));
     VIOLA_CHECK_ARG(m >= 0 && h >= 0 && k >= 0 && ar > 0 && br > 0 && limit > 0.0f);
     VIOLA_CHECK_ARG(activation >= VIOLA_SILU && activation <= VIOLA_RELU && (!bias || viola_is_float(bias_dtype)));
@@ -711,7 +711,7 @@ extern "C" int viola_varlen_group_gemm(const void* a, int a_dtype, const void* b
                                        const float* sb, const int64_t* offsets, int groups, int64_t m_total, int64_t n,
                                        int64_t k, int ar, int ak, int br, int bk, int64_t b_group_stride,
                                        int64_t sb_group_stride, void* out, int out_dtype, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_fp8(a_dtype) && viola_is_fp8(b_dtype) && viola_is_float(out_dtype));
     VIOLA_CHECK_ARG(m_total >= 0 && n >= 0 && k >= 0 && groups > 0 && ar == 1 && br > 0 && pow2(ak) && pow2(bk) && ak >= 32 && bk >= 32);
     if (m_total == 0 || n == 0) return 0;
@@ -733,7 +733,7 @@ extern "C" int viola_varlen_group_gemm(const void* a, int a_dtype, const void* b
 extern "C" int viola_varlen_wgrad_gemm(const void* at, int a_dtype, const void* bt, int b_dtype, const float* sat,
                                        const float* sbt, const int64_t* poffsets, int groups, int64_t t_total, int64_t n,
                                        int64_t kout, void* out, int out_dtype, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_fp8(a_dtype) && viola_is_fp8(b_dtype) && viola_is_float(out_dtype));
     VIOLA_CHECK_ARG(t_total >= 0 && t_total % 32 == 0 && n >= 0 && kout >= 0 && groups > 0 && groups <= 65535);
     if (n == 0 || kout == 0) return 0;

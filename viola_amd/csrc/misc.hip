@@ -31,11 +31,8 @@ __global__ __launch_bounds__(256) void comm_pack_kernel(const float* __restrict_
 
 // tile == 256, x 16-byte aligned: one wavefront per tile, one float4 per lane.
 template <typename TQ>
-__global__ __launch_bounds__(256) void comm_pack256_kernel(const float* __restrict__ x, int64_t n, uint8_t* __restrict__ packet,
-                                                            int64_t rows, int64_t groups, int64_t stride) {
-    const int64_t unit = (int64_t)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
-    if (unit >= rows * groups) return;
-    const int lane = threadIdx.x % WAVE;
+__device__ __forceinline__ void comm_pack256_tile(const float* __restrict__ x, int64_t n, uint8_t* __restrict__ packet, int64_t groups,
+                                                  int64_t stride, int64_t unit, int lane) {
     const int64_t row = unit / groups, group = unit % groups;
     const int64_t base = (row * groups + group) * 256 + lane * 4;
     float v[4] = {0, 0, 0, 0};
@@ -62,6 +59,27 @@ __global__ __launch_bounds__(256) void comm_pack256_kernel(const float* __restri
     }
     *reinterpret_cast<uint32_t*>(packet + row * stride + group * 256 + lane * 4) = w;
     if (lane == 0) reinterpret_cast<float*>(packet + row * stride + groups * 256)[group] = s;
+}
+
+template <typename TQ>
+__global__ __launch_bounds__(256) void comm_pack256_kernel(const float* __restrict__ x, int64_t n, uint8_t* __restrict__ packet,
+                                                            int64_t rows, int64_t groups, int64_t stride) {
+    const int64_t unit = (int64_t)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (unit >= rows * groups) return;
+    comm_pack256_tile<TQ>(x, n, packet, groups, stride, unit, threadIdx.x % WAVE);
+}
+
+// Many buckets, one launch: row blockIdx.y of the table names the bucket {x, n, packet, rows, groups, -, -, -}.
+constexpr int COMM_ROW = 8;                                                   // int64 words per table row
+template <typename TQ>
+__global__ __launch_bounds__(256) void comm_pack256_table_kernel(const int64_t* __restrict__ table) {
+    const int64_t* bucket = table + (int64_t)blockIdx.y * COMM_ROW;
+    const int64_t n = bucket[1], rows = bucket[3], groups = bucket[4];
+    const int64_t unit = (int64_t)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (unit >= rows * groups) return;
+    const int64_t stride = (groups * (256 + 4) + 15) / 16 * 16;
+    comm_pack256_tile<TQ>(reinterpret_cast<const float*>(bucket[0]), n, reinterpret_cast<uint8_t*>(bucket[2]), groups, stride, unit,
+                          threadIdx.x % WAVE);
 }
 
 template <typename TQ>
@@ -100,12 +118,11 @@ template <> __device__ __forceinline__ void decode4<e5m2_t>(uint32_t word, float
 // out 16-byte aligned: four consecutive elements per thread (one code word, one scale, one 16-byte store). The
 // hardware decoders equal the table decode on all 256 codes (checked by the device self test below).
 template <typename TQ, bool REDUCE>
-__global__ __launch_bounds__(256) void comm_unpack_quads_kernel(const uint8_t* __restrict__ packet, float* __restrict__ out,
-                                                                 int64_t n, int64_t rows, int64_t width, int tile_shift,
-                                                                 int64_t stride) {
+__device__ __forceinline__ void comm_unpack_quads(const uint8_t* __restrict__ packet, float* __restrict__ out, int64_t n, int64_t rows,
+                                                  int64_t width, int tile_shift, int64_t stride, int64_t first, int64_t step) {
     const int64_t quads_per_row = width / 4;
     const int64_t total = (REDUCE ? 1 : rows) * quads_per_row;
-    for (int64_t quad = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; quad < total; quad += (int64_t)gridDim.x * blockDim.x) {
+    for (int64_t quad = first; quad < total; quad += step) {
         const int64_t row = (REDUCE || rows == 1) ? 0 : quad / quads_per_row;
         const int64_t col = (quad - row * quads_per_row) * 4;
         const int64_t idx = row * width + col;
@@ -137,6 +154,25 @@ __global__ __launch_bounds__(256) void comm_unpack_quads_kernel(const uint8_t* _
         }
     }
 }
+
+template <typename TQ, bool REDUCE>
+__global__ __launch_bounds__(256) void comm_unpack_quads_kernel(const uint8_t* __restrict__ packet, float* __restrict__ out,
+                                                                 int64_t n, int64_t rows, int64_t width, int tile_shift,
+                                                                 int64_t stride) {
+    comm_unpack_quads<TQ, REDUCE>(packet, out, n, rows, width, tile_shift, stride, (int64_t)blockIdx.x * blockDim.x + threadIdx.x,
+                                  (int64_t)gridDim.x * blockDim.x);
+}
+
+// Many buckets, one launch: row blockIdx.y of the table names the bucket {packet, n, out, rows, groups, -, -, -}.
+template <typename TQ, bool REDUCE>
+__global__ __launch_bounds__(256) void comm_unpack_quads_table_kernel(const int64_t* __restrict__ table, int tile, int tile_shift) {
+    const int64_t* bucket = table + (int64_t)blockIdx.y * COMM_ROW;
+    const int64_t n = bucket[1], rows = bucket[3], groups = bucket[4];
+    const int64_t width = groups * tile, stride = (groups * (tile + 4) + 15) / 16 * 16;
+    comm_unpack_quads<TQ, REDUCE>(reinterpret_cast<const uint8_t*>(bucket[0]), reinterpret_cast<float*>(bucket[2]), n, rows, width,
+                                  tile_shift, stride, (int64_t)blockIdx.x * blockDim.x + threadIdx.x, (int64_t)gridDim.x * blockDim.x);
+}
+
 
 // ------------------------------------------------------------------ gated activations
 __device__ __forceinline__ float load_half(const void* p, int64_t i, int dtype) {
@@ -348,7 +384,7 @@ using namespace viola;
 
 extern "C" int viola_comm_pack(const float* x, int64_t n, void* packet, int64_t rows, int64_t groups, int tile, int fp8_dtype,
                                viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_fp8(fp8_dtype) && n >= 0 && rows >= 0 && groups >= 0 && tile >= 32 && (tile & (tile - 1)) == 0);
     if (rows == 0 || groups == 0) return 0;
     VIOLA_CHECK_ARG(packet && (n == 0 || x) && reinterpret_cast<uintptr_t>(packet) % 4 == 0);
@@ -360,7 +396,7 @@ extern "C" int viola_comm_pack(const float* x, int64_t n, void* packet, int64_t 
 
 extern "C" int viola_comm_unpack(const void* packet, float* out, int64_t n, int64_t rows, int64_t groups, int tile,
                                  int fp8_dtype, int reduce, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_fp8(fp8_dtype) && n >= 0 && rows >= 0 && groups >= 0 && tile >= 32 && (tile & (tile - 1)) == 0);
     if (rows == 0 || groups == 0 || n == 0) return 0;
     VIOLA_CHECK_ARG(packet && out && reinterpret_cast<uintptr_t>(packet) % 4 == 0);
@@ -383,9 +419,37 @@ extern "C" int viola_comm_unpack(const void* packet, float* out, int64_t n, int6
     return viola_launch_status();
 }
 
+extern "C" int viola_comm_pack_table(const int64_t* table, int64_t buckets, int64_t max_units, int tile, int fp8_dtype,
+                                     viola_stream_t stream_) {
+    hipStream_t stream = viola_enter(stream_);
+    VIOLA_CHECK_ARG(viola_is_fp8(fp8_dtype) && buckets >= 0 && max_units >= 0 && tile >= 32 && (tile & (tile - 1)) == 0);
+    if (buckets == 0 || max_units == 0) return 0;
+    VIOLA_CHECK_ARG(table && buckets <= 65535 && (max_units + 3) / 4 < (1ll << 31));
+    if (tile != 256) return VIOLA_EUNSUPPORTED;                                    // other tiles: one viola_comm_pack per bucket
+    const dim3 grid((unsigned)((max_units + 3) / 4), (unsigned)buckets);
+    if (fp8_dtype == VIOLA_E4M3) VIOLA_LAUNCH(comm_pack256_table_kernel<e4m3_t>, grid, dim3(256), 0, stream, table);
+    else VIOLA_LAUNCH(comm_pack256_table_kernel<e5m2_t>, grid, dim3(256), 0, stream, table);
+    return viola_launch_status();
+}
+
+extern "C" int viola_comm_unpack_table(const int64_t* table, int64_t buckets, int64_t max_elements, int tile, int fp8_dtype,
+                                       int reduce, viola_stream_t stream_) {
+    hipStream_t stream = viola_enter(stream_);
+    VIOLA_CHECK_ARG(viola_is_fp8(fp8_dtype) && buckets >= 0 && max_elements >= 0 && tile >= 32 && (tile & (tile - 1)) == 0);
+    if (buckets == 0 || max_elements == 0) return 0;
+    VIOLA_CHECK_ARG(table && buckets <= 65535);
+    const int shift = __builtin_ctz((unsigned)tile);
+    const dim3 grid(grid_for(max_elements / 4), (unsigned)buckets);
+#define VIOLA_UNPACK(TQ, REDUCE) VIOLA_LAUNCH((comm_unpack_quads_table_kernel<TQ, REDUCE>), grid, dim3(256), 0, stream, table, tile, shift)
+    if (fp8_dtype == VIOLA_E4M3) { if (reduce) VIOLA_UNPACK(e4m3_t, true); else VIOLA_UNPACK(e4m3_t, false); }
+    else { if (reduce) VIOLA_UNPACK(e5m2_t, true); else VIOLA_UNPACK(e5m2_t, false); }
+#undef VIOLA_UNPACK
+    return viola_launch_status();
+}
+
 extern "C" int viola_gated_forward(const void* z, void* out, int64_t rows, int64_t h, int dtype, int activation,
                                    viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_float(dtype) && rows >= 0 && h >= 0 && activation >= VIOLA_SILU && activation <= VIOLA_RELU);
     if (rows == 0 || h == 0) return 0;
     VIOLA_CHECK_ARG(z && out);
@@ -396,7 +460,7 @@ extern "C" int viola_gated_forward(const void* z, void* out, int64_t rows, int64
 
 extern "C" int viola_gated_backward(const void* z, const void* dy, void* dz, int64_t rows, int64_t h, int dtype,
                                     int activation, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_float(dtype) && rows >= 0 && h >= 0 && activation >= VIOLA_SILU && activation <= VIOLA_RELU);
     if (rows == 0 || h == 0) return 0;
     VIOLA_CHECK_ARG(z && dy && dz);
@@ -406,14 +470,14 @@ extern "C" int viola_gated_backward(const void* z, const void* dy, void* dz, int
 }
 
 extern "C" int viola_selftest_fp8(uint64_t* counts, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(counts);
     VIOLA_LAUNCH(selftest_fp8_kernel, dim3(4096), dim3(256), 0, stream, reinterpret_cast<unsigned long long*>(counts));
     return viola_launch_status();
 }
 
 extern "C" int viola_selftest_philox(const uint64_t* triples, uint32_t* out, int64_t count, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(count >= 0);
     if (count == 0) return 0;
     VIOLA_CHECK_ARG(triples && out);

@@ -534,10 +534,32 @@ static int ns_static_workspace(float** workspace) {
 
 using namespace viola;
 
+// A product of a matrix with its own transpose is multiplied on and above the diagonal only and mirrored. A transposed
+// result keeps the full kernel: there the [n, m] store is the only placement, and the mirrored tiles have none of their own.
+static bool ns_is_mirrored(const void* a, const void* bmat, int transpose_b, int64_t m, int64_t n, int transpose_out) {
+    return transpose_b && a == bmat && m == n && !transpose_out;
+}
+
+extern "C" int viola_ns_plan(int64_t batch, int64_t m, int64_t n, int64_t k, int transpose_b, int same_operand,
+                             int transpose_out, int* plan) {
+    VIOLA_CHECK_ARG(plan && batch >= 0 && m >= 0 && n >= 0 && k >= 0);
+    const void* const one = reinterpret_cast<const void*>(uintptr_t(4096));          // stand-ins: aligned, equal or not
+    const void* const two = reinterpret_cast<const void*>(uintptr_t(8192));
+    NsArgs probe{static_cast<const uint16_t*>(one), static_cast<const uint16_t*>(same_operand ? one : two), nullptr, nullptr, nullptr,
+                 batch, m, n, k, 0.0f, transpose_out, ns_is_mirrored(one, same_operand ? one : two, transpose_b, m, n, transpose_out), 0, 0, 0};
+    static const int shapes[6][2] = {{NBM, NBN}, {64, 64}, {128, 64}, {128, 128}, {192, 192}, {384, 192}};
+    const NsTile tile = batch > 0 && m > 0 && n > 0 && ns_fast_takes(probe) ? ns_choose_tile(batch, m, n, probe.symmetric != 0) : NS_TILE_GENERIC;
+    plan[0] = shapes[tile][0];
+    plan[1] = shapes[tile][1];
+    plan[2] = tile != NS_TILE_GENERIC && probe.symmetric;
+    plan[3] = (int)tile;
+    return 0;
+}
+
 extern "C" int viola_ns_gemm(const void* a, const void* bmat, const void* residual, void* out, int dtype, int transpose_b,
                              int epilogue, int64_t batch, int64_t m, int64_t n, int64_t k, float add_diag, void* out_diag,
                              int transpose_out, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG((dtype == VIOLA_BF16 || dtype == VIOLA_F16) && epilogue >= 0 && epilogue <= 2);
     VIOLA_CHECK_ARG(batch >= 0 && m >= 0 && n >= 0 && k >= 0);
     if (batch == 0 || m == 0 || n == 0) return 0;
@@ -545,7 +567,7 @@ extern "C" int viola_ns_gemm(const void* a, const void* bmat, const void* residu
     if (k > 0) {
         NsArgs fast{static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(bmat), static_cast<const uint16_t*>(residual),
                     static_cast<uint16_t*>(out), static_cast<uint16_t*>(out_diag), batch, m, n, k, add_diag, transpose_out,
-                    transpose_b && a == bmat && m == n, 0, 0, 0};
+                    ns_is_mirrored(a, bmat, transpose_b, m, n, transpose_out), 0, 0, 0};
         if (launch_ns_gemm_fast(fast, dtype == VIOLA_BF16, !transpose_b, epilogue, stream)) return viola_launch_status();
     }
     const int64_t gx = (n + NBN - 1) / NBN, gy = (m + NBM - 1) / NBM;
@@ -567,7 +589,7 @@ extern "C" int viola_ns_gemm(const void* a, const void* bmat, const void* residu
 
 extern "C" int viola_ns_prepare(const void* in, int in_dtype, void* out, int dtype, int64_t batch, int64_t rows,
                                 int64_t cols, float* workspace, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG((dtype == VIOLA_BF16 || dtype == VIOLA_F16) && viola_is_float(in_dtype));
     VIOLA_CHECK_ARG(batch >= 0 && rows >= 0 && cols >= 0 && batch <= 65535 && (rows + 31) / 32 <= 65535);
     if (batch == 0 || rows == 0 || cols == 0) return 0;

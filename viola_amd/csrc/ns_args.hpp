@@ -19,6 +19,12 @@ struct NsArgs {
     int64_t tiles;              // batch * tiles_m * tiles_n
 };
 
+// Tile shapes of the tiled kernel (rows x columns of output per block); NS_TILE_GENERIC is the kernel in ns.hip that
+// takes every shape the tiled one refuses.
+enum NsTile { NS_TILE_GENERIC = 0, NS_TILE_64x64 = 1, NS_TILE_128x64 = 2, NS_TILE_128x128 = 3, NS_TILE_192x192 = 4, NS_TILE_384x192 = 5 };
+NsTile ns_choose_tile(int64_t batch, int64_t m, int64_t n, bool symmetric);
+bool ns_fast_takes(const NsArgs& args);
+
 // Launches the tiled kernel when the shape qualifies (16-byte aligned rows, k and n multiples of 8,
 // one matrix below 2 GiB); returns false without launching otherwise.
 bool launch_ns_gemm_fast(const NsArgs& args, bool is_bf16, bool b_kn, int epilogue, hipStream_t stream);

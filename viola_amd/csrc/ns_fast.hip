@@ -415,36 +415,52 @@ static void launch_tiles(NsArgs p, int epilogue, hipStream_t stream) {
     else VIOLA_LAUNCH((ns_gemm_fast<IS_BF16, B_KN, 2, WM, WN, WAVES_M, WAVES_N, SBK, STAGES>), dim3(grid), dim3(THREADS), 0, stream, p);
 }
 
-template <bool IS_BF16, bool B_KN>
-static void launch_shape(const NsArgs& p, int epilogue, hipStream_t stream) {
-    // Every tile shape of ns_gemm_fast gives an output element the same arithmetic (k walked in steps of 16 into one
-    // FP32 accumulator, rounded once), so the choice below is about filling the GPU only and may look at the batch.
-    auto area = [&](int64_t tm, int64_t tn) { return ((p.m + tm - 1) / tm) * ((p.n + tn - 1) / tn) * tm * tn; };
+// Which tile shape a product runs on. Every shape of ns_gemm_fast gives an output element the same arithmetic (k walked
+// in steps of 16 into one FP32 accumulator, rounded once), so the choice is about filling the GPU only and may look at
+// the batch.
+NsTile ns_choose_tile(int64_t batch, int64_t m, int64_t n, bool symmetric) {
+    auto area = [&](int64_t tm, int64_t tn) { return ((m + tm - 1) / tm) * ((n + tn - 1) / tn) * tm * tn; };
     auto blocks = [&](int64_t tm, int64_t tn) {
-        const int64_t rows = (p.m + tm - 1) / tm, cols = (p.n + tn - 1) / tn;
-        return p.batch * (p.symmetric ? cols * (cols + 1) / 2 : rows * cols);
+        const int64_t rows = (m + tm - 1) / tm, cols = (n + tn - 1) / tn;
+        return batch * (symmetric ? cols * (cols + 1) / 2 : rows * cols);
     };
     // 192-wide tiles move a third less operand data per flop; take them unless their padding costs more
     // than that (1152 = 6 x 192 and its multiples fit exactly)
     const bool wide = area(192, 192) * 20 <= area(128, 128) * 21 && blocks(192, 192) >= NS_FILL;
     // 384 x 192 blocks with whole-line loads when they fit as well as the 192s and still give every CU a few tiles
     // (a Gram product keeps square tiles for its mirrored stores)
-    const bool big = wide && !p.symmetric && area(384, 192) <= area(192, 192) && blocks(384, 192) >= 3 * 256;
-    if (big) launch_tiles<IS_BF16, B_KN, 3, 3, 4, 2, 64, 2>(p, epilogue, stream);
-    else if (wide) launch_tiles<IS_BF16, B_KN, 3, 3, 2, 2, 32, 3>(p, epilogue, stream);
-    else if (blocks(128, 128) >= NS_FILL) launch_tiles<IS_BF16, B_KN, 2, 2, 2, 2, 32, 3>(p, epilogue, stream);
+    const bool big = wide && !symmetric && area(384, 192) <= area(192, 192) && blocks(384, 192) >= 3 * 256;
+    if (big) return NS_TILE_384x192;
+    if (wide) return NS_TILE_192x192;
+    if (blocks(128, 128) >= NS_FILL) return NS_TILE_128x128;
     // fewer 128 x 128 tiles than compute units (one matrix of a thousand rows): smaller tiles put more of the chip to work
-    else if (!p.symmetric && blocks(128, 64) >= NS_FILL) launch_tiles<IS_BF16, B_KN, 2, 1, 2, 2, 32, 3>(p, epilogue, stream);
-    else launch_tiles<IS_BF16, B_KN, 1, 1, 2, 2, NS_SMALL_SBK, NS_SMALL_STAGES>(p, epilogue, stream);
+    if (!symmetric && blocks(128, 64) >= NS_FILL) return NS_TILE_128x64;
+    return NS_TILE_64x64;
 }
 
-bool launch_ns_gemm_fast(const NsArgs& p, bool is_bf16, bool b_kn, int epilogue, hipStream_t stream) {
+template <bool IS_BF16, bool B_KN>
+static void launch_shape(const NsArgs& p, int epilogue, hipStream_t stream) {
+    switch (ns_choose_tile(p.batch, p.m, p.n, p.symmetric != 0)) {
+        case NS_TILE_384x192: launch_tiles<IS_BF16, B_KN, 3, 3, 4, 2, 64, 2>(p, epilogue, stream); break;
+        case NS_TILE_192x192: launch_tiles<IS_BF16, B_KN, 3, 3, 2, 2, 32, 3>(p, epilogue, stream); break;
+        case NS_TILE_128x128: launch_tiles<IS_BF16, B_KN, 2, 2, 2, 2, 32, 3>(p, epilogue, stream); break;
+        case NS_TILE_128x64: launch_tiles<IS_BF16, B_KN, 2, 1, 2, 2, 32, 3>(p, epilogue, stream); break;
+        default: launch_tiles<IS_BF16, B_KN, 1, 1, 2, 2, NS_SMALL_SBK, NS_SMALL_STAGES>(p, epilogue, stream); break;
+    }
+}
+
+bool ns_fast_takes(const NsArgs& p) {
     auto aligned = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
     if (p.k % 8 || p.n % 8 || p.k == 0) return false;
     if (!aligned(p.a) || !aligned(p.b) || !aligned(p.out) || !aligned(p.residual) || !aligned(p.out_diag)) return false;
     const int64_t limit = (1ll << 31) - 65536;
     if (p.m * p.k * 2 >= limit || p.n * p.k * 2 >= limit || p.m * p.n * 2 >= limit) return false;
     if (p.batch * ((p.m + 127) / 128) * ((p.n + 127) / 128) >= (1ll << 31) - 8) return false;
+    return true;
+}
+
+bool launch_ns_gemm_fast(const NsArgs& p, bool is_bf16, bool b_kn, int epilogue, hipStream_t stream) {
+    if (!ns_fast_takes(p)) return false;
     if (is_bf16) { if (b_kn) launch_shape<true, true>(p, epilogue, stream); else launch_shape<true, false>(p, epilogue, stream); }
     else { if (b_kn) launch_shape<false, true>(p, epilogue, stream); else launch_shape<false, false>(p, epilogue, stream); }
     return true;

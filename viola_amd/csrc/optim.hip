@@ -377,7 +377,7 @@ extern "C" int viola_momentum_update(const void* grad, int grad_dtype, const voi
                                      float inv_loss_scale, int nesterov, int granularity, int tile_size, int64_t planes,
                                      int64_t rows, int64_t cols, int tr, int tc, int rounding, int64_t rounding_step,
                                      int64_t rounding_key, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_float(grad_dtype) && n >= 0 && (granularity == 0 || granularity == 1));
     VIOLA_CHECK_ARG(rounding == VIOLA_NEAREST || rounding == VIOLA_STOCHASTIC);
     if (n == 0) return 0;
@@ -433,7 +433,7 @@ extern "C" int viola_momentum_update(const void* grad, int grad_dtype, const voi
 extern "C" int viola_momentum_update_table(const int64_t* table, int64_t tensors, int64_t tiles, int grad_dtype, int tile_size,
                                            float beta, float inv_loss_scale, int nesterov, int rounding, int64_t rounding_step,
                                            viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_float(grad_dtype) && tensors >= 0 && tensors <= 65535 && tiles >= 0 && (tiles + 3) / 4 < (1ll << 31));
     VIOLA_CHECK_ARG(tile_size == 256 || tile_size == 512 || tile_size == 1024);
     VIOLA_CHECK_ARG(rounding == VIOLA_NEAREST || rounding == VIOLA_STOCHASTIC);
@@ -455,7 +455,7 @@ extern "C" int viola_momentum_update_table(const int64_t* table, int64_t tensors
 
 extern "C" int viola_weight_update_table(const int64_t* table, int64_t tensors, int64_t count, int grad_dtype, float lr,
                                          float decay, float update_scale, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_float(grad_dtype) && tensors >= 0 && tensors <= 65535 && count >= 0 && count % 4 == 0);
     if (tensors == 0 || count == 0) return 0;
     VIOLA_CHECK_ARG(table);
@@ -471,7 +471,7 @@ extern "C" int viola_weight_update_table(const int64_t* table, int64_t tensors, 
 extern "C" int viola_weight_update(void* weight, int weight_dtype, const void* grad, int grad_dtype, int64_t n, float lr,
                                    float decay, float update_scale, int rounding, int64_t rounding_step,
                                    int64_t rounding_key, int64_t offset, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_float(weight_dtype) && viola_is_float(grad_dtype) && n >= 0);
     if (n == 0) return 0;
     VIOLA_CHECK_ARG(weight && grad);
@@ -499,7 +499,7 @@ extern "C" int viola_adam_update(void* weight, int weight_dtype, const void* gra
                                  int state_dtype, int64_t n, float lr, float decay, float b1, float b2, float inv_c1,
                                  float inv_c2, float eps, int rounding, int64_t rounding_step, int64_t rounding_key,
                                  int64_t offset, int adamw, int maximize, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_float(weight_dtype) && viola_is_float(grad_dtype) && viola_is_float(state_dtype) && n >= 0);
     if (n == 0) return 0;
     VIOLA_CHECK_ARG(weight && grad && first && second);
@@ -515,7 +515,7 @@ extern "C" int viola_adam_update_table(const int64_t* table, int64_t tensors, in
                                        int state_dtype, float lr, float decay, float b1, float b2, float inv_c1, float inv_c2,
                                        float eps, int rounding, int64_t rounding_step, int adamw, int maximize,
                                        viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_float(weight_dtype) && viola_is_float(grad_dtype) && viola_is_float(state_dtype));
     VIOLA_CHECK_ARG(tensors >= 0 && tensors <= 65535 && max_count >= 0);
     if (tensors == 0 || max_count == 0) return 0;
@@ -532,7 +532,7 @@ extern "C" int viola_adam_update_table(const int64_t* table, int64_t tensors, in
 
 extern "C" int viola_copy_scaled(const void* update, int update_dtype, void* out, int out_dtype, int64_t src, int64_t dst,
                                  int64_t count, float scale, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_float(update_dtype) && viola_is_float(out_dtype) && src >= 0 && dst >= 0 && count >= 0);
     if (count == 0) return 0;
     VIOLA_CHECK_ARG(update && out);
@@ -543,7 +543,7 @@ extern "C" int viola_copy_scaled(const void* update, int update_dtype, void* out
 extern "C" int viola_momentum_dequantize(const void* q, const float* scale, float* out, int64_t n, int granularity,
                                          int tile_size, int64_t planes, int64_t rows, int64_t cols, int tr, int tc,
                                          viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(n >= 0 && (granularity == 0 ? tile_size > 0 : (rows > 0 && cols > 0 && tr > 0 && tc > 0 && planes * rows * cols == n)));
     if (n == 0) return 0;
     VIOLA_CHECK_ARG(q && scale && out);

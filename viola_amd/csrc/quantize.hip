@@ -901,7 +901,7 @@ extern "C" int viola_group_quantize(const void* x, int x_dtype, int64_t rows, in
                                     void* scale_, int gr, int gc, float limit, int transposed,
                                     const void* source_scale_, int source_gr, int source_gc, int scale_format,
                                     viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     float* scale = static_cast<float*>(scale_);
     const float* source_scale = static_cast<const float*>(source_scale_);
     VIOLA_CHECK_ARG(scale_format == VIOLA_SCALE_F32 || scale_format == VIOLA_SCALE_E8M0);
@@ -926,7 +926,7 @@ extern "C" int viola_group_quantize(const void* x, int x_dtype, int64_t rows, in
 extern "C" int viola_group_quantize_dual(const void* x, int x_dtype, int64_t rows, int64_t cols, void* q, void* scale_,
                                          void* qt, void* scale_t_, int q_dtype, int gc, float limit,
                                          float* column_partial, int scale_format, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     float* scale = static_cast<float*>(scale_);
     float* scale_t = static_cast<float*>(scale_t_);
     VIOLA_CHECK_ARG(scale_format == VIOLA_SCALE_F32 || scale_format == VIOLA_SCALE_E8M0);
@@ -950,7 +950,7 @@ extern "C" int viola_group_quantize_dual(const void* x, int x_dtype, int64_t row
 extern "C" int viola_gated_quantize_dual(const void* z, int z_dtype, int64_t rows, int64_t cols, int activation, void* q,
                                          void* scale, void* qt, void* scale_t, int q_dtype, int gc, float limit,
                                          int scale_format, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(scale_format == VIOLA_SCALE_F32 || scale_format == VIOLA_SCALE_E8M0);
     VIOLA_CHECK_ARG(activation == VIOLA_SILU || activation == VIOLA_GELU || activation == VIOLA_RELU);
     VIOLA_CHECK_ARG(viola_is_fp8(q_dtype) && viola_is_float(z_dtype) && rows >= 0 && cols >= 0 && limit > 0.0f);
@@ -979,7 +979,7 @@ extern "C" int viola_gated_quantize_dual(const void* z, int z_dtype, int64_t row
 
 extern "C" int viola_column_reduce(const float* partial, int64_t parts, int64_t cols, void* out, int out_dtype,
                                    viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_float(out_dtype) && parts >= 0 && cols >= 0);
     if (cols == 0) return 0;
     VIOLA_CHECK_ARG(out && (parts == 0 || partial));
@@ -994,7 +994,7 @@ extern "C" int viola_varlen_quantize_transposed(const void* x, int x_dtype, int6
                                                 const int64_t* offsets, const int64_t* poffsets, int groups,
                                                 int64_t t_total, void* qt, float* scale_t, int q_dtype, float limit,
                                                 void* q, float* scale, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_fp8(q_dtype) && viola_is_float(x_dtype) && rows >= 0 && cols >= 0 && groups > 0);
     VIOLA_CHECK_ARG(t_total >= 0 && t_total % 32 == 0 && limit > 0.0f);
     if (t_total == 0 || cols == 0) return 0;
@@ -1013,7 +1013,7 @@ extern "C" int viola_varlen_quantize_transposed(const void* x, int x_dtype, int6
 
 extern "C" int viola_group_dequantize(const void* q, int q_dtype, const float* scale, int64_t rows, int64_t cols, int gr,
                                       int gc, float* out, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_fp8(q_dtype) && rows >= 0 && cols >= 0 && gr > 0 && gc > 0);
     if (rows == 0 || cols == 0) return 0;
     VIOLA_CHECK_ARG(q && scale && out);
@@ -1028,7 +1028,7 @@ extern "C" int viola_group_dequantize(const void* q, int q_dtype, const float* s
 
 extern "C" int viola_block_transpose(const void* x, void* out, int64_t rows, int64_t cols, const void* scale, void* scale_out,
                                      int gr, int gc, int scale_format, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(rows >= 0 && cols >= 0 && gr > 0 && gc > 0 && (scale_format == VIOLA_SCALE_F32 || scale_format == VIOLA_SCALE_E8M0));
     if (rows == 0 || cols == 0) return 0;
     VIOLA_CHECK_ARG(x && out && scale && scale_out && (rows + 63) / 64 <= 65535);
@@ -1043,7 +1043,7 @@ extern "C" int viola_block_transpose(const void* x, void* out, int64_t rows, int
 }
 
 extern "C" int viola_fp8_transpose(const void* x, void* out, int64_t batch, int64_t rows, int64_t cols, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(batch >= 0 && rows >= 0 && cols >= 0);
     if (batch == 0 || rows == 0 || cols == 0) return 0;
     VIOLA_CHECK_ARG(x && out && (rows + 63) / 64 <= 65535 && batch <= 65535);

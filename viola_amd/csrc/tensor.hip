@@ -349,7 +349,7 @@ static int launch_tensor_quantize(const void* x, const float* scale, void* q, vo
 using namespace viola;
 
 extern "C" int viola_tensor_amax(const void* x, int x_dtype, int64_t n, float* maxima, int64_t parts, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_float(x_dtype) && n >= 0 && parts > 0 && parts <= 65535 && maxima && (n == 0 || x));
     const dim3 grid((unsigned)parts);
     if (x_dtype == VIOLA_F32) VIOLA_LAUNCH(tensor_amax_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(x), n, maxima);
@@ -360,7 +360,7 @@ extern "C" int viola_tensor_amax(const void* x, int x_dtype, int64_t n, float* m
 
 extern "C" int viola_tensor_scale(const float* maxima, int64_t parts, float* history, int history_len, int64_t index,
                                   int delayed, float limit, float* scale, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(maxima && parts > 0 && history && history_len > 0 && index >= 0 && limit > 0.0f && scale);
     VIOLA_LAUNCH(tensor_scale_kernel, dim3(1), dim3(256), 0, stream, maxima, parts, history, history_len, index, delayed, limit, scale);
     return viola_launch_status();
@@ -368,7 +368,7 @@ extern "C" int viola_tensor_scale(const float* maxima, int64_t parts, float* his
 
 extern "C" int viola_tensor_amax_columns(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t slices, float* maxima,
                                          float* column_partial, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_float(x_dtype) && rows > 0 && cols > 0 && slices > 0 && slices <= 65535 && x && maxima && column_partial);
     const int piece = 16 / viola_dtype_size(x_dtype);
     VIOLA_CHECK_ARG(cols % piece == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(column_partial) % 16 == 0);
@@ -433,7 +433,7 @@ extern "C" int viola_rotation_quantize(const void* x, int x_dtype, int64_t rows,
 
 extern "C" int viola_rotation_amax(const void* x, int x_dtype, int64_t rows, int64_t cols, float* maxima, int64_t parts,
                                    viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_float(x_dtype) && rows > 0 && cols > 0 && x && maxima && (rows + 63) / 64 <= 65535);
     const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64));
     VIOLA_CHECK_ARG(parts == (int64_t)grid.x * grid.y);
@@ -445,7 +445,7 @@ extern "C" int viola_rotation_amax(const void* x, int x_dtype, int64_t rows, int
 }
 
 extern "C" int viola_rotation_inverse(void* x, int x_dtype, int64_t rows, int64_t cols, viola_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    hipStream_t stream = viola_enter(stream_);
     VIOLA_CHECK_ARG(viola_is_float(x_dtype) && rows >= 0 && cols >= 0);
     if (rows == 0 || cols == 0) return 0;
     VIOLA_CHECK_ARG(x && (rows + 63) / 64 <= 65535);

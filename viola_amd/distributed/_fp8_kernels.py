@@ -34,3 +34,41 @@ def unpack(packet, out, tile_size, fp8_dtype, *, reduce=False):
     assert out.dtype == torch.float32 and out.is_contiguous()
     _lib.call("viola_comm_unpack", _lib.ptr(packet), _lib.ptr(out), out.numel(), rows, groups, tile_size,
               _lib.code(fp8_dtype), int(reduce))
+
+
+def _table(rows, device, cache):
+    from ..optim._kernels import _device_table
+    return _device_table(rows, device, cache)
+
+
+def pack_many(sources, packets, tile_size, fp8_dtype, *, cache=None):
+    """pack() for a list of buckets in ONE launch (the reference drains its buckets one launch at a time,
+    viola/distributed/gradients.py:101-125); same bytes as bucket-by-bucket calls, which is also what shapes
+    the table kernel does not take fall back to. cache: a dict that keeps the device-side table between calls."""
+    geometry = [_geometry(packet, tile_size) for packet in packets]
+    assert len(sources) == len(packets) and all(s.dtype == torch.float32 and s.is_contiguous() for s in sources)
+    together = tile_size == 256 and len(packets) > 1 and all(s.data_ptr() % 16 == 0 for s in sources)
+    if together:
+        rows = [(s.data_ptr(), s.numel(), p.data_ptr(), r, g, 0, 0, 0) for s, p, (r, g) in zip(sources, packets, geometry)]
+        table = _table(rows, packets[0].device, cache)
+        status = _lib.call("viola_comm_pack_table", _lib.ptr(table), len(rows), max(r * g for r, g in geometry), tile_size,
+                           _lib.code(fp8_dtype), unsupported_ok=True)
+        together = status == 0
+    if not together:
+        for source, packet in zip(sources, packets):
+            pack(source, packet, tile_size, fp8_dtype)
+
+
+def unpack_many(packets, outs, tile_size, fp8_dtype, *, reduce=False, cache=None):
+    """unpack() for a list of buckets in ONE launch; same values as bucket-by-bucket calls."""
+    geometry = [_geometry(packet, tile_size) for packet in packets]
+    assert len(outs) == len(packets) and all(o.dtype == torch.float32 and o.is_contiguous() for o in outs)
+    capacity = [(1 if reduce else r) * g * tile_size for r, g in geometry]
+    assert all(o.numel() <= c for o, c in zip(outs, capacity))
+    if len(packets) > 1 and all(o.data_ptr() % 16 == 0 for o in outs):
+        rows = [(p.data_ptr(), o.numel(), o.data_ptr(), r, g, 0, 0, 0) for p, o, (r, g) in zip(packets, outs, geometry)]
+        table = _table(rows, packets[0].device, cache)
+        _lib.call("viola_comm_unpack_table", _lib.ptr(table), len(rows), max(capacity), tile_size, _lib.code(fp8_dtype), int(reduce))
+        return
+    for packet, out in zip(packets, outs):
+        unpack(packet, out, tile_size, fp8_dtype, reduce=reduce)

@@ -28,6 +28,14 @@ def gemm(a, b, sa, sb, *, layer, out_dtype, activation, backward=False, aux=None
     if getattr(layer, "accum_dtype", "fp32") == "fp16":
         # the FP16-accumulator model exists for the plain product: the same values as a fused epilogue from the plain
         # GEMM (which rounds g, u and d to out_dtype as the epilogue does) and the elementwise kernels
+        if not layer._grouped_scaling:
+            # Per-tensor scales: the reference's MLP kernel clears its FP16 partial every accum_block_size k counted in
+            # 32-k steps (viola/nn/_mlp_kernels.py:19-20,129-130), its Linear kernel, which the plain product here
+            # models, after whole 64-k chunks (viola/nn/_linear_kernels.py:150-153). The two agree for 32 and for
+            # multiples of 64; other periods are refused rather than computed with the wrong clearing points.
+            block = getattr(layer, "accum_block_size", 0)
+            assert block in (0, 32) or block % 64 == 0, \
+                "MLP with per-tensor scaling and accum_dtype='fp16' takes accum_block_size 0, 32 or a multiple of 64"
         plain = (lambda bias_: layer._group_gemm(a, b, sa, sb, tuple(group_a or layer.input_group_shape),
                                                  tuple(group_b or layer.weight_group_shape), out_dtype=out_dtype, bias=bias_)) \
             if layer._grouped_scaling else (lambda bias_: layer._tensor_gemm(a, b, sa, sb, out_dtype=out_dtype, bias=bias_))

@@ -24,6 +24,16 @@ def _matmul(a, b, *, transpose_b=False, residual=None, epilogue=0, add_diag=None
     return out if add_diag is None else (out, second)
 
 
+def plan(batch, m, n, k, *, transpose_b=False, same_operand=False, transpose_out=False):
+    """The tile shape one chain GEMM of this size runs on (the counterpart of the reference's timed `plan`,
+    viola/optim/_orthogonalize_kernels.py:114): host arithmetic of the library, usable without a GPU."""
+    import ctypes
+    out = (ctypes.c_int * 4)()
+    status = _lib.library().viola_ns_plan(batch, m, n, k, int(transpose_b), int(same_operand), int(transpose_out), out)
+    assert status == 0, status
+    return dict(bm=out[0], bn=out[1], mirrored=bool(out[2]), kernel=("generic", "64x64", "128x64", "128x128", "192x192", "384x192")[out[3]])
+
+
 def prepare(matrix, dtype):
     """[B, rows, cols] (any float dtype) -> dtype, transposed if tall, divided by (||.||_F + 1e-7)."""
     batch, rows, cols = matrix.shape
