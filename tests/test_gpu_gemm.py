@@ -240,20 +240,3 @@ def test_varlen_segmented_quantizer_rowwise_byproduct(counts, dtype):
             assert torch.equal(got, oq.view(torch.uint8))
             assert torch.equal(st[:, padded[group] // 32:padded[group] // 32 + (count + 31) // 32].cpu(), os_)
 
-
-def test_chunk_loop_probe_runs_and_checks_its_arguments():
-    """viola_probe_chunk_loop (measurement support): every combination of parts launches and finishes; arguments that
-    would send its loads outside `src` are refused before anything is launched."""
-    blocks, chunks, lda = 16, 8, 1024
-    out = torch.empty(blocks * 256, device="cuda")
-    src = torch.randint(0, 255, (72 * 128 * lda,), device="cuda", dtype=torch.uint8)
-    for parts in range(8):
-        _lib.call("viola_probe_chunk_loop", parts, _lib.ptr(out), _lib.ptr(src), src.numel(), blocks, chunks, lda)
-    torch.cuda.synchronize()
-    lib = _lib.library()
-    assert lib.viola_probe_chunk_loop(4, _lib.ptr(out), _lib.ptr(src), src.numel() - 1, blocks, chunks, lda, _lib.stream()) == -1
-    assert lib.viola_probe_chunk_loop(4, _lib.ptr(out), None, 0, blocks, chunks, lda, _lib.stream()) == -1
-    assert lib.viola_probe_chunk_loop(0, _lib.ptr(out), None, 0, blocks, chunks + 1, lda, _lib.stream()) == -1
-    assert lib.viola_probe_chunk_loop(8, _lib.ptr(out), None, 0, blocks, chunks, lda, _lib.stream()) == -1
-    assert lib.viola_probe_chunk_loop(0, _lib.ptr(out), None, 0, blocks, chunks, lda, _lib.stream()) == 0
-    torch.cuda.synchronize()
