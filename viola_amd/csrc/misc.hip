@@ -69,17 +69,78 @@ __global__ __launch_bounds__(256) void comm_pack256_kernel(const float* __restri
     comm_pack256_tile<TQ>(x, n, packet, groups, stride, unit, threadIdx.x % WAVE);
 }
 
+// max over the 16 lanes of a DPP row: quad permutes, then the row's two mirrors (lane i with 7 - i, then with 15 - i), all
+// inside the vector ALU (a shuffle goes through the LDS crossbar and its wait)
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, quad_xor<1>(v));
+    v = fmaxf(v, quad_xor<2>(v));
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x141, 0xf, 0xf, true)));   // row_half_mirror
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x140, 0xf, 0xf, true)));   // row_mirror
+    return v;
+}
+
+// tile == 256 for launches with many tiles: sixteen lanes per tile (lane j takes floats 4 j + 64 i, i = 0 .. 3, so every
+// load instruction of a 16-lane row covers 256 contiguous bytes and a lane has four loads in flight), a wavefront four
+// tiles at a time, the blocks walking the tiles with the grid's stride. Same bytes as comm_pack256_tile.
+template <typename TQ>
+__device__ __forceinline__ void comm_pack256_rows(const float* __restrict__ x, int64_t n, uint8_t* __restrict__ packet, int64_t rows,
+                                                  int64_t groups, int64_t stride, int64_t first_block, int64_t block_step) {
+    const int sub = threadIdx.x % 16;
+    const int64_t units = rows * groups;
+    for (int64_t unit = first_block * 16 + threadIdx.x / 16; unit < units; unit += block_step * 16) {
+        const int64_t row = unit / groups, group = unit - row * groups;
+        const int64_t base = unit * 256 + sub * 4;
+        float v[4][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int64_t at = base + 64 * i;
+            if (at + 3 < n) {
+                const float4 raw = *reinterpret_cast<const float4*>(x + at);
+                v[i][0] = raw.x; v[i][1] = raw.y; v[i][2] = raw.z; v[i][3] = raw.w;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[i][e] = at + e < n ? x[at + e] : 0.0f;
+            }
+        }
+        float amax = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) amax = fmaxf(amax, v[i][e] != v[i][e] ? __uint_as_float(0x7f800000u) : fabsf(v[i][e]));
+        amax = row16_max(amax);
+        const float s = scale_of(amax, fp8_traits<TQ>::max);
+        const SharedDivisor divisor(s, 0.0f);                    // declines an infinite scale (a tile with a NaN or an Inf)
+        uint8_t* codes = packet + row * stride + group * 256 + sub * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t w = 0;
+            if (divisor.fast) {
+                w = hw_encode4<TQ>(divisor.quotient(v[i][0]), divisor.quotient(v[i][1]), divisor.quotient(v[i][2]), divisor.quotient(v[i][3]));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) w |= (uint32_t)from_f32<TQ>(v[i][e] / s).bits << (8 * e);
+            }
+            *reinterpret_cast<uint32_t*>(codes + 64 * i) = w;
+        }
+        if (sub == 0) reinterpret_cast<float*>(packet + row * stride + groups * 256)[group] = s;
+    }
+}
+
+template <typename TQ>
+__global__ __launch_bounds__(256) void comm_pack256_rows_kernel(const float* __restrict__ x, int64_t n, uint8_t* __restrict__ packet,
+                                                                 int64_t rows, int64_t groups, int64_t stride) {
+    comm_pack256_rows<TQ>(x, n, packet, rows, groups, stride, blockIdx.x, gridDim.x);
+}
+
 // Many buckets, one launch: row blockIdx.y of the table names the bucket {x, n, packet, rows, groups, -, -, -}.
 constexpr int COMM_ROW = 8;                                                   // int64 words per table row
 template <typename TQ>
 __global__ __launch_bounds__(256) void comm_pack256_table_kernel(const int64_t* __restrict__ table) {
     const int64_t* bucket = table + (int64_t)blockIdx.y * COMM_ROW;
     const int64_t n = bucket[1], rows = bucket[3], groups = bucket[4];
-    const int64_t unit = (int64_t)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
-    if (unit >= rows * groups) return;
     const int64_t stride = (groups * (256 + 4) + 15) / 16 * 16;
-    comm_pack256_tile<TQ>(reinterpret_cast<const float*>(bucket[0]), n, reinterpret_cast<uint8_t*>(bucket[2]), groups, stride, unit,
-                          threadIdx.x % WAVE);
+    comm_pack256_rows<TQ>(reinterpret_cast<const float*>(bucket[0]), n, reinterpret_cast<uint8_t*>(bucket[2]), rows, groups, stride,
+                          blockIdx.x, gridDim.x);
 }
 
 template <typename TQ>
@@ -119,38 +180,61 @@ template <> __device__ __forceinline__ void decode4<e5m2_t>(uint32_t word, float
 // hardware decoders equal the table decode on all 256 codes (checked by the device self test below).
 template <typename TQ, bool REDUCE>
 __device__ __forceinline__ void comm_unpack_quads(const uint8_t* __restrict__ packet, float* __restrict__ out, int64_t n, int64_t rows,
-                                                  int64_t width, int tile_shift, int64_t stride, int64_t first, int64_t step) {
+                                                  int64_t width, int tile_shift, int64_t stride, int64_t first_block, int64_t block_step) {
     const int64_t quads_per_row = width / 4;
     const int64_t total = (REDUCE ? 1 : rows) * quads_per_row;
-    for (int64_t quad = first; quad < total; quad += step) {
-        const int64_t row = (REDUCE || rows == 1) ? 0 : quad / quads_per_row;
-        const int64_t col = (quad - row * quads_per_row) * 4;
-        const int64_t idx = row * width + col;
-        if (idx >= n) continue;
-        float result[4];
-        if constexpr (REDUCE) {
-            result[0] = result[1] = result[2] = result[3] = 0.0f;
-            for (int64_t rank = 0; rank < rows; ++rank) {
-                const uint8_t* base = packet + rank * stride;
-                const float s = reinterpret_cast<const float*>(base + width)[col >> tile_shift];
-                float v[4];
-                decode4<TQ>(*reinterpret_cast<const uint32_t*>(base + col), v);
+    // a block takes four runs of 256 quads per step: the code words and scales of all four are asked for before the
+    // first is used, so a thread has eight loads in flight; every load and store instruction stays contiguous over the block
+    constexpr int RUNS = 4;
+    for (int64_t chunk = first_block * RUNS * 256; chunk < total; chunk += block_step * RUNS * 256) {
+        uint32_t word[RUNS];
+        float s[RUNS];
+        int64_t index[RUNS];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) { const float term = v[i] * s; result[i] += term; }
+        for (int u = 0; u < RUNS; ++u) {
+            const int64_t quad = chunk + u * 256 + threadIdx.x;
+            const int64_t row = (REDUCE || rows == 1) ? 0 : quad / quads_per_row;
+            const int64_t col = (quad - row * quads_per_row) * 4;
+            index[u] = quad < total ? row * width + col : n;
+            word[u] = 0;
+            s[u] = 0.0f;
+            if (index[u] < n) {
+                if constexpr (REDUCE) {
+                    index[u] = col;                                      // the ranks' rows are summed below
+                } else {
+                    const uint8_t* base = packet + row * stride;
+                    word[u] = *reinterpret_cast<const uint32_t*>(base + col);
+                    s[u] = reinterpret_cast<const float*>(base + width)[col >> tile_shift];
+                }
             }
-        } else {
-            const uint8_t* base = packet + row * stride;
-            const float s = reinterpret_cast<const float*>(base + width)[col >> tile_shift];
-            float v[4];
-            decode4<TQ>(*reinterpret_cast<const uint32_t*>(base + col), v);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) result[i] = v[i] * s;
         }
-        if (idx + 3 < n) {
-            *reinterpret_cast<float4*>(out + idx) = make_float4(result[0], result[1], result[2], result[3]);
-        } else {
-            for (int i = 0; i < 4; ++i)
-                if (idx + i < n) out[idx + i] = result[i];
+#pragma unroll
+        for (int u = 0; u < RUNS; ++u) {
+            const int64_t idx = index[u];
+            if (idx >= n) continue;
+            float result[4];
+            if constexpr (REDUCE) {
+                result[0] = result[1] = result[2] = result[3] = 0.0f;
+                for (int64_t rank = 0; rank < rows; ++rank) {
+                    const uint8_t* base = packet + rank * stride;
+                    const float scale = reinterpret_cast<const float*>(base + width)[idx >> tile_shift];
+                    float v[4];
+                    decode4<TQ>(*reinterpret_cast<const uint32_t*>(base + idx), v);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { const float term = v[i] * scale; result[i] += term; }
+                }
+            } else {
+                float v[4];
+                decode4<TQ>(word[u], v);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) result[i] = v[i] * s[u];
+            }
+            if (idx + 3 < n) {
+                *reinterpret_cast<float4*>(out + idx) = make_float4(result[0], result[1], result[2], result[3]);
+            } else {
+                for (int i = 0; i < 4; ++i)
+                    if (idx + i < n) out[idx + i] = result[i];
+            }
         }
     }
 }
@@ -159,8 +243,7 @@ template <typename TQ, bool REDUCE>
 __global__ __launch_bounds__(256) void comm_unpack_quads_kernel(const uint8_t* __restrict__ packet, float* __restrict__ out,
                                                                  int64_t n, int64_t rows, int64_t width, int tile_shift,
                                                                  int64_t stride) {
-    comm_unpack_quads<TQ, REDUCE>(packet, out, n, rows, width, tile_shift, stride, (int64_t)blockIdx.x * blockDim.x + threadIdx.x,
-                                  (int64_t)gridDim.x * blockDim.x);
+    comm_unpack_quads<TQ, REDUCE>(packet, out, n, rows, width, tile_shift, stride, blockIdx.x, gridDim.x);
 }
 
 // Many buckets, one launch: row blockIdx.y of the table names the bucket {packet, n, out, rows, groups, -, -, -}.
@@ -170,7 +253,7 @@ __global__ __launch_bounds__(256) void comm_unpack_quads_table_kernel(const int6
     const int64_t n = bucket[1], rows = bucket[3], groups = bucket[4];
     const int64_t width = groups * tile, stride = (groups * (tile + 4) + 15) / 16 * 16;
     comm_unpack_quads<TQ, REDUCE>(reinterpret_cast<const uint8_t*>(bucket[0]), reinterpret_cast<float*>(bucket[2]), n, rows, width,
-                                  tile_shift, stride, (int64_t)blockIdx.x * blockDim.x + threadIdx.x, (int64_t)gridDim.x * blockDim.x);
+                                  tile_shift, stride, blockIdx.x, gridDim.x);
 }
 
 
@@ -364,11 +447,26 @@ static unsigned grid_for(int64_t n) {
     return (unsigned)(blocks < 1 ? 1 : blocks > 65536 * 8 ? 65536 * 8 : blocks);
 }
 
+// Blocks for a launch whose blocks walk `steps` steps of work with the grid's stride, `lanes` such walks side by side
+// (buckets): enough blocks to keep every CU's wavefront slots filled a few times over, no more.
+#ifndef COMM_BLOCKS_PER_CU
+#define COMM_BLOCKS_PER_CU 64
+#endif
+#ifndef COMM_ROWS_FROM
+#define COMM_ROWS_FROM 4096                                              // tiles from which one bucket takes the row-per-tile kernel
+#endif
+static unsigned comm_walkers(int64_t steps, int64_t lanes) {
+    const int64_t budget = (256 * COMM_BLOCKS_PER_CU + lanes - 1) / lanes;
+    return (unsigned)(steps < 1 ? 1 : steps < budget ? steps : budget);
+}
+
 template <typename TQ>
 static int launch_pack(const float* x, int64_t n, uint8_t* packet, int64_t rows, int64_t groups, int tile, int64_t stride,
                        hipStream_t stream) {
     const int64_t units = rows * groups;
-    if (tile == 256 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(packet) % 4 == 0) {
+    if (tile == 256 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(packet) % 4 == 0 && units >= COMM_ROWS_FROM) {
+        VIOLA_LAUNCH(comm_pack256_rows_kernel<TQ>, dim3(comm_walkers((units + 15) / 16, 1)), dim3(256), 0, stream, x, n, packet, rows, groups, stride);
+    } else if (tile == 256 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(packet) % 4 == 0) {
         VIOLA_LAUNCH(comm_pack256_kernel<TQ>, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x, n, packet, rows, groups, stride);
     } else if (tile >= 64) {
         VIOLA_LAUNCH((comm_pack_kernel<TQ, 64>), dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, x, n, packet, rows, groups, tile, stride);
@@ -407,7 +505,7 @@ extern "C" int viola_comm_unpack(const void* packet, float* out, int64_t n, int6
     if (reinterpret_cast<uintptr_t>(out) % 16 == 0) {
         const int64_t width = groups * tile;
         const int shift = __builtin_ctz((unsigned)tile);
-        const dim3 grid(grid_for(total / 4));
+        const dim3 grid(comm_walkers((total / 4 + 1023) / 1024, 1));
 #define VIOLA_UNPACK(TQ, REDUCE) VIOLA_LAUNCH((comm_unpack_quads_kernel<TQ, REDUCE>), grid, dim3(256), 0, stream, pk, out, n, rows, width, shift, stride)
         if (fp8_dtype == VIOLA_E4M3) { if (reduce) VIOLA_UNPACK(e4m3_t, true); else VIOLA_UNPACK(e4m3_t, false); }
         else { if (reduce) VIOLA_UNPACK(e5m2_t, true); else VIOLA_UNPACK(e5m2_t, false); }
@@ -426,7 +524,7 @@ extern "C" int viola_comm_pack_table(const int64_t* table, int64_t buckets, int6
     if (buckets == 0 || max_units == 0) return 0;
     VIOLA_CHECK_ARG(table && buckets <= 65535 && (max_units + 3) / 4 < (1ll << 31));
     if (tile != 256) return VIOLA_EUNSUPPORTED;                                    // other tiles: one viola_comm_pack per bucket
-    const dim3 grid((unsigned)((max_units + 3) / 4), (unsigned)buckets);
+    const dim3 grid(comm_walkers((max_units + 15) / 16, buckets), (unsigned)buckets);
     if (fp8_dtype == VIOLA_E4M3) VIOLA_LAUNCH(comm_pack256_table_kernel<e4m3_t>, grid, dim3(256), 0, stream, table);
     else VIOLA_LAUNCH(comm_pack256_table_kernel<e5m2_t>, grid, dim3(256), 0, stream, table);
     return viola_launch_status();
@@ -439,7 +537,7 @@ extern "C" int viola_comm_unpack_table(const int64_t* table, int64_t buckets, in
     if (buckets == 0 || max_elements == 0) return 0;
     VIOLA_CHECK_ARG(table && buckets <= 65535);
     const int shift = __builtin_ctz((unsigned)tile);
-    const dim3 grid(grid_for(max_elements / 4), (unsigned)buckets);
+    const dim3 grid(comm_walkers((max_elements / 4 + 1023) / 1024, buckets), (unsigned)buckets);
 #define VIOLA_UNPACK(TQ, REDUCE) VIOLA_LAUNCH((comm_unpack_quads_table_kernel<TQ, REDUCE>), grid, dim3(256), 0, stream, table, tile, shift)
     if (fp8_dtype == VIOLA_E4M3) { if (reduce) VIOLA_UNPACK(e4m3_t, true); else VIOLA_UNPACK(e4m3_t, false); }
     else { if (reduce) VIOLA_UNPACK(e5m2_t, true); else VIOLA_UNPACK(e5m2_t, false); }
