@@ -40,6 +40,55 @@ def test_linear_gemms_at_8192x1024x4096(name, m, k, n, gb):
     assert torch.equal(g.gemm(qa, qb, sa, sb, (1, 32), gb, out_dtype=torch.bfloat16, bias=bias), (out + bias).bfloat16())
 
 
+@pytest.mark.parametrize("name,m,k,n,gb", [("forward", 8192, 1024, 4096, (32, 32)), ("dgrad", 8192, 4096, 1024, (32, 32)),
+                                          ("wgrad", 4096, 8192, 1024, (1, 32))])
+def test_linear_gemms_at_8192x1024x4096_against_the_cpu_oracle(name, m, k, n, gb):
+    """The same three products held to the CPU oracle itself, on a sample the oracle finishes in seconds: 96 rows of the
+    output spread over the whole matrix (first, last, one per 128-row tile boundary region, random ones) with every
+    column, from the device's own codes and scales (which other tests pin to the oracle's bit for bit); the sum is
+    taken in float64 on the CPU (the reference's witness, viola/nn/_grouped_tuning.py:40-46)."""
+    from oracle import grouped as og
+    from viola_amd.nn import _grouped_kernels as g
+    _, qa, sa = _quantized(m, k, (1, 32), 1)
+    _, qb, sb = _quantized(n, k, gb, 2)
+    bias = torch.randn(n, device="cuda")
+    out = g.gemm(qa, qb, sa, sb, (1, 32), gb, out_dtype=torch.float32, bias=bias)
+    half = g.gemm(qa, qb, sa, sb, (1, 32), gb, out_dtype=torch.bfloat16, bias=bias)
+    generator = torch.Generator().manual_seed(5)
+    rows = torch.cat([torch.tensor([0, 1, 127, 128, m // 2 - 1, m // 2, m - 129, m - 128, m - 1]),
+                      torch.randint(0, m, (87,), generator=generator)]).unique()
+    witness = og.gemm(qa[rows.cuda()].cpu(), qb.cpu(), sa[rows.cuda()].cpu(), sb.cpu(), (1, 32), gb, bias=bias.cpu(), witness=True,
+                      out_dtype=torch.float64)
+    assert rel_l2(out[rows.cuda()], witness) < 2e-5                              # checks/check_grouped_linear.py:36-41
+    assert rel_l2(half[rows.cuda()], witness) < 3e-3
+    assert (out[rows.cuda()].cpu().double() - witness).abs().max() <= 1e-4 * witness.abs().max()
+
+
+@pytest.mark.parametrize("rows,cols", [(8192, 1024), (8192, 4096)])
+def test_dual_quantizer_at_full_size_against_the_cpu_oracle(rows, cols):
+    """X and dY of the benchmark's Linear through the one-read dual-layout quantizer, against the CPU oracle on samples
+    that cover both layouts: whole rows for the row-wise codes and scales (a row's groups depend on that row only) and
+    whole columns for the transposed ones (a column's groups run along the tokens), bit for bit; the column sums the
+    same pass produces against a float64 sum."""
+    from oracle import grouped as og
+    from viola_amd.nn import _grouped_kernels as g
+    torch.manual_seed(6)
+    x = (torch.randn(rows, cols, device="cuda") * torch.exp2(torch.randint(-6, 7, (rows, 1), device="cuda").float())).bfloat16()
+    q, s, qt, st, column_sum = g.quantize_dual(x, E4, (1, 32), column_sum_dtype=torch.float32)
+    generator = torch.Generator().manual_seed(7)
+    some_rows = torch.cat([torch.tensor([0, 31, 32, rows - 1]), torch.randint(0, rows, (60,), generator=generator)]).unique()
+    some_cols = torch.cat([torch.tensor([0, 63, 64, cols - 1]), torch.randint(0, cols, (60,), generator=generator)]).unique()
+    host = x.cpu()
+    want_q, want_s = og.quantize(host[some_rows], E4, (1, 32))
+    assert torch.equal(q[some_rows.cuda()].cpu().view(torch.uint8), want_q.view(torch.uint8))
+    assert torch.equal(s[some_rows.cuda()].cpu(), want_s)
+    want_qt, want_st = og.quantize(host[:, some_cols].contiguous(), E4, (1, 32), transposed=True)
+    assert torch.equal(qt[some_cols.cuda()].cpu().view(torch.uint8), want_qt.view(torch.uint8))
+    assert torch.equal(st[some_cols.cuda()].cpu(), want_st)
+    exact = host.double().sum(0)
+    assert (column_sum.cpu().double() - exact).abs().max() <= 1e-5 * host.double().abs().sum(0).max()
+
+
 def test_linear_module_at_8192x1024x4096():
     import viola_amd
     viola_amd.set_gradient_dtype("bf16")
