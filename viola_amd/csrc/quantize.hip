@@ -439,6 +439,165 @@ __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x
     }
 }
 
+// ------------------------------------------------------------------ 16-bit inputs: both layouts from a 64 x 64 tile
+// A block of 256 threads per tile, one tile per block: eight blocks are resident on a compute unit at 62 registers, and
+// the launch is timed 15 - 25 % below the persistent 128 x 64 kernel above on every shape tried (8192 x 4096 bf16:
+// 27.7 against 36.2 us). Row-wise: thread (row tid / 4, 16 columns) loads 32 bytes, a 32-column group is a pair of
+// lanes; four neighbouring lanes store 64 consecutive bytes of codes. The raw 16-bit values are parked in LDS
+// ([row][64 + 4 values], the four 16-column blocks of a row permuted by row / 16 so that the transposed phase's four
+// row chunks read distinct banks). After one barrier wavefront w takes columns 16 w .. + 15: lane (column lane / 4,
+// rows 16 (lane % 4) .. + 15) reads its 16 values, a 32-row group is again a pair of lanes, and four neighbouring lanes
+// store 64 consecutive bytes of one transposed row (with the group's halves 32 lanes apart instead, the same stores
+// left as 16-byte pieces and the launch took 31 us).
+template <typename TIn, typename TOut>
+__global__ __launch_bounds__(256) void quantize_dual16_tile64(const TIn* __restrict__ x, uint8_t* __restrict__ q,
+                                                               float* __restrict__ scale, uint8_t* __restrict__ qt,
+                                                               float* __restrict__ scale_t, int64_t rows, int64_t cols,
+                                                               float limit, float* __restrict__ column_partial, int e8m0, int xcd_walk) {
+    constexpr int LDV = 64 + 4;                                              // values per parked row (34 dwords)
+    __shared__ __attribute__((aligned(16))) uint16_t park[64 * LDV];
+    const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+    // blocks are dispatched in index order: those in flight together take 32 row tiles of one column tile, then the next
+    // column tile, so the transposed output is written in 2 KB runs per row however wide the matrix is
+    constexpr int64_t BAND = 32;
+    const int64_t tiles_x = (cols + 63) / 64, tiles_y = (rows + 63) / 64;
+    int64_t id = blockIdx.x;
+    if (xcd_walk) {
+        // consecutive block indices go to the eight XCDs in turn: give each XCD one contiguous eighth of the walk, so the
+        // halves of a 128-byte line of the transposed output (two row tiles) meet in one L2
+        const int64_t per_xcd = (tiles_x * tiles_y + 7) / 8;
+        id = (id % 8) * per_xcd + id / 8;
+    }
+    if (id >= tiles_x * tiles_y) return;
+    const int64_t patch = id / (BAND * tiles_x), within = id % (BAND * tiles_x);
+    const int64_t tall = tiles_y - patch * BAND < BAND ? tiles_y - patch * BAND : BAND;
+    const int64_t r0 = (patch * BAND + within % tall) * 64, c0 = within / tall * 64;
+    const int64_t nc = (cols + 31) / 32, nr = (rows + 31) / 32;
+    constexpr uint32_t MAGNITUDE = 0x7fff7fffu, INF16 = std::is_same<TIn, bf16_t>::value ? 0x7f80u : 0x7c00u;
+    const bool clamp_free = limit == fp8_traits<TOut>::max;
+
+    // ---- row-wise
+    const int lr = tid / 4, lc = (tid % 4) * 16;
+    const int64_t row = r0 + lr, col = c0 + lc;
+    uint4 raw[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+    if (row < rows) {
+        if (col < cols) raw[0] = *reinterpret_cast<const uint4*>(x + row * cols + col);          // cols % 8 == 0: whole pieces
+        if (col + 8 < cols) raw[1] = *reinterpret_cast<const uint4*>(x + row * cols + col + 8);
+    }
+    {
+        uint2* mine = reinterpret_cast<uint2*>(&park[lr * LDV + (lc ^ (((lr >> 4) & 3) << 4))]);       // 16-column blocks swapped by row chunk
+        mine[0] = make_uint2(raw[0].x, raw[0].y); mine[1] = make_uint2(raw[0].z, raw[0].w);
+        mine[2] = make_uint2(raw[1].x, raw[1].y); mine[3] = make_uint2(raw[1].z, raw[1].w);
+    }
+    const uint32_t words[8] = {raw[0].x, raw[0].y, raw[0].z, raw[0].w, raw[1].x, raw[1].y, raw[1].z, raw[1].w};
+    float v[16];
+    uint32_t top = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        v[2 * e] = widen16<TIn>(words[e] & 0xffffu);
+        v[2 * e + 1] = widen16<TIn>(words[e] >> 16);
+        top = pk_max_u16(top, words[e] & MAGNITUDE);
+    }
+    top = (top & 0xffffu) > (top >> 16) ? (top & 0xffffu) : (top >> 16);
+    {
+        const uint32_t other = (uint32_t)__builtin_amdgcn_mov_dpp((int)top, 0xB1, 0xf, 0xf, true);   // the pair's other lane
+        top = top > other ? top : other;
+    }
+    float s_row = group_scale(widen16<TIn>(top), limit, e8m0);
+    const SharedDivisor d_row(s_row, top >= INF16 ? __uint_as_float(0x7fc00000u) : 0.0f);
+    uint32_t codes[4];
+    if (__builtin_amdgcn_ballot_w64(!d_row.fast) == 0) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            codes[k] = clamp_free ? fast_encode4_unclamped<TOut>(d_row, v[4 * k], v[4 * k + 1], v[4 * k + 2], v[4 * k + 3])
+                                  : fast_encode4<TOut>(d_row, limit, v[4 * k], v[4 * k + 1], v[4 * k + 2], v[4 * k + 3]);
+    } else {
+        // an Inf or a NaN in some group of the wavefront, or a scale outside the quotient route's domain: the maxima as the
+        // reference's kernel takes them (fmax ignores NaN), true division, software encoder
+        float amax = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(v[e]));
+        amax = fmaxf(amax, quad_xor<1>(amax));
+        s_row = group_scale(amax, limit, e8m0);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            codes[k] = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) codes[k] |= (uint32_t)encode_clamped<TOut>(v[4 * k + e], s_row, limit) << (8 * e);
+        }
+    }
+    if (row < rows && col < cols) {
+        uint8_t* dst = q + row * cols + col;
+        if (col + 16 <= cols && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+            *reinterpret_cast<uint4*>(dst) = make_uint4(codes[0], codes[1], codes[2], codes[3]);
+        } else {
+            *reinterpret_cast<uint2*>(dst) = make_uint2(codes[0], codes[1]);                         // q is 8-byte aligned, cols % 8 == 0
+            if (col + 8 < cols) *reinterpret_cast<uint2*>(dst + 8) = make_uint2(codes[2], codes[3]);
+        }
+        if (tid % 2 == 0) put_scale(scale, row * nc + col / 32, s_row, e8m0);
+    }
+    __syncthreads();
+
+    // ---- transposed: wavefront w takes columns 16 w .. + 15 of the tile; lane = (column lane / 4, rows 16 (lane % 4) .. + 15), so four
+    // neighbouring lanes write 64 consecutive bytes of one transposed row and a 32-row group is a pair of lanes
+    const int tc = wave * 16 + lane / 4, chunk = lane % 4;
+    const int64_t tcol = c0 + tc, trow = r0 + chunk * 16;                    // first of the lane's 16 rows
+    float w[16];
+    uint32_t top_col = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const uint32_t bits = park[(chunk * 16 + i) * LDV + (tc ^ (chunk << 4))];
+        w[i] = widen16<TIn>(bits);
+        const uint32_t magnitude = bits & 0x7fffu;
+        top_col = top_col > magnitude ? top_col : magnitude;
+    }
+    {
+        const uint32_t other = (uint32_t)__builtin_amdgcn_mov_dpp((int)top_col, 0xB1, 0xf, 0xf, true);   // the pair's other lane
+        top_col = top_col > other ? top_col : other;
+    }
+    float s_col = group_scale(widen16<TIn>(top_col), limit, e8m0);
+    const SharedDivisor d_col(s_col, top_col >= INF16 ? __uint_as_float(0x7fc00000u) : 0.0f);
+    uint32_t tcodes[4];
+    if (__builtin_amdgcn_ballot_w64(!d_col.fast) == 0) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            tcodes[k] = clamp_free ? fast_encode4_unclamped<TOut>(d_col, w[4 * k], w[4 * k + 1], w[4 * k + 2], w[4 * k + 3])
+                                   : fast_encode4<TOut>(d_col, limit, w[4 * k], w[4 * k + 1], w[4 * k + 2], w[4 * k + 3]);
+    } else {
+        float amax = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(w[i]));
+        amax = fmaxf(amax, quad_xor<1>(amax));
+        s_col = group_scale(amax, limit, e8m0);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            tcodes[k] = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) tcodes[k] |= (uint32_t)encode_clamped<TOut>(w[4 * k + e], s_col, limit) << (8 * e);
+        }
+    }
+    float sum = 0.0f;
+    if (column_partial) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sum += w[i];
+        const float other = quad_xor<1>(sum);
+        sum = chunk % 2 == 0 ? sum + other : other + sum;                     // rows 0 .. 15 first, then 16 .. 31
+    }
+    if (tcol < cols && trow < rows) {
+        uint8_t* dst = qt + tcol * rows + trow;
+        if (trow + 16 <= rows && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+            *reinterpret_cast<uint4*>(dst) = make_uint4(tcodes[0], tcodes[1], tcodes[2], tcodes[3]);
+        } else {
+            const int count = (int)(rows - trow < 16 ? rows - trow : 16);
+            for (int i = 0; i < count; ++i) dst[i] = (uint8_t)(tcodes[i >> 2] >> (8 * (i & 3)));
+        }
+        if (chunk % 2 == 0) {
+            put_scale(scale_t, tcol * nr + trow / 32, s_col, e8m0);
+            if (column_partial) column_partial[(trow / 32) * cols + tcol] = sum;
+        }
+    }
+}
+
 // ------------------------------------------------------------------ column sums from 32-row partials
 // out[c] = sum over p of partial[p][c] in a fixed order: 8 threads per column each add a contiguous eighth of the
 // parts in ascending order (loads issued eight at a time), then the eighths are added in order.
@@ -859,6 +1018,16 @@ static int launch_dual(const void* x, int64_t rows, int64_t cols, void* q, float
     const TIn* xp = static_cast<const TIn*>(x);
     if constexpr (sizeof(TIn) == 2) {
         if (vec && reinterpret_cast<uintptr_t>(q) % 8 == 0) {
+            const int64_t tiles64 = ((cols + 63) / 64) * ((rows + 63) / 64);
+            if (tiles64 + 8 < (1ll << 31)) {
+                // one to four rounds of resident blocks (eight per compute unit): the XCD-contiguous walk measured faster
+                // (8192 x 4096: 29.7 -> 27.7 us); longer launches are faster with the eight XCDs streaming one region
+                // (16384 x 4096: 68 against 76 us), shorter ones leave XCDs uneven
+                const int xcd_walk = tiles64 >= 2048 && tiles64 <= 8192;
+                VIOLA_LAUNCH((quantize_dual16_tile64<TIn, TOut>), dim3((unsigned)((tiles64 + 7) / 8 * 8)), dim3(256), 0, stream, xp,
+                             static_cast<uint8_t*>(q), scale, static_cast<uint8_t*>(qt), scale_t, rows, cols, limit, column_partial, e8m0, xcd_walk);
+                return viola_launch_status();
+            }
             const int64_t tiles16 = ((cols + 63) / 64) * ((rows + 127) / 128);
             const dim3 grid16((unsigned)(tiles16 < 256 * 6 ? tiles16 : 256 * 6));
             VIOLA_LAUNCH((quantize_dual16<TIn, TOut, true>), grid16, dim3(256), 0, stream, xp, static_cast<uint8_t*>(q), scale,
