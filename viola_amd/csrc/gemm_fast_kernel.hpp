@@ -28,6 +28,9 @@ typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int FBK = 64, FKG = FBK / 32;                           // k bytes and K groups per LDS stage
 constexpr int FTHREADS = 256, FSTAGES = 3;
+#ifndef VIOLA_OUTER_SCALES
+#define VIOLA_OUTER_SCALES 1                                       // row-wise b scales: sa[m] * sb[n] per K group from an fp32 MFMA
+#endif
 #ifndef VIOLA_BIG_STAGES
 #define VIOLA_BIG_STAGES 3                                         // ring depth of the 256 x 256 tile kernels (4 measured the same)
 #endif
@@ -316,7 +319,23 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
 
     // Four 16-register accumulators: two receive the MFMAs of the current pair of (K group, sub-tile) units while the
     // two of the pair before are folded into the totals (across chunk boundaries when CARRY).
-    constexpr bool CARRY = !B_ROWSCALE;
+    // Row-wise b scales: every output element has its own product sa[m] * sb[n] per K group. One
+    // v_mfma_f32_32x32x1_2b_f32 forms the 2 x 32 x 32 products of a pair of units (a sub-tiles 0 and 1 against one b
+    // sub-tile) as an outer product on the matrix pipe, in the accumulators' own layout and rounded exactly as
+    // v_mul_f32 rounds them; the fold is then one FMA per element, as with uniform b scales. The products of a pair are
+    // issued among its MFMAs and read while the next pair's MFMAs run: into the other of two buffers where the registers
+    // allow it (TN = 1), else into the one buffer once the fold before has read it.
+    constexpr bool OUTER = B_ROWSCALE && TM == 2 && VIOLA_OUTER_SCALES;
+    constexpr bool CARRY = !B_ROWSCALE || OUTER;
+    constexpr int PBUF = TN == 1 ? 2 : 1;
+    typedef float f32x32 __attribute__((ext_vector_type(32)));
+    f32x32 prod[PBUF];
+    if constexpr (OUTER) {
+#pragma unroll
+        for (int b = 0; b < PBUF; ++b)
+#pragma unroll
+            for (int r = 0; r < 32; ++r) prod[b][r] = 0.0f;
+    }
     f32x16 acc[4];
     float pending_scale[2] = {0.0f, 0.0f};                                   // sa * sb of the pending pair (uniform b scales)
 #pragma unroll
@@ -377,10 +396,17 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
             for (int j = 0; j < TM; ++j) o.a[kg][j] = *reinterpret_cast<const uint4*>(tile_a + ((rd_a + j * 32 * FBK) ^ (kg * 32)));
 #pragma unroll
             for (int i = 0; i < TN; ++i) o.b[kg][i] = *reinterpret_cast<const uint4*>(tile_b + ((rd_b + (b_sub(i) - b_sub(0)) * FBK) ^ (kg * 32)));
+            if constexpr (OUTER) {                                           // compute() fetches the scales itself
 #pragma unroll
-            for (int j = 0; j < TM; ++j) o.sa[kg][j] = scale_a[kg * BM + a_sub(j) + l32];
+                for (int j = 0; j < TM; ++j) o.sa[kg][j] = 0.0f;
 #pragma unroll
-            for (int i = 0; i < TN; ++i) o.sb[kg][i] = B_ROWSCALE ? 0.0f : scale_b[kg * BM + b_sub(i)];
+                for (int i = 0; i < TN; ++i) o.sb[kg][i] = 0.0f;
+            } else {
+#pragma unroll
+                for (int j = 0; j < TM; ++j) o.sa[kg][j] = scale_a[kg * BM + a_sub(j) + l32];
+#pragma unroll
+                for (int i = 0; i < TN; ++i) o.sb[kg][i] = B_ROWSCALE ? 0.0f : scale_b[kg * BM + b_sub(i)];
+            }
         }
     };
 
@@ -427,6 +453,8 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
             for (int r = 8 * h; r < 8 * h + 8; ++r) {
                 if constexpr (!B_ROWSCALE) {
                     total[i][j][r] = fmaf(acc[buf][r], scale, total[i][j][r]);
+                } else if constexpr (OUTER) {
+                    total[i][j][r] = fmaf(acc[buf][r], prod[slot % PBUF][16 * j + r], total[i][j][r]);
                 } else {
                     const float4 q = sb_q[slot][r / 4];
                     const float sbv = r % 4 == 0 ? q.x : r % 4 == 1 ? q.y : r % 4 == 2 ? q.z : q.w;
@@ -452,7 +480,19 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
                 pkg[h] = prev / (TN * TM); pi[h] = prev / TM % TN; pj[h] = prev % TM;
                 prev_scale[h] = B_ROWSCALE ? (pair > 0 ? o.sa[pkg[h]][pj[h]] : 0.0f) : pending_scale[h];
             }
-            if constexpr (B_ROWSCALE) {
+            // operands of the scale products' MFMA: lanes 0..31 / 32..63 carry the a scales of sub-tile 0 / 1, every lane the
+            // b scale of row l32 of the pair's b sub-tile
+            float outer_a = 0.0f, outer_b = 0.0f;
+            if constexpr (OUTER) {
+                static_assert(PAIRS % 2 == 0, "the two product buffers alternate across chunk boundaries");
+                outer_a = (scale_b - F_SBLOCK / 4)[kg[0] * BM + a_sub(lhi) + l32];
+                outer_b = scale_b[kg[0] * BM + b_sub(ti[0]) + l32];
+            }
+            auto issue_products = [&]() {
+                const f32x32 zero32 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                prod[pair % PBUF] = __builtin_amdgcn_mfma_f32_32x32x1f32(outer_b, outer_a, zero32, 0, 0, 0);
+            };
+            if constexpr (B_ROWSCALE && !OUTER) {
 #pragma unroll
                 for (int r4 = 0; r4 < 4; ++r4)
                     sb_q[pair & 1][r4] = *reinterpret_cast<const float4*>(&scale_b[kg[0] * BM + b_sub(ti[0]) + r4 * 8 + lhi * 4]);
@@ -465,6 +505,11 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
                 else acc[base + h] = mfma32<A_BF8, B_BF8>(as_long(ob.z, ob.w), as_long(oa.z, oa.w), acc[base + h]);
                 if (fold_prev) fold_half(other + (step >> 1), pi[step >> 1], pj[step >> 1], before & 1, step & 1, prev_scale[step >> 1]);
                 asm volatile("" : "+v"(total[pi[step >> 1]][pj[step >> 1]]));
+                if constexpr (OUTER) {
+                    // with two buffers after the second MFMA of the pair (the scales have arrived from LDS by then), with one
+                    // after the last fold that reads it
+                    if (step == (PBUF == 2 ? 1 : 3)) issue_products();
+                }
                 __builtin_amdgcn_sched_barrier(0);
                 between(pair * 4 + step);
             }
@@ -548,7 +593,8 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
         for (int h = 0; h < 2; ++h) {
             const int unit = 2 * last_pair + h, li = unit / TM % TN, lj = unit % TM;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) total[li][lj][r] = fmaf(acc[(last_pair & 1) * 2 + h][r], pending_scale[h], total[li][lj][r]);
+            for (int r = 0; r < 16; ++r)
+                total[li][lj][r] = fmaf(acc[(last_pair & 1) * 2 + h][r], OUTER ? prod[last_pair % PBUF][16 * lj + r] : pending_scale[h], total[li][lj][r]);
         }
     }
 
