@@ -78,7 +78,8 @@ def test_quantize_transposed(in_dtype, fp8, group, shape):
 
 
 @pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float16, torch.float32])
-@pytest.mark.parametrize("shape", [(65, 128), (128, 64), (300, 200), (1, 32), (129, 72), (8192, 1024), (176, 200), (16, 64), (144, 72), (272, 136)])
+@pytest.mark.parametrize("shape", [(65, 128), (128, 64), (300, 200), (1, 32), (129, 72), (8192, 1024), (176, 200), (16, 64), (144, 72), (272, 136),
+                                   (2064, 4104), (1048, 8200)])     # the last two: ragged on both sides at sizes that take the XCD-contiguous walk
 def test_quantize_dual_equals_two_passes(in_dtype, shape):
     g = _gpu()
     x = _input(shape, in_dtype, seed=11)
@@ -124,7 +125,7 @@ def test_quantize_rounding_ties_over_all_magnitudes(fp8, limit):
 
 
 @pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float16, torch.float32])
-@pytest.mark.parametrize("shape", [(65, 128), (300, 200), (129, 72), (8192, 1024), (32, 64), (176, 200), (144, 72)])
+@pytest.mark.parametrize("shape", [(65, 128), (300, 200), (129, 72), (8192, 1024), (32, 64), (176, 200), (144, 72), (2064, 4104)])
 def test_quantize_dual_column_sums(in_dtype, shape):
     """x.sum(0) from the quantizer's own read: fp32 accumulation in a fixed order, same codes as without it."""
     g = _gpu()
@@ -141,6 +142,27 @@ def test_quantize_dual_column_sums(in_dtype, shape):
         assert ((total.cpu().double() - ref).abs() <= bound + 1e-30).all()
     again = g.quantize_dual(x.cuda(), E4, (1, 32), column_sum_dtype=torch.float32)[-1]
     assert torch.equal(again, g.quantize_dual(x.cuda(), E4, (1, 32), column_sum_dtype=torch.float32)[-1])    # deterministic
+
+
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float16])
+def test_quantize_dual_nonfinite_tiny_and_huge_groups(in_dtype):
+    """Groups that leave the quotient route in either layout: a NaN, an Inf, magnitudes whose scale underflows the route's
+    domain, the format's largest values, all-zero groups; next to ordinary groups of the same wavefront and tile."""
+    g = _gpu()
+    torch.manual_seed(17)
+    x = torch.randn(200, 136)
+    x[3, 5], x[70, 100], x[130, 40] = float("nan"), float("inf"), float("-inf")
+    x[10:12, :64] = 0.0
+    x[20:52, 32:64] *= 1e-30 if in_dtype == torch.bfloat16 else 6e-8         # subnormal in fp16
+    x[64:96, 64:96] *= 3e38 if in_dtype == torch.bfloat16 else 6e4
+    x[100, 0:32] = torch.finfo(in_dtype).max
+    x = x.to(in_dtype)
+    q, s, qt, st = g.quantize_dual(x.cuda(), E4, (1, 32))
+    for got, got_scale, transposed in ((q, s, False), (qt, st, True)):
+        rq, rs = og.quantize(x, E4, (1, 32), transposed=transposed)
+        a, b = got.float().cpu(), rq.float()
+        assert torch.equal(got_scale.cpu().isnan(), rs.isnan()) and torch.equal(got_scale.cpu().nan_to_num(7.0), rs.nan_to_num(7.0))
+        assert torch.equal(a.isnan(), b.isnan()) and torch.equal(a.nan_to_num(9.0), b.nan_to_num(9.0))
 
 
 def test_quantize_limit_and_out_arguments():
