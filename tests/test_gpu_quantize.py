@@ -160,9 +160,9 @@ def test_quantize_dual_nonfinite_tiny_and_huge_groups(in_dtype):
     q, s, qt, st = g.quantize_dual(x.cuda(), E4, (1, 32))
     for got, got_scale, transposed in ((q, s, False), (qt, st, True)):
         rq, rs = og.quantize(x, E4, (1, 32), transposed=transposed)
-        a, b = got.float().cpu(), rq.float()
         assert torch.equal(got_scale.cpu().isnan(), rs.isnan()) and torch.equal(got_scale.cpu().nan_to_num(7.0), rs.nan_to_num(7.0))
-        assert torch.equal(a.isnan(), b.isnan()) and torch.equal(a.nan_to_num(9.0), b.nan_to_num(9.0))
+        # code bytes, the NaN codes included: 0x7f | sign from the software encoder, never the hardware converters' 0xff
+        assert torch.equal(got.cpu().view(torch.uint8), rq.view(torch.uint8))
 
 
 def test_quantize_limit_and_out_arguments():

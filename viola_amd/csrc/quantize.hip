@@ -440,7 +440,7 @@ __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x
 }
 
 // ------------------------------------------------------------------ 16-bit inputs: both layouts from a 64 x 64 tile
-// A block of 256 threads per tile, one tile per block: eight blocks are resident on a compute unit at 62 registers, and
+// A block of 256 threads per tile, one tile per block: eight blocks are resident on a compute unit at 64 registers, and
 // the launch is timed 15 - 25 % below the persistent 128 x 64 kernel above on every shape tried (8192 x 4096 bf16:
 // 27.7 against 36.2 us). Row-wise: thread (row tid / 4, 16 columns) loads 32 bytes, a 32-column group is a pair of
 // lanes; four neighbouring lanes store 64 consecutive bytes of codes. The raw 16-bit values are parked in LDS
@@ -449,153 +449,217 @@ __global__ __launch_bounds__(256) void quantize_dual16(const TIn* __restrict__ x
 // rows 16 (lane % 4) .. + 15) reads its 16 values, a 32-row group is again a pair of lanes, and four neighbouring lanes
 // store 64 consecutive bytes of one transposed row (with the group's halves 32 lanes apart instead, the same stores
 // left as 16-byte pieces and the launch took 31 us).
-template <typename TIn, typename TOut>
-__global__ __launch_bounds__(256) void quantize_dual16_tile64(const TIn* __restrict__ x, uint8_t* __restrict__ q,
-                                                               float* __restrict__ scale, uint8_t* __restrict__ qt,
-                                                               float* __restrict__ scale_t, int64_t rows, int64_t cols,
-                                                               float limit, float* __restrict__ column_partial, int e8m0, int xcd_walk) {
-    constexpr int LDV = 64 + 4;                                              // values per parked row (34 dwords)
-    __shared__ __attribute__((aligned(16))) uint16_t park[64 * LDV];
-    const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
-    // blocks are dispatched in index order: those in flight together take 32 row tiles of one column tile, then the next
-    // column tile, so the transposed output is written in 2 KB runs per row however wide the matrix is
-    constexpr int64_t BAND = 32;
-    const int64_t tiles_x = (cols + 63) / 64, tiles_y = (rows + 63) / 64;
-    int64_t id = blockIdx.x;
-    if (xcd_walk) {
-        // consecutive block indices go to the eight XCDs in turn: give each XCD one contiguous eighth of the walk, so the
-        // halves of a 128-byte line of the transposed output (two row tiles) meet in one L2
-        const int64_t per_xcd = (tiles_x * tiles_y + 7) / 8;
-        id = (id % 8) * per_xcd + id / 8;
-    }
-    if (id >= tiles_x * tiles_y) return;
-    const int64_t patch = id / (BAND * tiles_x), within = id % (BAND * tiles_x);
-    const int64_t tall = tiles_y - patch * BAND < BAND ? tiles_y - patch * BAND : BAND;
-    const int64_t r0 = (patch * BAND + within % tall) * 64, c0 = within / tall * 64;
-    const int64_t nc = (cols + 31) / 32, nr = (rows + 31) / 32;
-    constexpr uint32_t MAGNITUDE = 0x7fff7fffu, INF16 = std::is_same<TIn, bf16_t>::value ? 0x7f80u : 0x7c00u;
-    const bool clamp_free = limit == fp8_traits<TOut>::max;
+// INTERIOR: the tile lies wholly inside the matrix and every 16-byte piece of either output is aligned (the launcher
+// says so in `aligned`): no bounds checks, tile base pointers in scalar registers with 32-bit offsets per lane.
 
-    // ---- row-wise
-    const int lr = tid / 4, lc = (tid % 4) * 16;
-    const int64_t row = r0 + lr, col = c0 + lc;
-    uint4 raw[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
-    if (row < rows) {
-        if (col < cols) raw[0] = *reinterpret_cast<const uint4*>(x + row * cols + col);          // cols % 8 == 0: whole pieces
-        if (col + 8 < cols) raw[1] = *reinterpret_cast<const uint4*>(x + row * cols + col + 8);
-    }
-    {
-        uint2* mine = reinterpret_cast<uint2*>(&park[lr * LDV + (lc ^ (((lr >> 4) & 3) << 4))]);       // 16-column blocks swapped by row chunk
-        mine[0] = make_uint2(raw[0].x, raw[0].y); mine[1] = make_uint2(raw[0].z, raw[0].w);
-        mine[2] = make_uint2(raw[1].x, raw[1].y); mine[3] = make_uint2(raw[1].z, raw[1].w);
-    }
-    const uint32_t words[8] = {raw[0].x, raw[0].y, raw[0].z, raw[0].w, raw[1].x, raw[1].y, raw[1].z, raw[1].w};
-    float v[16];
+// 16 values as 8 words of two (rows or columns) -> group scale with the pair's other lane, codes; `slow` receives
+// whether the wavefront must take the exact route instead.
+template <typename TIn, typename TOut>
+__device__ __forceinline__ bool encode_words16(const uint32_t (&words)[8], float limit, int e8m0, bool clamp_free, float& s, uint32_t (&codes)[4],
+                                               bool& nonfinite) {
+    constexpr uint32_t MAGNITUDE = 0x7fff7fffu, INF16 = std::is_same<TIn, bf16_t>::value ? 0x7f80u : 0x7c00u;
     uint32_t top = 0;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        v[2 * e] = widen16<TIn>(words[e] & 0xffffu);
-        v[2 * e + 1] = widen16<TIn>(words[e] >> 16);
-        top = pk_max_u16(top, words[e] & MAGNITUDE);
-    }
+    for (int e = 0; e < 8; ++e) top = pk_max_u16(top, words[e] & MAGNITUDE);
     top = (top & 0xffffu) > (top >> 16) ? (top & 0xffffu) : (top >> 16);
     {
         const uint32_t other = (uint32_t)__builtin_amdgcn_mov_dpp((int)top, 0xB1, 0xf, 0xf, true);   // the pair's other lane
         top = top > other ? top : other;
     }
-    float s_row = group_scale(widen16<TIn>(top), limit, e8m0);
-    const SharedDivisor d_row(s_row, top >= INF16 ? __uint_as_float(0x7fc00000u) : 0.0f);
-    uint32_t codes[4];
-    if (__builtin_amdgcn_ballot_w64(!d_row.fast) == 0) {
+    nonfinite = top >= INF16;
+    s = group_scale(widen16<TIn>(top), limit, e8m0);
+    const SharedDivisor d(s, nonfinite ? __uint_as_float(0x7fc00000u) : 0.0f);
+    if (__builtin_amdgcn_ballot_w64(!d.fast) != 0) return false;
 #pragma unroll
-        for (int k = 0; k < 4; ++k)
-            codes[k] = clamp_free ? fast_encode4_unclamped<TOut>(d_row, v[4 * k], v[4 * k + 1], v[4 * k + 2], v[4 * k + 3])
-                                  : fast_encode4<TOut>(d_row, limit, v[4 * k], v[4 * k + 1], v[4 * k + 2], v[4 * k + 3]);
-    } else {
-        // an Inf or a NaN in some group of the wavefront, or a scale outside the quotient route's domain: the maxima as the
-        // reference's kernel takes them (fmax ignores NaN), true division, software encoder
-        float amax = 0.0f;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(v[e]));
-        amax = fmaxf(amax, quad_xor<1>(amax));
-        s_row = group_scale(amax, limit, e8m0);
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            codes[k] = 0;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) codes[k] |= (uint32_t)encode_clamped<TOut>(v[4 * k + e], s_row, limit) << (8 * e);
-        }
+    for (int k = 0; k < 4; ++k) {
+        const float a = widen16<TIn>(words[2 * k] & 0xffffu), b = widen16<TIn>(words[2 * k] >> 16);
+        const float c = widen16<TIn>(words[2 * k + 1] & 0xffffu), e = widen16<TIn>(words[2 * k + 1] >> 16);
+        codes[k] = clamp_free ? fast_encode4_unclamped<TOut>(d, a, b, c, e) : fast_encode4<TOut>(d, limit, a, b, c, e);
     }
-    if (row < rows && col < cols) {
-        uint8_t* dst = q + row * cols + col;
-        if (col + 16 <= cols && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
-            *reinterpret_cast<uint4*>(dst) = make_uint4(codes[0], codes[1], codes[2], codes[3]);
-        } else {
-            *reinterpret_cast<uint2*>(dst) = make_uint2(codes[0], codes[1]);                         // q is 8-byte aligned, cols % 8 == 0
-            if (col + 8 < cols) *reinterpret_cast<uint2*>(dst + 8) = make_uint2(codes[2], codes[3]);
+    return true;
+}
+// The same for 16 finite values already widened: the maximum is taken in floating point, three values per instruction.
+__device__ __forceinline__ float max3_abs(float acc, float a, float b) {
+    float r;
+    asm("v_max3_f32 %0, %1, |%2|, |%3|" : "=v"(r) : "v"(acc), "v"(a), "v"(b));
+    return r;
+}
+template <typename TOut>
+__device__ __forceinline__ bool encode_finite16(const float (&v)[16], float limit, int e8m0, bool clamp_free, float& s, uint32_t (&codes)[4]) {
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i += 2) amax = max3_abs(amax, v[i], v[i + 1]);
+    {
+        const float other = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(amax), 0xB1, 0xf, 0xf, true));   // the pair's other lane
+        amax = max3_abs(amax, other, other);
+    }
+    s = group_scale(amax, limit, e8m0);
+    const SharedDivisor d(s, 0.0f);
+    if (__builtin_amdgcn_ballot_w64(!d.fast) != 0) return false;
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+        codes[k] = clamp_free ? fast_encode4_unclamped<TOut>(d, v[4 * k], v[4 * k + 1], v[4 * k + 2], v[4 * k + 3])
+                              : fast_encode4<TOut>(d, limit, v[4 * k], v[4 * k + 1], v[4 * k + 2], v[4 * k + 3]);
+    return true;
+}
+// The exact route: an Inf or a NaN in some group of the wavefront, or a scale outside the quotient route's domain. The
+// maximum as the reference's kernel takes it (fmax ignores NaN), true division, software encoder.
+struct Exact16 { uint32_t c0, c1, c2, c3; float s; };
+template <typename TIn, typename TOut>
+__device__ __noinline__ Exact16 encode_words16_exact(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3, uint32_t w4, uint32_t w5, uint32_t w6,
+                                                     uint32_t w7, float limit, int e8m0) {
+    const uint32_t words[8] = {w0, w1, w2, w3, w4, w5, w6, w7};
+    float v[16], amax = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        v[2 * e] = widen16<TIn>(words[e] & 0xffffu);
+        v[2 * e + 1] = widen16<TIn>(words[e] >> 16);
+        amax = fmaxf(amax, fmaxf(fabsf(v[2 * e]), fabsf(v[2 * e + 1])));
+    }
+    amax = fmaxf(amax, quad_xor<1>(amax));
+    Exact16 out;
+    out.s = group_scale(amax, limit, e8m0);
+    uint32_t codes[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        codes[k] = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) codes[k] |= (uint32_t)encode_clamped<TOut>(v[4 * k + e], out.s, limit) << (8 * e);
+    }
+    out.c0 = codes[0]; out.c1 = codes[1]; out.c2 = codes[2]; out.c3 = codes[3];
+    return out;
+}
+
+template <typename TIn, typename TOut, bool INTERIOR>
+__device__ __forceinline__ void dual16_tile64(const TIn* __restrict__ x, uint8_t* __restrict__ q, float* __restrict__ scale,
+                                              uint8_t* __restrict__ qt, float* __restrict__ scale_t, int64_t rows, int64_t cols,
+                                              float limit, float* __restrict__ column_partial, int e8m0, int64_t r0, int64_t c0,
+                                              uint16_t* park, int* flags) {
+    constexpr int LDV = 64 + 4;                                              // values per parked row (34 dwords)
+    const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+    const int64_t nc = (cols + 31) / 32, nr = (rows + 31) / 32;
+    const bool clamp_free = limit == fp8_traits<TOut>::max;
+
+    // ---- row-wise
+    {
+        const int lr = tid / 4, lc = (tid % 4) * 16;
+        const int64_t row = r0 + lr, col = c0 + lc;
+        const uint32_t offset = (uint32_t)lr * (uint32_t)cols + (uint32_t)lc;   // from the tile's first element (INTERIOR: < 2^31)
+        uint4 raw[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+        if constexpr (INTERIOR) {
+            const TIn* tile = x + r0 * cols + c0;
+            raw[0] = *reinterpret_cast<const uint4*>(tile + offset);
+            raw[1] = *reinterpret_cast<const uint4*>(tile + offset + 8);
+        } else if (row < rows) {
+            if (col < cols) raw[0] = *reinterpret_cast<const uint4*>(x + row * cols + col);      // cols % 8 == 0: whole pieces
+            if (col + 8 < cols) raw[1] = *reinterpret_cast<const uint4*>(x + row * cols + col + 8);
         }
-        if (tid % 2 == 0) put_scale(scale, row * nc + col / 32, s_row, e8m0);
+        {
+            uint2* mine = reinterpret_cast<uint2*>(&park[lr * LDV + (lc ^ (((lr >> 4) & 3) << 4))]);   // 16-column blocks swapped by row chunk
+            mine[0] = make_uint2(raw[0].x, raw[0].y); mine[1] = make_uint2(raw[0].z, raw[0].w);
+            mine[2] = make_uint2(raw[1].x, raw[1].y); mine[3] = make_uint2(raw[1].z, raw[1].w);
+        }
+        const uint32_t words[8] = {raw[0].x, raw[0].y, raw[0].z, raw[0].w, raw[1].x, raw[1].y, raw[1].z, raw[1].w};
+        float s_row;
+        uint32_t codes[4];
+        bool nonfinite;
+        if (!encode_words16<TIn, TOut>(words, limit, e8m0, clamp_free, s_row, codes, nonfinite)) {
+            const Exact16 r = encode_words16_exact<TIn, TOut>(words[0], words[1], words[2], words[3], words[4], words[5], words[6], words[7], limit, e8m0);
+            codes[0] = r.c0; codes[1] = r.c1; codes[2] = r.c2; codes[3] = r.c3; s_row = r.s;
+        }
+        if constexpr (INTERIOR) {
+            *reinterpret_cast<uint4*>(q + r0 * cols + c0 + offset) = make_uint4(codes[0], codes[1], codes[2], codes[3]);
+            if (tid % 2 == 0) put_scale(scale, (r0 * nc + c0 / 32) + (int64_t)((uint32_t)lr * (uint32_t)nc + (uint32_t)(lc / 32)), s_row, e8m0);
+        } else if (row < rows && col < cols) {
+            uint8_t* dst = q + row * cols + col;
+            if (col + 16 <= cols && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+                *reinterpret_cast<uint4*>(dst) = make_uint4(codes[0], codes[1], codes[2], codes[3]);
+            } else {
+                *reinterpret_cast<uint2*>(dst) = make_uint2(codes[0], codes[1]);                     // q is 8-byte aligned, cols % 8 == 0
+                if (col + 8 < cols) *reinterpret_cast<uint2*>(dst + 8) = make_uint2(codes[2], codes[3]);
+            }
+            if (tid % 2 == 0) put_scale(scale, row * nc + col / 32, s_row, e8m0);
+        }
+        const bool any_nonfinite = __builtin_amdgcn_ballot_w64(nonfinite) != 0;   // over the whole wavefront: outside the branch
+        if (lane == 0) flags[wave] = any_nonfinite;
     }
     __syncthreads();
+    // no NaN and no Inf anywhere in the tile: the transposed phase may then take its maxima in floating point
+    const bool plain = (flags[0] | flags[1] | flags[2] | flags[3]) == 0;
 
     // ---- transposed: wavefront w takes columns 16 w .. + 15 of the tile; lane = (column lane / 4, rows 16 (lane % 4) .. + 15), so four
     // neighbouring lanes write 64 consecutive bytes of one transposed row and a 32-row group is a pair of lanes
-    const int tc = wave * 16 + lane / 4, chunk = lane % 4;
-    const int64_t tcol = c0 + tc, trow = r0 + chunk * 16;                    // first of the lane's 16 rows
-    float w[16];
-    uint32_t top_col = 0;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const uint32_t bits = park[(chunk * 16 + i) * LDV + (tc ^ (chunk << 4))];
-        w[i] = widen16<TIn>(bits);
-        const uint32_t magnitude = bits & 0x7fffu;
-        top_col = top_col > magnitude ? top_col : magnitude;
-    }
     {
-        const uint32_t other = (uint32_t)__builtin_amdgcn_mov_dpp((int)top_col, 0xB1, 0xf, 0xf, true);   // the pair's other lane
-        top_col = top_col > other ? top_col : other;
-    }
-    float s_col = group_scale(widen16<TIn>(top_col), limit, e8m0);
-    const SharedDivisor d_col(s_col, top_col >= INF16 ? __uint_as_float(0x7fc00000u) : 0.0f);
-    uint32_t tcodes[4];
-    if (__builtin_amdgcn_ballot_w64(!d_col.fast) == 0) {
+        const int tc = wave * 16 + lane / 4, chunk = lane % 4;
+        const int64_t tcol = c0 + tc, trow = r0 + chunk * 16;                // first of the lane's 16 rows
+        uint32_t bits[16];
 #pragma unroll
-        for (int k = 0; k < 4; ++k)
-            tcodes[k] = clamp_free ? fast_encode4_unclamped<TOut>(d_col, w[4 * k], w[4 * k + 1], w[4 * k + 2], w[4 * k + 3])
-                                   : fast_encode4<TOut>(d_col, limit, w[4 * k], w[4 * k + 1], w[4 * k + 2], w[4 * k + 3]);
-    } else {
-        float amax = 0.0f;
+        for (int i = 0; i < 16; ++i) bits[i] = park[(chunk * 16 + i) * LDV + (tc ^ (chunk << 4))];
+        float w[16];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(w[i]));
-        amax = fmaxf(amax, quad_xor<1>(amax));
-        s_col = group_scale(amax, limit, e8m0);
+        for (int i = 0; i < 16; ++i) w[i] = widen16<TIn>(bits[i]);
+        float s_col;
+        uint32_t tcodes[4];
+        if (!plain || !encode_finite16<TOut>(w, limit, e8m0, clamp_free, s_col, tcodes)) {
+            const Exact16 r = encode_words16_exact<TIn, TOut>(bits[0] | bits[1] << 16, bits[2] | bits[3] << 16, bits[4] | bits[5] << 16, bits[6] | bits[7] << 16,
+                                                              bits[8] | bits[9] << 16, bits[10] | bits[11] << 16, bits[12] | bits[13] << 16,
+                                                              bits[14] | bits[15] << 16, limit, e8m0);
+            tcodes[0] = r.c0; tcodes[1] = r.c1; tcodes[2] = r.c2; tcodes[3] = r.c3; s_col = r.s;
+        }
+        float sum = 0.0f;
+        if (column_partial) {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            tcodes[k] = 0;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) tcodes[k] |= (uint32_t)encode_clamped<TOut>(w[4 * k + e], s_col, limit) << (8 * e);
+            for (int i = 0; i < 16; ++i) sum += w[i];
+            const float other = quad_xor<1>(sum);
+            sum = chunk % 2 == 0 ? sum + other : other + sum;                 // rows 0 .. 15 first, then 16 .. 31
+        }
+        if constexpr (INTERIOR) {
+            *reinterpret_cast<uint4*>(qt + c0 * rows + r0 + ((uint32_t)tc * (uint32_t)rows + (uint32_t)(chunk * 16))) = make_uint4(tcodes[0], tcodes[1], tcodes[2], tcodes[3]);
+            if (chunk % 2 == 0) {
+                put_scale(scale_t, (c0 * nr + r0 / 32) + (int64_t)((uint32_t)tc * (uint32_t)nr + (uint32_t)(chunk / 2)), s_col, e8m0);
+                if (column_partial) (column_partial + (r0 / 32) * cols + c0)[(uint32_t)(chunk / 2) * (uint32_t)cols + (uint32_t)tc] = sum;
+            }
+        } else if (tcol < cols && trow < rows) {
+            uint8_t* dst = qt + tcol * rows + trow;
+            if (trow + 16 <= rows && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+                *reinterpret_cast<uint4*>(dst) = make_uint4(tcodes[0], tcodes[1], tcodes[2], tcodes[3]);
+            } else {
+                const int count = (int)(rows - trow < 16 ? rows - trow : 16);
+                for (int i = 0; i < count; ++i) dst[i] = (uint8_t)(tcodes[i >> 2] >> (8 * (i & 3)));
+            }
+            if (chunk % 2 == 0) {
+                put_scale(scale_t, tcol * nr + trow / 32, s_col, e8m0);
+                if (column_partial) column_partial[(trow / 32) * cols + tcol] = sum;
+            }
         }
     }
-    float sum = 0.0f;
-    if (column_partial) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) sum += w[i];
-        const float other = quad_xor<1>(sum);
-        sum = chunk % 2 == 0 ? sum + other : other + sum;                     // rows 0 .. 15 first, then 16 .. 31
+}
+
+template <typename TIn, typename TOut>
+__global__ __launch_bounds__(256, 8) void quantize_dual16_tile64(const TIn* __restrict__ x, uint8_t* __restrict__ q,
+                                                               float* __restrict__ scale, uint8_t* __restrict__ qt,
+                                                               float* __restrict__ scale_t, int64_t rows, int64_t cols,
+                                                               float limit, float* __restrict__ column_partial, int e8m0, int xcd_walk,
+                                                               int aligned) {
+    __shared__ __attribute__((aligned(16))) uint16_t park[64 * (64 + 4)];
+    __shared__ __attribute__((aligned(16))) int flags[4];                   // per wavefront: its rows hold a NaN or an Inf
+    // blocks are dispatched in index order: those in flight together take 32 row tiles of one column tile, then the next
+    // column tile, so the transposed output is written in 2 KB runs per row however wide the matrix is (the launcher
+    // keeps the tile count below 2^31)
+    constexpr uint32_t BAND = 32;
+    const uint32_t tiles_x = (uint32_t)((cols + 63) / 64), tiles_y = (uint32_t)((rows + 63) / 64), tiles = tiles_x * tiles_y;
+    uint32_t id = blockIdx.x;
+    if (xcd_walk) {
+        // consecutive block indices go to the eight XCDs in turn: give each XCD one contiguous eighth of the walk, so the
+        // halves of a 128-byte line of the transposed output (two row tiles) meet in one L2
+        id = (id % 8) * ((tiles + 7) / 8) + id / 8;
     }
-    if (tcol < cols && trow < rows) {
-        uint8_t* dst = qt + tcol * rows + trow;
-        if (trow + 16 <= rows && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
-            *reinterpret_cast<uint4*>(dst) = make_uint4(tcodes[0], tcodes[1], tcodes[2], tcodes[3]);
-        } else {
-            const int count = (int)(rows - trow < 16 ? rows - trow : 16);
-            for (int i = 0; i < count; ++i) dst[i] = (uint8_t)(tcodes[i >> 2] >> (8 * (i & 3)));
-        }
-        if (chunk % 2 == 0) {
-            put_scale(scale_t, tcol * nr + trow / 32, s_col, e8m0);
-            if (column_partial) column_partial[(trow / 32) * cols + tcol] = sum;
-        }
-    }
+    if (id >= tiles) return;
+    const uint32_t patch = id / (BAND * tiles_x), within = id % (BAND * tiles_x);
+    const uint32_t tall = tiles_y - patch * BAND < BAND ? tiles_y - patch * BAND : BAND;
+    const int64_t r0 = (int64_t)(patch * BAND + within % tall) * 64, c0 = (int64_t)(within / tall) * 64;
+    if (aligned && r0 + 64 <= rows && c0 + 64 <= cols) dual16_tile64<TIn, TOut, true>(x, q, scale, qt, scale_t, rows, cols, limit, column_partial, e8m0, r0, c0, park, flags);
+    else dual16_tile64<TIn, TOut, false>(x, q, scale, qt, scale_t, rows, cols, limit, column_partial, e8m0, r0, c0, park, flags);
 }
 
 // ------------------------------------------------------------------ column sums from 32-row partials
@@ -1024,8 +1088,12 @@ static int launch_dual(const void* x, int64_t rows, int64_t cols, void* q, float
                 // (8192 x 4096: 29.7 -> 27.7 us); longer launches are faster with the eight XCDs streaming one region
                 // (16384 x 4096: 68 against 76 us), shorter ones leave XCDs uneven
                 const int xcd_walk = tiles64 >= 2048 && tiles64 <= 8192;
+                // whole tiles may skip their bounds checks and address a lane's pieces by 32-bit offsets from the tile
+                const int aligned = cols % 16 == 0 && rows % 16 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0 &&
+                                    reinterpret_cast<uintptr_t>(qt) % 16 == 0 && cols < (1ll << 24) && rows < (1ll << 24);
                 VIOLA_LAUNCH((quantize_dual16_tile64<TIn, TOut>), dim3((unsigned)((tiles64 + 7) / 8 * 8)), dim3(256), 0, stream, xp,
-                             static_cast<uint8_t*>(q), scale, static_cast<uint8_t*>(qt), scale_t, rows, cols, limit, column_partial, e8m0, xcd_walk);
+                             static_cast<uint8_t*>(q), scale, static_cast<uint8_t*>(qt), scale_t, rows, cols, limit, column_partial, e8m0, xcd_walk,
+                             aligned);
                 return viola_launch_status();
             }
             const int64_t tiles16 = ((cols + 63) / 64) * ((rows + 127) / 128);
