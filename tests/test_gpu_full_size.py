@@ -155,6 +155,44 @@ def test_gated_mlp_gemms_at_16384x4096x11008():
     assert rel_l2(dz[rows], expect) < 6e-3
 
 
+def test_gated_mlp_gemms_at_16384x4096x11008_against_the_cpu_oracle():
+    """The gated forward and backward GEMMs of the MLP at full size, held to the CPU oracle itself on a row sample the
+    oracle finishes in seconds (a row of either product depends on that row of the activations only): [g | u] against
+    the float64 witness of oracle.grouped.gemm, h and dz against oracle.linear.gated_forward / gated_backward applied to
+    the rounded values, as the fused kernels do (viola/nn/_mlp_kernels.py:158-194)."""
+    import types
+    from oracle import grouped as og, linear as ol
+    from viola_amd.nn import _grouped_kernels as g, _mlp_kernels as mk
+    m, d, h = 16384, 4096, 11008
+    _, qx, sx = _quantized(m, d, (1, 32), 4)
+    torch.manual_seed(5)
+    w = torch.empty(2 * h, d, device="cuda").uniform_(-1 / 64, 1 / 64)
+    qw, sw = g.quantize(w, E4, (32, 32))
+    del w
+    recipe = types.SimpleNamespace(_native_scaling=False, _grouped_scaling=True, input_group_shape=(1, 32), weight_group_shape=(32, 32))
+    out, aux, _ = mk.gemm(qx, qw, sx, sw, layer=recipe, out_dtype=torch.bfloat16, activation="silu", save=True)
+    generator = torch.Generator().manual_seed(9)
+    rows = torch.cat([torch.tensor([0, 1, 127, 128, m // 2, m - 129, m - 1]), torch.randint(0, m, (25,), generator=generator)]).unique()
+    on_gpu = rows.cuda()
+    z = og.gemm(qx[on_gpu].cpu(), qw.cpu(), sx[on_gpu].cpu(), sw.cpu(), (1, 32), (32, 32), witness=True, out_dtype=torch.float64)
+    assert rel_l2(aux[on_gpu], z) < 3e-3                                      # one bf16 rounding of [g | u]
+    z16 = z.to(torch.bfloat16)
+    assert (aux[on_gpu].cpu() == z16).float().mean() > 0.99                  # and the same rounded values but for summation order
+    gate, up = aux[on_gpu, :h].cpu(), aux[on_gpu, h:].cpu()
+    assert rel_l2(out[on_gpu], ol.gated_forward(gate, up, "silu")) < 4e-3
+    del qx, sx, qw, sw, z, z16
+    _, qg, sg = _quantized(m, d, (1, 32), 6)
+    torch.manual_seed(7)
+    w2 = torch.empty(h, d, device="cuda").uniform_(-1 / 64, 1 / 64)
+    qw2, sw2 = g.quantize(w2, E4, (32, 32))
+    del w2
+    dz, _, _ = mk.gemm(qg, qw2, sg, sw2, layer=recipe, out_dtype=torch.bfloat16, activation="silu", backward=True, aux=aux,
+                       group_a=(1, 32), group_b=(32, 32))
+    dh = og.gemm(qg[on_gpu].cpu(), qw2.cpu(), sg[on_gpu].cpu(), sw2.cpu(), (1, 32), (32, 32), witness=True, out_dtype=torch.float64)
+    dgate, dup = ol.gated_backward(dh.to(torch.bfloat16), gate, up, "silu")
+    assert rel_l2(dz[on_gpu], torch.cat([dgate, dup], 1)) < 6e-3
+
+
 def test_mlp_module_at_16384x4096x11008():
     """The whole viola_amd.nn.MLP forward + backward at the benchmark's size (grouped recipe, FP8 weight storage, memory
     mode) against fp32 GPU math on dequantized operands: y and dx on a row sample (row-wise quantization is per row, so
@@ -319,6 +357,42 @@ def test_variable_groups_at_16x32768x4096x1024():
         xt = g.dequantize(*g.quantize(x.detach()[rows].contiguous(), E4, (1, 32), transposed=True), (1, 32))
         gt = g.dequantize(*g.quantize(dy[rows].contiguous(), E4, (1, 32), transposed=True), (1, 32))
         assert rel_l2(experts.weight.grad[group], gt @ xt.T) < 3e-3, group
+
+
+def test_variable_groups_at_16x32768x4096x1024_against_the_cpu_oracle():
+    """The variable-group step at full size against the CPU oracle's Linear (oracle.linear.linear, which
+    oracle.linear.varlen_linear applies per group): y and dx on a few rows of a full group, of the 3-row group and of the
+    largest one (row-wise quantization makes a row's result depend on that row and the group's weight only), and the
+    whole weight gradient of the 3-row group and of one full group."""
+    from oracle import linear as ol
+    from viola_amd.nn import _varlen as v
+    groups, k, n, total = 16, 4096, 1024, 32768
+    generator = torch.Generator().manual_seed(6)
+    counts = torch.bincount(torch.multinomial(torch.ones(groups) / groups, total, replacement=True, generator=generator), minlength=groups)
+    counts[3] += counts[5] - 3
+    counts[5] = 3
+    counts[7] += counts[9]
+    counts[9] = 0
+    counts = counts.tolist()
+    torch.manual_seed(7)
+    x = torch.randn(total, k, device="cuda").bfloat16().requires_grad_()
+    dy = torch.randn(total, n, device="cuda").bfloat16()
+    experts = v.GroupedExperts(groups, k, n, device="cuda")
+    y = experts(x, counts)
+    y.backward(dy)
+    weights = experts.dequantize_weight().float().cpu()
+    starts = [sum(counts[:group]) for group in range(groups)]
+    for group in (0, 5, 3):
+        begin, count = starts[group], counts[group]
+        picks = torch.tensor(sorted({0, 1, count // 2, count - 1} & set(range(count)))) + begin
+        want = ol.linear(x.detach()[picks.cuda()].cpu(), weights[group], None, dy[picks.cuda()].cpu())
+        assert rel_l2(y[picks.cuda()], want["y"]) < 3e-3, group
+        assert rel_l2(x.grad[picks.cuda()], want["dx"]) < 3e-3, group
+    for group in (5, 0):
+        rows = slice(starts[group], starts[group] + counts[group])
+        want = ol.linear(x.detach()[rows].cpu(), weights[group], None, dy[rows].cpu(), grad_dtype=torch.float32)
+        assert rel_l2(experts.weight.grad[group], want["dw"]) < 3e-3, group
+    assert experts.weight.grad[9].count_nonzero() == 0
 
 
 @pytest.mark.parametrize("method", ["standard", "gram"])
