@@ -28,21 +28,18 @@ typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int FBK = 64, FKG = FBK / 32;                           // k bytes and K groups per LDS stage
 constexpr int FTHREADS = 256, FSTAGES = 3;
-#ifndef VIOLA_OUTER_SCALES
-#define VIOLA_OUTER_SCALES 1                                       // row-wise b scales: sa[m] * sb[n] per K group from an fp32 MFMA
-#endif
 #ifndef VIOLA_BIG_STAGES
 #define VIOLA_BIG_STAGES 3                                         // ring depth of the 256 x 256 tile kernels (4 measured the same)
 #endif
 constexpr int F_TILE = BM * FBK;                                  // bytes of one operand tile
 constexpr int F_STAGE = 2 * F_TILE;
 // Scales travel in blocks of 8 K groups (4 chunks): 32 bytes per row and operand, fetched as two 16-byte pieces
-// ("raw", piece = 4 groups of one row) and then rearranged in LDS to [group][row] floats, double-buffered.
+// (piece = 4 groups of one row; thread t brings piece t / 128 of row t % 128), double-buffered, and read from LDS in
+// that layout: the scale of (row, group g of the block) is float ((g / 4) * 128 + row) * 4 + g % 4.
 constexpr int F_SGROUPS = 8, F_SCHUNKS = F_SGROUPS / FKG;
 constexpr int F_SBLOCK = F_SGROUPS * BM * 4;                      // bytes of one operand's scale block
-constexpr int F_RAW = FSTAGES * F_STAGE;                          // raw a block, raw b block
-constexpr int F_SCALE = F_RAW + 2 * F_SBLOCK;                     // [buffer][operand][group][row]
-constexpr int F_LDS = F_SCALE + 4 * F_SBLOCK;
+constexpr int F_RAW = FSTAGES * F_STAGE;                          // scale blocks as fetched: [buffer][operand][half][row][4 groups]
+constexpr int F_LDS = F_RAW + 4 * F_SBLOCK;
 
 // 64 lanes x 16 (or 4) bytes from a raw buffer straight into LDS at lds_addr + 16 (4) * lane. The compiler
 // is not told that these touch LDS (it would drain every outstanding load before each LDS read); the kernel
@@ -272,7 +269,7 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
     // and operand; a piece wholly past the k range is not fetched
     auto issue_scales = [&](int block) {
         const bool inside = block * F_SGROUPS + shalf * 4 < groups_total;
-        const uint32_t at = lds_base + F_RAW + (uint32_t)wave * 1024;
+        const uint32_t at = lds_base + F_RAW + (uint32_t)(block & 1) * 2 * F_SBLOCK + (uint32_t)wave * 1024;
         load16_to_lds(res_sa, at, inside ? sa_off : OUTSIDE, (uint32_t)(block * F_SGROUPS * 4));
         load16_to_lds(res_sb, at + F_SBLOCK, inside ? sb_off : OUTSIDE, (uint32_t)(block * F_SGROUPS * 4));
     };
@@ -286,22 +283,6 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
         const uint32_t at = lds_base + K_RAW + (uint32_t)(block & 1) * K_MX_BLOCK + (uint32_t)wave * 1024;
         load16_to_lds(wave < TBM / 64 ? res_mxa : res_mxb, at, inside ? mx_off : OUTSIDE, (uint32_t)(block * MX_GROUPS));
     };
-    // raw area -> [group][row] floats of scale buffer `block & 1`; groups past the k range become zero (their
-    // products are zero too, and a neighbouring row's value must not meet them)
-    auto arrange_scales = [&](int block) {
-        const float4 va = *reinterpret_cast<const float4*>(lds + F_RAW + tid * 16);
-        const float4 vb = *reinterpret_cast<const float4*>(lds + F_RAW + F_SBLOCK + tid * 16);
-        float* ta = reinterpret_cast<float*>(lds + F_SCALE + (block & 1) * 2 * F_SBLOCK);
-        float* tb = ta + F_SBLOCK / 4;
-        const int left = groups_total - (int)(block * F_SGROUPS + shalf * 4);
-        const float a4[4] = {va.x, va.y, va.z, va.w}, b4[4] = {vb.x, vb.y, vb.z, vb.w};
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            ta[(shalf * 4 + q) * BM + srow] = q < left ? a4[q] : 0.0f;
-            tb[(shalf * 4 + q) * BM + srow] = q < left ? b4[q] : 0.0f;
-        }
-    };
-
     // ---- MFMA operand reads: 16 bytes = this lane's half (lhi) of K group kg for row l32 of a sub-tile
     auto a_sub = [&](int j) -> int { return (wm * TM + j) * 32; };
     auto b_sub = [&](int i) -> int { return GATED ? i * PANEL + wn * 32 : (wn * TN + i) * 32; };
@@ -325,7 +306,8 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
     // v_mul_f32 rounds them; the fold is then one FMA per element, as with uniform b scales. The products of a pair are
     // issued among its MFMAs and read while the next pair's MFMAs run: into the other of two buffers where the registers
     // allow it (TN = 1), else into the one buffer once the fold before has read it.
-    constexpr bool OUTER = B_ROWSCALE && TM == 2 && VIOLA_OUTER_SCALES;
+    constexpr bool OUTER = B_ROWSCALE;
+    static_assert(!B_ROWSCALE || TM == 2, "the two blocks of the scale products' MFMA are the wave's two a sub-tiles");
     constexpr bool CARRY = !B_ROWSCALE || OUTER;
     constexpr int PBUF = TN == 1 ? 2 : 1;
     typedef float f32x32 __attribute__((ext_vector_type(32)));
@@ -351,14 +333,17 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
         i32x8 wide_a[TM], wide_b[TN];                                        // TENSOR / MX: 16 k of either K group of a sub-tile row
         int mx_a[(TM + 1) / 2], mx_b[(TN + 1) / 2];                          // MX: the rows' scale bytes of K group lhi, sub-tile t in byte 2 (t & 1) of word t / 2
     };
-    auto scale_block = [&](int c) -> const float* {                      // a scales of chunk c: [kg][row]; b scales F_SBLOCK later
-        return reinterpret_cast<const float*>(lds + F_SCALE + ((c / F_SCHUNKS) & 1) * 2 * F_SBLOCK) + (c % F_SCHUNKS) * FKG * BM;
+    // scale of tile row `row` for K group kg of chunk c (operand 0: a, 1: b); a group past the k range gives zero (its
+    // products are zero too, and whatever the piece holds there, a neighbouring row's value perhaps, must not meet them)
+    auto scale_at = [&](int operand, int c, int kg, int row) -> float {
+        const int g8 = (c % F_SCHUNKS) * FKG + kg;                          // group of the block: uniform, like the test below
+        const float* block = reinterpret_cast<const float*>(lds + F_RAW + ((c / F_SCHUNKS) & 1) * 2 * F_SBLOCK + operand * F_SBLOCK);
+        const float v = block[((g8 >> 2) * BM + row) * 4 + (g8 & 3)];
+        return c * FKG + kg < groups_total ? v : 0.0f;
     };
     auto read_operands = [&](int stage, int c, Operands& o) {
         const uint8_t* tile_a = lds + stage * K_STAGE;
         const uint8_t* tile_b = tile_a + K_TILE_A;
-        const float* scale_a = scale_block(c);
-        const float* scale_b = scale_a + F_SBLOCK / 4;
         if constexpr (NOFOLD) {
             // the lane's 16 bytes of either K group (slots lhi and lhi + 2)
             const int first_a = rd_a, first_b = rd_b;
@@ -403,9 +388,9 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
                 for (int i = 0; i < TN; ++i) o.sb[kg][i] = 0.0f;
             } else {
 #pragma unroll
-                for (int j = 0; j < TM; ++j) o.sa[kg][j] = scale_a[kg * BM + a_sub(j) + l32];
+                for (int j = 0; j < TM; ++j) o.sa[kg][j] = scale_at(0, c, kg, a_sub(j) + l32);
 #pragma unroll
-                for (int i = 0; i < TN; ++i) o.sb[kg][i] = B_ROWSCALE ? 0.0f : scale_b[kg * BM + b_sub(i)];
+                for (int i = 0; i < TN; ++i) o.sb[kg][i] = scale_at(1, c, kg, b_sub(i));
             }
         }
     };
@@ -443,22 +428,14 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
             }
             return;
         }
-        // row-wise b scales of the lane's 16 columns for one pair of units (both share K group and b sub-tile): two
-        // slots, pair p loads slot p & 1 before its MFMAs and its fold reads it during pair p + 1
-        float4 sb_q[2][4];
-        const float* scale_b = scale_block(c) + F_SBLOCK / 4;
         // fold half `h` (registers 8h .. 8h+7) of accumulator `buf` into total[i][j]
         auto fold_half = [&](int buf, int i, int j, int slot, int h, float scale) {
 #pragma unroll
             for (int r = 8 * h; r < 8 * h + 8; ++r) {
                 if constexpr (!B_ROWSCALE) {
                     total[i][j][r] = fmaf(acc[buf][r], scale, total[i][j][r]);
-                } else if constexpr (OUTER) {
-                    total[i][j][r] = fmaf(acc[buf][r], prod[slot % PBUF][16 * j + r], total[i][j][r]);
                 } else {
-                    const float4 q = sb_q[slot][r / 4];
-                    const float sbv = r % 4 == 0 ? q.x : r % 4 == 1 ? q.y : r % 4 == 2 ? q.z : q.w;
-                    total[i][j][r] = fmaf(acc[buf][r], scale * sbv, total[i][j][r]);
+                    total[i][j][r] = fmaf(acc[buf][r], prod[slot % PBUF][16 * j + r], total[i][j][r]);
                 }
             }
         };
@@ -485,18 +462,13 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
             float outer_a = 0.0f, outer_b = 0.0f;
             if constexpr (OUTER) {
                 static_assert(PAIRS % 2 == 0, "the two product buffers alternate across chunk boundaries");
-                outer_a = (scale_b - F_SBLOCK / 4)[kg[0] * BM + a_sub(lhi) + l32];
-                outer_b = scale_b[kg[0] * BM + b_sub(ti[0]) + l32];
+                outer_a = scale_at(0, c, kg[0], a_sub(lhi) + l32);
+                outer_b = scale_at(1, c, kg[0], b_sub(ti[0]) + l32);
             }
             auto issue_products = [&]() {
                 const f32x32 zero32 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                 prod[pair % PBUF] = __builtin_amdgcn_mfma_f32_32x32x1f32(outer_b, outer_a, zero32, 0, 0, 0);
             };
-            if constexpr (B_ROWSCALE && !OUTER) {
-#pragma unroll
-                for (int r4 = 0; r4 < 4; ++r4)
-                    sb_q[pair & 1][r4] = *reinterpret_cast<const float4*>(&scale_b[kg[0] * BM + b_sub(ti[0]) + r4 * 8 + lhi * 4]);
-            }
 #pragma unroll
             for (int step = 0; step < 4; ++step) {
                 const int h = step & 1, ks = step >> 1;
@@ -535,8 +507,9 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
     // for everybody and nobody reads chunk c's stage any more. Then: the loads of chunk c+3 into that stage (one
     // instruction every few MFMAs, so the waves of a CU do not queue up at the memory pipe), the LDS reads of chunk
     // c+1 into the other register set, the math of chunk c. Scale block b (K groups 8b ..) is fetched in iteration
-    // 4b-4, rearranged in 4b-2 and first read in 4b-1; it is issued before the chunk loads of its iteration, so the
-    // waits below cover it one iteration later.
+    // 4b-4 into the buffer that block b-2 left at the barrier of that iteration, has landed for every wave at the barrier
+    // of iteration 4b-2 and is first read in 4b-1; it is issued before the chunk loads of its iteration, so the waits
+    // below cover it one iteration later.
     constexpr int STEPS = FKG * TN * TM * 2, STRIDE = STEPS / CHUNK_LOADS;
     int stage_now = 0, stage_next = 1;
     auto chunk_step = [&](int c, const Operands& now, Operands& next) {
@@ -548,7 +521,6 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
         __syncthreads();
         if constexpr (!NOFOLD) {
             if (c % F_SCHUNKS == 0) issue_scales(c / F_SCHUNKS + 1);
-            if (c % F_SCHUNKS == 2) arrange_scales(c / F_SCHUNKS + 1);
         }
         if constexpr (MX) {
             if (c % MX_CHUNKS == 0) issue_mx_scales(c / MX_CHUNKS + 1);
@@ -568,10 +540,6 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
     for (int s = 0; s < K_STAGES; ++s) issue(s, s);
     __builtin_amdgcn_s_waitcnt(0x0F70 | ((K_STAGES - 1) * CHUNK_LOADS));                   // scale block 0 and chunk 0 are in LDS
     __syncthreads();
-    if constexpr (!NOFOLD) {
-        arrange_scales(0);
-        __syncthreads();
-    }
     Operands set0, set1;
     read_operands(0, 0, set0);
     for (int c = 0; c < chunks; c += 2) {
