@@ -45,6 +45,30 @@ def test_group_gemm(ga, gb, formats, shape, out_dtype):
     assert rel_l2(nobias, og.gemm(qa, qb, sa, sb, ga, gb, witness=True, out_dtype=torch.float64)) < 2e-5
 
 
+@pytest.mark.parametrize("gb", [(32, 32), (1, 32)])
+@pytest.mark.parametrize("k", [96, 160, 224, 288, 32])
+def test_group_gemm_scales_past_the_k_range_do_not_leak(gb, k):
+    """Scales are stored [rows, k / 32], so what follows a row's last scale in memory is the next row's first one. The
+    kernel fetches scales in 16-byte pieces; when k / 32 is not a multiple of four, the last piece of a row reaches into
+    the next row, and a NaN or an Inf there (the scale of a group that holds one) must not reach this row's sums."""
+    from viola_amd.nn import _grouped_kernels as g
+    m, n = 130, 128
+    (qa, sa), (qb, sb) = _operands(m, k, n, (1, 32), gb, E4, E4, seed=77)
+    qa, sa, qb, sb = qa.cuda(), sa.cuda(), qb.cuda(), sb.cuda()
+    clean = g.gemm(qa, qb, sa, sb, (1, 32), gb, out_dtype=torch.float32)
+    sa2, sb2 = sa.clone(), sb.clone()
+    sa2[5, 0], sa2[77, 0], sa2[129, 0] = float("nan"), float("inf"), float("nan")
+    bad_columns = []
+    if gb == (1, 32):
+        sb2[9, 0] = float("nan")
+        bad_columns = [9]
+    dirty = g.gemm(qa, qb, sa2, sb2, (1, 32), gb, out_dtype=torch.float32)
+    rows = torch.tensor([r for r in range(m) if r not in (5, 77, 129)], device="cuda")
+    columns = torch.tensor([c for c in range(n) if c not in bad_columns], device="cuda")
+    assert torch.equal(dirty[rows][:, columns], clean[rows][:, columns])
+    assert not torch.isfinite(dirty[5]).any() and not torch.isfinite(dirty[129]).any()
+
+
 def test_group_gemm_special_structure():
     """Identity-like operands make the expected value exact: catches a transposed operand or a wrong scale index."""
     from viola_amd.nn import _grouped_kernels as g

@@ -273,6 +273,19 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
         load16_to_lds(res_sa, at, inside ? sa_off : OUTSIDE, (uint32_t)(block * F_SGROUPS * 4));
         load16_to_lds(res_sb, at + F_SBLOCK, inside ? sb_off : OUTSIDE, (uint32_t)(block * F_SGROUPS * 4));
     };
+    // The one scale block that straddles the end of the k range holds, past that end, whatever follows in memory (the
+    // next row's first scales, perhaps a NaN): the thread that fetched a piece clears those entries once its loads
+    // have landed. Their products are zero, and zero times the cleared scale stays zero. (Pieces wholly past the end
+    // were not fetched and read as zero already.)
+    auto clear_past_the_end = [&](int block) {
+        const int left = groups_total - (int)(block * F_SGROUPS + shalf * 4);
+        if (left <= 0 || left >= 4) return;
+        float* mine = reinterpret_cast<float*>(lds + F_RAW + (block & 1) * 2 * F_SBLOCK + tid * 16);
+#pragma unroll
+        for (int q = 1; q < 4; ++q)
+            if (q >= left) { mine[q] = 0.0f; mine[F_SBLOCK / 4 + q] = 0.0f; }
+    };
+    const int last_scale_block = (groups_total - 1) / F_SGROUPS;             // the only block that can straddle
     // MX: scale block `block` (K groups 16 block ..) -> buffer block & 1: waves 0, 1 fetch the a rows' pieces, waves 2, 3 the b rows'
     const i32x4 res_mxa = raw_resource(p.sa, p.sa_bytes);
     const i32x4 res_mxb = raw_resource(sbptr, p.sb_bytes);
@@ -333,13 +346,11 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
         i32x8 wide_a[TM], wide_b[TN];                                        // TENSOR / MX: 16 k of either K group of a sub-tile row
         int mx_a[(TM + 1) / 2], mx_b[(TN + 1) / 2];                          // MX: the rows' scale bytes of K group lhi, sub-tile t in byte 2 (t & 1) of word t / 2
     };
-    // scale of tile row `row` for K group kg of chunk c (operand 0: a, 1: b); a group past the k range gives zero (its
-    // products are zero too, and whatever the piece holds there, a neighbouring row's value perhaps, must not meet them)
+    // scale of tile row `row` for K group kg of chunk c (operand 0: a, 1: b); groups past the k range read as zero
     auto scale_at = [&](int operand, int c, int kg, int row) -> float {
-        const int g8 = (c % F_SCHUNKS) * FKG + kg;                          // group of the block: uniform, like the test below
+        const int g8 = (c % F_SCHUNKS) * FKG + kg;                          // group of the block (uniform)
         const float* block = reinterpret_cast<const float*>(lds + F_RAW + ((c / F_SCHUNKS) & 1) * 2 * F_SBLOCK + operand * F_SBLOCK);
-        const float v = block[((g8 >> 2) * BM + row) * 4 + (g8 & 3)];
-        return c * FKG + kg < groups_total ? v : 0.0f;
+        return block[((g8 >> 2) * BM + row) * 4 + (g8 & 3)];
     };
     auto read_operands = [&](int stage, int c, Operands& o) {
         const uint8_t* tile_a = lds + stage * K_STAGE;
@@ -521,6 +532,9 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
         __syncthreads();
         if constexpr (!NOFOLD) {
             if (c % F_SCHUNKS == 0) issue_scales(c / F_SCHUNKS + 1);
+            // the wait above has seen this wave's loads of that block land; the next barrier shows the fix to every wave
+            // before the block's first use, one iteration later
+            if (c % F_SCHUNKS == 2 && c / F_SCHUNKS + 1 == last_scale_block) clear_past_the_end(last_scale_block);
         }
         if constexpr (MX) {
             if (c % MX_CHUNKS == 0) issue_mx_scales(c / MX_CHUNKS + 1);
@@ -540,6 +554,12 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
     for (int s = 0; s < K_STAGES; ++s) issue(s, s);
     __builtin_amdgcn_s_waitcnt(0x0F70 | ((K_STAGES - 1) * CHUNK_LOADS));                   // scale block 0 and chunk 0 are in LDS
     __syncthreads();
+    if constexpr (!NOFOLD) {
+        if (last_scale_block == 0 && groups_total % 4 != 0) {                // a k range of one scale block: uniform
+            clear_past_the_end(0);
+            __syncthreads();
+        }
+    }
     Operands set0, set1;
     read_operands(0, 0, set0);
     for (int c = 0; c < chunks; c += 2) {
