@@ -69,6 +69,32 @@ def test_group_gemm_scales_past_the_k_range_do_not_leak(gb, k):
     assert not torch.isfinite(dirty[5]).any() and not torch.isfinite(dirty[129]).any()
 
 
+@pytest.mark.parametrize("formats", [(E4, E4), (E5, E4)])
+@pytest.mark.parametrize("k", [2048, 2064, 2336, 4000, 6176])
+def test_group_gemm_rowwise_long_k_few_tiles(k, formats):
+    """Row-wise scales on both operands, a long k and few output tiles (the weight-gradient shape): the kernel splits the
+    k range of a tile over two teams of waves and adds their sums. k values around the split's granularity (256) and with
+    a ragged last scale piece; a NaN / Inf scale in a neighbouring row must stay in its row."""
+    from viola_amd.nn import _grouped_kernels as g
+    m, n = 130, 200
+    (qa, sa), (qb, sb) = _operands(m, k, n, (1, 32), (1, 32), *formats, seed=k, spread=2)    # sums stay inside fp16
+    bias = torch.randn(n)
+    expected = og.gemm(qa, qb, sa, sb, (1, 32), (1, 32), bias=bias, witness=True, out_dtype=torch.float64)
+    qa, sa, qb, sb = qa.cuda(), sa.cuda(), qb.cuda(), sb.cuda()
+    for out_dtype, bound in ((torch.float32, 2e-5), (torch.bfloat16, 3e-3), (torch.float16, 1e-3)):
+        actual = g.gemm(qa, qb, sa, sb, (1, 32), (1, 32), out_dtype=out_dtype, bias=bias.cuda())
+        assert actual.dtype == out_dtype and rel_l2(actual, expected) < bound
+        assert torch.equal(actual, g.gemm(qa, qb, sa, sb, (1, 32), (1, 32), out_dtype=out_dtype, bias=bias.cuda()))
+    clean = g.gemm(qa, qb, sa, sb, (1, 32), (1, 32), out_dtype=torch.float32)
+    sa2, sb2 = sa.clone(), sb.clone()
+    sa2[5, 0], sa2[129, 0], sb2[9, 0] = float("nan"), float("inf"), float("nan")
+    dirty = g.gemm(qa, qb, sa2, sb2, (1, 32), (1, 32), out_dtype=torch.float32)
+    rows = torch.tensor([r for r in range(m) if r not in (5, 129)], device="cuda")
+    columns = torch.tensor([c for c in range(n) if c != 9], device="cuda")
+    assert torch.equal(dirty[rows][:, columns], clean[rows][:, columns])
+    assert not torch.isfinite(dirty[5]).any() and not torch.isfinite(dirty[:, 9]).any()
+
+
 def test_group_gemm_special_structure():
     """Identity-like operands make the expected value exact: catches a transposed operand or a wrong scale index."""
     from viola_amd.nn import _grouped_kernels as g

@@ -4,13 +4,25 @@
 
 namespace viola {
 
-template <int MODE, bool B_ROWSCALE, typename TO, int TN>
+template <int MODE, bool B_ROWSCALE, typename TO, int TN, bool KSPLIT = false>
 static void launch_formats(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, dim3 grid, hipStream_t stream) {
     const bool a5 = a_dtype == VIOLA_E5M2, b5 = b_dtype == VIOLA_E5M2;
-    if (!a5 && !b5) VIOLA_LAUNCH((group_gemm_fast<MODE, false, false, B_ROWSCALE, TO, TN>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else if (a5 && !b5) VIOLA_LAUNCH((group_gemm_fast<MODE, true, false, B_ROWSCALE, TO, TN>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else if (!a5 && b5) VIOLA_LAUNCH((group_gemm_fast<MODE, false, true, B_ROWSCALE, TO, TN>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else VIOLA_LAUNCH((group_gemm_fast<MODE, true, true, B_ROWSCALE, TO, TN>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    const dim3 block(KSPLIT ? 2 * FTHREADS : FTHREADS);
+    if (!a5 && !b5) VIOLA_LAUNCH((group_gemm_fast<MODE, false, false, B_ROWSCALE, TO, TN, false, false, false, KSPLIT>), grid, block, 0, stream, p, bias_dtype);
+    else if (a5 && !b5) VIOLA_LAUNCH((group_gemm_fast<MODE, true, false, B_ROWSCALE, TO, TN, false, false, false, KSPLIT>), grid, block, 0, stream, p, bias_dtype);
+    else if (!a5 && b5) VIOLA_LAUNCH((group_gemm_fast<MODE, false, true, B_ROWSCALE, TO, TN, false, false, false, KSPLIT>), grid, block, 0, stream, p, bias_dtype);
+    else VIOLA_LAUNCH((group_gemm_fast<MODE, true, true, B_ROWSCALE, TO, TN, false, false, false, KSPLIT>), grid, block, 0, stream, p, bias_dtype);
+}
+
+// plain mode, row-wise b scales, the k range of a 128 x 128 tile split over two teams of waves
+static int launch_split(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, dim3 grid, hipStream_t stream) {
+    switch (out_dtype) {
+        case VIOLA_F32: launch_formats<MODE_PLAIN, true, float, 2, true>(p, a_dtype, b_dtype, bias_dtype, grid, stream); break;
+        case VIOLA_BF16: launch_formats<MODE_PLAIN, true, bf16_t, 2, true>(p, a_dtype, b_dtype, bias_dtype, grid, stream); break;
+        case VIOLA_F16: launch_formats<MODE_PLAIN, true, f16_t, 2, true>(p, a_dtype, b_dtype, bias_dtype, grid, stream); break;
+        default: return VIOLA_EINVAL;
+    }
+    return viola_launch_status();
 }
 
 template <int MODE, int TN>
@@ -29,6 +41,11 @@ static int launch_mode(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dty
     return viola_launch_status();
 }
 
+#ifndef VIOLA_SPLIT_MIN_K
+#define VIOLA_SPLIT_MIN_K 2048
+#endif
+constexpr int64_t SPLIT_MIN_K = VIOLA_SPLIT_MIN_K;
+
 int launch_group_gemm_fast(const GemmArgs& args, int mode, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, bool rowscale,
                            dim3 grid, hipStream_t stream) {
     GemmArgs p = args;
@@ -36,13 +53,18 @@ int launch_group_gemm_fast(const GemmArgs& args, int mode, int a_dtype, int b_dt
     p.sa_bytes = (p.m + p.ar - 1) / p.ar * p.ldsa * 4;
     p.sb_bytes = (b_rows + p.br - 1) / p.br * p.ldsb * 4;
     // Two blocks fit a CU: with fewer than 512 tiles of 128 x 128, halve the tile in n so that all 256 CUs get two.
-    const bool narrow = mode == MODE_PLAIN && (int64_t)grid.x * grid.y * grid.z < 512 && p.n > 64;
+    // Row-wise b scales over a long k instead keep the tile and split its k range inside the block (one block of twice the
+    // waves per CU).
+    const bool few = mode == MODE_PLAIN && (int64_t)grid.x * grid.y * grid.z < 512;
+    const bool split = few && rowscale && !p.offsets && !p.koffsets && p.k >= SPLIT_MIN_K;
+    const bool narrow = few && !split && p.n > 64;
     if (narrow) grid.x = (unsigned)((p.n + 63) / 64);
     if (!p.offsets && (int64_t)grid.x * grid.y < (1 << 30)) {
         p.tiles_n = (int)grid.x;
         p.tiles_m = (int)grid.y;
         grid = dim3((grid.x * grid.y + 7) / 8 * 8, 1, grid.z);
     }
+    if (split) return launch_split(p, a_dtype, b_dtype, bias_dtype, out_dtype, grid, stream);
     if (narrow) return launch_mode<MODE_PLAIN, 1>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
     if (mode == MODE_PLAIN) return launch_mode<MODE_PLAIN, 2>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
     if (mode == MODE_GATED_FWD) return launch_mode<MODE_GATED_FWD, 2>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);

@@ -125,8 +125,16 @@ constexpr int MX_GROUPS = 16, MX_CHUNKS = MX_GROUPS / FKG, MX_BLOCK = 2 * BM * M
 // sub-tiles, one block per CU. Without the per-group fold these kernels are bound by the L2 -> LDS stream (taking the
 // global loads out of the 128 x 128 kernel brings it from 1.7 to 4.4 PFLOP/s on a 16384 x 22016 x 4096 product, taking
 // the LDS reads out changes nothing); the larger tile moves half the bytes per flop.
-template <int MODE, bool A_BF8, bool B_BF8, bool B_ROWSCALE, typename TO, int TN, bool TENSOR = false, bool MX = false, bool BIG = false>
-__global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) void group_gemm_fast(GemmArgs p, int bias_dtype) {
+// KSPLIT (row-wise b scales, plain mode): for products with fewer than 512 tiles of 128 x 128 and a long k. A block
+// of 512 threads is two teams of 2 x 2 waves, each with a stage ring and scale buffers of its own, that compute the
+// same 128 x 128 tile over the two halves of the k range (cut at a multiple of 256 k, one scale block); at the end
+// team 1 hands its totals over in LDS and team 0 adds them to its own (always in that order) and stores the tile.
+// Against the 128 x 64 tiles such products would otherwise get, a wave has the 2 x 2 sub-tiles' better ratio of MFMAs to
+// global loads and LDS reads, and a CU still holds eight waves.
+template <int MODE, bool A_BF8, bool B_BF8, bool B_ROWSCALE, typename TO, int TN, bool TENSOR = false, bool MX = false, bool BIG = false,
+          bool KSPLIT = false>
+__global__ __launch_bounds__(BIG || KSPLIT ? 512 : FTHREADS, BIG || KSPLIT ? 1 : TENSOR ? 3 : 2) void group_gemm_fast(GemmArgs p, int bias_dtype) {
+    static_assert(!KSPLIT || (B_ROWSCALE && MODE == MODE_PLAIN && TN == 2 && !TENSOR && !MX && !BIG), "the split exists for the weight-gradient shape");
     static_assert(!TENSOR || !B_ROWSCALE, "per-tensor scaling has no row scales");
     static_assert(!MX || !TENSOR, "one scaling recipe per kernel");
     static_assert(!BIG || ((TENSOR || MX) && TN == 2), "the large tile exists for the fold-free kernels");
@@ -137,7 +145,7 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
     constexpr int K_STAGES = BIG ? VIOLA_BIG_STAGES : FSTAGES, K_RAW = K_STAGES * K_STAGE;   // ring depth: loads run K_STAGES chunks ahead
     constexpr int K_MX_BLOCK = BIG ? 2 * MX_BLOCK : MX_BLOCK;
     // without scale blocks the ring plus the epilogue's bias row is all the LDS a block needs: three blocks share a CU
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[TENSOR ? K_RAW + 1024 : MX ? K_RAW + 2 * K_MX_BLOCK : F_LDS];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_all[TENSOR ? K_RAW + 1024 : MX ? K_RAW + 2 * K_MX_BLOCK : KSPLIT ? 2 * F_LDS : F_LDS];
 
     // wave grid 2 (m) x 2 (n), 2 x 2 sub-tiles each. Plain / gated backward: sub-tile i of wave wn covers b rows
     // 64 wn + 32 i. Gated forward: the tile's b rows are 64 gate rows then the 64 up rows of the same n, and
@@ -146,7 +154,10 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
     constexpr int TM = BIG ? 4 : 2;
     constexpr int PANEL = GATED ? 32 * WAVES_N : 32 * TN * WAVES_N;
     static_assert(!GATED || TN == 2, "gated forward pairs a gate and an up sub-tile");
-    const int tid = threadIdx.x, lane = tid % WAVE;
+    // KSPLIT: `team` is the half of the k range this wave works on; tid, wave and lds are the team's own
+    const int team = KSPLIT ? __builtin_amdgcn_readfirstlane((int)threadIdx.x / FTHREADS) : 0;
+    const int tid = KSPLIT ? (int)threadIdx.x % FTHREADS : (int)threadIdx.x, lane = tid % WAVE;
+    uint8_t* const lds = lds_all + team * (KSPLIT ? F_LDS : 0);
     const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int l32 = lane % 32, lhi = lane / 32;
@@ -192,6 +203,14 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
         outptr += (int64_t)g * p.out_group_stride * (int64_t)sizeof(TO);
     }
     if (m_begin >= m_end) return;
+    int split_chunks = 0;                                                    // KSPLIT: chunks of the longer (first) half
+    if constexpr (KSPLIT) {
+        const int64_t len = k_end - k_begin, blocks = (len + F_SGROUPS * 32 - 1) / (F_SGROUPS * 32);
+        const int64_t first = (blocks + 1) / 2 * (F_SGROUPS * 32) < len ? (blocks + 1) / 2 * (F_SGROUPS * 32) : len;
+        split_chunks = (int)((first + FBK - 1) / FBK);
+        if (team == 0) k_end = k_begin + first;
+        else k_begin += first;
+    }
     const int64_t n_begin = (int64_t)tile_n * PANEL;
     const int64_t b_rows_total = GATED ? 2 * p.n : p.n;
     auto b_global_row = [&](int r) -> int64_t {                               // tile-local b row -> row of b
@@ -215,7 +234,9 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
     constexpr uint32_t OUTSIDE = 0x80000000u;
     const int64_t k_len = k_end - k_begin;
     const int groups_total = (int)((k_len + 31) / 32);
-    const int chunks = (int)((k_len + FBK - 1) / FBK);
+    // (KSPLIT: both teams walk the first half's chunk count, they share the barriers; past its own range a team loads
+    // zero codes and zero scales)
+    const int chunks = KSPLIT ? split_chunks : (int)((k_len + FBK - 1) / FBK);
     const int full_chunks = (int)(k_len / FBK);                             // chunks wholly inside the k range
     // Offsets of the thread's 16-byte pieces. Chunks wholly inside the k range use them as they are; for the one chunk
     // that straddles the end of the range the pieces past it are redirected outside the buffer (they read zero), and
@@ -554,7 +575,10 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
     for (int s = 0; s < K_STAGES; ++s) issue(s, s);
     __builtin_amdgcn_s_waitcnt(0x0F70 | ((K_STAGES - 1) * CHUNK_LOADS));                   // scale block 0 and chunk 0 are in LDS
     __syncthreads();
-    if constexpr (!NOFOLD) {
+    if constexpr (KSPLIT) {                                                  // the condition differs between the teams, the barrier must not
+        if (last_scale_block == 0 && groups_total % 4 != 0) clear_past_the_end(0);
+        __syncthreads();
+    } else if constexpr (!NOFOLD) {
         if (last_scale_block == 0 && groups_total % 4 != 0) {                // a k range of one scale block: uniform
             clear_past_the_end(0);
             __syncthreads();
@@ -583,6 +607,37 @@ __global__ __launch_bounds__(BIG ? 512 : FTHREADS, BIG ? 1 : TENSOR ? 3 : 2) voi
 #pragma unroll
             for (int r = 0; r < 16; ++r)
                 total[li][lj][r] = fmaf(acc[(last_pair & 1) * 2 + h][r], OUTER ? prod[last_pair % PBUF][16 * lj + r] : pending_scale[h], total[li][lj][r]);
+        }
+    }
+
+    if constexpr (KSPLIT) {
+        // team 1's totals -> LDS (the first team's ring, idle now) as [register quad][thread], team 0 adds them. Team 1 then
+        // walks the epilogue with an empty row range: it stores nothing and meets the barriers there.
+        __syncthreads();
+        float4* handover = reinterpret_cast<float4*>(lds_all);
+        static_assert(TN * TM * 16 * 4 * FTHREADS <= F_LDS, "a team's totals fit the other team's LDS");
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+            for (int j = 0; j < TM; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float4* at = &handover[((i * TM + j) * 4 + q) * FTHREADS + tid];
+                    if (team == 1) *at = make_float4(total[i][j][4 * q], total[i][j][4 * q + 1], total[i][j][4 * q + 2], total[i][j][4 * q + 3]);
+                }
+        __syncthreads();
+        if (team == 0) {
+#pragma unroll
+            for (int i = 0; i < TN; ++i)
+#pragma unroll
+                for (int j = 0; j < TM; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const float4 t = handover[((i * TM + j) * 4 + q) * FTHREADS + tid];
+                        total[i][j][4 * q] += t.x; total[i][j][4 * q + 1] += t.y; total[i][j][4 * q + 2] += t.z; total[i][j][4 * q + 3] += t.w;
+                    }
+        } else {
+            m_end = m_begin;
         }
     }
 
