@@ -69,30 +69,38 @@ def test_group_gemm_scales_past_the_k_range_do_not_leak(gb, k):
     assert not torch.isfinite(dirty[5]).any() and not torch.isfinite(dirty[129]).any()
 
 
-@pytest.mark.parametrize("formats", [(E4, E4), (E5, E4)])
-@pytest.mark.parametrize("k", [2048, 2064, 2336, 4000, 6176])
-def test_group_gemm_rowwise_long_k_few_tiles(k, formats):
-    """Row-wise scales on both operands, a long k and few output tiles (the weight-gradient shape): the kernel splits the
-    k range of a tile over two teams of waves and adds their sums. k values around the split's granularity (256) and with
-    a ragged last scale piece; a NaN / Inf scale in a neighbouring row must stay in its row."""
+@pytest.mark.parametrize("gb", [(1, 32), (32, 32)])
+@pytest.mark.parametrize("k,formats", [(2048, (E4, E4)), (2064, (E5, E4)), (2336, (E4, E4)), (4000, (E4, E5)), (6176, (E5, E5))])
+def test_group_gemm_long_k_few_tiles(k, formats, gb):
+    """A long k and 129 .. 511 output tiles of 128 x 128 (a weight gradient; a small-batch dgrad): the kernel splits the k
+    range of a tile over two teams of waves and adds their sums. k values around the split's granularity (256) and with a
+    ragged last scale piece; a NaN / Inf scale in a neighbouring row must stay in its row."""
     from viola_amd.nn import _grouped_kernels as g
-    m, n = 130, 200
-    (qa, sa), (qb, sb) = _operands(m, k, n, (1, 32), (1, 32), *formats, seed=k, spread=2)    # sums stay inside fp16
+    m, n = 1930, 1100                                                         # 16 x 9 tiles, ragged in both directions
+    (qa, sa), (qb, sb) = _operands(m, k, n, (1, 32), gb, *formats, seed=k, spread=2)    # sums stay inside fp16
     bias = torch.randn(n)
-    expected = og.gemm(qa, qb, sa, sb, (1, 32), (1, 32), bias=bias, witness=True, out_dtype=torch.float64)
+    rows = torch.cat([torch.arange(0, 140), torch.arange(1900, m)])           # the oracle on row samples: first tiles and the ragged last
+    expected = og.gemm(qa[rows], qb, sa[rows], sb, (1, 32), gb, bias=bias, witness=True, out_dtype=torch.float64)
     qa, sa, qb, sb = qa.cuda(), sa.cuda(), qb.cuda(), sb.cuda()
     for out_dtype, bound in ((torch.float32, 2e-5), (torch.bfloat16, 3e-3), (torch.float16, 1e-3)):
-        actual = g.gemm(qa, qb, sa, sb, (1, 32), (1, 32), out_dtype=out_dtype, bias=bias.cuda())
-        assert actual.dtype == out_dtype and rel_l2(actual, expected) < bound
-        assert torch.equal(actual, g.gemm(qa, qb, sa, sb, (1, 32), (1, 32), out_dtype=out_dtype, bias=bias.cuda()))
-    clean = g.gemm(qa, qb, sa, sb, (1, 32), (1, 32), out_dtype=torch.float32)
+        actual = g.gemm(qa, qb, sa, sb, (1, 32), gb, out_dtype=out_dtype, bias=bias.cuda())
+        assert actual.dtype == out_dtype and rel_l2(actual[rows.cuda()], expected) < bound
+        assert torch.equal(actual, g.gemm(qa, qb, sa, sb, (1, 32), gb, out_dtype=out_dtype, bias=bias.cuda()))
+    # every row against an FP32 matmul of the dequantized operands (sums of a different order)
+    reference = g.dequantize(qa, sa, (1, 32)).float() @ g.dequantize(qb, sb, gb).float().t() + bias.cuda()
+    assert rel_l2(g.gemm(qa, qb, sa, sb, (1, 32), gb, out_dtype=torch.float32, bias=bias.cuda()), reference) < 2e-5
+    clean = g.gemm(qa, qb, sa, sb, (1, 32), gb, out_dtype=torch.float32)
     sa2, sb2 = sa.clone(), sb.clone()
-    sa2[5, 0], sa2[129, 0], sb2[9, 0] = float("nan"), float("inf"), float("nan")
-    dirty = g.gemm(qa, qb, sa2, sb2, (1, 32), (1, 32), out_dtype=torch.float32)
-    rows = torch.tensor([r for r in range(m) if r not in (5, 129)], device="cuda")
-    columns = torch.tensor([c for c in range(n) if c != 9], device="cuda")
-    assert torch.equal(dirty[rows][:, columns], clean[rows][:, columns])
-    assert not torch.isfinite(dirty[5]).any() and not torch.isfinite(dirty[:, 9]).any()
+    sa2[5, 0], sa2[m - 1, 0] = float("nan"), float("inf")
+    bad_columns = []
+    if gb == (1, 32):
+        sb2[9, 0] = float("nan")
+        bad_columns = [9]
+    dirty = g.gemm(qa, qb, sa2, sb2, (1, 32), gb, out_dtype=torch.float32)
+    keep = torch.tensor([r for r in range(m) if r not in (5, m - 1)], device="cuda")
+    columns = torch.tensor([c for c in range(n) if c not in bad_columns], device="cuda")
+    assert torch.equal(dirty[keep][:, columns], clean[keep][:, columns])
+    assert not torch.isfinite(dirty[5]).any() and not torch.isfinite(dirty[m - 1]).any()
 
 
 def test_group_gemm_special_structure():

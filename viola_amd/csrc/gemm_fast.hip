@@ -14,14 +14,19 @@ static void launch_formats(const GemmArgs& p, int a_dtype, int b_dtype, int bias
     else VIOLA_LAUNCH((group_gemm_fast<MODE, true, true, B_ROWSCALE, TO, TN, false, false, false, KSPLIT>), grid, block, 0, stream, p, bias_dtype);
 }
 
-// plain mode, row-wise b scales, the k range of a 128 x 128 tile split over two teams of waves
-static int launch_split(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, dim3 grid, hipStream_t stream) {
+// plain mode, the k range of a 128 x 128 tile split over two teams of waves
+static int launch_split(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, bool rowscale, dim3 grid,
+                        hipStream_t stream) {
+#define VIOLA_SPLIT(TO)                                                                                        \
+    if (rowscale) launch_formats<MODE_PLAIN, true, TO, 2, true>(p, a_dtype, b_dtype, bias_dtype, grid, stream); \
+    else launch_formats<MODE_PLAIN, false, TO, 2, true>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
     switch (out_dtype) {
-        case VIOLA_F32: launch_formats<MODE_PLAIN, true, float, 2, true>(p, a_dtype, b_dtype, bias_dtype, grid, stream); break;
-        case VIOLA_BF16: launch_formats<MODE_PLAIN, true, bf16_t, 2, true>(p, a_dtype, b_dtype, bias_dtype, grid, stream); break;
-        case VIOLA_F16: launch_formats<MODE_PLAIN, true, f16_t, 2, true>(p, a_dtype, b_dtype, bias_dtype, grid, stream); break;
+        case VIOLA_F32: VIOLA_SPLIT(float) break;
+        case VIOLA_BF16: VIOLA_SPLIT(bf16_t) break;
+        case VIOLA_F16: VIOLA_SPLIT(f16_t) break;
         default: return VIOLA_EINVAL;
     }
+#undef VIOLA_SPLIT
     return viola_launch_status();
 }
 
@@ -46,6 +51,7 @@ static int launch_mode(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dty
 #endif
 constexpr int64_t SPLIT_MIN_K = VIOLA_SPLIT_MIN_K;
 
+
 int launch_group_gemm_fast(const GemmArgs& args, int mode, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, bool rowscale,
                            dim3 grid, hipStream_t stream) {
     GemmArgs p = args;
@@ -53,10 +59,11 @@ int launch_group_gemm_fast(const GemmArgs& args, int mode, int a_dtype, int b_dt
     p.sa_bytes = (p.m + p.ar - 1) / p.ar * p.ldsa * 4;
     p.sb_bytes = (b_rows + p.br - 1) / p.br * p.ldsb * 4;
     // Two blocks fit a CU: with fewer than 512 tiles of 128 x 128, halve the tile in n so that all 256 CUs get two.
-    // Row-wise b scales over a long k instead keep the tile and split its k range inside the block (one block of twice the
-    // waves per CU).
-    const bool few = mode == MODE_PLAIN && (int64_t)grid.x * grid.y * grid.z < 512;
-    const bool split = few && rowscale && !p.offsets && !p.koffsets && p.k >= SPLIT_MIN_K;
+    // Over a long k, and with enough tiles to give half the CUs one each, keep the tile instead and split its k range inside
+    // the block (one block of twice the waves per CU): 7-12 % faster from 256 tiles up, slower at 64 (half as many CUs busy).
+    const int64_t tiles = (int64_t)grid.x * grid.y * grid.z;
+    const bool few = mode == MODE_PLAIN && tiles < 512;
+    const bool split = few && tiles > 128 && !p.offsets && !p.koffsets && p.k >= SPLIT_MIN_K;
     const bool narrow = few && !split && p.n > 64;
     if (narrow) grid.x = (unsigned)((p.n + 63) / 64);
     if (!p.offsets && (int64_t)grid.x * grid.y < (1 << 30)) {
@@ -64,7 +71,7 @@ int launch_group_gemm_fast(const GemmArgs& args, int mode, int a_dtype, int b_dt
         p.tiles_m = (int)grid.y;
         grid = dim3((grid.x * grid.y + 7) / 8 * 8, 1, grid.z);
     }
-    if (split) return launch_split(p, a_dtype, b_dtype, bias_dtype, out_dtype, grid, stream);
+    if (split) return launch_split(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
     if (narrow) return launch_mode<MODE_PLAIN, 1>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
     if (mode == MODE_PLAIN) return launch_mode<MODE_PLAIN, 2>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
     if (mode == MODE_GATED_FWD) return launch_mode<MODE_GATED_FWD, 2>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);

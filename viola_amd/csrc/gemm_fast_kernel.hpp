@@ -125,16 +125,16 @@ constexpr int MX_GROUPS = 16, MX_CHUNKS = MX_GROUPS / FKG, MX_BLOCK = 2 * BM * M
 // sub-tiles, one block per CU. Without the per-group fold these kernels are bound by the L2 -> LDS stream (taking the
 // global loads out of the 128 x 128 kernel brings it from 1.7 to 4.4 PFLOP/s on a 16384 x 22016 x 4096 product, taking
 // the LDS reads out changes nothing); the larger tile moves half the bytes per flop.
-// KSPLIT (row-wise b scales, plain mode): for products with fewer than 512 tiles of 128 x 128 and a long k. A block
-// of 512 threads is two teams of 2 x 2 waves, each with a stage ring and scale buffers of its own, that compute the
-// same 128 x 128 tile over the two halves of the k range (cut at a multiple of 256 k, one scale block); at the end
+// KSPLIT (plain mode): for products with fewer than 512 tiles of 128 x 128 and a long k, such as a weight gradient. A
+// block of 512 threads is two teams of 2 x 2 waves, each with a stage ring and scale buffers of its own, that compute
+// the same 128 x 128 tile over the two halves of the k range (cut at a multiple of 256 k, one scale block); at the end
 // team 1 hands its totals over in LDS and team 0 adds them to its own (always in that order) and stores the tile.
 // Against the 128 x 64 tiles such products would otherwise get, a wave has the 2 x 2 sub-tiles' better ratio of MFMAs to
 // global loads and LDS reads, and a CU still holds eight waves.
 template <int MODE, bool A_BF8, bool B_BF8, bool B_ROWSCALE, typename TO, int TN, bool TENSOR = false, bool MX = false, bool BIG = false,
           bool KSPLIT = false>
 __global__ __launch_bounds__(BIG || KSPLIT ? 512 : FTHREADS, BIG || KSPLIT ? 1 : TENSOR ? 3 : 2) void group_gemm_fast(GemmArgs p, int bias_dtype) {
-    static_assert(!KSPLIT || (B_ROWSCALE && MODE == MODE_PLAIN && TN == 2 && !TENSOR && !MX && !BIG), "the split exists for the weight-gradient shape");
+    static_assert(!KSPLIT || (MODE == MODE_PLAIN && TN == 2 && !TENSOR && !MX && !BIG), "the split exists for plain products of the grouped recipe");
     static_assert(!TENSOR || !B_ROWSCALE, "per-tensor scaling has no row scales");
     static_assert(!MX || !TENSOR, "one scaling recipe per kernel");
     static_assert(!BIG || ((TENSOR || MX) && TN == 2), "the large tile exists for the fold-free kernels");
