@@ -31,8 +31,8 @@ PEAK = {"fp8_tflops": 5000.0, "bf16_tflops": 2500.0, "hbm_gbs": 8000.0}
 # L2<->fabric bytes per grouped-scale GEMM launch, mean of the step's three launches (fwd, dgrad, wgrad), from two
 # `rocprofv3 --pmc` runs of `bench.py --skip-cpu --skip-muon --steps 5 --warmup 3 --calibrate` (FETCH_SIZE, then WRITE_SIZE, KiB per
 # dispatch), each scaled by the same counter's reading for the 256 MiB copy_scaled_kernel launch (factors 2.00 and 1.00):
-# fetch (2 * 58.2 + 121.7) / 3 MB, write (2 * 41.9 + 8.8) / 3 MB. The algorithmic figure is 65 MB per launch.
-GEMM_TRAFFIC_BYTES = 79.4e6 + 30.9e6
+# fetch (2 * 58.3 + 113.5) / 3 MB, write (2 * 41.9 + 8.4) / 3 MB. The algorithmic figure is 65 MB per launch.
+GEMM_TRAFFIC_BYTES = 76.7e6 + 30.8e6
 WARM_MS = 100.0
 
 
