@@ -134,7 +134,7 @@ constexpr int MX_GROUPS = 16, MX_CHUNKS = MX_GROUPS / FKG, MX_BLOCK = 2 * BM * M
 template <int MODE, bool A_BF8, bool B_BF8, bool B_ROWSCALE, typename TO, int TN, bool TENSOR = false, bool MX = false, bool BIG = false,
           bool KSPLIT = false>
 __global__ __launch_bounds__(BIG || KSPLIT ? 512 : FTHREADS, BIG || KSPLIT ? 1 : TENSOR ? 3 : 2) void group_gemm_fast(GemmArgs p, int bias_dtype) {
-    static_assert(!KSPLIT || (MODE == MODE_PLAIN && TN == 2 && !TENSOR && !MX && !BIG), "the split exists for plain products of the grouped recipe");
+    static_assert(!KSPLIT || (MODE == MODE_PLAIN && TN == 2 && !BIG), "the split exists for plain products on 128 x 128 tiles");
     static_assert(!TENSOR || !B_ROWSCALE, "per-tensor scaling has no row scales");
     static_assert(!MX || !TENSOR, "one scaling recipe per kernel");
     static_assert(!BIG || ((TENSOR || MX) && TN == 2), "the large tile exists for the fold-free kernels");
@@ -145,7 +145,8 @@ __global__ __launch_bounds__(BIG || KSPLIT ? 512 : FTHREADS, BIG || KSPLIT ? 1 :
     constexpr int K_STAGES = BIG ? VIOLA_BIG_STAGES : FSTAGES, K_RAW = K_STAGES * K_STAGE;   // ring depth: loads run K_STAGES chunks ahead
     constexpr int K_MX_BLOCK = BIG ? 2 * MX_BLOCK : MX_BLOCK;
     // without scale blocks the ring plus the epilogue's bias row is all the LDS a block needs: three blocks share a CU
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_all[TENSOR ? K_RAW + 1024 : MX ? K_RAW + 2 * K_MX_BLOCK : KSPLIT ? 2 * F_LDS : F_LDS];
+    constexpr int TEAM_LDS = TENSOR ? K_RAW + 1024 : MX ? K_RAW + 2 * K_MX_BLOCK : F_LDS;
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_all[(KSPLIT ? 2 : 1) * TEAM_LDS];
 
     // wave grid 2 (m) x 2 (n), 2 x 2 sub-tiles each. Plain / gated backward: sub-tile i of wave wn covers b rows
     // 64 wn + 32 i. Gated forward: the tile's b rows are 64 gate rows then the 64 up rows of the same n, and
@@ -157,7 +158,7 @@ __global__ __launch_bounds__(BIG || KSPLIT ? 512 : FTHREADS, BIG || KSPLIT ? 1 :
     // KSPLIT: `team` is the half of the k range this wave works on; tid, wave and lds are the team's own
     const int team = KSPLIT ? __builtin_amdgcn_readfirstlane((int)threadIdx.x / FTHREADS) : 0;
     const int tid = KSPLIT ? (int)threadIdx.x % FTHREADS : (int)threadIdx.x, lane = tid % WAVE;
-    uint8_t* const lds = lds_all + team * (KSPLIT ? F_LDS : 0);
+    uint8_t* const lds = lds_all + team * (KSPLIT ? TEAM_LDS : 0);
     const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int l32 = lane % 32, lhi = lane / 32;
@@ -205,8 +206,9 @@ __global__ __launch_bounds__(BIG || KSPLIT ? 512 : FTHREADS, BIG || KSPLIT ? 1 :
     if (m_begin >= m_end) return;
     int split_chunks = 0;                                                    // KSPLIT: chunks of the longer (first) half
     if constexpr (KSPLIT) {
-        const int64_t len = k_end - k_begin, blocks = (len + F_SGROUPS * 32 - 1) / (F_SGROUPS * 32);
-        const int64_t first = (blocks + 1) / 2 * (F_SGROUPS * 32) < len ? (blocks + 1) / 2 * (F_SGROUPS * 32) : len;
+        constexpr int64_t CUT = (MX ? MX_GROUPS : F_SGROUPS) * 32;            // a scale block belongs to one team
+        const int64_t len = k_end - k_begin, blocks = (len + CUT - 1) / CUT;
+        const int64_t first = (blocks + 1) / 2 * CUT < len ? (blocks + 1) / 2 * CUT : len;
         split_chunks = (int)((first + FBK - 1) / FBK);
         if (team == 0) k_end = k_begin + first;
         else k_begin += first;
@@ -575,7 +577,7 @@ __global__ __launch_bounds__(BIG || KSPLIT ? 512 : FTHREADS, BIG || KSPLIT ? 1 :
     for (int s = 0; s < K_STAGES; ++s) issue(s, s);
     __builtin_amdgcn_s_waitcnt(0x0F70 | ((K_STAGES - 1) * CHUNK_LOADS));                   // scale block 0 and chunk 0 are in LDS
     __syncthreads();
-    if constexpr (KSPLIT) {                                                  // the condition differs between the teams, the barrier must not
+    if constexpr (KSPLIT && !NOFOLD) {                                       // the condition differs between the teams, the barrier must not
         if (last_scale_block == 0 && groups_total % 4 != 0) clear_past_the_end(0);
         __syncthreads();
     } else if constexpr (!NOFOLD) {
@@ -591,15 +593,7 @@ __global__ __launch_bounds__(BIG || KSPLIT ? 512 : FTHREADS, BIG || KSPLIT ? 1 :
         if (c + 1 < chunks) chunk_step(c + 1, set1, set0);
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);     // drain the trailing loads before the LDS allocation is released
-    if constexpr (TENSOR) {
-        const float sa = p.sa[0], sb = p.sb[0];
-#pragma unroll
-        for (int i = 0; i < TN; ++i)
-#pragma unroll
-            for (int j = 0; j < TM; ++j)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) { const float t = total[i][j][r] * sa; total[i][j][r] = t * sb; }
-    } else if constexpr (CARRY && !MX) {
+    if constexpr (!TENSOR && CARRY && !MX) {
         constexpr int UNITS = FKG * TN * TM, last_pair = UNITS / 2 - 1;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
@@ -611,11 +605,11 @@ __global__ __launch_bounds__(BIG || KSPLIT ? 512 : FTHREADS, BIG || KSPLIT ? 1 :
     }
 
     if constexpr (KSPLIT) {
-        // team 1's totals -> LDS (the first team's ring, idle now) as [register quad][thread], team 0 adds them. Team 1 then
+        // team 1's totals -> LDS (the rings are idle now) as [register quad][thread], team 0 adds them. Team 1 then
         // walks the epilogue with an empty row range: it stores nothing and meets the barriers there.
         __syncthreads();
         float4* handover = reinterpret_cast<float4*>(lds_all);
-        static_assert(TN * TM * 16 * 4 * FTHREADS <= F_LDS, "a team's totals fit the other team's LDS");
+        static_assert(TN * TM * 16 * 4 * FTHREADS <= 2 * TEAM_LDS, "a team's totals fit the block's LDS");
 #pragma unroll
         for (int i = 0; i < TN; ++i)
 #pragma unroll
@@ -639,6 +633,15 @@ __global__ __launch_bounds__(BIG || KSPLIT ? 512 : FTHREADS, BIG || KSPLIT ? 1 :
         } else {
             m_end = m_begin;
         }
+    }
+    if constexpr (TENSOR) {
+        const float sa = p.sa[0], sb = p.sb[0];
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+            for (int j = 0; j < TM; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) { const float t = total[i][j][r] * sa; total[i][j][r] = t * sb; }
     }
 
     // ---- epilogue: for sub-tiles (i, j) the lane holds row m = 32*j + l32 and, per register quad r4, columns

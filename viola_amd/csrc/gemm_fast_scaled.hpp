@@ -7,13 +7,15 @@ namespace viola {
 
 // Per-tensor scales (TENSOR: args.sa / args.sb point at one float each) or E8M0 block scales (MX: they point at
 // bytes; ldsa / ldsb = bytes per scale row). grid: (n tiles, m tiles of 128); n tiles are 128 wide, 64 for gated forward.
-template <int MODE, typename TO, int TN, bool TENSOR, bool MX>
+// KSPLIT: the k range of a 128 x 128 tile split over two teams of waves in a 512-thread block (plain mode)
+template <int MODE, typename TO, int TN, bool TENSOR, bool MX, bool KSPLIT = false>
 static void launch_scaled_formats(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, dim3 grid, hipStream_t stream) {
     const bool a5 = a_dtype == VIOLA_E5M2, b5 = b_dtype == VIOLA_E5M2;
-    if (!a5 && !b5) VIOLA_LAUNCH((group_gemm_fast<MODE, false, false, false, TO, TN, TENSOR, MX>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else if (a5 && !b5) VIOLA_LAUNCH((group_gemm_fast<MODE, true, false, false, TO, TN, TENSOR, MX>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else if (!a5 && b5) VIOLA_LAUNCH((group_gemm_fast<MODE, false, true, false, TO, TN, TENSOR, MX>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
-    else VIOLA_LAUNCH((group_gemm_fast<MODE, true, true, false, TO, TN, TENSOR, MX>), grid, dim3(FTHREADS), 0, stream, p, bias_dtype);
+    const dim3 block(KSPLIT ? 2 * FTHREADS : FTHREADS);
+    if (!a5 && !b5) VIOLA_LAUNCH((group_gemm_fast<MODE, false, false, false, TO, TN, TENSOR, MX, false, KSPLIT>), grid, block, 0, stream, p, bias_dtype);
+    else if (a5 && !b5) VIOLA_LAUNCH((group_gemm_fast<MODE, true, false, false, TO, TN, TENSOR, MX, false, KSPLIT>), grid, block, 0, stream, p, bias_dtype);
+    else if (!a5 && b5) VIOLA_LAUNCH((group_gemm_fast<MODE, false, true, false, TO, TN, TENSOR, MX, false, KSPLIT>), grid, block, 0, stream, p, bias_dtype);
+    else VIOLA_LAUNCH((group_gemm_fast<MODE, true, true, false, TO, TN, TENSOR, MX, false, KSPLIT>), grid, block, 0, stream, p, bias_dtype);
 }
 
 // The 256 x 256 tile (one 512-thread block per CU) for products with at least two rounds of such tiles (8192 x 4096 x 1024: 52.9 us against 58.5; with fewer tiles the 128 x 128 kernel wins).
@@ -26,6 +28,9 @@ static void launch_big_formats(const GemmArgs& p, int a_dtype, int b_dtype, int 
     else VIOLA_LAUNCH((group_gemm_fast<MODE, true, true, false, TO, 2, TENSOR, MX, true>), grid, dim3(512), 0, stream, p, bias_dtype);
 }
 
+#ifndef VIOLA_SCALED_SPLIT_MIN_K
+#define VIOLA_SCALED_SPLIT_MIN_K 2048
+#endif
 #ifndef VIOLA_MX_BIG_GATED
 #define VIOLA_MX_BIG_GATED 0
 #endif
@@ -68,7 +73,12 @@ static int launch_scaled_gemm_fast(const GemmArgs& args, int mode, int a_dtype, 
         }
         return viola_launch_status();
     }
-    const bool narrow = mode == MODE_PLAIN && (int64_t)grid.x * grid.y < 512 && p.n > 64;
+    // fewer than 512 tiles of 128 x 128: over a long k keep the tile and split its k range inside the block (from 129
+    // tiles up, as for the grouped recipe), otherwise halve the tile in n
+    const int64_t tiles = (int64_t)grid.x * grid.y;
+    const bool few = mode == MODE_PLAIN && tiles < 512;
+    const bool split = few && tiles > 128 && p.k >= VIOLA_SCALED_SPLIT_MIN_K;
+    const bool narrow = few && !split && p.n > 64;
     if (narrow) grid.x = (unsigned)((p.n + 63) / 64);
     if ((int64_t)grid.x * grid.y < (1 << 30)) {
         p.tiles_n = (int)grid.x;
@@ -76,7 +86,8 @@ static int launch_scaled_gemm_fast(const GemmArgs& args, int mode, int a_dtype, 
         grid = dim3((grid.x * grid.y + 7) / 8 * 8, 1, 1);
     }
 #define VIOLA_SCALED(TO)                                                                                                        \
-    if (narrow) launch_scaled_formats<MODE_PLAIN, TO, 1, TENSOR, MX>(p, a_dtype, b_dtype, bias_dtype, grid, stream);             \
+    if (split) launch_scaled_formats<MODE_PLAIN, TO, 2, TENSOR, MX, true>(p, a_dtype, b_dtype, bias_dtype, grid, stream);        \
+    else if (narrow) launch_scaled_formats<MODE_PLAIN, TO, 1, TENSOR, MX>(p, a_dtype, b_dtype, bias_dtype, grid, stream);        \
     else if (mode == MODE_PLAIN) launch_scaled_formats<MODE_PLAIN, TO, 2, TENSOR, MX>(p, a_dtype, b_dtype, bias_dtype, grid, stream); \
     else if (mode == MODE_GATED_FWD) launch_scaled_formats<MODE_GATED_FWD, TO, 2, TENSOR, MX>(p, a_dtype, b_dtype, bias_dtype, grid, stream); \
     else launch_scaled_formats<MODE_GATED_BWD, TO, 2, TENSOR, MX>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
