@@ -664,7 +664,7 @@ __global__ __launch_bounds__(256, 8) void quantize_dual16_tile64(const TIn* __re
 
 // ------------------------------------------------------------------ column sums from 32-row partials
 // out[c] = sum over p of partial[p][c] in a fixed order: 8 threads per column each add a contiguous eighth of the
-// parts in ascending order (loads issued eight at a time), then the eighths are added in order.
+// parts in ascending order (loads issued 32 or eight at a time), then the eighths are added in order.
 template <typename TO>
 __global__ __launch_bounds__(256) void column_reduce_kernel(const float* __restrict__ partial, int64_t parts, int64_t cols,
                                                              TO* __restrict__ out) {
@@ -676,6 +676,13 @@ __global__ __launch_bounds__(256) void column_reduce_kernel(const float* __restr
     float sum = 0.0f;
     if (col < cols) {
         int64_t part = begin;
+        for (; part + 32 <= end; part += 32) {                              // same order of additions, four times the loads in flight
+            float v[32];
+#pragma unroll
+            for (int u = 0; u < 32; ++u) v[u] = partial[(part + u) * cols + col];
+#pragma unroll
+            for (int u = 0; u < 32; ++u) sum += v[u];
+        }
         for (; part + 8 <= end; part += 8) {
             float v[8];
 #pragma unroll
