@@ -70,16 +70,17 @@ def test_group_gemm_scales_past_the_k_range_do_not_leak(gb, k):
 
 
 @pytest.mark.parametrize("gb", [(1, 32), (32, 32)])
+@pytest.mark.parametrize("m,n", [(1930, 1100), (130, 200)])                  # 16 x 9 tiles of 128 x 128; 2 x 4 of 128 x 64
 @pytest.mark.parametrize("k,formats", [(2048, (E4, E4)), (2064, (E5, E4)), (2336, (E4, E4)), (4000, (E4, E5)), (6176, (E5, E5))])
-def test_group_gemm_long_k_few_tiles(k, formats, gb):
-    """A long k and 129 .. 511 output tiles of 128 x 128 (a weight gradient; a small-batch dgrad): the kernel splits the k
-    range of a tile over two teams of waves and adds their sums. k values around the split's granularity (256) and with a
-    ragged last scale piece; a NaN / Inf scale in a neighbouring row must stay in its row."""
+def test_group_gemm_long_k_few_tiles(k, formats, m, n, gb):
+    """A long k and fewer than 512 output tiles of 128 x 128 (a weight gradient; a small-batch dgrad): the kernel splits
+    the k range of a tile (128 x 128 from 129 tiles up, 128 x 64 below) over two teams of waves and adds their sums. k
+    values around the split's granularity (256) and with a ragged last scale piece; a NaN / Inf scale in a neighbouring
+    row must stay in its row."""
     from viola_amd.nn import _grouped_kernels as g
-    m, n = 1930, 1100                                                         # 16 x 9 tiles, ragged in both directions
     (qa, sa), (qb, sb) = _operands(m, k, n, (1, 32), gb, *formats, seed=k, spread=2)    # sums stay inside fp16
     bias = torch.randn(n)
-    rows = torch.cat([torch.arange(0, 140), torch.arange(1900, m)])           # the oracle on row samples: first tiles and the ragged last
+    rows = torch.cat([torch.arange(0, min(m, 140)), torch.arange(min(m, 1900), m)])   # the oracle on row samples: first tiles and the ragged last
     expected = og.gemm(qa[rows], qb, sa[rows], sb, (1, 32), gb, bias=bias, witness=True, out_dtype=torch.float64)
     qa, sa, qb, sb = qa.cuda(), sa.cuda(), qb.cuda(), sb.cuda()
     for out_dtype, bound in ((torch.float32, 2e-5), (torch.bfloat16, 3e-3), (torch.float16, 1e-3)):

@@ -14,12 +14,13 @@ static void launch_formats(const GemmArgs& p, int a_dtype, int b_dtype, int bias
     else VIOLA_LAUNCH((group_gemm_fast<MODE, true, true, B_ROWSCALE, TO, TN, false, false, false, KSPLIT>), grid, block, 0, stream, p, bias_dtype);
 }
 
-// plain mode, the k range of a 128 x 128 tile split over two teams of waves
+// plain mode, the k range of a tile split over two teams of waves
+template <int TN>
 static int launch_split(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, bool rowscale, dim3 grid,
                         hipStream_t stream) {
-#define VIOLA_SPLIT(TO)                                                                                        \
-    if (rowscale) launch_formats<MODE_PLAIN, true, TO, 2, true>(p, a_dtype, b_dtype, bias_dtype, grid, stream); \
-    else launch_formats<MODE_PLAIN, false, TO, 2, true>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
+#define VIOLA_SPLIT(TO)                                                                                         \
+    if (rowscale) launch_formats<MODE_PLAIN, true, TO, TN, true>(p, a_dtype, b_dtype, bias_dtype, grid, stream); \
+    else launch_formats<MODE_PLAIN, false, TO, TN, true>(p, a_dtype, b_dtype, bias_dtype, grid, stream);
     switch (out_dtype) {
         case VIOLA_F32: VIOLA_SPLIT(float) break;
         case VIOLA_BF16: VIOLA_SPLIT(bf16_t) break;
@@ -60,10 +61,13 @@ int launch_group_gemm_fast(const GemmArgs& args, int mode, int a_dtype, int b_dt
     p.sb_bytes = (b_rows + p.br - 1) / p.br * p.ldsb * 4;
     // Two blocks fit a CU: with fewer than 512 tiles of 128 x 128, halve the tile in n so that all 256 CUs get two.
     // Over a long k, and with enough tiles to give half the CUs one each, keep the tile instead and split its k range inside
-    // the block (one block of twice the waves per CU): 7-12 % faster from 256 tiles up, slower at 64 (half as many CUs busy).
+    // the block (one block of twice the waves per CU): 7-12 % faster from 256 tiles up. With 128 tiles or fewer the
+    // narrow tiles stay (more CUs busy) and their k range is split: a CU then holds eight waves instead of four
+    // (1024 x 1024 x 16384: 98 -> 76 us, 512 x 512 x 4096: 27.5 -> 22.3 us).
     const int64_t tiles = (int64_t)grid.x * grid.y * grid.z;
     const bool few = mode == MODE_PLAIN && tiles < 512;
-    const bool split = few && tiles > 128 && !p.offsets && !p.koffsets && p.k >= SPLIT_MIN_K;
+    const bool long_k = !p.offsets && !p.koffsets && p.k >= SPLIT_MIN_K;
+    const bool split = few && tiles > 128 && long_k;
     const bool narrow = few && !split && p.n > 64;
     if (narrow) grid.x = (unsigned)((p.n + 63) / 64);
     if (!p.offsets && (int64_t)grid.x * grid.y < (1 << 30)) {
@@ -71,7 +75,8 @@ int launch_group_gemm_fast(const GemmArgs& args, int mode, int a_dtype, int b_dt
         p.tiles_m = (int)grid.y;
         grid = dim3((grid.x * grid.y + 7) / 8 * 8, 1, grid.z);
     }
-    if (split) return launch_split(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
+    if (split) return launch_split<2>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
+    if (narrow && long_k) return launch_split<1>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
     if (narrow) return launch_mode<MODE_PLAIN, 1>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
     if (mode == MODE_PLAIN) return launch_mode<MODE_PLAIN, 2>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
     if (mode == MODE_GATED_FWD) return launch_mode<MODE_GATED_FWD, 2>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);

@@ -134,7 +134,7 @@ constexpr int MX_GROUPS = 16, MX_CHUNKS = MX_GROUPS / FKG, MX_BLOCK = 2 * BM * M
 template <int MODE, bool A_BF8, bool B_BF8, bool B_ROWSCALE, typename TO, int TN, bool TENSOR = false, bool MX = false, bool BIG = false,
           bool KSPLIT = false>
 __global__ __launch_bounds__(BIG || KSPLIT ? 512 : FTHREADS, BIG || KSPLIT ? 1 : TENSOR ? 3 : 2) void group_gemm_fast(GemmArgs p, int bias_dtype) {
-    static_assert(!KSPLIT || (MODE == MODE_PLAIN && TN == 2 && !BIG), "the split exists for plain products on 128 x 128 tiles");
+    static_assert(!KSPLIT || (MODE == MODE_PLAIN && !BIG), "the split exists for plain products on the small tiles");
     static_assert(!TENSOR || !B_ROWSCALE, "per-tensor scaling has no row scales");
     static_assert(!MX || !TENSOR, "one scaling recipe per kernel");
     static_assert(!BIG || ((TENSOR || MX) && TN == 2), "the large tile exists for the fold-free kernels");

@@ -73,11 +73,12 @@ static int launch_scaled_gemm_fast(const GemmArgs& args, int mode, int a_dtype, 
         }
         return viola_launch_status();
     }
-    // fewer than 512 tiles of 128 x 128: over a long k keep the tile and split its k range inside the block (from 129
-    // tiles up, as for the grouped recipe), otherwise halve the tile in n
+    // fewer than 512 tiles of 128 x 128: halve the tile in n, or from 129 tiles up and over a long k keep the tile and
+    // split its k range inside the block; the narrow tiles split a long k range as well (the grouped recipe's rule)
     const int64_t tiles = (int64_t)grid.x * grid.y;
     const bool few = mode == MODE_PLAIN && tiles < 512;
-    const bool split = few && tiles > 128 && p.k >= VIOLA_SCALED_SPLIT_MIN_K;
+    const bool long_k = p.k >= VIOLA_SCALED_SPLIT_MIN_K;
+    const bool split = few && tiles > 128 && long_k;
     const bool narrow = few && !split && p.n > 64;
     if (narrow) grid.x = (unsigned)((p.n + 63) / 64);
     if ((int64_t)grid.x * grid.y < (1 << 30)) {
@@ -87,6 +88,7 @@ static int launch_scaled_gemm_fast(const GemmArgs& args, int mode, int a_dtype, 
     }
 #define VIOLA_SCALED(TO)                                                                                                        \
     if (split) launch_scaled_formats<MODE_PLAIN, TO, 2, TENSOR, MX, true>(p, a_dtype, b_dtype, bias_dtype, grid, stream);        \
+    else if (narrow && long_k) launch_scaled_formats<MODE_PLAIN, TO, 1, TENSOR, MX, true>(p, a_dtype, b_dtype, bias_dtype, grid, stream); \
     else if (narrow) launch_scaled_formats<MODE_PLAIN, TO, 1, TENSOR, MX>(p, a_dtype, b_dtype, bias_dtype, grid, stream);        \
     else if (mode == MODE_PLAIN) launch_scaled_formats<MODE_PLAIN, TO, 2, TENSOR, MX>(p, a_dtype, b_dtype, bias_dtype, grid, stream); \
     else if (mode == MODE_GATED_FWD) launch_scaled_formats<MODE_GATED_FWD, TO, 2, TENSOR, MX>(p, a_dtype, b_dtype, bias_dtype, grid, stream); \
