@@ -277,14 +277,18 @@ def test_varlen_group_gemm_and_wgrad(counts):
             assert wparam.grad[g].count_nonzero() == 0
 
 
-@pytest.mark.parametrize("counts", [[130, 0, 3, 64, 1, 200], [31, 33]])
+@pytest.mark.parametrize("counts", [[130, 0, 3, 64, 1, 200], [31, 33], [96, 64, 0, 160, 7]])
+@pytest.mark.parametrize("cols", [136, 192])                                # rows of codes not / all 16-byte aligned
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
-def test_varlen_segmented_quantizer_rowwise_byproduct(counts, dtype):
+def test_varlen_segmented_quantizer_rowwise_byproduct(counts, cols, dtype):
     """The segmented transposed quantizer can emit the plain row-wise codes from the same read: both outputs must be the
-    ones the separate kernels give."""
+    ones the separate kernels give. Groups that fill whole 64-token tiles and groups that end inside one; a NaN and an Inf
+    send their wavefronts down the exact route."""
     from viola_amd.nn import _varlen as v, _grouped_kernels as g
     torch.manual_seed(12)
-    x = (torch.randn(sum(counts), 136) * 3).to(dtype).cuda()
+    x = (torch.randn(sum(counts), cols) * 3).to(dtype)
+    x[counts[0] // 2, 5], x[sum(counts) - 1, cols - 3] = float("nan"), float("inf")
+    x = x.cuda()
     offsets, padded, offsets_dev, padded_dev = v._offsets(counts, x.device)
     qt, st = v.quantize_transposed_segmented(x, E4, offsets_dev, padded_dev, len(counts), padded[-1])
     qt2, st2, q, s = v.quantize_transposed_segmented(x, E4, offsets_dev, padded_dev, len(counts), padded[-1], rowwise=True)
@@ -298,4 +302,7 @@ def test_varlen_segmented_quantizer_rowwise_byproduct(counts, dtype):
             got = qt[:, padded[group]:padded[group] + count].cpu().view(torch.uint8)
             assert torch.equal(got, oq.view(torch.uint8))
             assert torch.equal(st[:, padded[group] // 32:padded[group] // 32 + (count + 31) // 32].cpu(), os_)
+        # the padding behind a group's rows (to 32 tokens, and to 128 at the very end) holds zero codes
+        assert qt[:, padded[group] + count:padded[group + 1]].view(torch.uint8).count_nonzero() == 0
+    assert padded[-1] % 128 == 0 and qt.shape == (cols, padded[-1])
 

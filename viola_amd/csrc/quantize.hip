@@ -909,106 +909,164 @@ __global__ __launch_bounds__(64) void quantize_transposed_segmented(const TIn* _
     store_group32<TOut>(v, s, poison, limit, dst, 32, (reinterpret_cast<uintptr_t>(dst) & 15) == 0);
 }
 
-// 16-bit inputs: the same wavefront tile as quantize_dual16 over one 32-token slot x 64 columns, with the slot's rows
-// taken from its group (rows past the group's end read as zero) and, optionally, the row-wise layout of the valid rows
-// written in the same pass (q [rows, cols], scale [rows, ceil(cols/32)] in the unpadded row order).
-template <typename TIn, typename TOut, bool ROWWISE>
-__global__ __launch_bounds__(256) void quantize_segmented16(const TIn* __restrict__ x, const int64_t* __restrict__ offsets,
-                                                             const int64_t* __restrict__ poffsets, int groups, int64_t cols,
-                                                             int64_t t_total, uint8_t* __restrict__ qt, float* __restrict__ scale_t,
-                                                             uint8_t* __restrict__ q, float* __restrict__ scale, float limit) {
-    constexpr int LD = 64 + 32;
-    typedef short s16x4 __attribute__((ext_vector_type(4)));
-    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-    __shared__ __attribute__((aligned(16))) uint16_t park[4][32 * LD];
-    const int lane = threadIdx.x % WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);   // uniform: so is the buffer descriptor
-    uint16_t* mine = park[wave];
-    const int lr = lane / 8, ch = lane % 8;
-    const int64_t nc = (cols + 31) / 32;
-    const int64_t tiles_x = (cols + 63) / 64, slots = t_total / 32;
-    // a block takes four consecutive slots of one column tile, one per wavefront: their 32-byte runs of transposed
-    // codes are the four quarters of 128-byte lines (see quantize_dual16)
-    const int64_t first_slot = (int64_t)blockIdx.x / tiles_x * 4, slot = first_slot + wave, c0 = (int64_t)blockIdx.x % tiles_x * 64;
-    const bool active = slot < slots;                                        // a wavefront past the last slot reads zeros and stores nothing
-    const int64_t token = slot * 32;
-    int g = 0;
-    while (g + 1 < groups && poffsets[g + 1] <= token) ++g;
-    const int64_t first = offsets[g] + (token - poffsets[g]);
-    const int64_t left = offsets[g + 1] - first;                               // valid rows of this slot (may be <= 0)
-    const int valid = !active ? 0 : (int)(left < 0 ? 0 : left > 32 ? 32 : left);
-    const int64_t col8 = c0 + ch * 8;
+// 16-bit inputs: the 64 x 64 tile of quantize_dual16_tile64 over the padded token axis. A block takes two consecutive
+// 32-token slots of one column tile, each with its own group, first row and count of valid rows (rows past a group's end
+// are parked as zeros), so the transposed codes of a tile are again 64 consecutive bytes per column; optionally the
+// row-wise layout of the valid rows is written in the same pass (q [rows, cols], scale [rows, ceil(cols/32)] in the
+// unpadded row order). FP32 scales. (32768 x 4096 and x 1024 bf16, 16 groups, both layouts: 146 and 28.5 us against
+// 158 and 33 us for a kernel of one slot per wavefront; the plain dual-layout kernel takes 135 and 23.4 us.)
+// INTERIOR: both slots hold 32 valid rows, the tile lies inside the matrix and every 16-byte piece of either output is
+// aligned: no bounds checks, base pointers in scalar registers with 32-bit offsets per lane.
+template <typename TIn, typename TOut, bool ROWWISE, bool INTERIOR>
+__device__ __forceinline__ void segmented16_tile64(const TIn* __restrict__ x, int64_t cols, int64_t t_total, uint8_t* __restrict__ qt,
+                                                   float* __restrict__ scale_t, uint8_t* __restrict__ q, float* __restrict__ scale,
+                                                   float limit, int64_t pair, int64_t c0, const int64_t (&first)[2], const int (&valid)[2],
+                                                   uint16_t* park, int* flags) {
+    constexpr int LDV = 64 + 4;
+    const int tid = threadIdx.x, lane = tid % WAVE, wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+    const int64_t nc = (cols + 31) / 32, slots = t_total / 32;
+    const bool clamp_free = limit == fp8_traits<TOut>::max;
 
-    const __amdgpu_buffer_rsrc_t res = __builtin_amdgcn_make_buffer_rsrc(const_cast<TIn*>(x + first * cols), 0, (int)(valid * cols * 2), 0x00020000);
-    u32x4 raw[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-        raw[i] = __builtin_amdgcn_raw_buffer_load_b128(res, col8 < cols ? (int)(((lr + 8 * i) * cols + col8) * 2) : (int)0x80000000u, 0, 0);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(&mine[(lr + 8 * i) * LD + ch * 8]) = raw[i];
-
-    if constexpr (ROWWISE) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float v[8];
-            float amax = 0.0f, poison = 0.0f;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                v[e] = widen16<TIn>(e % 2 ? raw[i][e / 2] >> 16 : raw[i][e / 2] & 0xffffu);
-                amax = fmaxf(amax, fabsf(v[e]));
-                poison = poison_of(poison, v[e]);
-            }
-            amax = group_max<4>(amax);
-            poison += quad_xor<1>(poison);
-            poison += quad_xor<2>(poison);
-            const float s = group_scale(amax, limit);
-            const SharedDivisor divisor(s, poison);
-            const uint2 codes = encode8<TOut>(v, s, limit, divisor);
-            const int r = lr + 8 * i;
-            if (r < valid && col8 < cols) {
-                *reinterpret_cast<uint2*>(q + (first + r) * cols + col8) = codes;
-                if (ch % 4 == 0) scale[(first + r) * nc + col8 / 32] = s;
-            }
+    // ---- row-wise: thread (tile row tid / 4, 16 columns); wavefronts 0, 1 hold the first slot's rows, 2, 3 the second's
+    {
+        const int lr = tid / 4, lc = (tid % 4) * 16, half = wave / 2, in_slot = lr % 32;
+        const int64_t slot_first = half ? first[1] : first[0];
+        const bool live = INTERIOR || in_slot < (half ? valid[1] : valid[0]);
+        const int64_t row = slot_first + in_slot, col = c0 + lc;
+        const uint32_t offset = (uint32_t)in_slot * (uint32_t)cols + (uint32_t)lc;   // from the slot's first element of the tile
+        uint4 raw[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+        if constexpr (INTERIOR) {
+            const TIn* tile = x + slot_first * cols + c0;
+            raw[0] = *reinterpret_cast<const uint4*>(tile + offset);
+            raw[1] = *reinterpret_cast<const uint4*>(tile + offset + 8);
+        } else if (live) {
+            if (col < cols) raw[0] = *reinterpret_cast<const uint4*>(x + row * cols + col);      // cols % 8 == 0: whole pieces
+            if (col + 8 < cols) raw[1] = *reinterpret_cast<const uint4*>(x + row * cols + col + 8);
         }
-    }
-    const int64_t col = c0 + lane;
-    const int strip = (lane / 16) * 16, sub = lane & 15;
-    const uint16_t* at = &mine[(sub >> 2) * LD + strip + 4 * (sub & 3)];
-    float vc[32];
-    float amax = 0.0f, poison = 0.0f;
-#pragma unroll
-    for (int t = 0; t < 8; ++t) {
-        const s16x4 four = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at + 4 * t * LD));
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            vc[4 * t + e] = widen16<TIn>((uint16_t)four[e]);
-            amax = fmaxf(amax, fabsf(vc[4 * t + e]));
-            poison = poison_of(poison, vc[4 * t + e]);
+        {
+            uint2* mine = reinterpret_cast<uint2*>(&park[lr * LDV + (lc ^ (((lr >> 4) & 3) << 4))]);
+            mine[0] = make_uint2(raw[0].x, raw[0].y); mine[1] = make_uint2(raw[0].z, raw[0].w);
+            mine[2] = make_uint2(raw[1].x, raw[1].y); mine[3] = make_uint2(raw[1].z, raw[1].w);
         }
-    }
-    const float s = group_scale(amax, limit);
-    if (active && col < cols) scale_t[col * slots + slot] = s;
-    if ((reinterpret_cast<uintptr_t>(qt) & 15) != 0) {                        // (uniform) odd base: each wavefront stores its own runs
-        if (active && col < cols) store_group32<TOut>(vc, s, poison, limit, qt + col * t_total + token, 32, false);
-        return;
-    }
-    constexpr int XLD = 128 + 16;
-    __shared__ __attribute__((aligned(16))) uint8_t lines[64 * XLD];
-    if (active) {
-        uint32_t w[8];
-        encode_group32<TOut>(vc, s, poison, limit, w);
-        uint4* run = reinterpret_cast<uint4*>(&lines[lane * XLD + wave * 32]);
-        run[0] = make_uint4(w[0], w[1], w[2], w[3]);
-        run[1] = make_uint4(w[4], w[5], w[6], w[7]);
+        const uint32_t words[8] = {raw[0].x, raw[0].y, raw[0].z, raw[0].w, raw[1].x, raw[1].y, raw[1].z, raw[1].w};
+        bool nonfinite;
+        if constexpr (ROWWISE) {
+            float s_row;
+            uint32_t codes[4];
+            if (!encode_words16<TIn, TOut>(words, limit, 0, clamp_free, s_row, codes, nonfinite)) {
+                const Exact16 r = encode_words16_exact<TIn, TOut>(words[0], words[1], words[2], words[3], words[4], words[5], words[6], words[7], limit, 0);
+                codes[0] = r.c0; codes[1] = r.c1; codes[2] = r.c2; codes[3] = r.c3; s_row = r.s;
+            }
+            if constexpr (INTERIOR) {
+                *reinterpret_cast<uint4*>(q + slot_first * cols + c0 + offset) = make_uint4(codes[0], codes[1], codes[2], codes[3]);
+                if (tid % 2 == 0) (scale + slot_first * nc + c0 / 32)[(uint32_t)in_slot * (uint32_t)nc + (uint32_t)(lc / 32)] = s_row;
+            } else if (live && col < cols) {
+                uint8_t* dst = q + row * cols + col;
+                if (col + 16 <= cols && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+                    *reinterpret_cast<uint4*>(dst) = make_uint4(codes[0], codes[1], codes[2], codes[3]);
+                } else {
+                    *reinterpret_cast<uint2*>(dst) = make_uint2(codes[0], codes[1]);                 // q is 8-byte aligned, cols % 8 == 0
+                    if (col + 8 < cols) *reinterpret_cast<uint2*>(dst + 8) = make_uint2(codes[2], codes[3]);
+                }
+                if (tid % 2 == 0) scale[row * nc + col / 32] = s_row;
+            }
+        } else {
+            constexpr uint32_t MAGNITUDE = 0x7fff7fffu, INF16 = std::is_same<TIn, bf16_t>::value ? 0x7f80u : 0x7c00u;
+            uint32_t top = 0;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) top = pk_max_u16(top, words[e] & MAGNITUDE);
+            nonfinite = (top & 0xffffu) >= INF16 || (top >> 16) >= INF16;
+        }
+        const bool any_nonfinite = __builtin_amdgcn_ballot_w64(nonfinite) != 0;   // over the whole wavefront: outside any branch
+        if (lane == 0) flags[wave] = any_nonfinite;
     }
     __syncthreads();
+    const bool plain = (flags[0] | flags[1] | flags[2] | flags[3]) == 0;
+
+    // ---- transposed: wavefront w takes columns 16 w .. + 15; lane = (column lane / 4, tile rows 16 (lane % 4) .. + 15)
+    {
+        const int tc = wave * 16 + lane / 4, chunk = lane % 4;
+        const int64_t tcol = c0 + tc, token = pair * 64 + chunk * 16;
+        uint32_t bits[16];
 #pragma unroll
-    for (int it = 0; it < 2; ++it) {
-        const int id = it * 256 + (int)threadIdx.x, c = id >> 3, piece = id & 7;
-        const int64_t at_token = first_slot * 32 + piece * 16;               // t_total is a multiple of 32: whole pieces only
-        if (c0 + c < cols && at_token < t_total)
-            *reinterpret_cast<uint4*>(qt + (c0 + c) * t_total + at_token) = *reinterpret_cast<const uint4*>(&lines[c * XLD + piece * 16]);
+        for (int i = 0; i < 16; ++i) bits[i] = park[(chunk * 16 + i) * LDV + (tc ^ (chunk << 4))];
+        float w[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) w[i] = widen16<TIn>(bits[i]);
+        float s_col;
+        uint32_t tcodes[4];
+        if (!plain || !encode_finite16<TOut>(w, limit, 0, clamp_free, s_col, tcodes)) {
+            const Exact16 r = encode_words16_exact<TIn, TOut>(bits[0] | bits[1] << 16, bits[2] | bits[3] << 16, bits[4] | bits[5] << 16, bits[6] | bits[7] << 16,
+                                                              bits[8] | bits[9] << 16, bits[10] | bits[11] << 16, bits[12] | bits[13] << 16,
+                                                              bits[14] | bits[15] << 16, limit, 0);
+            tcodes[0] = r.c0; tcodes[1] = r.c1; tcodes[2] = r.c2; tcodes[3] = r.c3; s_col = r.s;
+        }
+        if constexpr (INTERIOR) {
+            *reinterpret_cast<uint4*>(qt + c0 * t_total + pair * 64 + ((uint32_t)tc * (uint32_t)t_total + (uint32_t)(chunk * 16))) = make_uint4(tcodes[0], tcodes[1], tcodes[2], tcodes[3]);
+            if (chunk % 2 == 0) (scale_t + c0 * slots + pair * 2)[(uint32_t)tc * (uint32_t)slots + (uint32_t)(chunk / 2)] = s_col;
+        } else if (tcol < cols && token < t_total) {                          // t_total is a multiple of 32: whole pieces only
+            uint8_t* dst = qt + tcol * t_total + token;
+            if ((reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+                *reinterpret_cast<uint4*>(dst) = make_uint4(tcodes[0], tcodes[1], tcodes[2], tcodes[3]);
+            } else {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) dst[4 * k + e] = (uint8_t)(tcodes[k] >> (8 * e));
+                }
+            }
+            if (chunk % 2 == 0) scale_t[tcol * slots + token / 32] = s_col;
+        }
     }
+}
+
+template <typename TIn, typename TOut, bool ROWWISE>
+__global__ __launch_bounds__(256, 8) void quantize_segmented16_tile64(const TIn* __restrict__ x, const int64_t* __restrict__ offsets,
+                                                                    const int64_t* __restrict__ poffsets, int groups, int64_t cols,
+                                                                    int64_t t_total, uint8_t* __restrict__ qt, float* __restrict__ scale_t,
+                                                                    uint8_t* __restrict__ q, float* __restrict__ scale, float limit, int aligned,
+                                                                    int xcd_walk) {
+    __shared__ __attribute__((aligned(16))) uint16_t park[64 * (64 + 4)];
+    __shared__ __attribute__((aligned(16))) int flags[4];
+    // the walk of quantize_dual16_tile64: blocks in flight together take 32 slot pairs of one column tile, then the next;
+    // with xcd_walk every XCD takes one contiguous eighth of it
+    constexpr uint32_t BAND = 32;
+    const int64_t slots = t_total / 32;
+    const uint32_t tiles_x = (uint32_t)((cols + 63) / 64), tiles_y = (uint32_t)((slots + 1) / 2), tiles = tiles_x * tiles_y;
+    uint32_t id = blockIdx.x;
+    if (xcd_walk) id = (id % 8) * ((tiles + 7) / 8) + id / 8;
+    if (id >= tiles) return;
+    const uint32_t patch = id / (BAND * tiles_x), within = id % (BAND * tiles_x);
+    const uint32_t tall = tiles_y - patch * BAND < BAND ? tiles_y - patch * BAND : BAND;
+    const int64_t pair = patch * BAND + within % tall, c0 = (int64_t)(within / tall) * 64;
+    // The two slots' groups and rows (uniform). A slot's group is the number of entries of poffsets[1 .. groups - 1] that are
+    // <= its first token (the table is nondecreasing): 64 entries per load and ballot instead of a chain of dependent loads.
+    int64_t first[2];
+    int valid[2];
+    {
+        const int lane = threadIdx.x % WAVE;
+        const int64_t token0 = 2 * pair * 32, token1 = token0 + 32;
+        int g0 = 0, g1 = 0;
+        for (int base = 1; base < groups; base += WAVE) {
+            const int at = base + lane;
+            const int64_t start = at < groups ? poffsets[at] : INT64_MAX;
+            g0 += __popcll(__builtin_amdgcn_ballot_w64(start <= token0));
+            g1 += __popcll(__builtin_amdgcn_ballot_w64(start <= token1));
+        }
+        const int gs[2] = {g0, g1};
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int64_t token = h ? token1 : token0;
+            first[h] = offsets[gs[h]] + (token - poffsets[gs[h]]);
+            const int64_t left = offsets[gs[h] + 1] - first[h];
+            valid[h] = token >= t_total ? 0 : (int)(left < 0 ? 0 : left > 32 ? 32 : left);
+        }
+    }
+    // (32-bit offsets inside a slot: 32 rows x cols and 64 columns x t_total stay below 2^31, the launcher sees to it)
+    if (aligned && valid[0] == 32 && valid[1] == 32 && c0 + 64 <= cols)
+        segmented16_tile64<TIn, TOut, ROWWISE, true>(x, cols, t_total, qt, scale_t, q, scale, limit, pair, c0, first, valid, park, flags);
+    else
+        segmented16_tile64<TIn, TOut, ROWWISE, false>(x, cols, t_total, qt, scale_t, q, scale, limit, pair, c0, first, valid, park, flags);
 }
 
 // ------------------------------------------------------------------ host dispatch
@@ -1120,11 +1178,16 @@ static int launch_segmented(const void* x, int64_t cols, const int64_t* offsets,
                             int64_t t_total, void* qt, float* scale_t, void* q, float* scale, float limit, hipStream_t stream) {
     if constexpr (sizeof(TIn) == 2) {
         const bool aligned = cols % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && (!q || reinterpret_cast<uintptr_t>(q) % 8 == 0);
-        const int64_t blocks = ((t_total / 32 + 3) / 4) * ((cols + 63) / 64);   // four slots x one column tile each
-        if (aligned && blocks < (1ll << 31)) {
-            const dim3 grid16((unsigned)blocks);
-            if (q) VIOLA_LAUNCH((quantize_segmented16<TIn, TOut, true>), grid16, dim3(256), 0, stream, static_cast<const TIn*>(x), offsets, poffsets, groups, cols, t_total, static_cast<uint8_t*>(qt), scale_t, static_cast<uint8_t*>(q), scale, limit);
-            else VIOLA_LAUNCH((quantize_segmented16<TIn, TOut, false>), grid16, dim3(256), 0, stream, static_cast<const TIn*>(x), offsets, poffsets, groups, cols, t_total, static_cast<uint8_t*>(qt), scale_t, nullptr, nullptr, limit);
+        const int64_t tiles64 = ((t_total / 32 + 1) / 2) * ((cols + 63) / 64);   // two slots x one column tile each
+        if (aligned && tiles64 + 8 < (1ll << 31)) {
+            const dim3 grid64((unsigned)((tiles64 + 7) / 8 * 8));
+            // an eighth of the walk per XCD pays for launches of this size (8272 tiles: 31.4 -> 28.5 us; 33088 tiles: 146 -> 156 us)
+            const int xcd_walk = tiles64 >= 2048 && tiles64 <= 16384;
+            // every 16-byte piece of the outputs aligned, 32-bit offsets inside a tile
+            const int interior = cols % 16 == 0 && reinterpret_cast<uintptr_t>(qt) % 16 == 0 && (!q || reinterpret_cast<uintptr_t>(q) % 16 == 0) &&
+                                 cols < (1 << 24) && t_total < (1 << 24);
+            if (q) VIOLA_LAUNCH((quantize_segmented16_tile64<TIn, TOut, true>), grid64, dim3(256), 0, stream, static_cast<const TIn*>(x), offsets, poffsets, groups, cols, t_total, static_cast<uint8_t*>(qt), scale_t, static_cast<uint8_t*>(q), scale, limit, interior, xcd_walk);
+            else VIOLA_LAUNCH((quantize_segmented16_tile64<TIn, TOut, false>), grid64, dim3(256), 0, stream, static_cast<const TIn*>(x), offsets, poffsets, groups, cols, t_total, static_cast<uint8_t*>(qt), scale_t, nullptr, nullptr, limit, interior, xcd_walk);
             return viola_launch_status();
         }
     }

@@ -29,6 +29,9 @@ def _offsets(counts, device):
     for c in counts:
         offsets.append(offsets[-1] + c)
         padded.append(padded[-1] + (c + 31) // 32 * 32)
+    # The padded token axis is the row length of the transposed codes: rounded up to 128 (empty slots at the end of the
+    # last group, zero codes) so that every row starts on a cache line and the quantizer's 64-byte pieces never straddle one.
+    padded[-1] = (padded[-1] + 127) // 128 * 128
     both = torch.tensor([offsets, padded], dtype=torch.int64).to(device, non_blocking=True)
     return offsets, padded, both[0], both[1]
 
