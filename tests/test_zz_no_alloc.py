@@ -3,6 +3,8 @@ kernels as viola_ns_prepare with the partial sums in an array built into the lib
 viola_ns_prepare's bit for bit: on two calls in a row, the second on a smaller input (the array keeps the first
 call's contents), for both working dtypes and the tall (transposed) case; sizes beyond the array are rejected."""
 
+import gc
+
 import pytest
 import torch
 
@@ -54,13 +56,19 @@ def test_static_scratch_prepare_allocates_nothing_and_matches_the_oracle(dtype):
     matrices = [torch.randn(28, 192, 576, device="cuda"), torch.randn(3, 96, 40, device="cuda") * 1e-3]
     outs = [torch.empty(m.shape[0], min(m.shape[1:]), max(m.shape[1:]), device="cuda", dtype=dtype) for m in matrices]
     host = [m.cpu() for m in matrices]
-    torch.cuda.synchronize()
-    before = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), _device_free_bytes())
-    for _ in range(3):
-        for matrix, out in zip(matrices, outs):
-            _lib.call("viola_ns_prepare_static", _lib.ptr(matrix), _lib.F32, _lib.ptr(out), _lib.code(dtype), *matrix.shape)
-    torch.cuda.synchronize()
-    after = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), _device_free_bytes())
+    # tensors that earlier tests left in reference cycles must not be collected (and freed) between the two readings
+    gc.collect()
+    gc.disable()
+    try:
+        torch.cuda.synchronize()
+        before = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), _device_free_bytes())
+        for _ in range(3):
+            for matrix, out in zip(matrices, outs):
+                _lib.call("viola_ns_prepare_static", _lib.ptr(matrix), _lib.F32, _lib.ptr(out), _lib.code(dtype), *matrix.shape)
+        torch.cuda.synchronize()
+        after = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), _device_free_bytes())
+    finally:
+        gc.enable()
     assert after == before, (before, after)
     ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
     for matrix, out in zip(host, outs):
