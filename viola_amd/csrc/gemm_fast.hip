@@ -47,10 +47,9 @@ static int launch_mode(const GemmArgs& p, int a_dtype, int b_dtype, int bias_dty
     return viola_launch_status();
 }
 
-#ifndef VIOLA_SPLIT_MIN_K
-#define VIOLA_SPLIT_MIN_K 2048
-#endif
-constexpr int64_t SPLIT_MIN_K = VIOLA_SPLIT_MIN_K;
+// shortest k ranges worth splitting (4096 x 1024 tiles of 128 x 128: k = 1024 14.4 -> 15.1 us, k = 1536 17.7 -> 17.1 us; 1024 x 1024
+// on 128 x 64 tiles: k = 512 slower, k = 1024 9.8 -> 9.1 us, k = 1536 12.6 -> 11.1 us)
+constexpr int64_t SPLIT_MIN_K = 1536, NARROW_SPLIT_MIN_K = 1024;
 
 
 int launch_group_gemm_fast(const GemmArgs& args, int mode, int a_dtype, int b_dtype, int bias_dtype, int out_dtype, bool rowscale,
@@ -61,13 +60,13 @@ int launch_group_gemm_fast(const GemmArgs& args, int mode, int a_dtype, int b_dt
     p.sb_bytes = (b_rows + p.br - 1) / p.br * p.ldsb * 4;
     // Two blocks fit a CU: with fewer than 512 tiles of 128 x 128, halve the tile in n so that all 256 CUs get two.
     // Over a long k, and with enough tiles to give half the CUs one each, keep the tile instead and split its k range inside
-    // the block (one block of twice the waves per CU): 7-12 % faster from 256 tiles up. With 128 tiles or fewer the
+    // the block (one block of twice the waves per CU): 7-12 % faster from 256 tiles up at k >= 2048. With 128 tiles or fewer the
     // narrow tiles stay (more CUs busy) and their k range is split: a CU then holds eight waves instead of four
     // (1024 x 1024 x 16384: 98 -> 76 us, 512 x 512 x 4096: 27.5 -> 22.3 us).
     const int64_t tiles = (int64_t)grid.x * grid.y * grid.z;
     const bool few = mode == MODE_PLAIN && tiles < 512;
-    const bool long_k = !p.offsets && !p.koffsets && p.k >= SPLIT_MIN_K;
-    const bool split = few && tiles > 128 && long_k;
+    const bool fixed_k = !p.offsets && !p.koffsets;
+    const bool split = few && tiles > 128 && fixed_k && p.k >= SPLIT_MIN_K;
     const bool narrow = few && !split && p.n > 64;
     if (narrow) grid.x = (unsigned)((p.n + 63) / 64);
     if (!p.offsets && (int64_t)grid.x * grid.y < (1 << 30)) {
@@ -76,7 +75,7 @@ int launch_group_gemm_fast(const GemmArgs& args, int mode, int a_dtype, int b_dt
         grid = dim3((grid.x * grid.y + 7) / 8 * 8, 1, grid.z);
     }
     if (split) return launch_split<2>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
-    if (narrow && long_k) return launch_split<1>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
+    if (narrow && fixed_k && p.k >= NARROW_SPLIT_MIN_K) return launch_split<1>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
     if (narrow) return launch_mode<MODE_PLAIN, 1>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
     if (mode == MODE_PLAIN) return launch_mode<MODE_PLAIN, 2>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
     if (mode == MODE_GATED_FWD) return launch_mode<MODE_GATED_FWD, 2>(p, a_dtype, b_dtype, bias_dtype, out_dtype, rowscale, grid, stream);
